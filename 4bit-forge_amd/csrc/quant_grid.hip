@@ -1,0 +1,295 @@
+// Group scale/zero search: min/max grid and MSE (Lp) shrink search.
+//
+// Arithmetic follows forge/backend/cuda/quant_grid.cu:42-183 of the reference: the same
+// fp32 formulas, the same first-strict-minimum rule and the same summation tree for the
+// candidate loss (32 partial sums of gs/32 elements each, then a halving tree), so that
+// only the hardware log2/exp2 approximations can make a near-tie resolve differently.
+//
+// Mapping to CDNA4: the min/max kernel is HBM-bound and gives half a wavefront to each
+// group (coalesced 128 B rows); the shrink search is VALU/transcendental-bound and gives
+// one LANE to each group: all gs values sit in that lane's registers, the P candidates
+// are evaluated without any cross-lane traffic, and the per-candidate scalar work
+// (scale, reciprocal, zero point) is paid once per group instead of once per lane.
+#include "common.h"
+#include <hip/hip_bf16.h>
+
+namespace {
+
+constexpr float kEps = 1e-12f;
+
+__device__ __forceinline__ float ld_as_f32(const float* p) { return *p; }
+__device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
+    return __uint_as_float(static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(p)) << 16);
+}
+
+__device__ __forceinline__ float clampf(float v, float lo, float hi) {
+    return fminf(fmaxf(v, lo), hi);
+}
+
+// Scale and zero of one group from its extrema (quant_grid.cu:74-97).
+__device__ __forceinline__ void meta_from_extrema(float xmin, float xmax, float maxq,
+                                                  bool symmetric, float& s, float& q0) {
+    if (symmetric) {
+        float amax = fmaxf(fabsf(xmin), fabsf(xmax));
+        s = __builtin_fmaf(2.0f / maxq, amax, kEps);
+        q0 = 0.5f * (maxq + 1.0f);
+    } else {
+        s = (xmax - xmin) / maxq + kEps;
+        q0 = clampf(__builtin_rintf(-xmin / s), 0.0f, maxq);
+    }
+}
+
+// ---------------------------------------------------------------- min/max grid
+// One half-wavefront (32 lanes) per group.  Group `g` of the flattened [batch*R*G] list
+// covers columns [grp*gs, grp*gs+gs) of row r, columns >= C read as zero.
+template <typename T>
+__global__ __launch_bounds__(256) void minmax_grid_kernel(
+    const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t gs,
+    int64_t G, int64_t n_groups, float maxq, bool symmetric, float* __restrict__ scales,
+    float* __restrict__ qzeros) {
+    const int lane = threadIdx.x & 31;
+    const int64_t half = (int64_t)blockIdx.x * (blockDim.x >> 5) + (threadIdx.x >> 5);
+    const int64_t stride = (int64_t)gridDim.x * (blockDim.x >> 5);
+    for (int64_t g = half; g < n_groups; g += stride) {
+        const int64_t b = g / (R * G);
+        const int64_t rg = g - b * R * G;
+        const int64_t r = rg / G, grp = rg - r * G;
+        const T* row = W + b * w_stride + r * ldw;
+        const int64_t c0 = grp * gs;
+        float lo = 1e30f, hi = -1e30f;
+        for (int64_t i = lane; i < gs; i += 32) {
+            const int64_t c = c0 + i;
+            const float v = (c < C) ? ld_as_f32(row + c) : 0.0f;
+            hi = fmaxf(hi, v);
+            lo = fminf(lo, v);
+        }
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) {
+            hi = fmaxf(hi, __shfl_down(hi, off, 32));
+            lo = fminf(lo, __shfl_down(lo, off, 32));
+        }
+        if (lane == 0) {
+            float s, q0;
+            meta_from_extrema(lo, hi, maxq, symmetric, s, q0);
+            scales[g] = s;
+            qzeros[g] = q0;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- shrink search
+// |diff|^norm as exp2(norm*log2(.)) on the hardware transcendental units (v_log_f32,
+// v_exp_f32: 1 ulp each); mathematically the reference's __expf(__logf(e)*norm).
+__device__ __forceinline__ float pow_abs(float e, float norm) {
+    return __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(e) * norm);
+}
+
+template <int GS>
+__device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, float rcp,
+                                                float q0, float maxq, float norm) {
+    constexpr int VPL = GS / 32;
+    float part[32];
+#pragma unroll
+    for (int l = 0; l < 32; ++l) {
+        float loss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const float x = v[l + 32 * i];
+            const float q = clampf(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq);
+            const float diff = __builtin_fmaf(q - q0, s, -x);
+            const float e = fmaxf(fabsf(diff), 1e-20f);
+            loss += pow_abs(e, norm);
+        }
+        part[l] = loss;
+    }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+#pragma unroll
+        for (int l = 0; l < off; ++l) part[l] += part[l + off];
+    }
+    return part[0];
+}
+
+// One lane per group.  FUSED: derive (sg, q0g) from the group's own extrema first;
+// otherwise read them from scales/qzeros (the reference's two-call protocol).
+template <typename T, int GS, bool FUSED>
+__global__ __launch_bounds__(64) void mse_grid_kernel(
+    const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t G,
+    int64_t n_groups, const float* __restrict__ cand, int P, float maxq, float norm,
+    bool symmetric, bool search, float* __restrict__ scales, float* __restrict__ qzeros) {
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= n_groups) return;
+    const int64_t b = g / (R * G);
+    const int64_t rg = g - b * R * G;
+    const int64_t r = rg / G, grp = rg - r * G;
+    const T* src = W + b * w_stride + r * ldw + grp * GS;
+    const int64_t valid = (C - grp * GS) < GS ? (C - grp * GS) : GS;
+
+    float v[GS];
+    if (valid == GS && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+        constexpr int PER = 16 / sizeof(T);
+        const uint4* s4 = reinterpret_cast<const uint4*>(src);
+#pragma unroll
+        for (int i = 0; i < GS / PER; ++i) {
+            const uint4 w = s4[i];
+            if constexpr (sizeof(T) == 4) {
+                v[4 * i + 0] = __uint_as_float(w.x);
+                v[4 * i + 1] = __uint_as_float(w.y);
+                v[4 * i + 2] = __uint_as_float(w.z);
+                v[4 * i + 3] = __uint_as_float(w.w);
+            } else {
+                v[8 * i + 0] = __uint_as_float(w.x << 16);
+                v[8 * i + 1] = __uint_as_float(w.x & 0xffff0000u);
+                v[8 * i + 2] = __uint_as_float(w.y << 16);
+                v[8 * i + 3] = __uint_as_float(w.y & 0xffff0000u);
+                v[8 * i + 4] = __uint_as_float(w.z << 16);
+                v[8 * i + 5] = __uint_as_float(w.z & 0xffff0000u);
+                v[8 * i + 6] = __uint_as_float(w.w << 16);
+                v[8 * i + 7] = __uint_as_float(w.w & 0xffff0000u);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < GS; ++i) v[i] = (i < valid) ? ld_as_f32(src + i) : 0.0f;
+    }
+
+    float sg, q0g;
+    if constexpr (FUSED) {
+        float lo = 1e30f, hi = -1e30f;
+#pragma unroll
+        for (int i = 0; i < GS; ++i) {
+            hi = fmaxf(hi, v[i]);
+            lo = fminf(lo, v[i]);
+        }
+        meta_from_extrema(lo, hi, maxq, symmetric, sg, q0g);
+    } else {
+        sg = scales[g];
+        q0g = qzeros[g];
+    }
+
+    float best_s = sg, best_q = q0g;
+    if (search) {
+        const float xmin = symmetric ? 0.0f : -(sg * q0g);
+        float best_loss = 3.402823466e+38f;
+        for (int p = 0; p < P; ++p) {
+            const float s = sg * cand[p];
+            const float rcp = 1.0f / (s + kEps);
+            const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
+            const float loss = candidate_loss<GS>(v, s, rcp, q0, maxq, norm);
+            if (loss < best_loss) {
+                best_loss = loss;
+                best_s = s;
+                best_q = q0;
+            }
+        }
+    }
+    scales[g] = best_s;
+    qzeros[g] = best_q;
+}
+
+template <typename T, bool FUSED>
+int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t gs,
+               int64_t G, int64_t n_groups, const float* cand, int64_t P, float maxq, float norm,
+               bool symmetric, bool search, float* scales, float* qzeros, hipStream_t st) {
+    const dim3 block(64), grid((unsigned)forge::ceil_div(n_groups, 64));
+#define FORGE_MSE_CASE(GS)                                                                    \
+    case GS:                                                                                  \
+        mse_grid_kernel<T, GS, FUSED><<<grid, block, 0, st>>>(W, w_stride, R, C, ldw, G,      \
+                                                              n_groups, cand, (int)P, maxq,   \
+                                                              norm, symmetric, search, scales, \
+                                                              qzeros);                        \
+        break;
+    switch (gs) {
+        FORGE_MSE_CASE(32)
+        FORGE_MSE_CASE(64)
+        FORGE_MSE_CASE(128)
+        default:
+            return forge::fail(FORGE_ERR_INVALID, "Unsupported group_size=%lld (expected 32/64/128)",
+                               (long long)gs);
+    }
+#undef FORGE_MSE_CASE
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+int check_bits(int bits) {
+    FORGE_REQUIRE(bits >= 1 && bits <= 8, "bits=%d outside 1..8", bits);
+    return FORGE_OK;
+}
+
+}  // namespace
+
+extern "C" int forge_build_group_meta_packed(const float* X, int64_t RG, int64_t gs, int bits,
+                                             int symmetric, float* scales, float* qzeros,
+                                             forge_stream_t stream) {
+    if (int e = check_bits(bits)) return e;
+    FORGE_REQUIRE(RG >= 0 && gs >= 1, "bad shape RG=%lld gs=%lld", (long long)RG, (long long)gs);
+    FORGE_REQUIRE(RG == 0 || (X && scales && qzeros), "null pointer");
+    if (RG == 0) return FORGE_OK;
+    const float maxq = (float)((1 << bits) - 1);
+    const int64_t halves_per_block = 8;
+    int64_t blocks = forge::ceil_div(RG, halves_per_block);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        X, 0, RG, gs, gs, gs, 1, RG, maxq, symmetric != 0, scales, qzeros);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_mse_scale_groups_packed(const float* X, float* scales, float* qzeros,
+                                             const float* candidates, int64_t RG, int64_t gs,
+                                             int64_t P, float norm, int bits, int symmetric,
+                                             forge_stream_t stream) {
+    if (int e = check_bits(bits)) return e;
+    FORGE_REQUIRE(gs == 32 || gs == 64 || gs == 128,
+                  "Unsupported group_size=%lld (expected 32/64/128)", (long long)gs);
+    FORGE_REQUIRE(RG >= 0 && P >= 0 && P < (1 << 30), "bad shape RG=%lld P=%lld", (long long)RG,
+                  (long long)P);
+    FORGE_REQUIRE(RG == 0 || (X && scales && qzeros && (candidates || P == 0)), "null pointer");
+    if (RG == 0) return FORGE_OK;
+    const float maxq = (float)((1 << bits) - 1);
+    return launch_mse<float, false>(X, 0, RG, gs, gs, gs, 1, RG, candidates, P, maxq, norm,
+                                    symmetric != 0, true, scales, qzeros, (hipStream_t)stream);
+}
+
+extern "C" int forge_quant_grid(const void* W, int w_dtype, int64_t batch, int64_t w_stride,
+                                int64_t R, int64_t C, int64_t ldw, int64_t gs, int bits,
+                                int symmetric, int mse, const float* candidates, int64_t P,
+                                float norm, float* scales, float* qzeros,
+                                forge_stream_t stream) {
+    if (int e = check_bits(bits)) return e;
+    FORGE_REQUIRE(w_dtype == FORGE_F32 || w_dtype == FORGE_BF16, "w_dtype=%d", w_dtype);
+    FORGE_REQUIRE(batch >= 0 && R >= 0 && C >= 1 && ldw >= C && gs >= 1,
+                  "bad shape batch=%lld R=%lld C=%lld ldw=%lld gs=%lld", (long long)batch,
+                  (long long)R, (long long)C, (long long)ldw, (long long)gs);
+    FORGE_REQUIRE(!mse || P == 0 || candidates, "candidates is null");
+    const int64_t G = forge::ceil_div(C, gs);
+    const int64_t n_groups = batch * R * G;
+    if (n_groups == 0) return FORGE_OK;
+    FORGE_REQUIRE(W && scales && qzeros, "null pointer");
+    const float maxq = (float)((1 << bits) - 1);
+    hipStream_t st = (hipStream_t)stream;
+    if (mse) {
+        FORGE_REQUIRE(gs == 32 || gs == 64 || gs == 128,
+                      "Unsupported group_size=%lld (expected 32/64/128)", (long long)gs);
+        if (w_dtype == FORGE_F32)
+            return launch_mse<float, true>((const float*)W, w_stride, R, C, ldw, gs, G, n_groups,
+                                           candidates, P, maxq, norm, symmetric != 0, true, scales,
+                                           qzeros, st);
+        return launch_mse<__hip_bfloat16, true>((const __hip_bfloat16*)W, w_stride, R, C, ldw, gs,
+                                                G, n_groups, candidates, P, maxq, norm,
+                                                symmetric != 0, true, scales, qzeros, st);
+    }
+    int64_t blocks = forge::ceil_div(n_groups, 8);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    if (w_dtype == FORGE_F32)
+        minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(
+            (const float*)W, w_stride, R, C, ldw, gs, G, n_groups, maxq, symmetric != 0, scales,
+            qzeros);
+    else
+        minmax_grid_kernel<__hip_bfloat16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(
+            (const __hip_bfloat16*)W, w_stride, R, C, ldw, gs, G, n_groups, maxq, symmetric != 0,
+            scales, qzeros);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}

@@ -1,0 +1,444 @@
+// Blocked GPTQ column sweep (dense and 1:4 joint solve) for gfx950.
+//
+// Arithmetic follows forge/backend/cuda/solver.cu:9-154 and
+// forge/backend/cuda/solver_sparsegptq14.cu:12-200: per column quantise with
+// q = clamp(rint(fma(x, 1/(s+eps), q0))), deq = fma(q, s, -q0*s), err = x - deq, then
+// x[k] = fma(-U[t,k], err, x[k]) for every later column k.  Every element therefore
+// receives its rank-1 updates as ONE fp32 fma chain in ascending t.  The trailing update
+// keeps that exact chain: on gfx950 v_mfma_f32_32x32x2_f32 accumulates
+// acc = fma(a[k], b[k], acc) one k after the other in fp32, so a GEMM whose accumulator
+// is initialised with the current weights and whose K loop runs in ascending t gives the
+// same bits as the scalar chain, for any blocking.  Two kernels:
+//
+//   sweep_block_kernel   one lane per output row, BW consecutive columns of that row in
+//                        registers; the serial quantise/propagate chain (VALU).
+//   chain_gemm_kernel    X[m, n] <- chain_k fma(-U[k, m], E[k, n], X[m, n]) on the f32
+//                        MFMA pipe, 128x128 tiles staged through LDS.
+//
+// The host schedules them left-looking (batched experts: each column block is brought
+// up to date with ONE long-K GEMM over all earlier errors, so the weights stream through
+// HBM once) or right-looking (a single matrix: more tiles in flight per step).
+#include "common.h"
+
+namespace {
+
+constexpr float kEps = 1e-12f;
+#ifndef FORGE_SWEEP_BW
+#define FORGE_SWEEP_BW 128
+#endif
+constexpr int forge_kBW = FORGE_SWEEP_BW;  // columns per in-register block
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct SweepArgs {
+    float* A;              // [C,R] per matrix: x on entry; on exit err (batched form) or deq
+    float* B;              // [C,R] per matrix: receives err in the per-element form
+    const float* U;        // [C,C] per matrix, row-normalised upper factor
+    const float* scales;   // PER_ELEM: [C,R]; else [G,R]
+    const float* qzeros;
+    const int32_t* g_idx;  // [C] per matrix (group of solver column), !PER_ELEM only
+    uint8_t* q;            // [C,R] per matrix
+    uint32_t* M;           // [ceil(C/32),R] per matrix (sparse only)
+    const float* uinv;     // [C] per matrix (sparse only)
+    int64_t C, R, G;
+    int64_t c0;            // first column of this block
+    int bw;                // columns in this block (<= BW)
+    int maxq;
+};
+
+// 16 consecutive floats of a row of U, wave-uniform, fetched with one s_load_dwordx16
+// (viewing U through the constant address space makes the compiler use scalar loads;
+// valid because no kernel in this file writes the factor it reads).
+typedef float f32x16_a4 __attribute__((ext_vector_type(16), aligned(4)));
+__device__ __forceinline__ f32x16 load_u16(const float* p) {
+    typedef const __attribute__((address_space(4))) f32x16_a4* vptr;
+    return *(vptr)(p);
+}
+
+// Quantise one value (solver.cu:9-23): code, dequantised value and error.
+__device__ __forceinline__ void quantize_scalar(float x, float s, float q0, float maxq, float& qf,
+                                                float& deq, float& err) {
+    const float inv_s = 1.0f / (s + kEps);
+    qf = fminf(fmaxf(__builtin_rintf(__builtin_fmaf(x, inv_s, q0)), 0.0f), maxq);
+    deq = __builtin_fmaf(qf, s, -(q0 * s));
+    err = x - deq;
+}
+
+// One wavefront = 64 rows, one lane per row; the row's BW block columns live in x[].
+// The block is walked in sub-blocks of 32 columns: the serial quantise/propagate chain on
+// x[0..31], then those 32 errors are pushed into the block's remaining columns, then x[]
+// is shifted down by 32 so that the next sub-block again sits in x[0..31] (this keeps the
+// unrolled code at one sub-block's size).  U[t,k] is wave-uniform: each 16-wide row
+// segment is fetched with a scalar load one step ahead of its use and v_fma takes it as
+// an SGPR operand; scheduling barriers keep the compiler from hoisting all those loads to
+// the top (which would spill SGPRs).  Lanes past the last row leave at once: nothing
+// below communicates across lanes.  TAIL is the guarded, slower variant for a block that
+// is not a whole number of 32-column sub-blocks.
+template <int BW, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL>
+__global__ __launch_bounds__(64) void sweep_block_kernel(SweepArgs a) {
+    constexpr int SB = 32, NSB = BW / SB;
+    const int64_t r = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (r >= a.R) return;
+    const int64_t b = blockIdx.y;
+    const int64_t C = a.C, R = a.R;
+    float* __restrict__ A = a.A + b * C * R + r;
+    float* __restrict__ Bo = ERR_IN_A ? nullptr : a.B + b * C * R + r;
+    const float* __restrict__ U = a.U + b * C * C;
+    const float* __restrict__ sc = a.scales + b * (PER_ELEM ? C * R : a.G * R) + r;
+    const float* __restrict__ qz = a.qzeros + b * (PER_ELEM ? C * R : a.G * R) + r;
+    const int32_t* __restrict__ gi = PER_ELEM ? nullptr : a.g_idx + b * C;
+    const float* __restrict__ uinv = SPARSE ? a.uinv + b * C : nullptr;
+    uint32_t* __restrict__ Mw = SPARSE ? a.M + b * ((C + 31) / 32) * R + r : nullptr;
+    uint8_t* __restrict__ q = a.q + b * C * R + r;
+    const int bw = a.bw;
+    const int nsub = (bw + SB - 1) / SB;
+    const float maxq = (float)a.maxq;
+
+    float x[BW];
+#pragma unroll
+    for (int i = 0; i < BW; ++i) x[i] = (i < bw) ? A[(a.c0 + i) * R] : 0.0f;
+
+    for (int sb = 0; sb < nsub; ++sb) {
+        const int64_t cs = a.c0 + (int64_t)sb * SB;   // first column of this sub-block
+        const int rem = bw - sb * SB;                 // block columns from cs on
+        float err[SB];
+        uint32_t mask = 0u;
+
+        auto select_and_quantize = [&](int t, int64_t c) {
+            bool keep = true;
+            if constexpr (SPARSE) {
+                if ((t & 3) == 0) {
+                    float best = -1e30f;
+                    int best_k = -1;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (!TAIL || c + k < C) {
+                            const float score = fabsf(x[t + k] * uinv[c + k]);
+                            if (best < score) { best = score; best_k = k; }
+                        }
+                    }
+                    if (best_k > -1) mask |= 1u << (t + best_k);
+                }
+                keep = (mask >> t) & 1u;
+            }
+            float s, q0;
+            if constexpr (PER_ELEM) {
+                s = sc[c * R];
+                q0 = qz[c * R];
+            } else {
+                const int64_t g = gi[c];
+                s = sc[g * R];
+                q0 = qz[g * R];
+            }
+            float e, deq, qf;
+            quantize_scalar(x[t], s, q0, maxq, qf, deq, e);
+            if constexpr (SPARSE) {
+                // pruned column: code 0, weight 0, the whole value becomes the error
+                qf = keep ? qf : 0.0f;
+                deq = keep ? deq : 0.0f;
+                e = keep ? e : x[t];
+            }
+            err[t] = e;
+            q[c * R] = (uint8_t)qf;
+            if constexpr (ERR_IN_A) {
+                A[c * R] = e;
+            } else {
+                A[c * R] = deq;
+                Bo[c * R] = e;
+            }
+        };
+
+        if constexpr (!TAIL) {
+            // serial chain inside the sub-block; U row t = two 16-wide halves
+            f32x16 cur = load_u16(U + cs * C + cs);
+#pragma unroll
+            for (int t = 0; t < SB; ++t) {
+                const f32x16 hi = load_u16(U + (cs + t) * C + cs + 16);
+                select_and_quantize(t, cs + t);
+                if (t < 15) {
+#pragma unroll
+                    for (int k = t + 1; k < 16; ++k) x[k] = __builtin_fmaf(-cur[k], err[t], x[k]);
+                }
+                if (t + 1 < SB) cur = load_u16(U + (cs + t + 1) * C + cs);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int k = (t + 1 > 16 ? t + 1 : 16); k < SB; ++k)
+                    x[k] = __builtin_fmaf(-hi[k - 16], err[t], x[k]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (SPARSE) Mw[(cs >> 5) * R] = mask;
+            // push the 32 errors into the rest of the block, 16 columns of one U row a step
+#pragma unroll
+            for (int u = 1; u < NSB; ++u) {
+                if (sb + u < nsub) {
+                    const float* Ub = U + cs * C + cs + u * SB;
+                    f32x16 c2 = load_u16(Ub);
+#pragma unroll
+                    for (int step = 0; step < 2 * SB; ++step) {
+                        const int t = step >> 1, h = step & 1;
+                        f32x16 n2 = c2;
+                        if (step + 1 < 2 * SB)
+                            n2 = load_u16(Ub + (int64_t)((step + 1) >> 1) * C + ((step + 1) & 1) * 16);
+#pragma unroll
+                        for (int k = 0; k < 16; ++k)
+                            x[u * SB + h * 16 + k] =
+                                __builtin_fmaf(-c2[k], err[t], x[u * SB + h * 16 + k]);
+                        c2 = n2;
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        } else {
+#pragma unroll 1
+            for (int t = 0; t < SB; ++t) {
+                err[t] = 0.0f;
+                if (t < rem) {
+                    select_and_quantize(t, cs + t);
+                    const float* __restrict__ Urow = U + (cs + t) * C + cs;
+                    for (int k = t + 1; k < rem; ++k)
+                        x[k] = __builtin_fmaf(-Urow[k], err[t], x[k]);
+                }
+            }
+            if constexpr (SPARSE) Mw[(cs >> 5) * R] = mask;
+        }
+#pragma unroll
+        for (int i = 0; i + SB < BW; ++i) x[i] = x[i + SB];
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// X[m, n] <- chain_{k=k0..k1-1} fma(-At[k, m], Bm[k, n], X[m, n])   for m in [m0, m1)
+// Tile 128 (m) x 128 (n); 4 wavefronts, each a 64x64 quadrant = 2x2 MFMA 32x32 tiles.
+constexpr int TM = 128, TN = 128, TK = 16;
+
+struct GemmArgs {
+    float* X;        // accumulator matrix, pitch ldx, batch stride xs
+    const float* At; // [K, M] operand (row k, column m), pitch lda, batch stride as
+    const float* Bm; // [K, N] operand, pitch ldb, batch stride bs
+    int64_t ldx, xs, lda, as, ldb, bs;
+    int m0, m1, n1, k0, k1;
+};
+
+__global__ __launch_bounds__(256) void chain_gemm_kernel(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) float As[2][TK][TM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TK][TN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t bz = blockIdx.z;
+    float* __restrict__ X = g.X + bz * g.xs;
+    const float* __restrict__ At = g.At + bz * g.as;
+    const float* __restrict__ Bm = g.Bm + bz * g.bs;
+    const int mt = g.m0 + blockIdx.y * TM;  // first row (m) of this tile
+    const int nt = blockIdx.x * TN;         // first column (n) of this tile
+
+    // accumulators <- current X
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = mt + wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int n = nt + wn * 64 + ni * 32 + (lane & 31);
+                acc[mi][ni][v] = (m < g.m1 && n < g.n1) ? X[(int64_t)m * g.ldx + n] : 0.0f;
+            }
+
+    // global -> LDS staging: thread loads rows (tid>>5) and (tid>>5)+8, 4 columns each
+    const int lrow = tid >> 5, lcol = (tid & 31) * 4;
+    float4 ra[2], rb[2];
+    auto fetch = [&](int kk) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = kk + lrow + 8 * h;
+            float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
+            if (k < g.k1) {
+                const float* pa = At + (int64_t)k * g.lda + mt + lcol;
+                const float* pb = Bm + (int64_t)k * g.ldb + nt + lcol;
+                if (mt + lcol + 3 < g.m1) {
+                    va = *reinterpret_cast<const float4*>(pa);
+                } else {
+                    if (mt + lcol + 0 < g.m1) va.x = pa[0];
+                    if (mt + lcol + 1 < g.m1) va.y = pa[1];
+                    if (mt + lcol + 2 < g.m1) va.z = pa[2];
+                }
+                if (nt + lcol + 3 < g.n1) {
+                    vb = *reinterpret_cast<const float4*>(pb);
+                } else {
+                    if (nt + lcol + 0 < g.n1) vb.x = pb[0];
+                    if (nt + lcol + 1 < g.n1) vb.y = pb[1];
+                    if (nt + lcol + 2 < g.n1) vb.z = pb[2];
+                }
+            }
+            ra[h] = make_float4(-va.x, -va.y, -va.z, -va.w);
+            rb[h] = vb;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
+            *reinterpret_cast<float4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
+        }
+    };
+
+    int buf = 0;
+    fetch(g.k0);
+    stage(0);
+    __syncthreads();
+    for (int kk = g.k0; kk < g.k1; kk += TK) {
+        const bool more = kk + TK < g.k1;
+        if (more) fetch(kk + TK);
+#pragma unroll
+        for (int kp = 0; kp < TK / 2; ++kp) {
+            const int kr = 2 * kp + (lane >> 5);
+            float av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                av[i] = As[buf][kr][wm * 64 + i * 32 + (lane & 31)];
+                bv[i] = Bs[buf][kr][wn * 64 + i * 32 + (lane & 31)];
+            }
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mi], bv[ni], acc[mi][ni],
+                                                                       0, 0, 0);
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = mt + wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int n = nt + wn * 64 + ni * 32 + (lane & 31);
+                if (m < g.m1 && n < g.n1) X[(int64_t)m * g.ldx + n] = acc[mi][ni][v];
+            }
+}
+
+// U[i, :] *= 1/U[i,i]; uinv[i] = 1/U[i,i]   (solver_sparsegptq14.cu:153-155)
+__global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ uinv, int64_t C) {
+    const int64_t i = blockIdx.x;
+    const float inv = 1.0f / U[i * C + i];
+    for (int64_t j = threadIdx.x; j < C; j += blockDim.x) U[i * C + j] = U[i * C + j] * inv;
+    if (threadIdx.x == 0) uinv[i] = inv;
+}
+
+int launch_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
+    if (g.m1 <= g.m0 || g.k1 <= g.k0 || g.n1 <= 0 || batch <= 0) return FORGE_OK;
+    dim3 grid((unsigned)forge::ceil_div(g.n1, TN), (unsigned)forge::ceil_div(g.m1 - g.m0, TM),
+              (unsigned)batch);
+    chain_gemm_kernel<<<grid, dim3(256), 0, st>>>(g);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+template <bool SPARSE, bool PER_ELEM>
+int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
+    dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
+    constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
+    if (a.bw % 32 == 0)
+        sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, false>
+            <<<grid, dim3(64), 0, st>>>(a);
+    else
+        sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, true>
+            <<<grid, dim3(64), 0, st>>>(a);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+int check_sweep_shape(int64_t C, int64_t R, int bits) {
+    FORGE_REQUIRE(bits >= 1 && bits <= 8, "bits=%d outside 1..8", bits);
+    FORGE_REQUIRE(C >= 1 && R >= 1 && C < (1 << 30) && R < (1 << 30), "bad shape C=%lld R=%lld",
+                  (long long)C, (long long)R);
+    FORGE_REQUIRE((R % 4) == 0 && (C % 4) == 0,
+                  "C and R must be multiples of 4 (C=%lld R=%lld)", (long long)C, (long long)R);
+    return FORGE_OK;
+}
+
+}  // namespace
+
+namespace forge {
+constexpr int kBW = forge_kBW;
+}
+
+// Right-looking schedule for one matrix with per-element metadata (reference signature).
+template <bool SPARSE>
+static int solve_single(float* W, const float* U, const float* scales, const float* qzeros,
+                        int bits, int64_t C, int64_t R, uint8_t* q, uint32_t* M, float* E,
+                        const float* uinv, hipStream_t st) {
+    for (int64_t start = 0; start < C; start += forge::kBW) {
+        const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
+        SweepArgs a{};
+        a.A = W; a.B = E; a.U = U; a.scales = scales; a.qzeros = qzeros; a.g_idx = nullptr;
+        a.q = q; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = 0; a.c0 = start; a.bw = bw;
+        a.maxq = (1 << bits) - 1;
+        if (int e = launch_block<SPARSE, true>(a, 1, st)) return e;
+        GemmArgs g{};
+        g.X = W; g.At = U; g.Bm = E; g.ldx = R; g.lda = C; g.ldb = R; g.xs = g.as = g.bs = 0;
+        g.m0 = (int)(start + bw); g.m1 = (int)C; g.n1 = (int)R; g.k0 = (int)start;
+        g.k1 = (int)(start + bw);
+        if (int e = launch_gemm(g, 1, st)) return e;
+    }
+    return FORGE_OK;
+}
+
+extern "C" int forge_gptq_solver(float* W, const float* U, const float* scales,
+                                 const float* qzeros, int bits, int64_t C, int64_t R,
+                                 uint8_t* qweight, float* E, forge_stream_t stream) {
+    if (int e = check_sweep_shape(C, R, bits)) return e;
+    FORGE_REQUIRE(W && U && scales && qzeros && qweight && E, "null pointer");
+    return solve_single<false>(W, U, scales, qzeros, bits, C, R, qweight, nullptr, E, nullptr,
+                               (hipStream_t)stream);
+}
+
+extern "C" int forge_sparsegptq14_solver(float* W, float* U, const float* scales,
+                                         const float* qzeros, int bits, int64_t C, int64_t R,
+                                         uint8_t* qweight, uint32_t* M, float* E, float* uinv,
+                                         forge_stream_t stream) {
+    if (int e = check_sweep_shape(C, R, bits)) return e;
+    FORGE_REQUIRE(W && U && scales && qzeros && qweight && M && E && uinv, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    row_normalise_kernel<<<dim3((unsigned)C), dim3(256), 0, st>>>(U, uinv, C);
+    FORGE_LAUNCH_CHECK();
+    return solve_single<true>(W, U, scales, qzeros, bits, C, R, qweight, M, E, uinv, st);
+}
+
+// Left-looking schedule for a batch of equally shaped matrices, errors kept in X.
+extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
+                                        const float* qzerosT, const int32_t* g_idx,
+                                        uint8_t* qweight, uint32_t* M, const float* uinv,
+                                        int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
+                                        int sparse14, forge_stream_t stream) {
+    if (int e = check_sweep_shape(C, R, bits)) return e;
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && G >= 1, "bad batch=%lld G=%lld", (long long)batch,
+                  (long long)G);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(X && U && scalesT && qzerosT && g_idx && qweight, "null pointer");
+    FORGE_REQUIRE(!sparse14 || (M && uinv), "sparse14 needs M and uinv");
+    hipStream_t st = (hipStream_t)stream;
+    for (int64_t start = 0; start < C; start += forge::kBW) {
+        const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
+        GemmArgs g{};
+        g.X = X; g.At = U; g.Bm = X; g.ldx = R; g.lda = C; g.ldb = R;
+        g.xs = C * R; g.as = C * C; g.bs = C * R;
+        g.m0 = (int)start; g.m1 = (int)(start + bw); g.n1 = (int)R; g.k0 = 0; g.k1 = (int)start;
+        if (int e = launch_gemm(g, batch, st)) return e;
+        SweepArgs a{};
+        a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
+        a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
+        a.maxq = (1 << bits) - 1;
+        int e = sparse14 ? launch_block<true, false>(a, batch, st)
+                         : launch_block<false, false>(a, batch, st);
+        if (e) return e;
+    }
+    return FORGE_OK;
+}

@@ -1,0 +1,311 @@
+"""Operator boundary of the MI355X backend.
+
+``kernels`` exposes the hot-path operators under the names the reference binds in
+forge/backend/cuda/kernels.cpp:92-120 (``build_group_meta_packed``,
+``mse_scale_groups_packed``, ``gptq_solver``, ``sparsegptq14_solver``) with the same
+positional signatures and return conventions, plus the batched entry points of
+include/forge_hip.h.  Everything goes through the C ABI of ``csrc/libforge_hip.so``
+(ctypes; device pointers and the current HIP stream), torch only provides the memory.
+
+There is no CPU fallback: without a GPU or without the built library every attribute
+access raises ``RuntimeError`` (the reference's stub does the same when CUDA is missing,
+forge/backend/cuda/__init__.py:74-87).
+"""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+from types import ModuleType
+
+import torch
+
+__all__ = ["kernels", "library_path", "load_library"]
+
+_CSRC = Path(__file__).resolve().parents[3] / "csrc"
+FORGE_F32, FORGE_BF16 = 0, 1
+
+
+def library_path() -> Path:
+    return _CSRC / "libforge_hip.so"
+
+
+def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
+    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+    sigs = {
+        "forge_hip_abi_version": ([], i32),
+        "forge_last_error": ([], ctypes.c_char_p),
+        "forge_build_group_meta_packed": ([vp, i64, i64, i32, i32, vp, vp, vp], i32),
+        "forge_mse_scale_groups_packed": ([vp, vp, vp, vp, i64, i64, i64, f32, i32, i32, vp], i32),
+        "forge_quant_grid": ([vp, i32, i64, i64, i64, i64, i64, i64, i32, i32, i32, vp, i64, f32,
+                              vp, vp, vp], i32),
+        "forge_gptq_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp], i32),
+        "forge_sparsegptq14_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp, vp, vp], i32),
+        "forge_gptq_sweep_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32,
+                                      vp], i32),
+        "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp], i32),
+        "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
+        "forge_chol_workspace_bytes": ([i64, i64], i64),
+        "forge_hessian_permute": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
+        "forge_weight_to_solver_order": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_pack_int4": ([vp, vp, vp, i64, i64, i64, vp], i32),
+    }
+    for name, (args, res) in sigs.items():
+        fn = getattr(lib, name)          # AttributeError here = library/header mismatch
+        fn.argtypes, fn.restype = args, res
+    return lib
+
+
+EXPORTED_SYMBOLS = (
+    "forge_hip_abi_version", "forge_last_error", "forge_build_group_meta_packed",
+    "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
+    "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_hessian_update_grouped",
+    "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
+    "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
+)
+
+
+def load_library() -> ctypes.CDLL:
+    """dlopen the C-ABI library and declare its prototypes (no GPU needed for this)."""
+    path = library_path()
+    if not path.exists():
+        raise RuntimeError(f"{path} is missing: run `python 4bit-forge_amd/build.py` "
+                           "(hipcc --offload-arch=gfx950)")
+    return _declare(ctypes.CDLL(str(path)))
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return FORGE_F32
+    if t.dtype == torch.bfloat16:
+        return FORGE_BF16
+    raise RuntimeError(f"unsupported dtype {t.dtype} (float32 or bfloat16 expected)")
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("forge HIP kernels need tensors on the GPU "
+                               f"(got a tensor on {t.device}); there is no CPU fallback")
+
+
+class _HipKernels:
+    """The operator table.  Method names and argument order follow kernels.cpp."""
+
+    def __init__(self, lib: ctypes.CDLL):
+        self._lib = lib
+
+    def _check(self, rc: int):
+        if rc != 0:
+            raise RuntimeError(self._lib.forge_last_error().decode())
+
+    # -- reference-signature operators -------------------------------------------------
+    def build_group_meta_packed(self, X, bit_width, symmetric):
+        _need_cuda(X)
+        if X.dtype != torch.float32 or not X.is_contiguous() or X.dim() != 2:
+            raise RuntimeError("build_group_meta_packed: X must be a contiguous f32 [RG, gs] tensor")
+        RG, gs = X.shape
+        scales = torch.empty(RG, dtype=torch.float32, device=X.device)
+        qzeros = torch.empty(RG, dtype=torch.float32, device=X.device)
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_build_group_meta_packed(
+                _ptr(X), RG, gs, int(bit_width), int(bool(symmetric)), _ptr(scales), _ptr(qzeros),
+                _stream()))
+        return scales, qzeros
+
+    def mse_scale_groups_packed(self, X, scales, qzeros, candidates, norm, bit_width, symmetric):
+        _need_cuda(X, scales, qzeros, candidates)
+        for t in (X, scales, qzeros, candidates):
+            if t.dtype != torch.float32 or not t.is_contiguous():
+                raise RuntimeError("mse_scale_groups_packed: contiguous f32 tensors expected")
+        RG, gs = X.shape
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_mse_scale_groups_packed(
+                _ptr(X), _ptr(scales), _ptr(qzeros), _ptr(candidates), RG, gs,
+                candidates.numel(), float(norm), int(bit_width), int(bool(symmetric)), _stream()))
+        return scales, qzeros
+
+    def gptq_solver(self, W, U, scales, qzeros, bits):
+        _need_cuda(W, U, scales, qzeros)
+        W = W.contiguous()          # as solver.cu:107: a non-contiguous W is solved on a copy
+        U, scales, qzeros = U.contiguous(), scales.contiguous(), qzeros.contiguous()
+        for t in (W, U, scales, qzeros):
+            if t.dtype != torch.float32:
+                raise RuntimeError("gptq_solver: f32 tensors expected")
+        C, R = W.shape
+        if tuple(U.shape) != (C, C) or tuple(scales.shape) != (C, R) or tuple(qzeros.shape) != (C, R):
+            raise RuntimeError("gptq_solver: shape mismatch (W [C,R], U [C,C], scales/qzeros [C,R])")
+        q = torch.empty((C, R), dtype=torch.uint8, device=W.device)
+        E = torch.empty((C, R), dtype=torch.float32, device=W.device)
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_gptq_solver(_ptr(W), _ptr(U), _ptr(scales), _ptr(qzeros),
+                                                    int(bits), C, R, _ptr(q), _ptr(E), _stream()))
+        return q
+
+    def sparsegptq14_solver(self, W, U, scales, qzeros, bits):
+        _need_cuda(W, U, scales, qzeros)
+        W = W.contiguous()
+        Uc = U.contiguous()
+        scales, qzeros = scales.contiguous(), qzeros.contiguous()
+        for t in (W, Uc, scales, qzeros):
+            if t.dtype != torch.float32:
+                raise RuntimeError("sparsegptq14_solver: f32 tensors expected")
+        C, R = W.shape
+        if tuple(Uc.shape) != (C, C) or tuple(scales.shape) != (C, R) or tuple(qzeros.shape) != (C, R):
+            raise RuntimeError("sparsegptq14_solver: shape mismatch")
+        q = torch.empty((C, R), dtype=torch.uint8, device=W.device)
+        M = torch.empty(((C + 31) // 32, R), dtype=torch.uint32, device=W.device)
+        E = torch.empty((C, R), dtype=torch.float32, device=W.device)
+        uinv = torch.empty(C, dtype=torch.float32, device=W.device)
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_sparsegptq14_solver(
+                _ptr(W), _ptr(Uc), _ptr(scales), _ptr(qzeros), int(bits), C, R, _ptr(q), _ptr(M),
+                _ptr(E), _ptr(uinv), _stream()))
+        if Uc.data_ptr() != U.data_ptr():
+            U.copy_(Uc)             # the reference row-normalises the caller's U in place
+        return q, M
+
+    # -- batched / fused entry points (no reference counterpart) -------------------------
+    def quant_grid(self, W, gs, bits, symmetric, mse, candidates=None, norm=2.4):
+        """W [R,C] or [B,R,C] (f32/bf16, last dim contiguous) -> scales, qzeros [B?, R*G]."""
+        _need_cuda(W, candidates)
+        squeeze = W.dim() == 2
+        W3 = W.unsqueeze(0) if squeeze else W
+        if W3.stride(2) != 1:
+            W3 = W3.contiguous()
+        B, R, C = W3.shape
+        G = (C + gs - 1) // gs
+        scales = torch.empty((B, R * G), dtype=torch.float32, device=W.device)
+        qzeros = torch.empty_like(scales)
+        P = 0 if candidates is None else candidates.numel()
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_quant_grid(
+                _ptr(W3), _dtype_code(W3), B, W3.stride(0), R, C, W3.stride(1), gs, int(bits),
+                int(bool(symmetric)), int(bool(mse)), _ptr(candidates), P, float(norm),
+                _ptr(scales), _ptr(qzeros), _stream()))
+        return (scales[0], qzeros[0]) if squeeze else (scales, qzeros)
+
+    def gptq_sweep_batched(self, X, U, scalesT, qzerosT, g_idx, bits, sparse14=False, uinv=None):
+        """X [B,C,R] f32 in/out (errors on exit); returns qweight [B,C,R] u8 (and M)."""
+        _need_cuda(X, U, scalesT, qzerosT, g_idx)
+        B, C, R = X.shape
+        G = scalesT.shape[1]
+        assert X.is_contiguous() and U.is_contiguous() and scalesT.is_contiguous()
+        assert qzerosT.is_contiguous() and g_idx.is_contiguous() and g_idx.dtype == torch.int32
+        assert tuple(U.shape) == (B, C, C) and tuple(scalesT.shape) == (B, G, R)
+        assert tuple(qzerosT.shape) == (B, G, R) and tuple(g_idx.shape) == (B, C)
+        q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
+        M = None
+        if sparse14:
+            M = torch.empty((B, (C + 31) // 32, R), dtype=torch.uint32, device=X.device)
+            assert uinv is not None and tuple(uinv.shape) == (B, C) and uinv.is_contiguous()
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_gptq_sweep_batched(
+                _ptr(X), _ptr(U), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q), _ptr(M),
+                _ptr(uinv), B, C, R, G, int(bits), int(bool(sparse14)), _stream()))
+        return (q, M) if sparse14 else q
+
+    def hessian_update_grouped(self, X, offsets, H, alpha, beta):
+        """X [T,C] (bf16/f32) rows grouped by expert; offsets: host int64 [E+1];
+        H [E,C,C] f32; alpha/beta: host float sequences [E]."""
+        _need_cuda(X, H)
+        E = H.shape[0]
+        C = H.shape[-1]
+        offs = (ctypes.c_int64 * (E + 1))(*[int(o) for o in offsets])
+        al = (ctypes.c_float * E)(*[float(a) for a in alpha])
+        be = (ctypes.c_float * E)(*[float(b) for b in beta])
+        assert X.stride(1) == 1 and H.is_contiguous() and H.dtype == torch.float32
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_hessian_update_grouped(
+                _ptr(X), _dtype_code(X), X.stride(0), C, offs, E, al, be, _ptr(H), _stream()))
+        return H
+
+    def chol_inv_upper_batched(self, H, damp, normalise=True):
+        """H [B,C,C] f32 (destroyed); damp [B] f32 -> U [B,C,C], udiag [B,C], info [B]."""
+        _need_cuda(H, damp)
+        B, C, _ = H.shape
+        assert H.is_contiguous() and H.dtype == torch.float32 and damp.dtype == torch.float32
+        U = torch.empty_like(H)
+        udiag = torch.empty((B, C), dtype=torch.float32, device=H.device)
+        info = torch.empty(B, dtype=torch.int32, device=H.device)
+        nbytes = int(self._lib.forge_chol_workspace_bytes(B, C))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=H.device)
+        with torch.cuda.device(H.device):
+            self._check(self._lib.forge_chol_inv_upper_batched(
+                _ptr(H), _ptr(damp), _ptr(U), _ptr(udiag), _ptr(info), B, C,
+                int(bool(normalise)), _ptr(ws), nbytes, _stream()))
+        return U, udiag, info
+
+    def hessian_permute(self, H, perm, dead, rel_damp):
+        _need_cuda(H, perm, dead)
+        B, C, _ = H.shape
+        assert H.is_contiguous() and perm.dtype == torch.int64 and perm.is_contiguous()
+        assert dead.dtype == torch.uint8 and dead.is_contiguous()
+        Hp = torch.empty_like(H)
+        damp = torch.empty(B, dtype=torch.float32, device=H.device)
+        with torch.cuda.device(H.device):
+            self._check(self._lib.forge_hessian_permute(
+                _ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
+                _stream()))
+        return Hp, damp
+
+    def weight_to_solver_order(self, W, perm, dead=None):
+        """W [B,R,C] (bf16/f32) -> [B,C,R] f32 with columns taken in perm order."""
+        _need_cuda(W, perm, dead)
+        B, R, C = W.shape
+        assert W.stride(2) == 1 and perm.dtype == torch.int64 and perm.is_contiguous()
+        out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_weight_to_solver_order(
+                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm), _ptr(dead),
+                _ptr(out), B, R, C, _stream()))
+        return out
+
+    def codes_to_layer_order(self, q, perm):
+        _need_cuda(q, perm)
+        B, C, R = q.shape
+        assert q.is_contiguous() and q.dtype == torch.uint8 and perm.is_contiguous()
+        out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
+        with torch.cuda.device(q.device):
+            self._check(self._lib.forge_codes_to_layer_order(_ptr(q), _ptr(perm), _ptr(out), B, R,
+                                                             C, _stream()))
+        return out
+
+    def pack_int4(self, codes, qzeros, group_size):
+        _need_cuda(codes, qzeros)
+        R, C = codes.shape
+        assert codes.is_contiguous() and codes.dtype == torch.uint8
+        out = torch.empty((R, (C + 7) // 8), dtype=torch.int32, device=codes.device)
+        with torch.cuda.device(codes.device):
+            self._check(self._lib.forge_pack_int4(_ptr(codes), _ptr(qzeros), _ptr(out), R, C,
+                                                  int(group_size), _stream()))
+        return out
+
+
+class _HipUnavailable(ModuleType):
+    def __init__(self, why: str) -> None:
+        super().__init__("forge.backend.hip.kernels")
+        self.__dict__["_why"] = why
+
+    def __getattr__(self, name: str):
+        raise RuntimeError(f"4Bit-Forge HIP kernels are unavailable: {self.__dict__['_why']}")
+
+
+def _make_kernels():
+    if not torch.cuda.is_available():
+        return _HipUnavailable("torch.cuda.is_available() is False (no MI355X visible)")
+    try:
+        return _HipKernels(load_library())
+    except (OSError, RuntimeError, AttributeError) as exc:
+        return _HipUnavailable(str(exc))
+
+
+kernels = _make_kernels()

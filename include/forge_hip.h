@@ -1,0 +1,154 @@
+/*
+ * forge_hip.h -- C ABI of libforge_hip.so, the MI355X (gfx950) implementation of
+ * 4Bit-Forge's GPTQ calibration-and-solve kernels.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the name ends in _host.
+ *   - Matrices are dense row-major; "ld" arguments are row pitches in elements.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All work is
+ *     enqueued asynchronously on it; no entry point synchronises unless it says so.
+ *   - Return value: 0 on success, FORGE_ERR_* otherwise; forge_last_error() then gives
+ *     a message (thread-local).  Invalid shapes are rejected BEFORE any launch.
+ *   - dtype codes: FORGE_F32 = 0, FORGE_BF16 = 1.
+ *
+ * The first four entry points are what the reference binds through pybind11 in
+ * forge/backend/cuda/kernels.cpp:92-120; the rest are batched forms of the same
+ * arithmetic plus the torch library calls of forge/gptq.py that sit on the hot path.
+ */
+#ifndef FORGE_HIP_H
+#define FORGE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FORGE_OK 0
+#define FORGE_ERR_INVALID 1   /* bad argument / unsupported shape */
+#define FORGE_ERR_HIP 2       /* a HIP runtime call failed */
+
+#define FORGE_F32 0
+#define FORGE_BF16 1
+
+typedef void* forge_stream_t;
+
+/* Library identification and error text. */
+int forge_hip_abi_version(void);
+const char* forge_last_error(void);
+
+/* ------------------------------------------------------------------ quant grid */
+
+/* Replaces kernels.build_group_meta_packed (kernels.cpp:93-97, quant_grid.cu:186-224).
+ * X [RG, gs] f32.  Writes scales[RG], qzeros[RG] (f32).  Any gs >= 1. */
+int forge_build_group_meta_packed(const float* X, int64_t RG, int64_t gs, int bits,
+                                  int symmetric, float* scales, float* qzeros,
+                                  forge_stream_t stream);
+
+/* Replaces kernels.mse_scale_groups_packed (kernels.cpp:98-102, quant_grid.cu:227-287).
+ * Overwrites scales/qzeros in place.  gs must be 32, 64 or 128 (as the reference). */
+int forge_mse_scale_groups_packed(const float* X, float* scales, float* qzeros,
+                                  const float* candidates, int64_t RG, int64_t gs, int64_t P,
+                                  float norm, int bits, int symmetric, forge_stream_t stream);
+
+/* Fused form of GPTQ._quant_grid (gptq.py:180-227) for `batch` weight matrices
+ * W[b] = W + b*w_stride, each [R, C] with row pitch ldw, dtype w_dtype: contiguous
+ * gs-wide column groups, the last one zero padded; min/max grid, then (if mse != 0)
+ * the shrink search over `candidates`[P].  scales/qzeros: [batch, R*G] f32, index
+ * r*G + g, G = ceil(C/gs).  gs in {32,64,128}. */
+int forge_quant_grid(const void* W, int w_dtype, int64_t batch, int64_t w_stride, int64_t R,
+                     int64_t C, int64_t ldw, int64_t gs, int bits, int symmetric, int mse,
+                     const float* candidates, int64_t P, float norm, float* scales,
+                     float* qzeros, forge_stream_t stream);
+
+/* ------------------------------------------------------------------ column sweep */
+
+/* Replaces kernels.gptq_solver (kernels.cpp:104-108, solver.cu:99-154).
+ * W [C, R] f32 contiguous: solver-order columns x rows; overwritten with the dequantised
+ * weights.  U [C, C] f32: row-normalised upper factor.  scales/qzeros [C, R] f32 per
+ * element.  qweight [C, R] u8 receives codes 0..2^bits-1.  E [C, R] f32 is workspace
+ * (receives the per-column errors). */
+int forge_gptq_solver(float* W, const float* U, const float* scales, const float* qzeros,
+                      int bits, int64_t C, int64_t R, uint8_t* qweight, float* E,
+                      forge_stream_t stream);
+
+/* Replaces kernels.sparsegptq14_solver (kernels.cpp:110-120,
+ * solver_sparsegptq14.cu:142-200).  U holds the UN-normalised upper factor and is
+ * row-normalised in place, as the reference does to its caller's tensor.
+ * M [ceil(C/32), R] u32: bit i of word w <-> solver column 32*w+i kept.
+ * uinv [C] f32 workspace (1/diag(U)). */
+int forge_sparsegptq14_solver(float* W, float* U, const float* scales, const float* qzeros,
+                              int bits, int64_t C, int64_t R, uint8_t* qweight, uint32_t* M,
+                              float* E, float* uinv, forge_stream_t stream);
+
+/* Batched sweep with per-group metadata (no [C,R] expansion, gptq.py:251-252 folded in).
+ * For b in [0,batch): X[b] [C, R] f32 workspace holding the permuted transposed weight on
+ * entry and the per-column errors on exit; U[b] [C, C]; scalesT/qzerosT[b] [G, R] f32
+ * (group-major); g_idx[b] [C] int32 = group of solver column c; qweight[b] [C, R] u8.
+ * sparse14 != 0 selects the 1:4 joint solve (then M[b] [ceil(C/32), R] u32 and
+ * uinv[b] [C] must be given and U must already be row-normalised). */
+int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
+                             const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
+                             uint32_t* M, const float* uinv, int64_t batch, int64_t C,
+                             int64_t R, int64_t G, int bits, int sparse14,
+                             forge_stream_t stream);
+
+/* ------------------------------------------------------------------ Hessian */
+
+/* Grouped ragged rank-k update, the batched form of GPTQ.update (gptq.py:61-80):
+ * for each group e in [0, n_groups): rows offsets_host[e] .. offsets_host[e+1] of X
+ * ([*, C], pitch ldx, dtype x_dtype) are that expert's tokens, and
+ *   H[e] <- beta[e]*H[e] + alpha[e] * X_e^T X_e      (H[e] = H + e*C*C, f32 [C,C], full)
+ * alpha_host/beta_host [n_groups] are host arrays (the caller owns the running-mean
+ * bookkeeping).  Groups with zero rows are left untouched.  bf16 inputs use bf16 MFMA with
+ * fp32 accumulation (products exact); f32 inputs use f32 MFMA. */
+int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_t C,
+                                 const int64_t* offsets_host, int64_t n_groups,
+                                 const float* alpha_host, const float* beta_host, float* H,
+                                 forge_stream_t stream);
+
+/* ------------------------------------------------------------------ factorisation */
+
+/* Batched form of GPTQ._h_factor's torch.linalg calls (gptq.py:152-175):
+ * for each b: A = H[b] + damp[b]*I (lower triangle of H[b] read), U0 = upper Cholesky
+ * factor of inv(A); writes U[b] = U0 / diag(U0)[:,None] (normalise != 0) or U0, upper
+ * triangle + zeroed lower; udiag[b] [C] receives diag(U0).  info[b] (int32) is 0 on
+ * success or the 1-based index of the first non-positive pivot, in which case U[b] = I.
+ * H[b] is destroyed (used as workspace).  ws: workspace of forge_chol_workspace_bytes. */
+int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
+                                 int32_t* info, int64_t batch, int64_t C, int normalise,
+                                 void* ws, int64_t ws_bytes, forge_stream_t stream);
+int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C);
+
+/* Fused gather for GPTQ._prep/_h_factor (gptq.py:100-117,145-154): for each b builds
+ * Hp[b][i][j] = H[b][perm[i]][perm[j]] with rows/cols flagged in dead[b] (u8, in PERMUTED
+ * position) zeroed and their diagonal set to 1; writes damp[b] = rel_damp * mean(diag). */
+int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
+                          float* damp, float rel_damp, int64_t batch, int64_t C,
+                          forge_stream_t stream);
+
+/* ------------------------------------------------------------------ layout helpers */
+
+/* Xout[b][c][r] = (f32) W[b][r][perm[b][c]]   (the W.T[perm] of gptq.py:133), W of dtype
+ * w_dtype [R, C] pitch ldw; columns flagged in dead[b] (original order, may be NULL) read
+ * as zero. */
+int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                                 const int64_t* perm, const uint8_t* dead, float* Xout,
+                                 int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
+
+/* qout[b][r][perm[b][c]] = qin[b][c][r]: back to [R, C] in original column order
+ * (qweight[perm_inv].T of gptq.py:139). */
+int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm, uint8_t* qout,
+                               int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
+
+/* Nibble packing of [R, C] u8 codes into the compressed-tensors "pack-quantized" int32
+ * layout consumed by pack_quantized.py:279-313: value = code - zero + 8 (offset binary of
+ * the zero-shifted int4), eight values per int32 along C, lowest nibble first.
+ * qzeros [R*G] f32 (NULL = 8 for every group).  packed [R, ceil(C/8)] int32. */
+int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_t* packed, int64_t R,
+                    int64_t C, int64_t gs, forge_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FORGE_HIP_H */

@@ -1,0 +1,243 @@
+/*
+ * CPU oracle for the GPTQ calibration-and-solve kernels of 4Bit-Forge.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, in scalar C, the arithmetic of the
+ * reference's CUDA kernels so that the HIP kernels can be checked against it.  It is
+ * never linked into, imported by, or called from the product library; only tests,
+ * the smoke check and the benchmark's cpu_baseline leg use it.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -shared -fPIC  (see oracle/Makefile).
+ * -ffp-contract=off matters: every fused multiply-add below is an explicit fmaf()
+ * and every other a*b+c must stay two roundings.
+ *
+ * Restated reference functions (paths relative to the reference checkout):
+ *   oracle_build_group_meta      forge/backend/cuda/quant_grid.cu:42-99
+ *   oracle_mse_scale_groups      forge/backend/cuda/quant_grid.cu:101-183
+ *   oracle_gptq_solver           forge/backend/cuda/solver.cu:9-154
+ *   oracle_sparsegptq14_solver   forge/backend/cuda/solver_sparsegptq14.cu:12-200
+ *
+ * Where the reference leaves fp32 bits undefined, the oracle fixes them as follows
+ * (each choice is within the reference's own numerical freedom):
+ *   - nvcc contracts `x*inv_s+q0` (solver.cu:13) and `(2/maxq)*amax+eps`
+ *     (quant_grid.cu:83) into one FMA by default (--fmad=true); written as fmaf here.
+ *   - __logf/__expf (quant_grid.cu:165-166) are hardware approximations whose bits are
+ *     not specified; the oracle uses libm logf/expf.  Only exact near-ties of the
+ *     candidate losses can therefore resolve differently.
+ *   - The trailing update W[end:,:] -= U[blk,end:]^T * Eblk is a cuBLAS SGEMM
+ *     (solver.cu:146-150) whose summation order is a library detail.  Two orders are
+ *     offered: TRAIL_CHAIN applies the block's rank-1 updates one after another,
+ *     x = fmaf(-U[t,k], err_t, x) for t ascending, i.e. the very chain the reference
+ *     uses inside a block (solver.cu:91-94); the result is then independent of the
+ *     block size.  TRAIL_GEMM accumulates acc = sum_t U[t,k]*err_t from zero with fmaf
+ *     in ascending t and then stores W - acc (alpha=-1, beta=1 epilogue).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <float.h>
+
+#define ORACLE_EPS 1e-12f
+
+static inline float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
+
+/* lrintf in the default rounding mode is round-to-nearest-even, like CUDA's lrintf. */
+static inline float rne(float v) { return nearbyintf(v); }
+
+/* quant_grid.cu:42-99.  X is [RG, gs] row-major fp32. */
+void oracle_build_group_meta(const float* X, int64_t RG, int64_t gs, int bits, int symmetric,
+                             float* scales, float* qzeros) {
+    const float maxq = (float)((1 << bits) - 1);
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < RG; ++g) {
+        const float* grp = X + g * gs;
+        float lo = 1e30f, hi = -1e30f;
+        for (int64_t i = 0; i < gs; ++i) { hi = fmaxf(hi, grp[i]); lo = fminf(lo, grp[i]); }
+        float s, q0;
+        if (symmetric) {
+            float amax = fmaxf(fabsf(lo), fabsf(hi));
+            s = fmaf(2.0f / maxq, amax, ORACLE_EPS);
+            q0 = 0.5f * (maxq + 1.0f);
+        } else {
+            s = (hi - lo) / maxq + ORACLE_EPS;
+            q0 = clampf(rne(-lo / s), 0.0f, maxq);
+        }
+        scales[g] = s;
+        qzeros[g] = q0;
+    }
+}
+
+/* Loss of one shrink candidate for one group, in the reference's summation order:
+ * 32 lanes, lane l adds elements l, l+32, l+64, ... in that order, then a shuffle-down
+ * tree with offsets 16,8,4,2,1 (quant_grid.cu:15-22,156-169). */
+static float group_loss(const float* grp, int64_t gs, float s, float rcp_s, float q0,
+                        float maxq, float norm) {
+    float lane[32];
+    const int64_t vpl = gs / 32;
+    for (int l = 0; l < 32; ++l) {
+        float loss = 0.0f;
+        for (int64_t i = 0; i < vpl; ++i) {
+            float v = grp[l + 32 * i];
+            float q = clampf(rne(fmaf(v, rcp_s, q0)), 0.0f, maxq);
+            float diff = fmaf(q - q0, s, -v);
+            float e = fmaxf(fabsf(diff), 1e-20f);
+            loss += expf(logf(e) * norm);
+        }
+        lane[l] = loss;
+    }
+    for (int off = 16; off > 0; off >>= 1)
+        for (int l = 0; l < off; ++l) lane[l] += lane[l + off];
+    return lane[0];
+}
+
+/* quant_grid.cu:101-183.  Overwrites scales/qzeros in place.  losses_out (optional,
+ * [RG,P]) receives every candidate's loss so that tests can recognise near-ties. */
+void oracle_mse_scale_groups(const float* X, float* scales, float* qzeros, const float* cand,
+                             int64_t RG, int64_t gs, int64_t P, int bits, float norm,
+                             int symmetric, float* losses_out) {
+    const float maxq = (float)((1 << bits) - 1);
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < RG; ++g) {
+        const float sg = scales[g], q0g = qzeros[g];
+        float xmin = 0.0f;
+        if (!symmetric) xmin = -(sg * q0g);
+        float best_s = sg, best_q = q0g, best_loss = FLT_MAX;
+        for (int64_t p = 0; p < P; ++p) {
+            float s = sg * cand[p];
+            float rcp_s = 1.0f / (s + ORACLE_EPS);
+            float q0;
+            if (symmetric) q0 = q0g;
+            else q0 = clampf(rne(-xmin * rcp_s), 0.0f, maxq);
+            float loss = group_loss(X + g * gs, gs, s, rcp_s, q0, maxq, norm);
+            if (losses_out) losses_out[g * P + p] = loss;
+            if (loss < best_loss) { best_loss = loss; best_s = s; best_q = q0; }
+        }
+        scales[g] = best_s;
+        qzeros[g] = best_q;
+    }
+}
+
+/* solver.cu:9-23 */
+static inline void quantize_scalar(float x, float inv_s, float s, float q0, int maxq_i,
+                                   float* err, uint8_t* qb, float* deq) {
+    float biased = fmaf(x, inv_s, q0);
+    long q = lrintf(biased);
+    if (q < 0) q = 0; else if (q > maxq_i) q = maxq_i;
+    *deq = fmaf((float)q, s, -q0 * s);
+    *err = x - *deq;
+    *qb = (uint8_t)q;
+}
+
+enum { TRAIL_CHAIN = 0, TRAIL_GEMM = 1 };
+
+/* Apply one finished block's errors to every later column.  E is [B, R]. */
+static void trailing_update(float* W, const float* U, const float* E, int64_t C, int64_t R,
+                            int64_t start, int64_t B, int mode) {
+    const int64_t end = start + B;
+#pragma omp parallel for schedule(static)
+    for (int64_t k = end; k < C; ++k) {
+        float* wk = W + k * R;
+        if (mode == TRAIL_CHAIN) {
+            for (int64_t t = 0; t < B; ++t) {
+                const float a = -U[(start + t) * C + k];
+                const float* e = E + t * R;
+                for (int64_t r = 0; r < R; ++r) wk[r] = fmaf(a, e[r], wk[r]);
+            }
+        } else {
+            float* acc = (float*)calloc((size_t)R, sizeof(float));
+            for (int64_t t = 0; t < B; ++t) {
+                const float a = U[(start + t) * C + k];
+                const float* e = E + t * R;
+                for (int64_t r = 0; r < R; ++r) acc[r] = fmaf(a, e[r], acc[r]);
+            }
+            for (int64_t r = 0; r < R; ++r) wk[r] = wk[r] - acc[r];
+            free(acc);
+        }
+    }
+}
+
+/* solver.cu:26-154.  W [C,R] fp32 is updated in place to the dequantised weights,
+ * qweight [C,R] receives the codes.  U [C,C] is the row-normalised upper factor.
+ * scales/qzeros are per element [C,R].  B is the in-block width (reference: 32). */
+void oracle_gptq_solver(float* W, const float* U, const float* scales, const float* qzeros,
+                        int bits, int64_t C, int64_t R, uint8_t* qweight, int trail_mode,
+                        int64_t B) {
+    const int maxq_i = (1 << bits) - 1;
+    float* E = (float*)malloc((size_t)(B * R) * sizeof(float));
+    for (int64_t start = 0; start < C; start += B) {
+        const int64_t Bc = (start + B <= C) ? B : (C - start);
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < R; ++r) {
+            float x[256];
+            for (int64_t i = 0; i < Bc; ++i) x[i] = W[(start + i) * R + r];
+            for (int64_t t = 0; t < Bc; ++t) {
+                const int64_t c = start + t;
+                const float s = scales[c * R + r], q0 = qzeros[c * R + r];
+                const float inv_s = 1.0f / (s + ORACLE_EPS);
+                float err, deq; uint8_t qb;
+                quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+                qweight[c * R + r] = qb;
+                W[c * R + r] = deq;
+                E[t * R + r] = err;
+                for (int64_t k = t + 1; k < Bc; ++k)
+                    x[k] = fmaf(-U[c * C + start + k], err, x[k]);
+            }
+        }
+        if (start + Bc < C) trailing_update(W, U, E, C, R, start, Bc, trail_mode);
+    }
+    free(E);
+}
+
+/* solver_sparsegptq14.cu:29-200.  U [C,C] holds the un-normalised upper factor on entry
+ * and is row-normalised in place (lines 153-155), as the reference does to the caller's
+ * tensor.  M is [ceil(C/32), R] uint32, bit i of word w <-> solver column 32*w+i. */
+void oracle_sparsegptq14_solver(float* W, float* U, const float* scales, const float* qzeros,
+                                int bits, int64_t C, int64_t R, uint8_t* qweight, uint32_t* M,
+                                int trail_mode) {
+    const int maxq_i = (1 << bits) - 1;
+    const int64_t B = 32;
+    float* Uinv = (float*)malloc((size_t)C * sizeof(float));
+    for (int64_t i = 0; i < C; ++i) Uinv[i] = 1.0f / U[i * C + i];
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < C; ++i)
+        for (int64_t j = 0; j < C; ++j) U[i * C + j] = U[i * C + j] * Uinv[i];
+    float* E = (float*)malloc((size_t)(B * R) * sizeof(float));
+    for (int64_t start = 0; start < C; start += B) {
+        const int64_t Bc = (start + B <= C) ? B : (C - start);
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < R; ++r) {
+            float x[32];
+            uint32_t mask = 0u;
+            for (int64_t i = 0; i < Bc; ++i) x[i] = W[(start + i) * R + r];
+            for (int64_t t = 0; t < Bc; ++t) {
+                const int64_t c = start + t;
+                if (t % 4 == 0) {
+                    float best = -1e30f; int best_k = -1;
+                    for (int k = 0; k < 4; ++k) {
+                        if (c + k >= C) continue;
+                        float score = fabsf(x[t + k] * Uinv[c + k]);
+                        if (best < score) { best = score; best_k = k; }
+                    }
+                    if (best_k > -1) mask |= (1u << (t + best_k));
+                }
+                float err, deq = 0.0f; uint8_t qb = 0;
+                if ((mask >> t) & 1u) {
+                    const float s = scales[c * R + r], q0 = qzeros[c * R + r];
+                    const float inv_s = 1.0f / (s + ORACLE_EPS);
+                    quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+                } else {
+                    err = x[t];
+                }
+                qweight[c * R + r] = qb;
+                W[c * R + r] = deq;
+                E[t * R + r] = err;
+                for (int64_t k = t + 1; k < Bc; ++k)
+                    x[k] = fmaf(-U[c * C + start + k], err, x[k]);
+            }
+            M[(start >> 5) * R + r] = mask;
+        }
+        if (start + Bc < C) trailing_update(W, U, E, C, R, start, Bc, trail_mode);
+    }
+    free(E);
+    free(Uinv);
+}
