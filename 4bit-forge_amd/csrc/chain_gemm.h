@@ -1,0 +1,29 @@
+// fp32 MFMA GEMM whose K loop is one fma chain per output element (see chain_gemm.hip).
+#pragma once
+#include "common.h"
+
+namespace forge {
+
+// X[m, n] <- chain_{k = k0 .. k1-1} fma(sA * At[k, m], Bm[k, n], acc),  m in [m0, m1),
+// n in [0, n1), acc starting from X[m, n] (or 0 when init_zero), sA = -1 when negate_a.
+// Operands are "K-major": row k of At holds the m index contiguously, row k of Bm the n
+// index.  All three may point into the same allocation as long as the rows written
+// ([m0, m1) of X) are not among the rows read ([k0, k1) of At/Bm), or, when they are
+// (in-place triangular solve), as long as n-tiles do not overlap: each workgroup reads
+// all of its K range before it writes.
+struct GemmArgs {
+    float* X;         // accumulator / output, pitch ldx, batch stride xs
+    const float* At;  // [K, M], pitch lda, batch stride as
+    const float* Bm;  // [K, N], pitch ldb, batch stride bs
+    int64_t ldx, xs, lda, as, ldb, bs;
+    int m0, m1, n0, n1, k0, k1;
+    bool negate_a;
+    bool init_zero;
+    bool b_upper_tri;  // Bm[k, n] == 0 for k > n: stop each tile's K loop at its last column
+    bool b_lower_tri;  // Bm[k, n] == 0 for k < n: start each tile's K loop at its first column
+    bool blocked_sum;  // sum K in blocks of 128 (more accurate; NOT the sweep's single chain)
+};
+
+int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);
+
+}  // namespace forge

@@ -1,0 +1,215 @@
+// fp32 GEMM on the gfx950 matrix cores with a defined summation order.
+//
+// v_mfma_f32_32x32x2_f32 computes, for each output element, acc = fma(a[k], b[k], acc)
+// for its two k values one after the other, in fp32 with round-to-nearest.  Chaining the
+// instruction over ascending k therefore reproduces, bit for bit, the scalar recurrence
+//     for k: x = fmaf(a_k, b_k, x)
+// which is exactly how the GPTQ sweep propagates quantisation errors.  The same kernel
+// serves the Cholesky / triangular-inverse updates, where only fp32 accuracy matters.
+//
+// Tile: 128 (m) x 128 (n) per workgroup of 4 wavefronts; each wavefront owns a 64x64
+// quadrant = 2x2 MFMA tiles (64 accumulator registers).  Operands are K-major in memory,
+// so a half-wavefront reads 32 consecutive floats of one k row: global loads are
+// coalesced float4, LDS reads are conflict-free ds_read_b32, and no transpose is needed.
+// K advances 16 rows per stage: the next stage's rows are fetched into registers while
+// the current stage's 32 MFMAs per wavefront run, all LDS operands of a stage are read
+// before its first MFMA so the matrix pipe is fed back to back, and the register budget
+// leaves room for two workgroups per CU to cover the barrier between stages.
+#include "chain_gemm.h"
+
+namespace forge {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int TM = 128, TN = 128, TK = 16;
+
+// EDGE: bounds-checked loads/stores for tiles that stick out of [m0,m1) x [n0,n1) or a K
+// range that is not a multiple of 16.  CHUNK > 0: every CHUNK k values the running
+// accumulators are folded into a second set and restarted from zero (blocked summation:
+// the rounding error of each fma is then relative to a short partial sum instead of the
+// whole accumulated value).  Used where only accuracy matters; CHUNK == 0 is the single
+// chain that the sweep's bit-exactness needs.
+template <bool EDGE, int CHUNK>
+__global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) float As[2][TK][TM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TK][TN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t bz = blockIdx.z;
+    float* __restrict__ X = g.X + bz * g.xs;
+    const float* __restrict__ At = g.At + bz * g.as;
+    const float* __restrict__ Bm = g.Bm + bz * g.bs;
+    const int mt = g.m0 + blockIdx.y * TM;  // first m of this tile
+    const int nt = g.n0 + blockIdx.x * TN;  // first n of this tile
+    int k0 = g.k0, k1 = g.k1;
+    if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
+    if (g.b_lower_tri && k0 < nt) k0 = nt;
+
+    // element (v, lane) of MFMA tile (mi, ni) <-> X[m_base + mi*32 + row(v), n_base + ni*32]
+    const int m_base = mt + wm * 64 + (lane >> 5) * 4;
+    const int n_base = nt + wn * 64 + (lane & 31);
+    float* __restrict__ Xw = X + (int64_t)m_base * g.ldx + n_base;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                float x = 0.0f;
+                if (!g.init_zero && (!EDGE || (m_base + dm < g.m1 && n_base + dn < g.n1)))
+                    x = Xw[(int64_t)dm * g.ldx + dn];
+                acc[mi][ni][v] = x;
+            }
+    f32x16 tot[2][2];
+    if constexpr (CHUNK > 0) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                tot[mi][ni] = acc[mi][ni];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+            }
+    }
+
+    // global -> LDS staging: thread loads k rows (tid>>5) and (tid>>5)+8, 4 columns each
+    const int lrow = tid >> 5, lcol = (tid & 31) * 4;
+    const float sign = g.negate_a ? -1.0f : 1.0f;
+    const float* pa = At + (int64_t)(k0 + lrow) * g.lda + mt + lcol;
+    const float* pb = Bm + (int64_t)(k0 + lrow) * g.ldb + nt + lcol;
+    const int64_t a_step8 = 8 * g.lda, b_step8 = 8 * g.ldb;
+    float4 ra[2], rb[2];
+    auto fetch = [&](int kk) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float4 va, vb;
+            if constexpr (!EDGE) {
+                va = *reinterpret_cast<const float4*>(pa + h * a_step8);
+                vb = *reinterpret_cast<const float4*>(pb + h * b_step8);
+            } else {
+                va = make_float4(0.f, 0.f, 0.f, 0.f);
+                vb = va;
+                if (kk + lrow + 8 * h < k1) {
+                    const float* qa = pa + h * a_step8;
+                    const float* qb = pb + h * b_step8;
+                    if (mt + lcol + 0 < g.m1) va.x = qa[0];
+                    if (mt + lcol + 1 < g.m1) va.y = qa[1];
+                    if (mt + lcol + 2 < g.m1) va.z = qa[2];
+                    if (mt + lcol + 3 < g.m1) va.w = qa[3];
+                    if (nt + lcol + 0 < g.n1) vb.x = qb[0];
+                    if (nt + lcol + 1 < g.n1) vb.y = qb[1];
+                    if (nt + lcol + 2 < g.n1) vb.z = qb[2];
+                    if (nt + lcol + 3 < g.n1) vb.w = qb[3];
+                }
+            }
+            ra[h] = make_float4(sign * va.x, sign * va.y, sign * va.z, sign * va.w);
+            rb[h] = vb;
+        }
+        pa += 2 * a_step8;
+        pb += 2 * b_step8;
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
+            *reinterpret_cast<float4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
+        }
+    };
+
+    const int a_off = wm * 64 + (lane & 31), b_off = wn * 64 + (lane & 31), kr0 = lane >> 5;
+    int buf = 0;
+    if (k0 < k1) {
+        fetch(k0);
+        stage(0);
+    }
+    __syncthreads();
+    int stage_no = 0;
+    for (int kk = k0; kk < k1; kk += TK) {
+        const bool more = kk + TK < k1;
+        if (more) fetch(kk + TK);
+        float av[TK / 2][2], bv[TK / 2][2];
+#pragma unroll
+        for (int kp = 0; kp < TK / 2; ++kp)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                av[kp][i] = As[buf][2 * kp + kr0][a_off + i * 32];
+                bv[kp][i] = Bs[buf][2 * kp + kr0][b_off + i * 32];
+            }
+#pragma unroll
+        for (int kp = 0; kp < TK / 2; ++kp)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[kp][mi], bv[kp][ni],
+                                                                       acc[mi][ni], 0, 0, 0);
+        if constexpr (CHUNK > 0) {
+            if (++stage_no == CHUNK / TK) {
+                stage_no = 0;
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni) {
+                        tot[mi][ni] += acc[mi][ni];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+                    }
+            }
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    if constexpr (CHUNK > 0) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = tot[mi][ni] + acc[mi][ni];
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                if (!EDGE || (m_base + dm < g.m1 && n_base + dn < g.n1))
+                    Xw[(int64_t)dm * g.ldx + dn] = acc[mi][ni][v];
+            }
+}
+
+}  // namespace
+
+int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
+    if (g.m1 <= g.m0 || g.n1 <= g.n0 || batch <= 0) return FORGE_OK;
+    if (g.k1 <= g.k0 && !g.init_zero) return FORGE_OK;
+    // float4 loads need 16-byte aligned rows; anything else takes the scalar EDGE path
+    const bool aligned = (g.lda % 4) == 0 && (g.ldb % 4) == 0 && (g.m0 % 4) == 0 &&
+                         (g.n0 % 4) == 0 && (g.as % 4) == 0 && (g.bs % 4) == 0 &&
+                         (reinterpret_cast<uintptr_t>(g.At) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(g.Bm) % 16) == 0;
+    dim3 grid((unsigned)ceil_div(g.n1 - g.n0, TN), (unsigned)ceil_div(g.m1 - g.m0, TM),
+              (unsigned)batch);
+    // the triangular K clipping keeps multiples of 16 only when tiles and K origin line up
+    const bool tri_ok = (!g.b_upper_tri || ((g.n0 + TN - g.k0) % TK) == 0) &&
+                        (!g.b_lower_tri || ((g.n0 - g.k0) % TK) == 0);
+    const bool edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
+                      ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned;
+    if (g.blocked_sum) {
+        if (edge) chain_gemm_kernel<true, 128><<<grid, dim3(256), 0, st>>>(g);
+        else chain_gemm_kernel<false, 128><<<grid, dim3(256), 0, st>>>(g);
+    } else {
+        if (edge) chain_gemm_kernel<true, 0><<<grid, dim3(256), 0, st>>>(g);
+        else chain_gemm_kernel<false, 0><<<grid, dim3(256), 0, st>>>(g);
+    }
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+}  // namespace forge

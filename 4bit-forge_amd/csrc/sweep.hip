@@ -13,12 +13,13 @@
 //   sweep_block_kernel   one lane per output row, BW consecutive columns of that row in
 //                        registers; the serial quantise/propagate chain (VALU).
 //   chain_gemm_kernel    X[m, n] <- chain_k fma(-U[k, m], E[k, n], X[m, n]) on the f32
-//                        MFMA pipe, 128x128 tiles staged through LDS.
+//                        MFMA pipe, 128x128 tiles staged through LDS (chain_gemm.hip).
 //
 // The host schedules them left-looking (batched experts: each column block is brought
 // up to date with ONE long-K GEMM over all earlier errors, so the weights stream through
 // HBM once) or right-looking (a single matrix: more tiles in flight per step).
 #include "common.h"
+#include "chain_gemm.h"
 
 namespace {
 
@@ -28,7 +29,6 @@ constexpr float kEps = 1e-12f;
 #endif
 constexpr int forge_kBW = FORGE_SWEEP_BW;  // columns per in-register block
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct SweepArgs {
     float* A;              // [C,R] per matrix: x on entry; on exit err (batched form) or deq
@@ -49,6 +49,7 @@ struct SweepArgs {
 // 16 consecutive floats of a row of U, wave-uniform, fetched with one s_load_dwordx16
 // (viewing U through the constant address space makes the compiler use scalar loads;
 // valid because no kernel in this file writes the factor it reads).
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x16_a4 __attribute__((ext_vector_type(16), aligned(4)));
 __device__ __forceinline__ f32x16 load_u16(const float* p) {
     typedef const __attribute__((address_space(4))) f32x16_a4* vptr;
@@ -206,139 +207,12 @@ __global__ __launch_bounds__(64) void sweep_block_kernel(SweepArgs a) {
     }
 }
 
-// ---------------------------------------------------------------------------------
-// X[m, n] <- chain_{k=k0..k1-1} fma(-At[k, m], Bm[k, n], X[m, n])   for m in [m0, m1)
-// Tile 128 (m) x 128 (n); 4 wavefronts, each a 64x64 quadrant = 2x2 MFMA 32x32 tiles.
-constexpr int TM = 128, TN = 128, TK = 16;
-
-struct GemmArgs {
-    float* X;        // accumulator matrix, pitch ldx, batch stride xs
-    const float* At; // [K, M] operand (row k, column m), pitch lda, batch stride as
-    const float* Bm; // [K, N] operand, pitch ldb, batch stride bs
-    int64_t ldx, xs, lda, as, ldb, bs;
-    int m0, m1, n1, k0, k1;
-};
-
-__global__ __launch_bounds__(256) void chain_gemm_kernel(GemmArgs g) {
-    __shared__ __attribute__((aligned(16))) float As[2][TK][TM];
-    __shared__ __attribute__((aligned(16))) float Bs[2][TK][TN];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int64_t bz = blockIdx.z;
-    float* __restrict__ X = g.X + bz * g.xs;
-    const float* __restrict__ At = g.At + bz * g.as;
-    const float* __restrict__ Bm = g.Bm + bz * g.bs;
-    const int mt = g.m0 + blockIdx.y * TM;  // first row (m) of this tile
-    const int nt = blockIdx.x * TN;         // first column (n) of this tile
-
-    // accumulators <- current X
-    f32x16 acc[2][2];
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = mt + wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                const int n = nt + wn * 64 + ni * 32 + (lane & 31);
-                acc[mi][ni][v] = (m < g.m1 && n < g.n1) ? X[(int64_t)m * g.ldx + n] : 0.0f;
-            }
-
-    // global -> LDS staging: thread loads rows (tid>>5) and (tid>>5)+8, 4 columns each
-    const int lrow = tid >> 5, lcol = (tid & 31) * 4;
-    float4 ra[2], rb[2];
-    auto fetch = [&](int kk) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int k = kk + lrow + 8 * h;
-            float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
-            if (k < g.k1) {
-                const float* pa = At + (int64_t)k * g.lda + mt + lcol;
-                const float* pb = Bm + (int64_t)k * g.ldb + nt + lcol;
-                if (mt + lcol + 3 < g.m1) {
-                    va = *reinterpret_cast<const float4*>(pa);
-                } else {
-                    if (mt + lcol + 0 < g.m1) va.x = pa[0];
-                    if (mt + lcol + 1 < g.m1) va.y = pa[1];
-                    if (mt + lcol + 2 < g.m1) va.z = pa[2];
-                }
-                if (nt + lcol + 3 < g.n1) {
-                    vb = *reinterpret_cast<const float4*>(pb);
-                } else {
-                    if (nt + lcol + 0 < g.n1) vb.x = pb[0];
-                    if (nt + lcol + 1 < g.n1) vb.y = pb[1];
-                    if (nt + lcol + 2 < g.n1) vb.z = pb[2];
-                }
-            }
-            ra[h] = make_float4(-va.x, -va.y, -va.z, -va.w);
-            rb[h] = vb;
-        }
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
-            *reinterpret_cast<float4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
-        }
-    };
-
-    int buf = 0;
-    fetch(g.k0);
-    stage(0);
-    __syncthreads();
-    for (int kk = g.k0; kk < g.k1; kk += TK) {
-        const bool more = kk + TK < g.k1;
-        if (more) fetch(kk + TK);
-#pragma unroll
-        for (int kp = 0; kp < TK / 2; ++kp) {
-            const int kr = 2 * kp + (lane >> 5);
-            float av[2], bv[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                av[i] = As[buf][kr][wm * 64 + i * 32 + (lane & 31)];
-                bv[i] = Bs[buf][kr][wn * 64 + i * 32 + (lane & 31)];
-            }
-#pragma unroll
-            for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mi], bv[ni], acc[mi][ni],
-                                                                       0, 0, 0);
-        }
-        if (more) stage(buf ^ 1);
-        __syncthreads();
-        buf ^= 1;
-    }
-
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = mt + wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                const int n = nt + wn * 64 + ni * 32 + (lane & 31);
-                if (m < g.m1 && n < g.n1) X[(int64_t)m * g.ldx + n] = acc[mi][ni][v];
-            }
-}
-
 // U[i, :] *= 1/U[i,i]; uinv[i] = 1/U[i,i]   (solver_sparsegptq14.cu:153-155)
 __global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ uinv, int64_t C) {
     const int64_t i = blockIdx.x;
     const float inv = 1.0f / U[i * C + i];
     for (int64_t j = threadIdx.x; j < C; j += blockDim.x) U[i * C + j] = U[i * C + j] * inv;
     if (threadIdx.x == 0) uinv[i] = inv;
-}
-
-int launch_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
-    if (g.m1 <= g.m0 || g.k1 <= g.k0 || g.n1 <= 0 || batch <= 0) return FORGE_OK;
-    dim3 grid((unsigned)forge::ceil_div(g.n1, TN), (unsigned)forge::ceil_div(g.m1 - g.m0, TM),
-              (unsigned)batch);
-    chain_gemm_kernel<<<grid, dim3(256), 0, st>>>(g);
-    FORGE_LAUNCH_CHECK();
-    return FORGE_OK;
 }
 
 template <bool SPARSE, bool PER_ELEM>
@@ -359,8 +233,6 @@ int check_sweep_shape(int64_t C, int64_t R, int bits) {
     FORGE_REQUIRE(bits >= 1 && bits <= 8, "bits=%d outside 1..8", bits);
     FORGE_REQUIRE(C >= 1 && R >= 1 && C < (1 << 30) && R < (1 << 30), "bad shape C=%lld R=%lld",
                   (long long)C, (long long)R);
-    FORGE_REQUIRE((R % 4) == 0 && (C % 4) == 0,
-                  "C and R must be multiples of 4 (C=%lld R=%lld)", (long long)C, (long long)R);
     return FORGE_OK;
 }
 
@@ -382,11 +254,11 @@ static int solve_single(float* W, const float* U, const float* scales, const flo
         a.q = q; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = 0; a.c0 = start; a.bw = bw;
         a.maxq = (1 << bits) - 1;
         if (int e = launch_block<SPARSE, true>(a, 1, st)) return e;
-        GemmArgs g{};
+        forge::GemmArgs g{};
         g.X = W; g.At = U; g.Bm = E; g.ldx = R; g.lda = C; g.ldb = R; g.xs = g.as = g.bs = 0;
         g.m0 = (int)(start + bw); g.m1 = (int)C; g.n1 = (int)R; g.k0 = (int)start;
-        g.k1 = (int)(start + bw);
-        if (int e = launch_gemm(g, 1, st)) return e;
+        g.k1 = (int)(start + bw); g.negate_a = true;
+        if (int e = forge::launch_chain_gemm(g, 1, st)) return e;
     }
     return FORGE_OK;
 }
@@ -427,11 +299,12 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
     hipStream_t st = (hipStream_t)stream;
     for (int64_t start = 0; start < C; start += forge::kBW) {
         const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
-        GemmArgs g{};
+        forge::GemmArgs g{};
         g.X = X; g.At = U; g.Bm = X; g.ldx = R; g.lda = C; g.ldb = R;
         g.xs = C * R; g.as = C * C; g.bs = C * R;
         g.m0 = (int)start; g.m1 = (int)(start + bw); g.n1 = (int)R; g.k0 = 0; g.k1 = (int)start;
-        if (int e = launch_gemm(g, batch, st)) return e;
+        g.negate_a = true;
+        if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
         SweepArgs a{};
         a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;

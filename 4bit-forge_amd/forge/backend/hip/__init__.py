@@ -42,7 +42,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_sparsegptq14_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp, vp, vp], i32),
         "forge_gptq_sweep_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32,
                                       vp], i32),
-        "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp], i32),
+        "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
+        "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
         "forge_chol_workspace_bytes": ([i64, i64], i64),
         "forge_hessian_permute": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
@@ -60,6 +61,7 @@ EXPORTED_SYMBOLS = (
     "forge_hip_abi_version", "forge_last_error", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
     "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_hessian_update_grouped",
+    "forge_hessian_workspace_bytes",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
 )
@@ -223,16 +225,21 @@ class _HipKernels:
         al = (ctypes.c_float * E)(*[float(a) for a in alpha])
         be = (ctypes.c_float * E)(*[float(b) for b in beta])
         assert X.stride(1) == 1 and H.is_contiguous() and H.dtype == torch.float32
+        total = int(offsets[-1]) - int(offsets[0])
+        nbytes = int(self._lib.forge_hessian_workspace_bytes(total, E, C, _dtype_code(X)))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=X.device)
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_hessian_update_grouped(
-                _ptr(X), _dtype_code(X), X.stride(0), C, offs, E, al, be, _ptr(H), _stream()))
+                _ptr(X), _dtype_code(X), X.stride(0), C, offs, E, al, be, _ptr(H), _ptr(ws),
+                nbytes, _stream()))
         return H
 
     def chol_inv_upper_batched(self, H, damp, normalise=True):
-        """H [B,C,C] f32 (destroyed); damp [B] f32 -> U [B,C,C], udiag [B,C], info [B]."""
+        """H [B,C,C] f32 (destroyed); damp [B] f32 or None -> U [B,C,C], udiag [B,C], info [B]."""
         _need_cuda(H, damp)
         B, C, _ = H.shape
-        assert H.is_contiguous() and H.dtype == torch.float32 and damp.dtype == torch.float32
+        assert H.is_contiguous() and H.dtype == torch.float32
+        assert damp is None or (damp.dtype == torch.float32 and damp.numel() == B)
         U = torch.empty_like(H)
         udiag = torch.empty((B, C), dtype=torch.float32, device=H.device)
         info = torch.empty(B, dtype=torch.int32, device=H.device)
@@ -257,26 +264,30 @@ class _HipKernels:
                 _stream()))
         return Hp, damp
 
-    def weight_to_solver_order(self, W, perm, dead=None):
-        """W [B,R,C] (bf16/f32) -> [B,C,R] f32 with columns taken in perm order."""
-        _need_cuda(W, perm, dead)
+    def weight_to_solver_order(self, W, perm_inv, dead=None):
+        """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c]."""
+        _need_cuda(W, perm_inv, dead)
         B, R, C = W.shape
-        assert W.stride(2) == 1 and perm.dtype == torch.int64 and perm.is_contiguous()
+        assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
+        assert tuple(perm_inv.shape) == (B, C)
+        assert dead is None or (dead.dtype == torch.uint8 and dead.is_contiguous())
         out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
         with torch.cuda.device(W.device):
             self._check(self._lib.forge_weight_to_solver_order(
-                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm), _ptr(dead),
+                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
                 _ptr(out), B, R, C, _stream()))
         return out
 
-    def codes_to_layer_order(self, q, perm):
-        _need_cuda(q, perm)
+    def codes_to_layer_order(self, q, perm_inv):
+        """q [B,C,R] u8 (solver order) -> [B,R,C] u8, out[b, r, c] = q[b, perm_inv[b,c], r]."""
+        _need_cuda(q, perm_inv)
         B, C, R = q.shape
-        assert q.is_contiguous() and q.dtype == torch.uint8 and perm.is_contiguous()
+        assert q.is_contiguous() and q.dtype == torch.uint8 and perm_inv.is_contiguous()
+        assert perm_inv.dtype == torch.int64 and tuple(perm_inv.shape) == (B, C)
         out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
         with torch.cuda.device(q.device):
-            self._check(self._lib.forge_codes_to_layer_order(_ptr(q), _ptr(perm), _ptr(out), B, R,
-                                                             C, _stream()))
+            self._check(self._lib.forge_codes_to_layer_order(_ptr(q), _ptr(perm_inv), _ptr(out), B,
+                                                             R, C, _stream()))
         return out
 
     def pack_int4(self, codes, qzeros, group_size):

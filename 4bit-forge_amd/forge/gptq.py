@@ -1,0 +1,204 @@
+"""Per-layer GPTQ handle on MI355X: drop-in for the reference's ``forge.gptq.GPTQ``.
+
+Same constructor, methods, attributes and return values as forge/gptq.py:10-276 of the
+reference (``update``/``add_batch`` accumulate the Hessian from calibration activations,
+``quantize`` returns ``(qweight [R,C] u8, scales [R*G] f32, qzeros [R*G] f32[, M])``), but
+every stage is a HIP kernel from ``forge.backend.hip``:
+
+=====================  ==============================================================
+reference (torch/CUDA)  here
+=====================  ==============================================================
+``H.addmm_``            ragged rank-k MFMA update (``hessian_update_grouped``)
+``H[perm][:, perm]``    fused gather + dead-column fix-up (``hessian_permute``)
+3 x cuSOLVER            one batched factorisation (``chol_inv_upper_batched``)
+grid kernels            ``quant_grid`` (min/max + shrink search, straight from bf16/f32)
+``repeat_interleave``   none: the sweep looks scales up by group (``g_idx = perm // gs``)
+32-column sweep + SGEMM  128-column register sweep + chained f32 MFMA GEMM
+=====================  ==============================================================
+
+There is no CPU path: tensors must live on the GPU and the HIP library must be built.
+"""
+from __future__ import annotations
+
+import uuid
+
+import torch
+
+from forge.backend.hip import kernels
+
+
+def _as_calibration_rows(X: torch.Tensor, device) -> torch.Tensor:
+    """Flatten to [n, C]; bf16 and f32 are consumed as they are, anything else as f32."""
+    X = X.reshape(-1, X.shape[-1]).to(device=device)
+    if X.dtype not in (torch.bfloat16, torch.float32):
+        X = X.to(torch.float32)
+    if X.stride(-1) != 1:
+        X = X.contiguous()
+    return X
+
+
+class GPTQ(object):
+    def __init__(self, layer, bits: int = 4, group_size: int = 128, symmetric: bool = False,
+                 quantization_scale: str = "mse", quantization_order: str = "activation",
+                 rel_damp: float = 1e-2, algorithm: str = "gptq", owner=None, device=None):
+        if algorithm not in ("gptq", "sparsegptq"):
+            raise NotImplementedError(f"algorithm={algorithm!r}: only 'gptq' and 'sparsegptq' "
+                                      "run on the HIP backend")
+        self.layer = layer
+        self.device = torch.device(device) if device is not None else layer.weight.device
+        if self.device.type != "cuda":
+            raise RuntimeError("forge.gptq.GPTQ runs on the GPU only (device must be a cuda "
+                               f"device, got {self.device}); there is no CPU fallback")
+        self.W = layer.weight.detach().clone().to(self.device)      # [R, C]
+        self.H = None
+        self.num_samples = torch.zeros((), device=self.device, dtype=torch.int64)
+        self._n_host = 0                    # same count, kept on the host: no sync per update
+        self.bits = bits
+        self.group_size = group_size
+        self.symmetric = symmetric
+        self.quantization_scale = quantization_scale
+        self.quantization_order = quantization_order
+        self.rel_damp = rel_damp
+        self.algorithm = algorithm
+        self.owner = owner if owner is not None else self
+        self.perm = None
+        self.perm_inv = None
+        self.pruned_ids = None
+        self.prepared = False
+        self.issue_non_invertible = False
+        self.G = None
+        self.id = uuid.uuid4()
+
+    def _is_owner(self):
+        return self.id == self.owner.id
+
+    # ------------------------------------------------------------------ state
+    @torch.no_grad()
+    def reset(self):
+        self.W = self.layer.weight.detach().clone().to(self.device)
+        self.H = None
+        self.num_samples = torch.zeros((), device=self.device, dtype=torch.int64)
+        self._n_host = 0
+        self.prepared = False
+        self.perm = self.perm_inv = self.pruned_ids = None
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ Hessian
+    @torch.no_grad()
+    def update(self, X: torch.Tensor):
+        """H <- (n/N) H + (2/N) X^T X with N = n + rows(X); the owner accumulates."""
+        if not self._is_owner():
+            return
+        o = self.owner
+        X = _as_calibration_rows(X, o.device)
+        new = int(X.shape[0])
+        if new == 0:
+            return
+        C = int(X.shape[1])
+        n = o._n_host
+        total = n + new
+        if o.H is None:
+            o.H = torch.empty((C, C), dtype=torch.float32, device=o.device)
+        # first call: beta == 0, H is written without being read
+        kernels.hessian_update_grouped(X, [0, new], o.H.view(1, C, C), [2.0 / total], [n / total])
+        o._n_host = total
+        o.num_samples.add_(new)
+
+    add_batch = update
+
+    # ------------------------------------------------------------------ prepare
+    def _copy_owner_state(self):
+        o = self.owner
+        self.H = o.H.clone()
+        self.pruned_ids = o.pruned_ids.clone()
+        self.perm = o.perm.clone()
+        self.perm_inv = o.perm_inv.clone()
+        self.W[:, self.pruned_ids] = 0
+        self.num_samples = o.num_samples.clone()
+        self._n_host = o._n_host
+        self.prepared = True
+
+    @torch.no_grad()
+    def _prep(self):
+        o = self.owner
+        if self._is_owner() and self.prepared:
+            return
+        if not self._is_owner() and o.prepared:
+            if not self.prepared:
+                self._copy_owner_state()
+            return
+        C = int(o.W.shape[-1])
+        if o.H is None or o._n_host == 0 or bool(torch.isnan(o.H).any()):
+            o.H = torch.eye(C, device=o.device, dtype=torch.float32)
+        dead = torch.diag(o.H) == 0
+        o.pruned_ids = dead
+        if o.quantization_order == "activation":
+            diag = torch.where(dead, torch.ones_like(torch.diag(o.H)), torch.diag(o.H))
+            o.perm = torch.argsort(diag, descending=True)
+        else:
+            o.perm = torch.arange(C, device=o.device)
+        o.perm_inv = torch.argsort(o.perm)
+        o.W[:, dead] = 0
+        # H[perm][:, perm] with the dead rows/columns cleared and their diagonal set to 1
+        Hp, _ = kernels.hessian_permute(o.H.view(1, C, C), o.perm.view(1, C),
+                                        dead[o.perm].to(torch.uint8).view(1, C), 0.0)
+        o.H = Hp[0]
+        o.prepared = True
+        if not self._is_owner():
+            self._copy_owner_state()
+
+    # ------------------------------------------------------------------ stages
+    @torch.no_grad()
+    def _quant_grid(self, max_shrink: float = 0.2, n_grid: int = 100, norm: float = 2.4):
+        R, C = self.W.shape
+        mse = self.quantization_scale == "mse"
+        cand = None
+        if mse:
+            cand = torch.linspace(1.0, max_shrink, n_grid, dtype=torch.float32, device=self.device)
+        W = self.W if self.W.dtype in (torch.float32, torch.bfloat16) else self.W.float()
+        scales, qzeros = kernels.quant_grid(W, self.group_size, self.bits, self.symmetric, mse,
+                                            cand, norm)
+        self.G = (C + self.group_size - 1) // self.group_size
+        return scales, qzeros
+
+    @torch.no_grad()
+    def _h_factor(self):
+        """Row-normalised ('gptq') or raw ('sparsegptq') upper Cholesky factor of
+        inv(H + damp I); identity when the factorisation fails.  As in the reference the
+        fix-ups and the damping are applied to self.H in place (forge/gptq.py:143-154), so
+        a non-owner that copies its owner's Hessian afterwards sees the damped matrix."""
+        H = self.H
+        C = int(self.W.shape[-1])
+        zero_cols = self.W.eq(0).all(dim=0)      # original column order, used on permuted H
+        if bool(zero_cols.any()):
+            H[zero_cols, :] = 0
+            H[:, zero_cols] = 0
+            H[zero_cols, zero_cols] = 1.0
+        H.diagonal().add_(float(self.rel_damp) * torch.diag(H).mean())
+        U, _, info = kernels.chol_inv_upper_batched(H.clone().view(1, C, C), None,
+                                                    normalise=self.algorithm == "gptq")
+        if int(info.item()) > 0:
+            self.issue_non_invertible = True
+        return U[0]
+
+    @torch.no_grad()
+    def quantize(self):
+        self._prep()
+        scales, qzeros = self._quant_grid()
+        U = self._h_factor()
+        R, C = self.W.shape
+        G, gs = self.G, self.group_size
+        W = self.W if self.W.dtype in (torch.float32, torch.bfloat16) else self.W.float()
+        X = kernels.weight_to_solver_order(W.view(1, R, C), self.perm_inv.view(1, C))
+        if self.algorithm == "sparsegptq":
+            s_e = scales.view(R, G).repeat_interleave(gs, dim=1)[:, :C].t()[self.perm].contiguous()
+            z_e = qzeros.view(R, G).repeat_interleave(gs, dim=1)[:, :C].t()[self.perm].contiguous()
+            q, M = kernels.sparsegptq14_solver(X[0], U, s_e, z_e, self.bits)
+            qw = kernels.codes_to_layer_order(q.view(1, C, R), self.perm_inv.view(1, C))[0]
+            return qw, scales, qzeros, M
+        g_idx = (self.perm // gs).to(torch.int32).view(1, C)
+        sT = scales.view(R, G).t().contiguous().view(1, G, R)
+        zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
+        q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
+        qw = kernels.codes_to_layer_order(q, self.perm_inv.view(1, C))[0]
+        return qw, scales, qzeros

@@ -100,12 +100,16 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * ([*, C], pitch ldx, dtype x_dtype) are that expert's tokens, and
  *   H[e] <- beta[e]*H[e] + alpha[e] * X_e^T X_e      (H[e] = H + e*C*C, f32 [C,C], full)
  * alpha_host/beta_host [n_groups] are host arrays (the caller owns the running-mean
- * bookkeeping).  Groups with zero rows are left untouched.  bf16 inputs use bf16 MFMA with
- * fp32 accumulation (products exact); f32 inputs use f32 MFMA. */
+ * bookkeeping); H[e] is not read when beta[e] == 0.  Groups with zero rows are left
+ * untouched.  bf16 inputs use bf16 MFMA with fp32 accumulation (products exact); f32
+ * inputs use f32 MFMA.  ws: device workspace of forge_hessian_workspace_bytes(total rows,
+ * n_groups, C, x_dtype).  Synchronises `stream` once (after uploading the group table). */
 int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_t C,
                                  const int64_t* offsets_host, int64_t n_groups,
                                  const float* alpha_host, const float* beta_host, float* H,
-                                 forge_stream_t stream);
+                                 void* ws, int64_t ws_bytes, forge_stream_t stream);
+int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int64_t C,
+                                      int x_dtype);
 
 /* ------------------------------------------------------------------ factorisation */
 
@@ -129,16 +133,17 @@ int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* de
 
 /* ------------------------------------------------------------------ layout helpers */
 
-/* Xout[b][c][r] = (f32) W[b][r][perm[b][c]]   (the W.T[perm] of gptq.py:133), W of dtype
- * w_dtype [R, C] pitch ldw; columns flagged in dead[b] (original order, may be NULL) read
- * as zero. */
+/* Xout[b][perm_inv[b][c]][r] = (f32) W[b][r][c]: the W.T[perm] of gptq.py:133 written as a
+ * scatter of whole rows (perm_inv = argsort(perm), gptq.py:113).  W of dtype w_dtype
+ * [R, C] pitch ldw; columns flagged in dead[b] (u8 [C], original order, may be NULL) read
+ * as zero (gptq.py:115). */
 int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
-                                 const int64_t* perm, const uint8_t* dead, float* Xout,
+                                 const int64_t* perm_inv, const uint8_t* dead, float* Xout,
                                  int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
 
-/* qout[b][r][perm[b][c]] = qin[b][c][r]: back to [R, C] in original column order
+/* qout[b][r][c] = qin[b][perm_inv[b][c]][r]: back to [R, C] in original column order
  * (qweight[perm_inv].T of gptq.py:139). */
-int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm, uint8_t* qout,
+int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm_inv, uint8_t* qout,
                                int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
 
 /* Nibble packing of [R, C] u8 codes into the compressed-tensors "pack-quantized" int32

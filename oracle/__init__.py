@@ -273,11 +273,16 @@ class GPTQ:
         if self.algorithm == "babai":
             raise NotImplementedError("babai is outside the restated path")
         L, info = torch.linalg.cholesky_ex(H, upper=False)
-        Hinv = torch.cholesky_inverse(L, upper=False)
-        U, info2 = torch.linalg.cholesky_ex(Hinv, upper=True)
-        info = info + info2
-        if self.algorithm == "gptq":
-            U = U / U.diag()[:, None]
+        try:
+            Hinv = torch.cholesky_inverse(L, upper=False)
+            U, info2 = torch.linalg.cholesky_ex(Hinv, upper=True)
+            info = info + info2
+            if self.algorithm == "gptq":
+                U = U / U.diag()[:, None]
+        except RuntimeError:
+            # torch's CPU potri raises on a singular factor instead of carrying on; the
+            # outcome the reference codes for is the identity fallback below
+            info = info + 1
         if int(info.item()) > 0:
             self.issue_non_invertible = True
             U = torch.eye(C, dtype=torch.float32)

@@ -1,0 +1,198 @@
+"""End-to-end: forge.gptq.GPTQ / forge.moe.ExpertGroupGPTQ on the GPU against oracle.GPTQ.
+
+Tolerances.  Scales and zeros: equal (MSE: except candidate ties, <= 0.1 % of groups,
+checked in test_gpu_grid).  Codes: with the SAME factor the sweep is bit-exact
+(test_gpu_sweep); end to end the factor comes from a different fp32 algorithm than
+LAPACK's, and GPTQ's rounding decisions amplify last-bit differences of U, so the oracle
+itself moves by FLOOR = flips(LAPACK fp32 factor vs float64 factor) when only its factor's
+rounding changes.  The GPU result must stay within max(1e-3, 3 * FLOOR) of the oracle and
+its layer output error ||WX - QX||^2 within 1 % of the oracle's.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import mathref
+from forge import synth
+from helpers import linear, flip_rate, expand_meta
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _noise_floor(W, o, scales, zeros):
+    """Flips of the oracle's own sweep when its fp32 LAPACK factor is replaced by the
+    float64 factor rounded to fp32 (same prepared Hessian, same grid)."""
+    R, C = W.shape
+    Hd = o.H.double().numpy().copy()                   # damped + permuted (after quantize)
+    U64 = torch.from_numpy(mathref.factor(Hd, 0.0)).float().contiguous()
+    L, _ = torch.linalg.cholesky_ex(o.H)
+    U32 = torch.linalg.cholesky_ex(torch.cholesky_inverse(L), upper=True)[0]
+    U32 = (U32 / U32.diag()[:, None]).contiguous()
+    Wt = o.W.float().t()[o.perm].contiguous()
+    se, ze = o._expand(scales, C, R), o._expand(zeros, C, R)
+    a = oracle.gptq_solver(Wt.clone(), U32, se, ze, 4)
+    b = oracle.gptq_solver(Wt.clone(), U64, se, ze, 4)
+    return flip_rate(a, b)
+
+
+def _run_pair(W, X, chunks=2, **kw):
+    from forge.gptq import GPTQ
+    o = oracle.GPTQ(linear(W), **kw)
+    g = GPTQ(linear(W).to(DEV), device=DEV, **kw)
+    for part in torch.chunk(X, chunks):
+        o.update(part)
+        g.add_batch(part.to(DEV))
+    assert int(g.num_samples) == int(o.num_samples) == X.shape[0]
+    Hrel = ((g.H.cpu().double() - o.H.double()).norm() / o.H.double().norm()).item()
+    assert Hrel < 2e-6
+    H = o.H.double().numpy().copy()
+    return o, g, H
+
+
+@pytest.mark.parametrize("kw", [
+    dict(symmetric=True, quantization_scale="absmax", quantization_order="default"),
+    dict(symmetric=True, quantization_scale="mse", quantization_order="default"),
+    dict(symmetric=False, quantization_scale="mse", quantization_order="activation"),
+    dict(symmetric=False, quantization_scale="absmax", quantization_order="activation", group_size=64),
+], ids=["sym-absmax", "sym-mse", "asym-mse-actorder", "asym-absmax-actorder-g64"])
+def test_dense_layer_end_to_end(kw):
+    case = synth.dense_outlier(R=256, C=1024, n=1024, seed=1)
+    kw = dict(bits=4, rel_damp=0.01, **kw)
+    kw.setdefault("group_size", 128)
+    o, g, H = _run_pair(case.W, case.X, **kw)
+    qo, so, zo = o.quantize()
+    qg, sg, zg = g.quantize()
+    assert qg.dtype == torch.uint8 and tuple(qg.shape) == (256, 1024) and qg.is_contiguous()
+    assert sg.shape == so.shape and zg.shape == zo.shape and g.G == o.G
+    same = so == sg.cpu()
+    assert float((~same).float().mean()) <= 1e-3
+    assert torch.equal(zo[same], zg.cpu()[same])
+    floor = _noise_floor(case.W, o, so, zo)
+    flips = flip_rate(qo, qg)
+    assert flips <= max(1e-3, 3 * floor), (flips, floor)
+    gs = kw["group_size"]
+    Wf = case.W.numpy()
+    eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, gs).numpy(), H)
+    eg = mathref.layer_error(Wf, oracle.dequantize(qg.cpu(), sg.cpu(), zg.cpu(), gs).numpy(), H)
+    assert abs(eg / eo - 1) < 0.01
+
+
+def test_fallbacks_zero_tokens_nan_dead_column_and_non_pd():
+    from forge.gptq import GPTQ
+    g0 = torch.Generator().manual_seed(2)
+    W = 0.02 * torch.randn(64, 256, generator=g0)
+    kw = dict(bits=4, symmetric=True, quantization_scale="absmax", quantization_order="activation")
+
+    def rtn_of(q, s, z):
+        se = expand_meta(s.cpu(), 64, 256, 128).t()
+        ze = expand_meta(z.cpu(), 64, 256, 128).t()
+        return np.array_equal(q.cpu().numpy(), mathref.rtn(W.numpy(), se.numpy(), ze.numpy(), 4))
+
+    h = GPTQ(linear(W).to(DEV), device=DEV, **kw)                        # no tokens: H = I
+    h.update(torch.empty(0, 256, device=DEV))
+    assert rtn_of(*h.quantize())
+    h = GPTQ(linear(W).to(DEV), device=DEV, **kw)                        # NaN activations: H = I
+    X = torch.randn(16, 256, generator=g0); X[3, 7] = float("nan")
+    h.update(X.to(DEV))
+    assert rtn_of(*h.quantize())
+    # dead input feature: pruned, weight column zeroed, same as the oracle
+    X = torch.randn(512, 256, generator=g0) * torch.linspace(0.5, 2.0, 256)
+    X[:, 9] = 0
+    o = oracle.GPTQ(linear(W), **kw); o.update(X)
+    h = GPTQ(linear(W).to(DEV), device=DEV, **kw); h.update(X.to(DEV))
+    qo, so, zo = o.quantize(); qg, sg, zg = h.quantize()
+    assert bool(h.pruned_ids[9]) and int(h.pruned_ids.sum()) == 1
+    assert torch.equal(so, sg.cpu()) and flip_rate(qo, qg) <= 2e-3
+    assert torch.equal(qo[:, 9], qg.cpu()[:, 9])
+    # not positive definite (rank 4, no damping): identity fallback + flag, like gptq.py:172-175
+    h = GPTQ(linear(W).to(DEV), device=DEV, rel_damp=0.0, **kw)
+    h.update((torch.randn(4, 256, generator=g0) + 0.5).to(DEV))
+    assert rtn_of(*h.quantize()) and h.issue_non_invertible
+
+
+def test_owner_sharing_reset_and_in_place_damping():
+    from forge.gptq import GPTQ
+    g0 = torch.Generator().manual_seed(3)
+    Wg, Wu = 0.02 * torch.randn(48, 256, generator=g0), 0.02 * torch.randn(48, 256, generator=g0)
+    X = torch.randn(400, 256, generator=g0) * torch.linspace(0.3, 2.0, 256)
+    kw = dict(bits=4, symmetric=False, quantization_scale="absmax", quantization_order="activation")
+    og = oracle.GPTQ(linear(Wg), **kw); ou = oracle.GPTQ(linear(Wu), owner=og, **kw)
+    hg = GPTQ(linear(Wg).to(DEV), device=DEV, **kw); hu = GPTQ(linear(Wu).to(DEV), device=DEV, owner=hg, **kw)
+    for h in (og, ou):
+        h.update(X)
+    for h in (hg, hu):
+        h.update(X.to(DEV))
+    assert hu.H is None and not hu._is_owner() and hg._is_owner()
+    # owner first, then the non-owner (quant.py:414,514): the non-owner re-damps the
+    # owner's already damped Hessian -- reproduced, see the oracle's host test
+    qo_g, _, _ = og.quantize(); qo_u, so_u, _ = ou.quantize()
+    qg_g, _, _ = hg.quantize(); qg_u, sg_u, _ = hu.quantize()
+    assert torch.equal(hu.perm.cpu(), ou.perm) and int(hu.num_samples) == 400
+    assert torch.equal(so_u, sg_u.cpu())
+    assert flip_rate(qo_g, qg_g) <= 3e-3 and flip_rate(qo_u, qg_u) <= 3e-3
+    ratio = (hu.H.diagonal().cpu() - ou.H.diagonal()).abs().max() / ou.H.diagonal().abs().max()
+    assert ratio < 1e-5                      # both damped twice
+    hg.reset()
+    assert hg.H is None and int(hg.num_samples) == 0 and not hg.prepared and hg.perm is None
+
+
+def test_sparse14_end_to_end():
+    from forge.gptq import GPTQ
+    case = synth.sparse14_down_proj(R=192, C=512, n=1024, seed=4)
+    kw = dict(bits=4, symmetric=True, quantization_scale="mse", quantization_order="default",
+              algorithm="sparsegptq")
+    o, g, H = _run_pair(case.W, case.X, **kw)
+    qo, so, zo, Mo = o.quantize()
+    qg, sg, zg, Mg = g.quantize()
+    assert tuple(Mg.shape) == (16, 192) and Mg.dtype == torch.uint32
+    assert float((so != sg.cpu()).float().mean()) <= 1e-3
+    mask_diff = (Mo.view(torch.int32) != Mg.cpu().view(torch.int32)).float().mean().item()
+    assert mask_diff <= 5e-3 and flip_rate(qo, qg) <= 5e-3
+    bits = lambda M: ((M.view(torch.int32).cpu().numpy().astype(np.uint32)[np.arange(512) // 32]
+                       >> (np.arange(512) % 32)[:, None]) & 1)
+    keep = bits(Mg)
+    assert np.all(keep.reshape(128, 4, 192).sum(axis=1) == 1)           # exactly 1 of 4 kept
+    dq = lambda q, s, z, M: (oracle.dequantize(q, s, z, 128) * torch.from_numpy(bits(M).T.copy()).float()).numpy()
+    eo = mathref.layer_error(case.W.float().numpy(), dq(qo, so, zo, Mo), H)
+    eg = mathref.layer_error(case.W.float().numpy(), dq(qg.cpu(), sg.cpu(), zg.cpu(), Mg), H)
+    assert abs(eg / eo - 1) < 0.01
+
+
+def test_expert_group_matches_per_expert_handles():
+    """Qwen3-shaped miniature: ragged routed tokens, a zero-token expert, gate/up sharing
+    one Hessian and one factorisation, down on its own."""
+    from forge.moe import ExpertGroupGPTQ
+    moe = synth.qwen3_moe(experts=6, n_experts=48, hidden=512, inter=256, tokens=1024, seed=5)
+    E = 6
+    moe.rows[4] = moe.rows[4][:0]                                        # expert without tokens
+    xs, hs = zip(*(moe.expert_inputs(e) for e in range(E)))
+    offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
+    kw = dict(bits=4, group_size=128, symmetric=False, quantization_scale="mse",
+              quantization_order="activation")
+    gu = ExpertGroupGPTQ([moe.Wg[:E].to(DEV), moe.Wu[:E].to(DEV)], device=DEV, **kw)
+    dn = ExpertGroupGPTQ([moe.Wd[:E].to(DEV)], device=DEV, **kw)
+    half = [x.shape[0] // 2 for x in xs]                                 # two ragged calibration passes
+    for sel in (lambda x, h: x[:h], lambda x, h: x[h:]):
+        px = [sel(x, h) for x, h in zip(xs, half)]
+        ph = [sel(y, h) for y, h in zip(hs, half)]
+        o2 = np.concatenate([[0], np.cumsum([p.shape[0] for p in px])])
+        gu.update(torch.cat(px).to(DEV), o2)
+        dn.update(torch.cat(ph).to(DEV), o2)
+    (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=4)
+    (qd, sd, zd), = dn.quantize(chunk=4)
+    worst = 0.0
+    for e in range(E):
+        for W, X, (q, s, z) in ((moe.Wg[e], xs[e], (qg, sg, zg)), (moe.Wu[e], xs[e], (qu, su, zu)),
+                                (moe.Wd[e], hs[e], (qd, sd, zd))):
+            o = oracle.GPTQ(linear(W), **kw)
+            o.update(X)
+            qo, so, zo = o.quantize()
+            assert float((so != s[e].cpu()).float().mean()) <= 2e-3
+            same = so == s[e].cpu()
+            assert torch.equal(zo[same], z[e].cpu()[same])
+            worst = max(worst, flip_rate(qo, q[e]))
+            if X.shape[0] == 0:
+                assert torch.equal(qo, q[e].cpu())                       # H = I: pure RTN, exact
+    assert worst <= 5e-3, worst

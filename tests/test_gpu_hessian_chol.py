@@ -1,0 +1,136 @@
+"""HIP Hessian accumulation, factorisation and layout kernels against float64 closed forms."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mathref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), torch.as_tensor(b).double()
+    return ((a - b).norm() / b.norm()).item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("C", [256, 200, 1000])
+def test_grouped_ragged_hessian(hip, dtype, C):
+    counts = [0, 3, 17, 300, 64, 0, 129]
+    offs = np.concatenate([[0], np.cumsum(counts)])
+    g = torch.Generator().manual_seed(C)
+    X = torch.randn(int(offs[-1]), C, generator=g).to(dtype)
+    E = len(counts)
+    H = torch.full((E, C, C), float("nan"), device=DEV)
+    hip.hessian_update_grouped(X.to(DEV), offs, H, [2.0 / max(c, 1) for c in counts], [0.0] * E)
+    for e, c in enumerate(counts):
+        if c == 0:
+            assert bool(torch.isnan(H[e]).all())            # zero-token expert: untouched
+            continue
+        ref = mathref.hessian([X[offs[e]:offs[e + 1]].double().numpy()])
+        assert _rel(H[e], ref) < 2e-6
+        assert torch.equal(H[e], H[e].t())                  # exactly symmetric
+    # second batch: running mean H <- (n/N) H + (2/N) X^T X   (gptq.py:73-79)
+    X2 = torch.randn(int(offs[-1]), C, generator=g).to(dtype)
+    hip.hessian_update_grouped(X2.to(DEV), offs, H, [2.0 / max(2 * c, 1) for c in counts], [0.5] * E)
+    for e in (1, 3, 6):
+        ref = mathref.hessian([X[offs[e]:offs[e + 1]].double().numpy(),
+                               X2[offs[e]:offs[e + 1]].double().numpy()])
+        assert _rel(H[e], ref) < 2e-6 and torch.equal(H[e], H[e].t())
+
+
+def test_hessian_strided_rows_and_empty_call(hip):
+    X = torch.randn(40, 300, device=DEV).bfloat16()[:, :256]          # row pitch 300
+    H = torch.zeros((1, 256, 256), device=DEV)
+    hip.hessian_update_grouped(X, [0, 40], H, [2.0 / 40], [0.0])
+    assert _rel(H[0], mathref.hessian([X.double().cpu().numpy()])) < 2e-6
+    before = H.clone()
+    hip.hessian_update_grouped(X, [7, 7], H, [1.0], [0.0])            # no rows: no-op
+    assert torch.equal(before, H)
+
+
+@pytest.mark.parametrize("C", [128, 256, 200, 36, 1024])
+@pytest.mark.parametrize("normalise", [True, False])
+def test_factor_matches_float64(hip, C, normalise):
+    B = 3
+    Hs = []
+    for b in range(B):
+        g = torch.Generator().manual_seed(10 * C + b)
+        X = torch.randn(2 * C if b < 2 else max(C // 2, 4), C, generator=g, dtype=torch.float64)
+        X[:, :3] *= 8
+        Hs.append((2.0 / X.shape[0]) * X.T @ X)
+    H = torch.stack(Hs).float()
+    damp = (0.01 * torch.diagonal(H, dim1=1, dim2=2).mean(1)).float()
+    U, ud, info = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV), normalise=normalise)
+    assert info.tolist() == [0] * B
+    for b in range(B):
+        Hd = H[b].double().numpy().copy()
+        Hd[np.diag_indices(C)] += float(damp[b])
+        U0 = np.linalg.cholesky(np.linalg.inv(Hd)).T
+        ref = U0 / np.diag(U0)[:, None] if normalise else U0
+        # rank-deficient Hessian (b == 2) is far worse conditioned
+        assert _rel(U[b], ref) < (2e-4 if b == 2 else 5e-6)
+        assert _rel(ud[b], np.diag(U0).copy()) < (1e-4 if b == 2 else 5e-6)
+        assert int((torch.tril(U[b], -1) != 0).sum()) == 0
+        if normalise:
+            assert bool((U[b].diagonal() == 1).all())
+
+
+def test_factor_failure_gives_identity(hip):
+    H = torch.eye(256).repeat(3, 1, 1)
+    H[1, 100, 100] = -1.0                               # not positive definite
+    H[2, 5, 5] = float("nan")
+    U, ud, info = hip.chol_inv_upper_batched(H.to(DEV), torch.zeros(3, device=DEV))
+    assert info[0].item() == 0 and info[1].item() > 0 and info[2].item() > 0
+    for b in range(3):
+        assert torch.equal(U[b].cpu(), torch.eye(256))
+
+
+def test_layout_kernels(hip):
+    B, R, C = 2, 192, 320
+    g = torch.Generator().manual_seed(0)
+    W = torch.randn(B, R, C, generator=g).bfloat16()
+    perm = torch.stack([torch.randperm(C, generator=g) for _ in range(B)])
+    pinv = torch.argsort(perm, dim=1)
+    dead = (torch.rand(B, C, generator=g) < 0.05).to(torch.uint8)
+    Xo = hip.weight_to_solver_order(W.to(DEV), pinv.to(DEV), dead.to(DEV))
+    q = torch.randint(0, 16, (B, C, R), dtype=torch.uint8, generator=g)
+    qo = hip.codes_to_layer_order(q.to(DEV), pinv.to(DEV))
+    Hh = torch.randn(B, C, C, generator=g)
+    Hh = Hh + Hh.transpose(1, 2)
+    Hp, dmp = hip.hessian_permute(Hh.to(DEV), perm.to(DEV), dead.to(DEV), 0.01)
+    for b in range(B):
+        Wz = W[b].float().clone()
+        Wz[:, dead[b].bool()] = 0
+        assert torch.equal(Xo[b].cpu(), Wz.t()[perm[b]].contiguous())          # W.T[perm]
+        assert torch.equal(qo[b].cpu(), q[b][pinv[b]].t().contiguous())        # q[perm_inv].T
+        ref = Hh[b][perm[b]][:, perm[b]].clone()
+        d = dead[b].bool()
+        ref[d, :] = 0; ref[:, d] = 0; ref[d, d] = 1
+        assert torch.equal(Hp[b].cpu(), ref)
+        assert dmp[b].item() == pytest.approx(0.01 * ref.diag().mean().item(), rel=1e-5)
+    Wf = torch.randn(1, 50, 70, generator=g)                                    # f32, ragged tile
+    ident = torch.arange(70).view(1, 70)
+    assert torch.equal(hip.weight_to_solver_order(Wf.to(DEV), ident.to(DEV)).cpu()[0], Wf[0].t().contiguous())
+
+
+def test_pack_int4_layout(hip):
+    """compressed-tensors 'pack-quantized' int4: eight (code - zero) values per int32,
+    offset binary (+8), lowest nibble first, along the input dimension
+    (consumer: pack_quantized.py:279-313).  parity unpinned against the third-party packer
+    itself (not installed here); pinned against its documented layout."""
+    R, C, gs = 33, 330, 128
+    g = torch.Generator().manual_seed(1)
+    codes = torch.randint(0, 16, (R, C), dtype=torch.uint8, generator=g)
+    G = (C + gs - 1) // gs
+    z = torch.randint(0, 16, (R * G,), generator=g).float()
+    pk = hip.pack_int4(codes.to(DEV), z.to(DEV), gs).cpu()
+    zz = z.view(R, G).repeat_interleave(gs, 1)[:, :C].to(torch.int64)
+    sh = (codes.to(torch.int64) - zz + 8) & 0xF
+    sh = torch.nn.functional.pad(sh, (0, (-C) % 8)).view(R, -1, 8)
+    ref = sum(sh[:, :, k] << (4 * k) for k in range(8))
+    assert torch.equal(pk.to(torch.int64) & 0xFFFFFFFF, ref)
+    pk8 = hip.pack_int4(codes.to(DEV), None, gs).cpu()                 # symmetric: zero = 8
+    sh = torch.nn.functional.pad(codes.to(torch.int64), (0, (-C) % 8)).view(R, -1, 8)
+    assert torch.equal(pk8.to(torch.int64) & 0xFFFFFFFF, sum(sh[:, :, k] << (4 * k) for k in range(8)))

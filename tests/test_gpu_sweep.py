@@ -1,0 +1,103 @@
+"""HIP column sweep against the oracle: bit-exact codes, weights and masks."""
+import pytest
+import torch
+
+import oracle
+from oracle import mathref
+from helpers import random_problem
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("C,R,sym", [(128, 64, True), (256, 130, False), (640, 96, True),
+                                     (200, 77, False), (36, 5, True), (1024, 512, True)])
+def test_gptq_solver_bit_exact(hip, C, R, sym):
+    pr = random_problem(C=C, R=R, sym=sym, seed=C + R)
+    Wt = pr["W"].t().contiguous()
+    q0 = oracle.gptq_solver(Wt.clone(), pr["U"], pr["se"], pr["ze"], 4)
+    W0 = oracle.gptq_solver.last_W
+    Wd = Wt.clone().to(DEV)
+    q1 = hip.gptq_solver(Wd, pr["U"].to(DEV), pr["se"].to(DEV), pr["ze"].to(DEV), 4)
+    assert torch.equal(q0, q1.cpu())
+    assert torch.equal(W0, Wd.cpu())            # contiguous W is overwritten with deq
+
+
+def test_gptq_solver_non_contiguous_input_is_left_alone(hip):
+    pr = random_problem(C=128, R=64)
+    Wd = pr["W"].to(DEV)
+    before = Wd.clone()
+    q1 = hip.gptq_solver(Wd.t(), pr["U"].to(DEV), pr["se"].to(DEV), pr["ze"].to(DEV), 4)
+    q0 = oracle.gptq_solver(pr["W"].t().contiguous(), pr["U"], pr["se"], pr["ze"], 4)
+    assert torch.equal(q0, q1.cpu()) and torch.equal(Wd, before)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 8])
+def test_other_bit_widths(hip, bits):
+    pr = random_problem(C=256, R=64)
+    s, z = oracle.build_group_meta_packed(pr["W"].reshape(-1, 128), bits, False)
+    from helpers import expand_meta
+    se, ze = expand_meta(s, 64, 256, 128), expand_meta(z, 64, 256, 128)
+    Wt = pr["W"].t().contiguous()
+    q0 = oracle.gptq_solver(Wt.clone(), pr["U"], se, ze, bits)
+    q1 = hip.gptq_solver(Wt.clone().to(DEV), pr["U"].to(DEV), se.to(DEV), ze.to(DEV), bits)
+    assert torch.equal(q0, q1.cpu()) and int(q0.max()) <= 2 ** bits - 1
+
+
+@pytest.mark.parametrize("C,R", [(256, 64), (384, 200), (100, 33)])
+def test_sparse14_solver_bit_exact(hip, C, R):
+    pr = random_problem(C=C, R=R, seed=C)
+    U0 = torch.from_numpy(mathref.factor(pr["H"].double().numpy(), 0.01, normalise=False)).float().contiguous()
+    Wt = pr["W"].t().contiguous()
+    Uo = U0.clone()
+    q0, M0 = oracle.sparsegptq14_solver(Wt.clone(), Uo, pr["se"], pr["ze"], 4)
+    W0 = oracle.sparsegptq14_solver.last_W
+    Ud, Wd = U0.clone().to(DEV), Wt.clone().to(DEV)
+    q1, M1 = hip.sparsegptq14_solver(Wd, Ud, pr["se"].to(DEV), pr["ze"].to(DEV), 4)
+    assert torch.equal(q0, q1.cpu())
+    assert torch.equal(M0.view(torch.int32), M1.cpu().view(torch.int32))
+    assert torch.equal(Uo, Ud.cpu())            # caller's U row-normalised in place
+    assert torch.equal(W0, Wd.cpu())
+
+
+@pytest.mark.parametrize("C,R", [(512, 192), (200, 70)])
+def test_batched_sweep_with_group_lookup_and_permutation(hip, C, R):
+    B, gs = 3, 128
+    G = (C + gs - 1) // gs
+    Xs, Us, sT, zT, gi, want = [], [], [], [], [], []
+    for b in range(B):
+        pr = random_problem(C=C, R=R, seed=100 + b, sym=bool(b % 2))
+        perm = torch.randperm(C, generator=torch.Generator().manual_seed(b))
+        Wt = pr["W"].t()[perm].contiguous()
+        se, ze = pr["se"][perm].contiguous(), pr["ze"][perm].contiguous()
+        want.append(oracle.gptq_solver(Wt.clone(), pr["U"], se, ze, 4))
+        Xs.append(Wt); Us.append(pr["U"])
+        sT.append(pr["s"].view(R, G).t().contiguous()); zT.append(pr["z"].view(R, G).t().contiguous())
+        gi.append((perm // gs).int())
+    X = torch.stack(Xs).to(DEV)
+    q = hip.gptq_sweep_batched(X, torch.stack(Us).to(DEV), torch.stack(sT).to(DEV),
+                               torch.stack(zT).to(DEV), torch.stack(gi).to(DEV), 4)
+    for b in range(B):
+        assert torch.equal(want[b], q[b].cpu())
+
+
+def test_full_size_sweep_properties(hip):
+    """Config-1 size (2048 x 2048): U = I must give round-to-nearest bit for bit, and the
+    batched (left-looking) and single-matrix (right-looking) schedules must agree."""
+    C = R = 2048
+    pr = random_problem(C=C, R=R, n=1024, seed=7)
+    Wt = pr["W"].t().contiguous().to(DEV)
+    se, ze = pr["se"].to(DEV), pr["ze"].to(DEV)
+    q_rtn = hip.gptq_solver(Wt.clone(), torch.eye(C, device=DEV), se, ze, 4)
+    ref = torch.clamp(torch.round(torch.addcmul(ze.double(), Wt.double(), (1.0 / (se + 1e-12)).double()).float()), 0, 15)
+    assert torch.equal(q_rtn.float(), ref)
+    U = pr["U"].to(DEV)
+    q_single = hip.gptq_solver(Wt.clone(), U, se, ze, 4)
+    G = C // 128
+    q_batched = hip.gptq_sweep_batched(Wt.clone().view(1, C, R), U.view(1, C, C),
+                                       pr["s"].view(R, G).t().contiguous().view(1, G, R).to(DEV),
+                                       pr["z"].view(R, G).t().contiguous().view(1, G, R).to(DEV),
+                                       (torch.arange(C) // 128).int().view(1, C).to(DEV), 4)
+    assert torch.equal(q_single, q_batched[0])
+    q0 = oracle.gptq_solver(pr["W"].t().contiguous(), pr["U"], pr["se"], pr["ze"], 4)
+    assert torch.equal(q0, q_single.cpu())
