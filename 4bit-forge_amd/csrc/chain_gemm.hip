@@ -201,6 +201,17 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
                         (!g.b_lower_tri || ((g.n0 - g.k0) % TK) == 0);
     const bool edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
                       ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned;
+    // useful flops: 2*M*N*K with K clipped per n-tile for the triangular variants
+    double kn = 0.0;
+    for (int nt = g.n0; nt < g.n1; nt += TN) {
+        int k0 = g.k0, k1 = g.k1;
+        if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
+        if (g.b_lower_tri && k0 < nt) k0 = nt;
+        const int ncols = (g.n1 - nt) < TN ? (g.n1 - nt) : TN;
+        if (k1 > k0) kn += (double)(k1 - k0) * ncols;
+    }
+    KernelTiming timing(g.blocked_sum ? "chain_gemm_blocked_sum" : "chain_gemm", st,
+                        2.0 * (g.m1 - g.m0) * kn * (double)batch, WORK_FLOPS);
     if (g.blocked_sum) {
         if (edge) chain_gemm_kernel<true, 128><<<grid, dim3(256), 0, st>>>(g);
         else chain_gemm_kernel<false, 128><<<grid, dim3(256), 0, st>>>(g);

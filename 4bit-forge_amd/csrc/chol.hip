@@ -189,7 +189,10 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
     FORGE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(diag_block_kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDiagLds));
     FORGE_HIP_CHECK(hipMemsetAsync(info, 0, batch * sizeof(int32_t), st));
-    FORGE_HIP_CHECK(hipMemsetAsync(U, 0, batch * C * C * sizeof(float), st));
+    {
+        forge::KernelTiming timing("chol_clear_u", st, 4.0 * C * C * (double)batch, forge::WORK_BYTES);
+        FORGE_HIP_CHECK(hipMemsetAsync(U, 0, batch * C * C * sizeof(float), st));
+    }
     if (damp) {
         add_damp_kernel<<<dim3((unsigned)forge::ceil_div(C, 256), (unsigned)batch), dim3(256), 0, st>>>(
             H, damp, C);
@@ -206,9 +209,13 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
             g.m0 = m0; g.m1 = m1; g.n0 = 0; g.n1 = m1; g.k0 = m1; g.k1 = (int)C; g.negate_a = true; g.blocked_sum = true;
             if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
         }
-        diag_block_kernel<<<dim3((unsigned)batch), dim3(256), kDiagLds, st>>>(
-            H, U, Dinv, udiag, info, C, a, nblk);
-        FORGE_LAUNCH_CHECK();
+        {
+            forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,
+                                       forge::WORK_FLOPS);
+            diag_block_kernel<<<dim3((unsigned)batch), dim3(256), kDiagLds, st>>>(
+                H, U, Dinv, udiag, info, C, a, nblk);
+            FORGE_LAUNCH_CHECK();
+        }
         // Dinv blocks addressed with global (k, m) indices: shift the base so that
         // element (m0 + k', m0 + m') lands on block entry (k', m').
         const int64_t shift = (int64_t)m0 * NB + m0;
@@ -233,6 +240,7 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
             if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
         }
     }
+    forge::KernelTiming timing("chol_finish_rows", st, 4.0 * C * C * (double)batch, forge::WORK_BYTES);
     finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(U, udiag, info, C,
                                                                                normalise != 0);
     FORGE_LAUNCH_CHECK();

@@ -29,4 +29,20 @@ int fail(int code, const char* fmt, ...);
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Optional per-kernel timing (forge_kernel_timing_* in forge_hip.h).  When enabled, a
+// KernelTiming object brackets one launch with two HIP events on the launch stream and
+// files the pair under `name` together with the launch's algorithmic work (flops or HBM
+// bytes).  Disabled (the default) it does nothing.
+enum WorkKind { WORK_FLOPS = 0, WORK_BYTES = 1 };
+class KernelTiming {
+public:
+    KernelTiming(const char* name, hipStream_t st, double work, WorkKind kind);
+    ~KernelTiming();
+    KernelTiming(const KernelTiming&) = delete;
+    KernelTiming& operator=(const KernelTiming&) = delete;
+private:
+    int slot_;
+    hipStream_t st_;
+};
+
 }  // namespace forge

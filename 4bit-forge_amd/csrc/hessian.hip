@@ -314,10 +314,17 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
         pack_bf16_kernel<<<dim3((unsigned)forge::ceil_div(C, 32), ychunks, (unsigned)n_groups),
                            dim3(64), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev, pack);
         FORGE_LAUNCH_CHECK();
+        // executed flops: tiles on and above the diagonal only
+        forge::KernelTiming timing("hessian_syrk_bf16", st,
+                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
+                                   forge::WORK_FLOPS);
         syrk_bf16_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev, H, C,
                                                                                NT);
         FORGE_LAUNCH_CHECK();
     } else {
+        forge::KernelTiming timing("hessian_syrk_f32", st,
+                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
+                                   forge::WORK_FLOPS);
         syrk_f32_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
             (const float*)X, ldx, gd_dev, H, C, NT);
         FORGE_LAUNCH_CHECK();

@@ -124,6 +124,9 @@ extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t 
     FORGE_REQUIRE(W && perm_inv && Xout, "null pointer");
     dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
     FORGE_REQUIRE(grid.y < 65536, "R too large");
+    forge::KernelTiming timing("weight_to_solver_order", (hipStream_t)stream,
+                               (double)batch * R * C * (4.0 + (w_dtype == FORGE_F32 ? 4.0 : 2.0)),
+                               forge::WORK_BYTES);
     if (w_dtype == FORGE_F32)
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
             (const float*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
@@ -142,6 +145,8 @@ extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* per
     FORGE_REQUIRE(qin && perm_inv && qout, "null pointer");
     dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
     FORGE_REQUIRE(grid.y < 65536, "R too large");
+    forge::KernelTiming timing("codes_to_layer_order", (hipStream_t)stream, 2.0 * batch * R * C,
+                               forge::WORK_BYTES);
     to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
@@ -155,6 +160,7 @@ extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const 
     FORGE_REQUIRE(H && perm && Hp && damp, "null pointer");
     FORGE_REQUIRE(H != Hp, "hessian_permute cannot run in place");
     hipStream_t st = (hipStream_t)stream;
+    forge::KernelTiming timing("hessian_permute", st, 8.0 * C * C * (double)batch, forge::WORK_BYTES);
     hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(H, perm, dead,
                                                                                    Hp, C);
     FORGE_LAUNCH_CHECK();
@@ -169,6 +175,8 @@ extern "C" int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_
     if (R == 0 || C == 0) return FORGE_OK;
     FORGE_REQUIRE(codes && packed, "null pointer");
     const int64_t n = R * ((C + 7) / 8);
+    forge::KernelTiming timing("pack_int4", (hipStream_t)stream,
+                               1.5 * R * C + 4.0 * R * forge::ceil_div(C, gs), forge::WORK_BYTES);
     pack_int4_kernel<<<dim3((unsigned)forge::ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream>>>(
         codes, qzeros, packed, R, C, gs, forge::ceil_div(C, gs));
     FORGE_LAUNCH_CHECK();

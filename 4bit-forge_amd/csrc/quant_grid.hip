@@ -192,6 +192,9 @@ int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, 
                int64_t G, int64_t n_groups, const float* cand, int64_t P, float maxq, float norm,
                bool symmetric, bool search, float* scales, float* qzeros, hipStream_t st) {
     const dim3 block(64), grid((unsigned)forge::ceil_div(n_groups, 64));
+    forge::KernelTiming timing(search ? "mse_grid" : "minmax_grid_lane", st,
+                               (double)n_groups * (gs * sizeof(T) + 8.0 + (FUSED ? 0.0 : 8.0)),
+                               forge::WORK_BYTES);
 #define FORGE_MSE_CASE(GS)                                                                    \
     case GS:                                                                                  \
         mse_grid_kernel<T, GS, FUSED><<<grid, block, 0, st>>>(W, w_stride, R, C, ldw, G,      \
@@ -230,6 +233,8 @@ extern "C" int forge_build_group_meta_packed(const float* X, int64_t RG, int64_t
     const int64_t halves_per_block = 8;
     int64_t blocks = forge::ceil_div(RG, halves_per_block);
     if (blocks > (1 << 20)) blocks = 1 << 20;
+    forge::KernelTiming timing("minmax_grid", (hipStream_t)stream, (double)RG * (gs * 4.0 + 8.0),
+                               forge::WORK_BYTES);
     minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
         X, 0, RG, gs, gs, gs, 1, RG, maxq, symmetric != 0, scales, qzeros);
     FORGE_LAUNCH_CHECK();
@@ -282,6 +287,10 @@ extern "C" int forge_quant_grid(const void* W, int w_dtype, int64_t batch, int64
     }
     int64_t blocks = forge::ceil_div(n_groups, 8);
     if (blocks > (1 << 20)) blocks = 1 << 20;
+    forge::KernelTiming timing("minmax_grid", st,
+                               (double)batch * R * C * (w_dtype == FORGE_F32 ? 4.0 : 2.0) +
+                                   8.0 * n_groups,
+                               forge::WORK_BYTES);
     if (w_dtype == FORGE_F32)
         minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(
             (const float*)W, w_stride, R, C, ldw, gs, G, n_groups, maxq, symmetric != 0, scales,

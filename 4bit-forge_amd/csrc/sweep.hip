@@ -219,6 +219,9 @@ template <bool SPARSE, bool PER_ELEM>
 int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
     dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
     constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
+    forge::KernelTiming timing(SPARSE ? "sweep_block_sparse14" : "sweep_block", st,
+                               (double)a.bw * (a.bw - 1) * (double)a.R * (double)batch,
+                               forge::WORK_FLOPS);
     if (a.bw % 32 == 0)
         sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, false>
             <<<grid, dim3(64), 0, st>>>(a);

@@ -34,6 +34,11 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     sigs = {
         "forge_hip_abi_version": ([], i32),
         "forge_last_error": ([], ctypes.c_char_p),
+        "forge_kernel_timing_enable": ([i32], i32),
+        "forge_kernel_timing_collect": ([], i32),
+        "forge_kernel_timing_get": ([i32, ctypes.c_char_p, i32, ctypes.POINTER(i64),
+                                     ctypes.POINTER(ctypes.c_double),
+                                     ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i32)], i32),
         "forge_build_group_meta_packed": ([vp, i64, i64, i32, i32, vp, vp, vp], i32),
         "forge_mse_scale_groups_packed": ([vp, vp, vp, vp, i64, i64, i64, f32, i32, i32, vp], i32),
         "forge_quant_grid": ([vp, i32, i64, i64, i64, i64, i64, i64, i32, i32, i32, vp, i64, f32,
@@ -58,7 +63,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
 
 
 EXPORTED_SYMBOLS = (
-    "forge_hip_abi_version", "forge_last_error", "forge_build_group_meta_packed",
+    "forge_hip_abi_version", "forge_last_error", "forge_kernel_timing_enable",
+    "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
     "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_hessian_update_grouped",
     "forge_hessian_workspace_bytes",
@@ -108,6 +114,27 @@ class _HipKernels:
     def _check(self, rc: int):
         if rc != 0:
             raise RuntimeError(self._lib.forge_last_error().decode())
+
+    # -- per-kernel timing (benchmarks) ------------------------------------------------
+    def timing_enable(self, on: bool):
+        self._check(self._lib.forge_kernel_timing_enable(int(bool(on))))
+
+    def timing_collect(self):
+        """-> {kernel name: dict(launches, ms, work, unit)} for the launches since enable."""
+        n = self._lib.forge_kernel_timing_collect()
+        if n < 0:
+            raise RuntimeError(self._lib.forge_last_error().decode())
+        out = {}
+        for i in range(n):
+            name = ctypes.create_string_buffer(64)
+            launches, ms, work, kind = (ctypes.c_int64(), ctypes.c_double(), ctypes.c_double(),
+                                        ctypes.c_int())
+            self._check(self._lib.forge_kernel_timing_get(i, name, 64, ctypes.byref(launches),
+                                                          ctypes.byref(ms), ctypes.byref(work),
+                                                          ctypes.byref(kind)))
+            out[name.value.decode()] = dict(launches=launches.value, ms=ms.value, work=work.value,
+                                            unit="flop" if kind.value == 0 else "byte")
+        return out
 
     # -- reference-signature operators -------------------------------------------------
     def build_group_meta_packed(self, X, bit_width, symmetric):

@@ -1,0 +1,230 @@
+"""Benchmark of the GPTQ calibration-and-solve path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config deepseek_v3|qwen3]
+
+Workload (default): the DeepSeek-V3-style MoE layer of the benchmark definition -- 256
+experts, gate/up 2048x7168 and down 7168x2048 (bf16 after an fp8-e4m3 128x128 block-scale
+round trip), 8192 bf16 tokens routed top-8 with Zipf(1.1) popularity, 4-bit symmetric
+g128, act-order, MSE scale search (the GPTQ class default), damp 0.01.  One STEP = one
+pass of the hot path over one chunk of experts, everything already resident in HBM:
+ragged Hessian accumulation for gate/up and for down, then per expert two factorisations
+(gate and up share theirs), three scale searches and three sweeps.  Successive steps walk
+through the layer's experts chunk by chunk (their routed-token lists differ).
+value = experts quantised per second = steps * chunk / elapsed.
+
+After the timed steps one more step runs with the library's per-kernel event timing
+switched on; its dominant kernel gives the `roofline` object.  `cpu_baseline` times the CPU
+oracle (reference-structured: 32-column C kernel + BLAS SGEMM trailing update, LAPACK
+factorisation, OpenMP grid search) on one expert of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
+
+PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, TFLOP/s, GB/s
+KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit)
+    "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s"),
+    "chain_gemm": ("mfma", "mfma_f32", "TFLOP/s"),
+    "hessian_syrk_bf16": ("mfma", "mfma_bf16", "TFLOP/s"),
+    "hessian_syrk_f32": ("mfma", "mfma_f32", "TFLOP/s"),
+}
+
+CONFIGS = {
+    "deepseek_v3": dict(n_experts=256, hidden=7168, inter=2048, tokens=8192, fp8=True,
+                        symmetric=True, order="activation", chunk=32),
+    "qwen3": dict(n_experts=128, hidden=2048, inter=768, tokens=4096, fp8=False,
+                  symmetric=False, order="default", chunk=64),
+}
+
+
+def make_workload(cfg, chunk, seed=0):
+    """Weights of `chunk` experts (reused by every step: values do not change the work) and
+    the routed, expert-sorted activations of ALL experts, on the GPU."""
+    import torch
+    from forge import synth
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(seed)
+    Hd, I, E = cfg["hidden"], cfg["inter"], cfg["n_experts"]
+    X = torch.randn(cfg["tokens"], Hd, generator=g, device=dev).to(torch.bfloat16)
+    rows = synth.route_topk(cfg["tokens"], E, 8, g, device=dev)
+
+    def w(R, C):
+        t = (0.02 * torch.randn(chunk, R, C, generator=g, device=dev)).to(torch.bfloat16)
+        if cfg["fp8"]:
+            for i in range(chunk):
+                t[i] = synth.fp8_block_roundtrip(t[i])
+        return t
+
+    Wg, Wu, Wd = w(I, Hd), w(I, Hd), w(Hd, I)
+    counts = [int(r.numel()) for r in rows]
+    xs = X[torch.cat(rows)].contiguous()                      # gate/up inputs, grouped by expert
+    # down-proj inputs silu(x Wg^T) * (x Wu^T) with the unquantised weights of the chunk's
+    # slot the expert will be solved in (one calibration forward, outside the timed region)
+    hs = torch.empty(xs.shape[0], I, dtype=torch.bfloat16, device=dev)
+    o = 0
+    for e, n in enumerate(counts):
+        if n:
+            x = xs[o:o + n]
+            slot = e % chunk
+            hs[o:o + n] = (torch.nn.functional.silu(x @ Wg[slot].T) * (x @ Wu[slot].T))
+        o += n
+    return dict(Wg=Wg, Wu=Wu, Wd=Wd, xs=xs, hs=hs, counts=counts)
+
+
+def run_step(wl, cfg, chunk, step, mse=True):
+    """Hot path for experts [step*chunk, (step+1)*chunk) of the layer."""
+    from forge.moe import ExpertGroupGPTQ
+    E = cfg["n_experts"]
+    e0 = (step * chunk) % E
+    ids = [(e0 + i) % E for i in range(chunk)]
+    starts = [0]
+    for c in wl["counts"]:
+        starts.append(starts[-1] + c)
+    import torch
+    if ids == list(range(ids[0], ids[0] + chunk)):
+        xs = wl["xs"][starts[ids[0]]:starts[ids[-1] + 1]]
+        hs = wl["hs"][starts[ids[0]]:starts[ids[-1] + 1]]
+    else:
+        xs = torch.cat([wl["xs"][starts[e]:starts[e + 1]] for e in ids])
+        hs = torch.cat([wl["hs"][starts[e]:starts[e + 1]] for e in ids])
+    offs = [0]
+    for e in ids:
+        offs.append(offs[-1] + wl["counts"][e])
+    kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"],
+              quantization_scale="mse" if mse else "absmax", quantization_order=cfg["order"],
+              rel_damp=0.01, device="cuda")
+    gu = ExpertGroupGPTQ([wl["Wg"], wl["Wu"]], **kw)
+    gu.update(xs, offs)
+    out_gu = gu.quantize(chunk=chunk)
+    del gu
+    dn = ExpertGroupGPTQ([wl["Wd"]], **kw)
+    dn.update(hs, offs)
+    out_dn = dn.quantize(chunk=chunk)
+    del dn
+    return out_gu, out_dn
+
+
+def cpu_baseline(wl, cfg, expert_slot=0):
+    """One expert (gate, up, down) on the host cores with the CPU oracle."""
+    import torch
+    import oracle
+    counts = wl["counts"]
+    # an expert with a median token count
+    order = sorted(range(len(counts)), key=lambda e: counts[e])
+    e = order[len(order) // 2]
+    start = sum(counts[:e])
+    x = wl["xs"][start:start + counts[e]].cpu()
+    h = wl["hs"][start:start + counts[e]].cpu()
+    slot = e % wl["Wg"].shape[0]
+    kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"], quantization_scale="mse",
+              quantization_order=cfg["order"], rel_damp=0.01, trail_mode=oracle.TRAIL_BLAS)
+
+    def lin(W):
+        layer = torch.nn.Linear(W.shape[1], W.shape[0], bias=False)
+        layer.weight.data = W.cpu().float().to(torch.bfloat16)
+        return layer
+
+    t0 = time.perf_counter()
+    gate = oracle.GPTQ(lin(wl["Wg"][slot]), **kw)
+    gate.update(x)
+    gate.quantize()
+    # up_proj is a non-owner of gate_proj's Hessian and re-factorises it, as in the
+    # reference's flow (quant.py:382-397,514-517)
+    up = oracle.GPTQ(lin(wl["Wu"][slot]), owner=gate, **kw)
+    up.quantize()
+    down = oracle.GPTQ(lin(wl["Wd"][slot]), **kw)
+    down.update(h)
+    down.quantize()
+    dt = time.perf_counter() - t0
+    return dict(value=1.0 / dt, unit="experts/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"1 expert (gate+up+down, {counts[e]} routed tokens) of the same layer, "
+                       f"{dt:.1f} s on the host; 3 factorisations as in the reference's flow")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", default="deepseek_v3", choices=sorted(CONFIGS))
+    ap.add_argument("--chunk", type=int, default=0, help="experts per step (0 = config default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+              "(experts would shard across GPUs without any exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from forge.backend.hip import kernels
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    cfg = CONFIGS[a.config]
+    chunk = a.chunk or cfg["chunk"]
+    wl = make_workload(cfg, chunk)
+    mse = not a.no_mse
+
+    for i in range(a.warmup):
+        run_step(wl, cfg, chunk, i, mse)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        run_step(wl, cfg, chunk, a.warmup + i, mse)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    # one more step with per-kernel HIP-event timing (on the stream the kernels run on)
+    kernels.timing_enable(True)
+    run_step(wl, cfg, chunk, a.warmup + a.steps, mse)
+    torch.cuda.synchronize()
+    stats = kernels.timing_collect()
+    kernels.timing_enable(False)
+    total_ms = sum(s["ms"] for s in stats.values())
+    breakdown = {}
+    for name, s in sorted(stats.items(), key=lambda kv: -kv[1]["ms"]):
+        rate = s["work"] / (s["ms"] * 1e-3) if s["ms"] > 0 else 0.0
+        breakdown[name] = dict(launches=s["launches"], ms=round(s["ms"], 3),
+                               avg_us=round(1e3 * s["ms"] / max(s["launches"], 1), 2),
+                               share=round(s["ms"] / total_ms, 4),
+                               rate=round(rate / (1e12 if s["unit"] == "flop" else 1e9), 2),
+                               rate_unit="TFLOP/s" if s["unit"] == "flop" else "GB/s")
+    dom = next(iter(breakdown))
+    bound, peak_key, unit = KERNEL_BOUND.get(dom, ("hbm", "hbm", "GB/s"))
+    roofline = dict(kernel=dom, bound=bound, achieved=breakdown[dom]["rate"], peak=PEAK[peak_key],
+                    unit=unit, frac=round(breakdown[dom]["rate"] / PEAK[peak_key], 4), traffic=None,
+                    avg_launch_us=breakdown[dom]["avg_us"], launches=breakdown[dom]["launches"])
+
+    out = {
+        "metric": "experts quantized/sec (GPTQ 4-bit g128)",
+        "value": round(a.steps * chunk / elapsed, 3),
+        "unit": "experts/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(1e3 * elapsed / a.steps, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{a.config}: {cfg['n_experts']} experts, gate/up {cfg['inter']}x{cfg['hidden']}"
+                               f" + down {cfg['hidden']}x{cfg['inter']}, {cfg['tokens']} tokens top-8 Zipf(1.1),"
+                               f" 4-bit {'sym' if cfg['symmetric'] else 'asym'} g128"
+                               f" {'act-order' if cfg['order'] == 'activation' else 'no act-order'}"
+                               f" {'mse' if mse else 'absmax'} grid",
+                   "experts_per_step": chunk},
+        "roofline": roofline,
+        "kernels": breakdown,
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, cfg)
+        out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

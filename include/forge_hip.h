@@ -37,6 +37,17 @@ typedef void* forge_stream_t;
 int forge_hip_abi_version(void);
 const char* forge_last_error(void);
 
+/* Optional per-kernel timing, for benchmarks: while enabled every kernel launch of this
+ * library is bracketed by two HIP events on its stream.  _enable(on) clears all records;
+ * _collect() waits for the bracketed launches and returns the number of distinct kernel
+ * names (negative on error); _get(i) returns name, launches, summed duration (ms) and
+ * summed algorithmic work of entry i (work_kind 0 = flops, 1 = HBM bytes).  No
+ * counterpart in the reference. */
+int forge_kernel_timing_enable(int on);
+int forge_kernel_timing_collect(void);
+int forge_kernel_timing_get(int index, char* name, int name_cap, int64_t* launches,
+                            double* total_ms, double* work, int* work_kind);
+
 /* ------------------------------------------------------------------ quant grid */
 
 /* Replaces kernels.build_group_meta_packed (kernels.cpp:93-97, quant_grid.cu:186-224).

@@ -37,6 +37,7 @@ _LIB = None
 
 TRAIL_CHAIN = 0
 TRAIL_GEMM = 1
+TRAIL_BLAS = 2      # in-block in C, trailing update with torch's CPU SGEMM (addmm_)
 
 
 def build(force: bool = False) -> Path:
@@ -60,8 +61,9 @@ def lib() -> ctypes.CDLL:
         L.oracle_mse_scale_groups.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, f32, i32, vp]
         L.oracle_gptq_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, i32, i64]
         L.oracle_sparsegptq14_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32]
+        L.oracle_gptq_inblock.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i64, vp, vp]
         for f in (L.oracle_build_group_meta, L.oracle_mse_scale_groups, L.oracle_gptq_solver,
-                  L.oracle_sparsegptq14_solver):
+                  L.oracle_sparsegptq14_solver, L.oracle_gptq_inblock):
             f.restype = None
         _LIB = L
     return _LIB
@@ -111,8 +113,20 @@ def gptq_solver(W, U, scales, qzeros, bits, trail_mode: int = TRAIL_CHAIN, block
     U = _f32c(U); scales = _f32c(scales); qzeros = _f32c(qzeros)
     C, R = W.shape
     q = torch.empty((C, R), dtype=torch.uint8)
-    lib().oracle_gptq_solver(W.data_ptr(), U.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-                             int(bits), C, R, q.data_ptr(), int(trail_mode), int(block))
+    if trail_mode == TRAIL_BLAS:
+        # the reference's host loop literally: 32-column kernel, then one SGEMM per block
+        E = torch.empty((block, R), dtype=torch.float32)
+        for start in range(0, C, block):
+            end = min(start + block, C)
+            lib().oracle_gptq_inblock(W.data_ptr(), U.data_ptr(), scales.data_ptr(),
+                                      qzeros.data_ptr(), int(bits), C, R, start, end - start,
+                                      q.data_ptr(), E.data_ptr())
+            if end < C:
+                W[end:].addmm_(U[start:end, end:].t(), E[:end - start], beta=1.0, alpha=-1.0)
+    else:
+        lib().oracle_gptq_solver(W.data_ptr(), U.data_ptr(), scales.data_ptr(),
+                                 qzeros.data_ptr(), int(bits), C, R, q.data_ptr(),
+                                 int(trail_mode), int(block))
     gptq_solver.last_W = W
     return q
 

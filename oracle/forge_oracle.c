@@ -156,6 +156,32 @@ static void trailing_update(float* W, const float* U, const float* E, int64_t C,
     }
 }
 
+/* The in-block kernel alone (solver.cu:26-96) for one block of B <= 256 columns starting at
+ * `start`; E [B,R] receives the errors.  Lets a caller do the trailing update with a BLAS
+ * SGEMM exactly as the reference's host loop does (solver.cu:146-150). */
+void oracle_gptq_inblock(float* W, const float* U, const float* scales, const float* qzeros,
+                         int bits, int64_t C, int64_t R, int64_t start, int64_t B,
+                         uint8_t* qweight, float* E) {
+    const int maxq_i = (1 << bits) - 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r) {
+        float x[256];
+        for (int64_t i = 0; i < B; ++i) x[i] = W[(start + i) * R + r];
+        for (int64_t t = 0; t < B; ++t) {
+            const int64_t c = start + t;
+            const float s = scales[c * R + r], q0 = qzeros[c * R + r];
+            const float inv_s = 1.0f / (s + ORACLE_EPS);
+            float err, deq; uint8_t qb;
+            quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+            qweight[c * R + r] = qb;
+            W[c * R + r] = deq;
+            E[t * R + r] = err;
+            for (int64_t k = t + 1; k < B; ++k)
+                x[k] = fmaf(-U[c * C + start + k], err, x[k]);
+        }
+    }
+}
+
 /* solver.cu:26-154.  W [C,R] fp32 is updated in place to the dequantised weights,
  * qweight [C,R] receives the codes.  U [C,C] is the row-normalised upper factor.
  * scales/qzeros are per element [C,R].  B is the in-block width (reference: 32). */
