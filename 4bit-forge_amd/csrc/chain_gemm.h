@@ -22,6 +22,9 @@ struct GemmArgs {
     bool b_upper_tri;  // Bm[k, n] == 0 for k > n: stop each tile's K loop at its last column
     bool b_lower_tri;  // Bm[k, n] == 0 for k < n: start each tile's K loop at its first column
     bool blocked_sum;  // sum K in blocks of 128 (more accurate; NOT the sweep's single chain)
+    // filled in by launch_chain_gemm
+    int n_tiles, m_tiles;
+    bool xcd_map;
 };
 
 int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);

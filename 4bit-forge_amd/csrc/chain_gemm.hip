@@ -11,7 +11,7 @@
 // quadrant = 2x2 MFMA tiles (64 accumulator registers).  Operands are K-major in memory,
 // so a half-wavefront reads 32 consecutive floats of one k row: global loads are
 // coalesced float4, LDS reads are conflict-free ds_read_b32, and no transpose is needed.
-// K advances 16 rows per stage: the next stage's rows are fetched into registers while
+// K advances TK rows per stage: the next stage's rows are fetched into registers while
 // the current stage's 32 MFMAs per wavefront run, all LDS operands of a stage are read
 // before its first MFMA so the matrix pipe is fed back to back, and the register budget
 // leaves room for two workgroups per CU to cover the barrier between stages.
@@ -21,7 +21,12 @@ namespace forge {
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr int TM = 128, TN = 128, TK = 16;
+constexpr int TM = 128, TN = 128;
+#ifndef FORGE_GEMM_TK
+#define FORGE_GEMM_TK 32
+#endif
+constexpr int TK = FORGE_GEMM_TK;   // k rows per LDS stage
+constexpr int NH = TK / 8;          // float4 loads per thread, operand and stage
 
 // EDGE: bounds-checked loads/stores for tiles that stick out of [m0,m1) x [n0,n1) or a K
 // range that is not a multiple of 16.  CHUNK > 0: every CHUNK k values the running
@@ -37,12 +42,27 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t bz = blockIdx.z;
-    float* __restrict__ X = g.X + bz * g.xs;
-    const float* __restrict__ At = g.At + bz * g.as;
-    const float* __restrict__ Bm = g.Bm + bz * g.bs;
-    const int mt = g.m0 + blockIdx.y * TM;  // first m of this tile
-    const int nt = g.n0 + blockIdx.x * TN;  // first n of this tile
+    // 1-D grid -> (n tile, m tile, matrix).  Workgroups are handed to the 8 XCDs round
+    // robin by linear id, and each XCD has its own L2.  With xcd_map, matrix e is served
+    // by XCD e % 8 only, so the At panel that all of its tiles share is fetched into one L2
+    // once instead of into all eight.
+    const int per_matrix = g.n_tiles * g.m_tiles;
+    int bz, tile;
+    if (g.xcd_map) {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        bz = xcd + 8 * (slot / per_matrix);
+        tile = slot % per_matrix;
+    } else {
+        bz = blockIdx.x / per_matrix;
+        tile = blockIdx.x % per_matrix;
+    }
+    float* __restrict__ X = g.X + (int64_t)bz * g.xs;
+    const float* __restrict__ At = g.At + (int64_t)bz * g.as;
+    const float* __restrict__ Bm = g.Bm + (int64_t)bz * g.bs;
+    const int mt = g.m0 + (tile / g.n_tiles) * TM;  // first m of this tile
+    // triangular operand: K grows with n, so hand out the long tiles first
+    const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile % g.n_tiles : tile % g.n_tiles;
+    const int nt = g.n0 + tn * TN;                  // first n of this tile
     int k0 = g.k0, k1 = g.k1;
     if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
     if (g.b_lower_tri && k0 < nt) k0 = nt;
@@ -83,10 +103,10 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
     const float* pa = At + (int64_t)(k0 + lrow) * g.lda + mt + lcol;
     const float* pb = Bm + (int64_t)(k0 + lrow) * g.ldb + nt + lcol;
     const int64_t a_step8 = 8 * g.lda, b_step8 = 8 * g.ldb;
-    float4 ra[2], rb[2];
+    float4 ra[NH], rb[NH];
     auto fetch = [&](int kk) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < NH; ++h) {
             float4 va, vb;
             if constexpr (!EDGE) {
                 va = *reinterpret_cast<const float4*>(pa + h * a_step8);
@@ -110,12 +130,12 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
             ra[h] = make_float4(sign * va.x, sign * va.y, sign * va.z, sign * va.w);
             rb[h] = vb;
         }
-        pa += 2 * a_step8;
-        pb += 2 * b_step8;
+        pa += NH * a_step8;
+        pb += NH * b_step8;
     };
     auto stage = [&](int buf) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < NH; ++h) {
             *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
             *reinterpret_cast<float4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
         }
@@ -132,22 +152,30 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
     for (int kk = k0; kk < k1; kk += TK) {
         const bool more = kk + TK < k1;
         if (more) fetch(kk + TK);
-        float av[TK / 2][2], bv[TK / 2][2];
+        // 16 k rows (8 MFMA k-pairs) at a time: all their LDS reads first, then 32 MFMAs
 #pragma unroll
-        for (int kp = 0; kp < TK / 2; ++kp)
+        for (int sub = 0; sub < TK / 16; ++sub) {
+            float av[8][2], bv[8][2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                av[kp][i] = As[buf][2 * kp + kr0][a_off + i * 32];
-                bv[kp][i] = Bs[buf][2 * kp + kr0][b_off + i * 32];
-            }
+            for (int kp = 0; kp < 8; ++kp)
 #pragma unroll
-        for (int kp = 0; kp < TK / 2; ++kp)
+                for (int i = 0; i < 2; ++i) {
+                    av[kp][i] = As[buf][sub * 16 + 2 * kp + kr0][a_off + i * 32];
+                    bv[kp][i] = Bs[buf][sub * 16 + 2 * kp + kr0][b_off + i * 32];
+                }
+            // keep every LDS read ahead of its MFMAs (the scheduler would otherwise sink
+            // each read next to its use and expose the LDS latency 8 times)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mi = 0; mi < 2; ++mi)
+            for (int kp = 0; kp < 8; ++kp)
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[kp][mi], bv[kp][ni],
-                                                                       acc[mi][ni], 0, 0, 0);
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[kp][mi], bv[kp][ni],
+                                                                           acc[mi][ni], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         if constexpr (CHUNK > 0) {
             if (++stage_no == CHUNK / TK) {
                 stage_no = 0;
@@ -186,7 +214,8 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
 
 }  // namespace
 
-int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
+int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
+    GemmArgs g = g_in;
     if (g.m1 <= g.m0 || g.n1 <= g.n0 || batch <= 0) return FORGE_OK;
     if (g.k1 <= g.k0 && !g.init_zero) return FORGE_OK;
     // float4 loads need 16-byte aligned rows; anything else takes the scalar EDGE path
@@ -194,8 +223,12 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
                          (g.n0 % 4) == 0 && (g.as % 4) == 0 && (g.bs % 4) == 0 &&
                          (reinterpret_cast<uintptr_t>(g.At) % 16) == 0 &&
                          (reinterpret_cast<uintptr_t>(g.Bm) % 16) == 0;
-    dim3 grid((unsigned)ceil_div(g.n1 - g.n0, TN), (unsigned)ceil_div(g.m1 - g.m0, TM),
-              (unsigned)batch);
+    g.n_tiles = (int)ceil_div(g.n1 - g.n0, TN);
+    g.m_tiles = (int)ceil_div(g.m1 - g.m0, TM);
+    g.xcd_map = (batch % 8) == 0;
+    const int64_t n_wg = (int64_t)g.n_tiles * g.m_tiles * batch;
+    FORGE_REQUIRE(n_wg < (1LL << 31), "chain_gemm: grid too large");
+    dim3 grid((unsigned)n_wg);
     // the triangular K clipping keeps multiples of 16 only when tiles and K origin line up
     const bool tri_ok = (!g.b_upper_tri || ((g.n0 + TN - g.k0) % TK) == 0) &&
                         (!g.b_lower_tri || ((g.n0 - g.k0) % TK) == 0);

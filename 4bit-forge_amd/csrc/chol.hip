@@ -36,15 +36,25 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
 }
 
 // 1b for one diagonal block of every matrix in the batch.  256 threads as a 16x16 grid,
-// thread (ty,tx) owns the 8x8 sub-block P[8ty.., 8tx..] in registers; the pivot row of
-// each elimination step is published through LDS.
+// thread (ty,tx) owns the 8x8 sub-block P[8ty.., 8tx..] in registers.  Each elimination
+// step publishes the (unscaled) pivot row through LDS and costs one barrier:
+//   P[i][j] -= (row[i] / piv) * row[j],   D[c][j] = row[j] / sqrt(piv) afterwards.
+__device__ __forceinline__ void select_row(const float (&P)[8][8], int which, float (&out)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = P[0][j];
+#pragma unroll
+    for (int i = 1; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = (which == i) ? P[i][j] : out[j];
+}
+
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
     float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
     extern __shared__ float smem[];                      // 2 * NB * LDP floats (135 KB)
     float (*Dm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem);
     float (*Zm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem + NB * LDP);
-    __shared__ float s_piv;
+    __shared__ float dsq[NB], drc[NB];
     __shared__ int s_fail;
 
     const int64_t b = blockIdx.x;
@@ -59,7 +69,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int r = 8 * ty + i, c = 8 * tx + j;
-            // symmetric tile: take the lower half that the GEMM keeps exact
+            // symmetric tile: both halves were produced by the same GEMM; read the lower one
             const int rr = r > c ? r : c, cc = r > c ? c : r;
             float v = (r == c) ? 1.0f : 0.0f;
             if (rr < n) v = Ab[(m0 + rr) * C + m0 + cc];
@@ -69,31 +79,20 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
 
     // ---- P = D^T D, eliminating from the last row upwards
     for (int c = NB - 1; c >= 0; --c) {
-        if (ty == (c >> 3) && tx == (c >> 3)) {
+        if (ty == (c >> 3)) {
+            float row[8];
+            select_row(P, c & 7, row);
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (i == (c & 7)) s_piv = P[i][i];
+            for (int j = 0; j < 8; ++j) Dm[c][8 * tx + j] = row[j];
         }
         __syncthreads();
-        const float piv = s_piv;
+        const float piv = Dm[c][c];
         const bool ok = piv > 0.0f;
         if (!ok && tid == 0 && s_fail == 0) s_fail = c + 1;
-        const float d = ok ? sqrtf(piv) : 1.0f;
-        if (ty == (c >> 3)) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (i == (c & 7)) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int col = 8 * tx + j;
-                        Dm[c][col] = col < c ? P[i][j] / d : (col == c ? d : 0.0f);
-                    }
-                }
-        }
-        __syncthreads();
+        const float inv = ok ? 1.0f / piv : 0.0f;
         float ri[8], rj[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ri[i] = Dm[c][8 * ty + i];
+        for (int i = 0; i < 8; ++i) ri[i] = Dm[c][8 * ty + i] * inv;
 #pragma unroll
         for (int j = 0; j < 8; ++j) rj[j] = Dm[c][8 * tx + j];
 #pragma unroll
@@ -101,6 +100,19 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
     }
+    __syncthreads();
+    if (tid < NB) {
+        const float piv = Dm[tid][tid];
+        const float d = piv > 0.0f ? sqrtf(piv) : 1.0f;
+        dsq[tid] = d;
+        drc[tid] = 1.0f / d;
+    }
+    __syncthreads();
+    for (int e = tid; e < NB * NB; e += 256) {
+        const int c = e >> 7, j = e & (NB - 1);
+        Dm[c][j] = j < c ? Dm[c][j] * drc[c] : (j == c ? dsq[c] : 0.0f);
+    }
+    __syncthreads();
 
     // ---- Z = D^-1 (lower), row by row from the top; P now accumulates D[i,k] Z[k,j]
 #pragma unroll
@@ -109,17 +121,14 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
     for (int k = 0; k < NB; ++k) {
         if (ty == (k >> 3)) {
-            const float dkk = Dm[k][k];
+            float row[8];
+            select_row(P, k & 7, row);
+            const float rc = drc[k];
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (i == (k & 7)) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int col = 8 * tx + j;
-                        const float rhs = (col == k ? 1.0f : 0.0f) - P[i][j];
-                        Zm[k][col] = col <= k ? rhs / dkk : 0.0f;
-                    }
-                }
+            for (int j = 0; j < 8; ++j) {
+                const int col = 8 * tx + j;
+                Zm[k][col] = col <= k ? ((col == k ? 1.0f : 0.0f) - row[j]) * rc : 0.0f;
+            }
         }
         __syncthreads();
         float di[8], zj[8];

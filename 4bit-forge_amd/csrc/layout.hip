@@ -6,6 +6,8 @@
 
 namespace {
 
+constexpr int64_t kPermuteLdsFloats = 16384;   // 64 KB of LDS per workgroup at most
+
 __device__ __forceinline__ float ld_as_f32(const float* p) { return *p; }
 __device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
     return __uint_as_float(static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(p)) << 16);
@@ -56,18 +58,25 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
 
 // Hp[b][i][j] = H[b][perm[i]][perm[j]], dead rows/columns zeroed with a unit diagonal
 // (forge/gptq.py:100-103,117,145-149).  One workgroup per output row: the source row is
-// read in scattered order but stays cache resident while it is consumed.
+// streamed into LDS with coalesced loads, gathered from there in permuted order and
+// written out coalesced, so HBM sees one sequential read and one sequential write.
 __global__ __launch_bounds__(256) void hessian_permute_kernel(
     const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
     float* __restrict__ Hp, int64_t C) {
+    extern __shared__ float srow[];                 // C floats, or nothing when C is too large
     const int64_t b = blockIdx.y, i = blockIdx.x;
     const int64_t* __restrict__ pb = perm + b * C;
     const uint8_t* __restrict__ db = dead ? dead + b * C : nullptr;
     const float* __restrict__ src = H + b * C * C + pb[i] * C;
     float* __restrict__ dst = Hp + b * C * C + i * C;
     const bool dead_i = db && db[i];
+    const bool staged = C <= kPermuteLdsFloats;
+    if (staged) {
+        for (int64_t j = threadIdx.x; j < C; j += blockDim.x) srow[j] = src[j];
+        __syncthreads();
+    }
     for (int64_t j = threadIdx.x; j < C; j += blockDim.x) {
-        float v = src[pb[j]];
+        float v = staged ? srow[pb[j]] : src[pb[j]];
         if (dead_i || (db && db[j])) v = (i == j) ? 1.0f : 0.0f;
         dst[j] = v;
     }
@@ -161,8 +170,9 @@ extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const 
     FORGE_REQUIRE(H != Hp, "hessian_permute cannot run in place");
     hipStream_t st = (hipStream_t)stream;
     forge::KernelTiming timing("hessian_permute", st, 8.0 * C * C * (double)batch, forge::WORK_BYTES);
-    hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(H, perm, dead,
-                                                                                   Hp, C);
+    const size_t lds = C <= kPermuteLdsFloats ? (size_t)C * sizeof(float) : 0;
+    hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), lds, st>>>(H, perm, dead,
+                                                                                     Hp, C);
     FORGE_LAUNCH_CHECK();
     damp_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(Hp, damp, rel_damp, C);
     FORGE_LAUNCH_CHECK();

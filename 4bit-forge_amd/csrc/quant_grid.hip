@@ -84,30 +84,51 @@ __device__ __forceinline__ float pow_abs(float e, float norm) {
     return __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(e) * norm);
 }
 
-template <int GS>
-__device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, float rcp,
-                                                float q0, float maxq, float norm) {
+// Loss of one element for one candidate (quant_grid.cu:159-167).
+__device__ __forceinline__ float element_loss(float x, float s, float rcp, float q0, float maxq,
+                                              float norm) {
+    const float q = clampf(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq);
+    const float diff = __builtin_fmaf(q - q0, s, -x);
+    return pow_abs(fmaxf(fabsf(diff), 1e-20f), norm);
+}
+
+// Sum over the 8 "reference lanes" l = Q, Q+4, ..., Q+28 (each the in-order sum of its
+// GS/32 elements), combined exactly as the reference's halving tree combines them:
+// ((p[Q] + p[Q+16]) + (p[Q+8] + p[Q+24])) + ((p[Q+4] + p[Q+20]) + (p[Q+12] + p[Q+28])).
+template <int GS, int Q>
+__device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, float rcp, float q0,
+                                              float maxq, float norm) {
     constexpr int VPL = GS / 32;
-    float part[32];
+    float p[8];
 #pragma unroll
-    for (int l = 0; l < 32; ++l) {
+    for (int j = 0; j < 8; ++j) {
+        const int l = Q + 4 * j;
         float loss = 0.0f;
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) {
-            const float x = v[l + 32 * i];
-            const float q = clampf(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq);
-            const float diff = __builtin_fmaf(q - q0, s, -x);
-            const float e = fmaxf(fabsf(diff), 1e-20f);
-            loss += pow_abs(e, norm);
-        }
-        part[l] = loss;
+        for (int i = 0; i < VPL; ++i) loss += element_loss(v[l + 32 * i], s, rcp, q0, maxq, norm);
+        p[j] = loss;
     }
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) {
-#pragma unroll
-        for (int l = 0; l < off; ++l) part[l] += part[l + off];
-    }
-    return part[0];
+    return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+}
+
+// Loss of one candidate in the reference's summation order (32 lane sums, then the
+// halving tree: total = (Q0 + Q2) + (Q1 + Q3) with Qi the quarter above).  Every term is
+// >= 0 and fp32 addition is monotone, so each partial sum is a lower bound of the total:
+// once it reaches `bound` for every group of the wavefront the candidate cannot be a new
+// strict minimum and the rest of its evaluation is skipped (returns +inf for it).  The
+// selected candidate and its loss are exactly those of the full evaluation.
+template <int GS>
+__device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, float rcp,
+                                                float q0, float maxq, float norm, float bound) {
+    constexpr float kInf = __builtin_inff();
+    const float a0 = quarter_loss<GS, 0>(v, s, rcp, q0, maxq, norm);
+    if (__builtin_amdgcn_ballot_w64(a0 < bound) == 0) return kInf;
+    const float h0 = a0 + quarter_loss<GS, 2>(v, s, rcp, q0, maxq, norm);
+    if (__builtin_amdgcn_ballot_w64(h0 < bound) == 0) return kInf;
+    const float a1 = quarter_loss<GS, 1>(v, s, rcp, q0, maxq, norm);
+    if (__builtin_amdgcn_ballot_w64(h0 + a1 < bound) == 0) return kInf;
+    const float h1 = a1 + quarter_loss<GS, 3>(v, s, rcp, q0, maxq, norm);
+    return h0 + h1;
 }
 
 // One lane per group.  FUSED: derive (sg, q0g) from the group's own extrema first;
@@ -117,8 +138,9 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t G,
     int64_t n_groups, const float* __restrict__ cand, int P, float maxq, float norm,
     bool symmetric, bool search, float* __restrict__ scales, float* __restrict__ qzeros) {
-    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (g >= n_groups) return;
+    // lanes past the end replay the last group (the wavefront votes together below)
+    const int64_t g_raw = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t g = g_raw < n_groups ? g_raw : n_groups - 1;
     const int64_t b = g / (R * G);
     const int64_t rg = g - b * R * G;
     const int64_t r = rg / G, grp = rg - r * G;
@@ -175,7 +197,7 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
             const float s = sg * cand[p];
             const float rcp = 1.0f / (s + kEps);
             const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
-            const float loss = candidate_loss<GS>(v, s, rcp, q0, maxq, norm);
+            const float loss = candidate_loss<GS>(v, s, rcp, q0, maxq, norm, best_loss);
             if (loss < best_loss) {
                 best_loss = loss;
                 best_s = s;
@@ -183,8 +205,10 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
             }
         }
     }
-    scales[g] = best_s;
-    qzeros[g] = best_q;
+    if (g_raw < n_groups) {
+        scales[g] = best_s;
+        qzeros[g] = best_q;
+    }
 }
 
 template <typename T, bool FUSED>

@@ -65,6 +65,10 @@ __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, floa
     err = x - deq;
 }
 
+// Four wavefronts of one matrix per workgroup: they walk the same U rows at the same
+// time, so one CU's scalar cache serves each row segment to all four.
+constexpr int kSweepThreads = 256;
+
 // One wavefront = 64 rows, one lane per row; the row's BW block columns live in x[].
 // The block is walked in sub-blocks of 32 columns: the serial quantise/propagate chain on
 // x[0..31], then those 32 errors are pushed into the block's remaining columns, then x[]
@@ -76,9 +80,9 @@ __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, floa
 // below communicates across lanes.  TAIL is the guarded, slower variant for a block that
 // is not a whole number of 32-column sub-blocks.
 template <int BW, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL>
-__global__ __launch_bounds__(64) void sweep_block_kernel(SweepArgs a) {
+__global__ __launch_bounds__(kSweepThreads) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
-    const int64_t r = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    const int64_t r = (int64_t)blockIdx.x * kSweepThreads + threadIdx.x;
     if (r >= a.R) return;
     const int64_t b = blockIdx.y;
     const int64_t C = a.C, R = a.R;
@@ -217,17 +221,17 @@ __global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ 
 
 template <bool SPARSE, bool PER_ELEM>
 int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
-    dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
+    dim3 grid((unsigned)forge::ceil_div(a.R, kSweepThreads), (unsigned)batch);
     constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
     forge::KernelTiming timing(SPARSE ? "sweep_block_sparse14" : "sweep_block", st,
                                (double)a.bw * (a.bw - 1) * (double)a.R * (double)batch,
                                forge::WORK_FLOPS);
     if (a.bw % 32 == 0)
         sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, false>
-            <<<grid, dim3(64), 0, st>>>(a);
+            <<<grid, dim3(kSweepThreads), 0, st>>>(a);
     else
         sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, true>
-            <<<grid, dim3(64), 0, st>>>(a);
+            <<<grid, dim3(kSweepThreads), 0, st>>>(a);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

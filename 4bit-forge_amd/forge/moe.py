@@ -83,24 +83,22 @@ class ExpertGroupGPTQ:
             self.H = torch.empty((E, C, C), dtype=torch.float32, device=dev)
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
         seen = torch.tensor([n > 0 for n in self.num_samples], device=dev)
-        bad = ~seen
-        if bool(seen.any()):
-            nan = torch.isnan(self.H[seen].diagonal(dim1=1, dim2=2)).any(dim=1)
-            bad[seen.nonzero().flatten()[nan]] = True
+        bad = (~seen) | torch.isnan(self.H.diagonal(dim1=1, dim2=2)).any(dim=1)
         if bool(bad.any()):
             self.H[bad] = torch.eye(C, device=dev, dtype=torch.float32)
+        failed = []
+        side = torch.cuda.Stream(device=dev)          # default priority
 
-        outs = [[None, None, None] for _ in self.W]
-        for i, W in enumerate(self.W):
-            R = W.shape[1]
-            outs[i][0] = torch.empty((E, R, C), dtype=torch.uint8, device=dev)
+        sizes = [int(W.shape[1]) for W in self.W]
+        outs = [[torch.empty((E, R, C), dtype=torch.uint8, device=dev),
+                 torch.empty((E, R * G), dtype=torch.float32, device=dev),
+                 torch.empty((E, R * G), dtype=torch.float32, device=dev)] for R in sizes]
         for e0 in range(0, E, chunk):
             e1 = min(E, e0 + chunk)
             B = e1 - e0
             H = self.H[e0:e1]
             diag = H.diagonal(dim1=1, dim2=2)
             dead = diag == 0                                             # [B, C]
-            has_dead = bool(dead.any())
             if self.quantization_order == "activation":
                 perm = torch.argsort(torch.where(dead, torch.ones_like(diag), diag), dim=1,
                                      descending=True)
@@ -114,34 +112,48 @@ class ExpertGroupGPTQ:
             # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149)
             masks = []
             for W in self.W:
-                Wc = W[e0:e1]
-                zero_cols = ((Wc == 0) | dead[:, None, :]).all(dim=1)
+                zero_cols = ((W[e0:e1] == 0) | dead[:, None, :]).all(dim=1)
                 masks.append((dead_perm | zero_cols).to(torch.uint8).contiguous())
-            shared = all(torch.equal(masks[0], m) for m in masks[1:])
-            U = None
-            for i, W in enumerate(self.W):
-                Wc = W[e0:e1]
+            same = torch.stack([(masks[0] == m).all() for m in masks[1:]] + [~dead.any()])
+            flags = same.cpu().tolist()                                  # the chunk's one host sync
+            shared, has_dead = all(flags[:-1]), not flags[-1]
+            # stacks that share the factor are swept as ONE tall matrix (rows are independent)
+            jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
+            for job in jobs:
+                Wc = self.W[job[0]][e0:e1] if len(job) == 1 else torch.cat(
+                    [self.W[i][e0:e1] for i in job], dim=1)
                 R = Wc.shape[1]
-                if U is None or not shared:
-                    Hp, damp = kernels.hessian_permute(H, perm, masks[i], float(self.rel_damp))
-                    U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True)
-                    del Hp
-                    self.issue_non_invertible[e0:e1] |= (info > 0).cpu()
-                # pruned columns are zero in the reference's W before the grid is built
-                Wsrc = Wc.masked_fill(dead[:, None, :], 0) if has_dead else Wc
-                scales, qzeros = kernels.quant_grid(Wsrc, gs, self.bits, self.symmetric, mse, cand,
-                                                    norm)
-                del Wsrc
+                # the scale search only needs the weights: it runs on a side stream so that
+                # its VALU/transcendental work shares the CUs with the MFMA-bound factorisation
+                main = torch.cuda.current_stream()
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    # pruned columns are zero in the reference's W before the grid is built
+                    Wsrc = Wc.masked_fill(dead[:, None, :], 0) if has_dead else Wc
+                    scales, qzeros = kernels.quant_grid(Wsrc, gs, self.bits, self.symmetric, mse,
+                                                        cand, norm)
+                    sT = scales.view(B, R, G).transpose(1, 2).contiguous()
+                    zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
+                    Wsrc.record_stream(side)
+                    del Wsrc
+                Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
+                U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True)
+                del Hp
+                failed.append((e0, info))
                 X = kernels.weight_to_solver_order(Wc, perm_inv, dead_u8)
-                sT = scales.view(B, R, G).transpose(1, 2).contiguous()
-                zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
+                main.wait_stream(side)
+                for t in (scales, qzeros, sT, zT):
+                    t.record_stream(main)
                 q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
-                del X
-                outs[i][0][e0:e1] = kernels.codes_to_layer_order(q, perm_inv)
-                if outs[i][1] is None:
-                    outs[i][1] = torch.empty((E, R * G), dtype=torch.float32, device=dev)
-                    outs[i][2] = torch.empty((E, R * G), dtype=torch.float32, device=dev)
-                outs[i][1][e0:e1] = scales
-                outs[i][2][e0:e1] = qzeros
-            del U
+                del X, U
+                q = kernels.codes_to_layer_order(q, perm_inv)
+                r0 = 0
+                for i in job:
+                    Ri = sizes[i]
+                    outs[i][0][e0:e1] = q[:, r0:r0 + Ri]
+                    outs[i][1][e0:e1] = scales.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
+                    outs[i][2][e0:e1] = qzeros.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
+                    r0 += Ri
+        for e0, info in failed:
+            self.issue_non_invertible[e0:e0 + info.numel()] |= (info > 0).cpu()
         return [tuple(o) for o in outs]
