@@ -173,6 +173,9 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="experts per step (0 = config default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run of "
+                         "this command shows what FETCH_SIZE/WRITE_SIZE read for known traffic")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -188,6 +191,13 @@ def main():
     mse = not a.no_mse
     STREAMS.extend([torch.cuda.Stream(), torch.cuda.Stream()])      # default priority
 
+    if a.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        src.zero_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for i in range(a.warmup):
         run_step(wl, cfg, chunk, i, mse)
     torch.cuda.synchronize()
