@@ -176,13 +176,13 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
     }
 
     float sg, q0g;
-    if constexpr (FUSED) {
-        float lo = 1e30f, hi = -1e30f;
+    float lo = 1e30f, hi = -1e30f;
 #pragma unroll
-        for (int i = 0; i < GS; ++i) {
-            hi = fmaxf(hi, v[i]);
-            lo = fminf(lo, v[i]);
-        }
+    for (int i = 0; i < GS; ++i) {
+        hi = fmaxf(hi, v[i]);
+        lo = fminf(lo, v[i]);
+    }
+    if constexpr (FUSED) {
         meta_from_extrema(lo, hi, maxq, symmetric, sg, q0g);
     } else {
         sg = scales[g];
@@ -197,6 +197,13 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
             const float s = sg * cand[p];
             const float rcp = 1.0f / (s + kEps);
             const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
+            // The group's extreme values are two of the summands; shrinking the scale clips
+            // them first.  A single summand is a lower bound of the (monotone, non-negative)
+            // fp32 sum, so once it reaches the best loss for every group of the wavefront
+            // the candidate is out without touching the other gs-2 elements.
+            const float clip = fmaxf(element_loss(lo, s, rcp, q0, maxq, norm),
+                                     element_loss(hi, s, rcp, q0, maxq, norm));
+            if (__builtin_amdgcn_ballot_w64(clip < best_loss) == 0) continue;
             const float loss = candidate_loss<GS>(v, s, rcp, q0, maxq, norm, best_loss);
             if (loss < best_loss) {
                 best_loss = loss;
