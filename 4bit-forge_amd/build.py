@@ -23,6 +23,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the register-resident sweep relies on `#pragma unroll` of large bodies being honoured
+    "-mllvm", "-pragma-unroll-threshold=200000",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 

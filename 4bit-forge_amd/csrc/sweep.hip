@@ -46,16 +46,6 @@ struct SweepArgs {
     int maxq;
 };
 
-// 16 consecutive floats of a row of U, wave-uniform, fetched with one s_load_dwordx16
-// (viewing U through the constant address space makes the compiler use scalar loads;
-// valid because no kernel in this file writes the factor it reads).
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x16_a4 __attribute__((ext_vector_type(16), aligned(4)));
-__device__ __forceinline__ f32x16 load_u16(const float* p) {
-    typedef const __attribute__((address_space(4))) f32x16_a4* vptr;
-    return *(vptr)(p);
-}
-
 // Quantise one value (solver.cu:9-23): code, dequantised value and error.
 __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, float maxq, float& qf,
                                                 float& deq, float& err) {
@@ -65,24 +55,29 @@ __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, floa
     err = x - deq;
 }
 
-// Four wavefronts of one matrix per workgroup: they walk the same U rows at the same
-// time, so one CU's scalar cache serves each row segment to all four.
-constexpr int kSweepThreads = 256;
+#ifndef FORGE_SWEEP_RING
+#define FORGE_SWEEP_RING 3
+#endif
 
-// One wavefront = 64 rows, one lane per row; the row's BW block columns live in x[].
-// The block is walked in sub-blocks of 32 columns: the serial quantise/propagate chain on
-// x[0..31], then those 32 errors are pushed into the block's remaining columns, then x[]
-// is shifted down by 32 so that the next sub-block again sits in x[0..31] (this keeps the
-// unrolled code at one sub-block's size).  U[t,k] is wave-uniform: each 16-wide row
-// segment is fetched with a scalar load one step ahead of its use and v_fma takes it as
-// an SGPR operand; scheduling barriers keep the compiler from hoisting all those loads to
-// the top (which would spill SGPRs).  Lanes past the last row leave at once: nothing
-// below communicates across lanes.  TAIL is the guarded, slower variant for a block that
-// is not a whole number of 32-column sub-blocks.
-template <int BW, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL>
-__global__ __launch_bounds__(kSweepThreads) void sweep_block_kernel(SweepArgs a) {
+// One lane per output row; the row's BW block columns live in x[].  The block is walked
+// in sub-blocks of 32 columns: the serial quantise/propagate chain on x[0..31], then
+// those 32 errors are pushed into the block's remaining columns, then x[] is shifted down
+// by 32 so that the next sub-block again sits in x[0..31] (this keeps the unrolled code at
+// one sub-block's size).  U[t,k] is the same for every lane: the workgroup stages the
+// 32-row panel of U that a sub-block needs in LDS (the next panel is fetched into
+// registers while the current one is used) and every fma takes its U operand from a
+// broadcast ds_read.  TAIL is the guarded, slower variant (U straight from global memory)
+// for blocks that are not a whole number of 32-column sub-blocks or whose U rows are not
+// 16-byte aligned.
+template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL>
+__global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
-    const int64_t r = (int64_t)blockIdx.x * kSweepThreads + threadIdx.x;
+    constexpr int RING = FORGE_SWEEP_RING;   // LDS read-ahead: RING-1 steps of 16 columns
+    __shared__ __attribute__((aligned(16))) float Up[TAIL ? 1 : 2][TAIL ? 1 : SB][TAIL ? 4 : BW];
+    // Lanes past the last row leave at once; that only happens in the TAIL variant (the
+    // LDS-staged variants are launched for whole wavefronts only: every lane loads its
+    // share of the panel and meets the others at the barriers).
+    const int64_t r = (int64_t)blockIdx.x * NT + threadIdx.x;
     if (r >= a.R) return;
     const int64_t b = blockIdx.y;
     const int64_t C = a.C, R = a.R;
@@ -102,6 +97,18 @@ __global__ __launch_bounds__(kSweepThreads) void sweep_block_kernel(SweepArgs a)
     float x[BW];
 #pragma unroll
     for (int i = 0; i < BW; ++i) x[i] = (i < bw) ? A[(a.c0 + i) * R] : 0.0f;
+
+    int buf = 0;
+    if constexpr (!TAIL) {
+        // first panel: rows c0..c0+31, columns c0..c0+bw-1
+        const int w4 = bw / 4;
+        for (int idx = threadIdx.x; idx < SB * w4; idx += NT) {
+            const int t = idx / w4, j = idx - t * w4;
+            *reinterpret_cast<float4*>(&Up[0][t][4 * j]) =
+                *reinterpret_cast<const float4*>(U + (a.c0 + t) * C + a.c0 + 4 * j);
+        }
+        __syncthreads();
+    }
 
     for (int sb = 0; sb < nsub; ++sb) {
         const int64_t cs = a.c0 + (int64_t)sb * SB;   // first column of this sub-block
@@ -154,45 +161,96 @@ __global__ __launch_bounds__(kSweepThreads) void sweep_block_kernel(SweepArgs a)
         };
 
         if constexpr (!TAIL) {
-            // serial chain inside the sub-block; U row t = two 16-wide halves
-            f32x16 cur = load_u16(U + cs * C + cs);
+            // fetch the next sub-block's panel (rows cs+32.., columns cs+32..) into registers
+            const bool more = sb + 1 < nsub;
+            float4 nxt[(NSB - 1) * (256 / NT)];
+            if (more) {
+                const int w4 = (rem - SB) / 4;               // float4 per panel row
 #pragma unroll
-            for (int t = 0; t < SB; ++t) {
-                const f32x16 hi = load_u16(U + (cs + t) * C + cs + 16);
-                select_and_quantize(t, cs + t);
-                if (t < 15) {
-#pragma unroll
-                    for (int k = t + 1; k < 16; ++k) x[k] = __builtin_fmaf(-cur[k], err[t], x[k]);
+                for (int i = 0; i < (NSB - 1) * (256 / NT); ++i) {
+                    const int idx = threadIdx.x + i * NT;
+                    if (idx < SB * w4) {
+                        const int t = idx / w4, j = idx - t * w4;
+                        nxt[i] = *reinterpret_cast<const float4*>(U + (cs + SB + t) * C + cs + SB + 4 * j);
+                    }
                 }
-                if (t + 1 < SB) cur = load_u16(U + (cs + t + 1) * C + cs);
-                __builtin_amdgcn_sched_barrier(0);
+            }
+            // U operands come from LDS 16 columns (4 broadcast ds_read_b128) at a time, read
+            // two steps ahead of their use; scheduling barriers pin that distance (left
+            // alone the scheduler hoists hundreds of reads and spills the x registers).
+            // serial chain inside the sub-block: step = (row t, half h) -> 2*SB steps
+            {
+                float4 ring[RING][4];
+                auto rd = [&](int step, float4 (&dst)[4]) {
+                    const float4* p = reinterpret_cast<const float4*>(&Up[buf][step >> 1][(step & 1) * 16]);
 #pragma unroll
-                for (int k = (t + 1 > 16 ? t + 1 : 16); k < SB; ++k)
-                    x[k] = __builtin_fmaf(-hi[k - 16], err[t], x[k]);
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int j = 0; j < 4; ++j) dst[j] = p[j];
+                };
+                rd(0, ring[0]);
+                if (RING > 2) rd(1, ring[1]);
+#pragma unroll
+                for (int step = 0; step < 2 * SB; ++step) {
+                    const int t = step >> 1, h = step & 1;
+                    if (step + RING - 1 < 2 * SB) rd(step + RING - 1, ring[(step + RING - 1) % RING]);
+                    if (h == 0) select_and_quantize(t, cs + t);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const float4(&u4)[4] = ring[step % RING];
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) {
+                        const int col = h * 16 + k;
+                        if (col > t) {
+                            const float4 q4 = u4[k >> 2];
+                            const float uv = (k & 3) == 0 ? q4.x : (k & 3) == 1 ? q4.y : (k & 3) == 2 ? q4.z : q4.w;
+                            x[col] = __builtin_fmaf(-uv, err[t], x[col]);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             if constexpr (SPARSE) Mw[(cs >> 5) * R] = mask;
-            // push the 32 errors into the rest of the block, 16 columns of one U row a step
+            // push the 32 errors into the rest of the block
 #pragma unroll
             for (int u = 1; u < NSB; ++u) {
                 if (sb + u < nsub) {
-                    const float* Ub = U + cs * C + cs + u * SB;
-                    f32x16 c2 = load_u16(Ub);
+                    float4 ring[RING][4];
+                    auto rd = [&](int step, float4 (&dst)[4]) {
+                        const float4* p = reinterpret_cast<const float4*>(
+                            &Up[buf][step >> 1][u * SB + (step & 1) * 16]);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) dst[j] = p[j];
+                    };
+                    rd(0, ring[0]);
+                    if (RING > 2) rd(1, ring[1]);
 #pragma unroll
                     for (int step = 0; step < 2 * SB; ++step) {
                         const int t = step >> 1, h = step & 1;
-                        f32x16 n2 = c2;
-                        if (step + 1 < 2 * SB)
-                            n2 = load_u16(Ub + (int64_t)((step + 1) >> 1) * C + ((step + 1) & 1) * 16);
+                        if (step + RING - 1 < 2 * SB) rd(step + RING - 1, ring[(step + RING - 1) % RING]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        const float4(&u4)[4] = ring[step % RING];
 #pragma unroll
-                        for (int k = 0; k < 16; ++k)
-                            x[u * SB + h * 16 + k] =
-                                __builtin_fmaf(-c2[k], err[t], x[u * SB + h * 16 + k]);
-                        c2 = n2;
+                        for (int k = 0; k < 16; ++k) {
+                            const int col = u * SB + h * 16 + k;
+                            const float4 q4 = u4[k >> 2];
+                            const float uv = (k & 3) == 0 ? q4.x : (k & 3) == 1 ? q4.y : (k & 3) == 2 ? q4.z : q4.w;
+                            x[col] = __builtin_fmaf(-uv, err[t], x[col]);
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
+            if (more) {
+                const int w4 = (rem - SB) / 4;
+#pragma unroll
+                for (int i = 0; i < (NSB - 1) * (256 / NT); ++i) {
+                    const int idx = threadIdx.x + i * NT;
+                    if (idx < SB * w4) {
+                        const int t = idx / w4, j = idx - t * w4;
+                        *reinterpret_cast<float4*>(&Up[buf ^ 1][t][4 * j]) = nxt[i];
+                    }
+                }
+            }
+            __syncthreads();
+            buf ^= 1;
         } else {
 #pragma unroll 1
             for (int t = 0; t < SB; ++t) {
@@ -221,17 +279,26 @@ __global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ 
 
 template <bool SPARSE, bool PER_ELEM>
 int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
-    dim3 grid((unsigned)forge::ceil_div(a.R, kSweepThreads), (unsigned)batch);
     constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
     forge::KernelTiming timing(SPARSE ? "sweep_block_sparse14" : "sweep_block", st,
                                (double)a.bw * (a.bw - 1) * (double)a.R * (double)batch,
                                forge::WORK_FLOPS);
-    if (a.bw % 32 == 0)
-        sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, false>
-            <<<grid, dim3(kSweepThreads), 0, st>>>(a);
-    else
-        sweep_block_kernel<forge_kBW, SPARSE, PER_ELEM, ERR_IN_A, true>
-            <<<grid, dim3(kSweepThreads), 0, st>>>(a);
+    // the LDS-staged variants need whole wavefronts (every lane helps to load the panel)
+    const bool fast = a.bw % 32 == 0 && a.C % 4 == 0 && a.c0 % 4 == 0 && a.R % 64 == 0 &&
+                      (reinterpret_cast<uintptr_t>(a.U) % 16) == 0;
+    if (fast && a.R % 256 == 0) {
+        dim3 grid((unsigned)(a.R / 256), (unsigned)batch);
+        sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false>
+            <<<grid, dim3(256), 0, st>>>(a);
+    } else {
+        dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
+        if (fast)
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, false>
+                <<<grid, dim3(64), 0, st>>>(a);
+        else
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, true>
+                <<<grid, dim3(64), 0, st>>>(a);
+    }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }
