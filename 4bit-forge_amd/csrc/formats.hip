@@ -1,0 +1,137 @@
+// Data formats either side of the solve: the fp8 block-scaled checkpoint weights that
+// come in, and the 1:4 sparse int4 words that go out.  Both are HBM-bound byte movers.
+#include "common.h"
+
+namespace {
+
+// OCP float8 e4m3fn (1-4-3, bias 7, no infinities, 0x7f/0xff = NaN) -> f32, exact.
+__device__ __forceinline__ float e4m3fn_to_f32(uint32_t b) {
+    const uint32_t sign = (b & 0x80u) << 24;
+    const uint32_t exp = (b >> 3) & 0xFu, man = b & 0x7u;
+    uint32_t bits;
+    if (exp == 0xFu && man == 0x7u) {
+        bits = 0x7FC00000u;                                   // NaN
+    } else if (exp == 0) {
+        // subnormal: man * 2^-9  (exact in f32)
+        return __uint_as_float(sign | __float_as_uint((float)man * 0.001953125f));
+    } else {
+        bits = ((exp + 120u) << 23) | (man << 20);            // 127 - 7 = 120
+    }
+    return __uint_as_float(sign | bits);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);   // quiet NaN
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// w = fp8.to(f32) * scale_inv[row / so][col / si] -> bf16 (or f32); 16 bytes in per thread
+// (forge/utils/io.py:533-563, 863-872).
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void fp8_block_dequant_kernel(
+    const uint8_t* __restrict__ w, const float* __restrict__ sinv, void* __restrict__ out,
+    int64_t O, int64_t I, int64_t so, int64_t si, int64_t nO, int64_t nI, int64_t batch) {
+    const int64_t per_row = (I + 15) / 16;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= batch * O * per_row) return;
+    const int64_t b = idx / (O * per_row);
+    const int64_t rem = idx - b * O * per_row;
+    const int64_t r = rem / per_row, c0 = (rem - r * per_row) * 16;
+    const uint8_t* src = w + (b * O + r) * I + c0;
+    const float* srow = sinv + (b * nO + r / so) * nI;
+    const int n = (int)((I - c0) < 16 ? (I - c0) : 16);
+    uint8_t v[16];
+    if (n == 16 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(src);
+    } else {
+        for (int i = 0; i < n; ++i) v[i] = src[i];
+    }
+    for (int i = 0; i < n; ++i) {
+        const float f = e4m3fn_to_f32(v[i]) * srow[(c0 + i) / si];
+        const int64_t o = (b * O + r) * I + c0 + i;
+        if (OUT_BF16) reinterpret_cast<uint16_t*>(out)[o] = f32_to_bf16_rne(f);
+        else reinterpret_cast<float*>(out)[o] = f;
+    }
+}
+
+// One thread per (pair of 32-column words, row): two u64 =
+//   bf16(scale) << 48 | idx16 << 32 | qw32
+// qw32: eight 4-bit codes (default 8 = zero weight), idx16: eight 2-bit positions of the
+// kept column inside its group of four (bitpacking_sparsegptq14.cu:58-107).
+__global__ __launch_bounds__(256) void pack_sparse14_kernel(
+    const uint8_t* __restrict__ q_rc, const uint32_t* __restrict__ M,
+    const float* __restrict__ scales, uint64_t* __restrict__ out, int64_t C, int64_t R, int64_t G32) {
+    const int64_t G2 = (G32 + 1) >> 1;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t r = tid % R, g2 = tid / R;
+    if (g2 >= G2) return;
+    uint64_t word[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int64_t gid = 2 * g2 + h;
+        uint64_t packed = 0ull;
+        if (gid < G32) {
+            const uint32_t bitmask = M[gid * R + r];
+            uint32_t idx16 = 0, qw32 = 0x88888888u;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t sub = (bitmask >> (4 * i)) & 0xFu;
+                if (sub == 0u) continue;
+                const int c = __ffs((int)sub) - 1;
+                idx16 |= (uint32_t)(c & 3) << (2 * i);
+                const int64_t cid = gid * 32 + i * 4 + c;
+                if (cid < C) {
+                    const uint32_t q = q_rc[r * C + cid] & 0xFu;
+                    qw32 = (qw32 & ~(0xFu << (4 * i))) | (q << (4 * i));
+                }
+            }
+            packed = ((uint64_t)f32_to_bf16_rne(scales[gid * R + r]) << 48) |
+                     ((uint64_t)(idx16 & 0xFFFFu) << 32) | (uint64_t)qw32;
+        }
+        word[h] = packed;
+    }
+    out[(g2 * R + r) * 2 + 0] = word[0];
+    out[(g2 * R + r) * 2 + 1] = word[1];
+}
+
+}  // namespace
+
+extern "C" int forge_fp8_e4m3_block_dequant(const uint8_t* w, const float* scale_inv, void* out,
+                                            int out_dtype, int64_t batch, int64_t O, int64_t I,
+                                            int64_t so, int64_t si, forge_stream_t stream) {
+    FORGE_REQUIRE(out_dtype == FORGE_F32 || out_dtype == FORGE_BF16, "out_dtype=%d", out_dtype);
+    FORGE_REQUIRE(batch >= 0 && O >= 0 && I >= 0 && so >= 1 && si >= 1, "bad shape");
+    if (batch == 0 || O == 0 || I == 0) return FORGE_OK;
+    FORGE_REQUIRE(w && scale_inv && out, "null pointer");
+    const int64_t nO = forge::ceil_div(O, so), nI = forge::ceil_div(I, si);
+    const int64_t n = batch * O * forge::ceil_div(I, 16);
+    forge::KernelTiming timing("fp8_block_dequant", (hipStream_t)stream,
+                               (double)batch * O * I * (out_dtype == FORGE_BF16 ? 3.0 : 5.0),
+                               forge::WORK_BYTES);
+    dim3 grid((unsigned)forge::ceil_div(n, 256));
+    if (out_dtype == FORGE_BF16)
+        fp8_block_dequant_kernel<true><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
+            w, scale_inv, out, O, I, so, si, nO, nI, batch);
+    else
+        fp8_block_dequant_kernel<false><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
+            w, scale_inv, out, O, I, so, si, nO, nI, batch);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_pack_sparsegptq14_to_u64x2(const uint8_t* qweight_rc, const uint32_t* M,
+                                                const float* scales, uint64_t* out, int64_t R,
+                                                int64_t C, forge_stream_t stream) {
+    FORGE_REQUIRE(R >= 0 && C >= 0, "bad shape");
+    if (R == 0 || C == 0) return FORGE_OK;
+    FORGE_REQUIRE(qweight_rc && M && scales && out, "null pointer");
+    const int64_t G32 = forge::ceil_div(C, 32), G2 = (G32 + 1) >> 1;
+    forge::KernelTiming timing("pack_sparse14_u64x2", (hipStream_t)stream,
+                               (double)R * C / 4.0 + 8.0 * G32 * R + 16.0 * G2 * R, forge::WORK_BYTES);
+    pack_sparse14_kernel<<<dim3((unsigned)forge::ceil_div(G2 * R, 256)), dim3(256), 0,
+                           (hipStream_t)stream>>>(qweight_rc, M, scales, out, C, R, G32);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}

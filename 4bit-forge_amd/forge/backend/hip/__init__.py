@@ -55,6 +55,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_weight_to_solver_order": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_pack_int4": ([vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_fp8_e4m3_block_dequant": ([vp, vp, vp, i32, i64, i64, i64, i64, i64, vp], i32),
+        "forge_pack_sparsegptq14_to_u64x2": ([vp, vp, vp, vp, i64, i64, vp], i32),
     }
     for name, (args, res) in sigs.items():
         fn = getattr(lib, name)          # AttributeError here = library/header mismatch
@@ -70,6 +72,7 @@ EXPORTED_SYMBOLS = (
     "forge_hessian_workspace_bytes",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
+    "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
 )
 
 
@@ -325,6 +328,44 @@ class _HipKernels:
         with torch.cuda.device(codes.device):
             self._check(self._lib.forge_pack_int4(_ptr(codes), _ptr(qzeros), _ptr(out), R, C,
                                                   int(group_size), _stream()))
+        return out
+
+
+    def fp8_block_dequant(self, w, scale_inv, dtype=torch.bfloat16):
+        """w [O,I] or [B,O,I] float8_e4m3fn (or its uint8 view), scale_inv [.., nO, nI] f32 ->
+        dequantised weights; tile sizes are inferred as forge/utils/io.py:533-548 does."""
+        _need_cuda(w, scale_inv)
+        squeeze = w.dim() == 2
+        w3 = (w.unsqueeze(0) if squeeze else w).contiguous()
+        s3 = (scale_inv.unsqueeze(0) if squeeze else scale_inv).contiguous().float()
+        B, O, I = w3.shape
+        nO, nI = s3.shape[1:]
+        if I % nI:
+            raise RuntimeError("fp8_block_dequant: I must be a multiple of the scale grid width")
+        si = I // nI
+        so = si if (O + si - 1) // si == nO else (O + nO - 1) // nO
+        out = torch.empty((B, O, I), dtype=dtype, device=w.device)
+        with torch.cuda.device(w.device):
+            self._check(self._lib.forge_fp8_e4m3_block_dequant(
+                _ptr(w3.view(torch.uint8)), _ptr(s3), _ptr(out), _dtype_code(out), B, O, I, so, si,
+                _stream()))
+        return out[0] if squeeze else out
+
+    def pack_sparsegptq14_to_u64x2(self, qweight_rc, M, scales):
+        """kernels.cpp:122-126: qweight_rc [R,C] u8, M [G32,R] u32, scales [G32,R] f32 ->
+        uint64 [G2, R, 2]."""
+        _need_cuda(qweight_rc, M, scales)
+        qweight_rc, M, scales = qweight_rc.contiguous(), M.contiguous(), scales.contiguous()
+        if qweight_rc.dim() != 2 or M.dim() != 2 or scales.dim() != 2:
+            raise RuntimeError("pack_sparsegptq14_to_u64x2: 2-d tensors expected")
+        R, C = qweight_rc.shape
+        G32 = (C + 31) // 32
+        if M.shape[0] != G32 or M.shape[1] != R or tuple(scales.shape) != (G32, R):
+            raise RuntimeError("pack_sparsegptq14_to_u64x2: M/scales must be [ceil(C/32), R]")
+        out = torch.empty(((G32 + 1) // 2, R, 2), dtype=torch.uint64, device=qweight_rc.device)
+        with torch.cuda.device(qweight_rc.device):
+            self._check(self._lib.forge_pack_sparsegptq14_to_u64x2(
+                _ptr(qweight_rc), _ptr(M), _ptr(scales.float()), _ptr(out), R, C, _stream()))
         return out
 
 

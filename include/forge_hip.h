@@ -164,6 +164,24 @@ int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm_inv, uint
 int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_t* packed, int64_t R,
                     int64_t C, int64_t gs, forge_stream_t stream);
 
+/* ------------------------------------------------------------------ formats around the path */
+
+/* DeepSeek-style fp8 checkpoint weights -> bf16/f32 (forge/utils/io.py:533-563,863-872):
+ * out[b][r][c] = (f32) w[b][r][c] * scale_inv[b][r / so][c / si], w holding OCP float8
+ * e4m3fn bytes [batch, O, I], scale_inv [batch, ceil(O/so), ceil(I/si)] f32; the product is
+ * rounded to out_dtype (FORGE_BF16: round to nearest even, or FORGE_F32). */
+int forge_fp8_e4m3_block_dequant(const uint8_t* w, const float* scale_inv, void* out,
+                                 int out_dtype, int64_t batch, int64_t O, int64_t I, int64_t so,
+                                 int64_t si, forge_stream_t stream);
+
+/* Replaces kernels.pack_sparsegptq14_to_u64x2 (kernels.cpp:122-126,
+ * bitpacking_sparsegptq14.cu:58-172): qweight_rc [R, C] u8 codes, M [ceil(C/32), R] u32 keep
+ * masks, scales [ceil(C/32), R] f32 -> out [ceil(ceil(C/32)/2), R, 2] u64, each
+ * bf16(scale) << 48 | idx16 << 32 | qw32. */
+int forge_pack_sparsegptq14_to_u64x2(const uint8_t* qweight_rc, const uint32_t* M,
+                                     const float* scales, uint64_t* out, int64_t R, int64_t C,
+                                     forge_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

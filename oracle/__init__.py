@@ -62,6 +62,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_gptq_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, i32, i64]
         L.oracle_sparsegptq14_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32]
         L.oracle_gptq_inblock.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i64, vp, vp]
+        L.oracle_pack_sparsegptq14.argtypes = [vp, vp, vp, vp, i64, i64]
+        L.oracle_pack_sparsegptq14.restype = None
         for f in (L.oracle_build_group_meta, L.oracle_mse_scale_groups, L.oracle_gptq_solver,
                   L.oracle_sparsegptq14_solver, L.oracle_gptq_inblock):
             f.restype = None
@@ -146,11 +148,40 @@ def sparsegptq14_solver(W, U, scales, qzeros, bits, trail_mode: int = TRAIL_CHAI
     return q, M.view(torch.uint32) if hasattr(torch, "uint32") else M
 
 
+def pack_sparsegptq14_to_u64x2(qweight_rc, M, scales):
+    """kernels.cpp:122-126 -> bitpacking_sparsegptq14.cu:110-172.  Returns int64 [G2,R,2]
+    holding the u64 bit patterns."""
+    q = qweight_rc.contiguous()
+    R, C = q.shape
+    G32 = (C + 31) // 32
+    Mi = M.contiguous().view(torch.int32)
+    sc = _f32c(scales)
+    assert tuple(Mi.shape) == (G32, R) and tuple(sc.shape) == (G32, R) and q.dtype == torch.uint8
+    out = torch.empty(((G32 + 1) // 2, R, 2), dtype=torch.int64)
+    lib().oracle_pack_sparsegptq14(q.data_ptr(), Mi.data_ptr(), sc.data_ptr(), out.data_ptr(), R, C)
+    return out
+
+
+def fp8_block_dequant(w_fp8, scale_inv, dtype=torch.bfloat16):
+    """The reference's own torch expression for DeepSeek fp8 weights
+    (forge/utils/io.py:533-563,863-872): f32(w) * scale_inv per so x si tile -> dtype."""
+    w = w_fp8.to(torch.float32)
+    O, I = w.shape
+    nO, nI = scale_inv.shape
+    assert I % nI == 0
+    si = I // nI
+    so = si if (O + si - 1) // si == nO else (O + nO - 1) // nO
+    rows = torch.arange(O) // so
+    cols = torch.arange(I) // si
+    return (w * scale_inv.float()[rows][:, cols]).to(dtype)
+
+
 kernels = SimpleNamespace(
     build_group_meta_packed=build_group_meta_packed,
     mse_scale_groups_packed=mse_scale_groups_packed,
     gptq_solver=gptq_solver,
     sparsegptq14_solver=sparsegptq14_solver,
+    pack_sparsegptq14_to_u64x2=pack_sparsegptq14_to_u64x2,
 )
 
 

@@ -15,6 +15,7 @@
  *   oracle_mse_scale_groups      forge/backend/cuda/quant_grid.cu:101-183
  *   oracle_gptq_solver           forge/backend/cuda/solver.cu:9-154
  *   oracle_sparsegptq14_solver   forge/backend/cuda/solver_sparsegptq14.cu:12-200
+ *   oracle_pack_sparsegptq14     forge/backend/cuda/bitpacking_sparsegptq14.cu:58-107
  *
  * Where the reference leaves fp32 bits undefined, the oracle fixes them as follows
  * (each choice is within the reference's own numerical freedom):
@@ -266,4 +267,43 @@ void oracle_sparsegptq14_solver(float* W, float* U, const float* scales, const f
     }
     free(E);
     free(Uinv);
+}
+
+/* bitpacking_sparsegptq14.cu:58-107.  q_rc [R,C] codes, M [G32,R], scales [G32,R] ->
+ * out [G2,R,2] u64 = bf16(scale) << 48 | idx16 << 32 | qw32. */
+static uint16_t bf16_rne_bits(float x) {
+    uint32_t u; memcpy(&u, &x, 4);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+void oracle_pack_sparsegptq14(const uint8_t* q_rc, const uint32_t* M, const float* scales,
+                              uint64_t* out, int64_t R, int64_t C) {
+    const int64_t G32 = (C + 31) / 32, G2 = (G32 + 1) / 2;
+    for (int64_t g2 = 0; g2 < G2; ++g2)
+        for (int64_t r = 0; r < R; ++r)
+            for (int h = 0; h < 2; ++h) {
+                const int64_t gid = 2 * g2 + h;
+                uint64_t packed = 0;
+                if (gid < G32) {
+                    const uint32_t bitmask = M[gid * R + r];
+                    uint32_t idx16 = 0, qw32 = 0x88888888u;
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t sub = (bitmask >> (4 * i)) & 0xFu;
+                        if (!sub) continue;
+                        int c = 0;
+                        while (!((sub >> c) & 1u)) ++c;            /* __ffs(sub) - 1 */
+                        idx16 |= (uint32_t)(c & 3) << (2 * i);
+                        const int64_t cid = gid * 32 + i * 4 + c;
+                        if (cid < C) {
+                            const uint32_t q = q_rc[r * C + cid] & 0xFu;
+                            qw32 = (qw32 & ~(0xFu << (4 * i))) | (q << (4 * i));
+                        }
+                    }
+                    packed = ((uint64_t)bf16_rne_bits(scales[gid * R + r]) << 48) |
+                             ((uint64_t)(idx16 & 0xFFFFu) << 32) | (uint64_t)qw32;
+                }
+                out[(g2 * R + r) * 2 + h] = packed;
+            }
 }
