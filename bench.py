@@ -32,6 +32,13 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
 
 PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, TFLOP/s, GB/s
+# HBM bytes per launch of the factorisation GEMM on the default workload (64 experts per
+# step), from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each
+# scaled by what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and
+# x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  Algorithmic bytes per
+# launch (operands + accumulator tile once) are ~1.8e9.
+MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 2.14e9}
+
 KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit)
     "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s"),
     "chain_gemm": ("mfma", "mfma_f32", "TFLOP/s"),
@@ -109,19 +116,30 @@ def run_step(wl, cfg, chunk, step, mse=True):
     # gate/up (shared Hessian) and down are independent: one host thread and one HIP stream
     # each, so that the MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale
     # search and the latency-bound diagonal blocks of the other
-    def solve(weights, rows, stream):
-        with torch.cuda.stream(stream):
-            grp = ExpertGroupGPTQ(weights, **kw)
-            grp.update(rows, offs)
-            return grp.quantize(chunk=chunk)
-
     cur = torch.cuda.current_stream()
     for s in STREAMS:
         s.wait_stream(cur)
-    with ThreadPoolExecutor(max_workers=2) as pool:
-        f_gu = pool.submit(solve, [wl["Wg"], wl["Wu"]], xs, STREAMS[0])
-        f_dn = pool.submit(solve, [wl["Wd"]], hs, STREAMS[1])
-        out_gu, out_dn = f_gu.result(), f_dn.result()
+    # SPLIT sub-batches of experts per group, each on its own stream
+    nsub = max(1, len(STREAMS) // 2)
+    per = (chunk + nsub - 1) // nsub
+    jobs = []
+    with ThreadPoolExecutor(max_workers=len(STREAMS)) as pool:
+        for j in range(nsub):
+            a, b = j * per, min(chunk, (j + 1) * per)
+            if a >= b:
+                continue
+            sub_offs = [o - offs[a] for o in offs[a:b + 1]]
+
+            def solve_sub(weights, rows, stream, a=a, b=b, sub_offs=sub_offs):
+                with torch.cuda.stream(stream):
+                    grp = ExpertGroupGPTQ([w[a:b] for w in weights], **kw)
+                    grp.update(rows[offs[a]:offs[b]], sub_offs)
+                    return grp.quantize(chunk=b - a)
+
+            jobs.append(pool.submit(solve_sub, [wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]))
+            jobs.append(pool.submit(solve_sub, [wl["Wd"]], hs, STREAMS[2 * j + 1]))
+        results = [j.result() for j in jobs]
+    out_gu, out_dn = results[0::2], results[1::2]
     for s in STREAMS:
         cur.wait_stream(s)
     return out_gu, out_dn
@@ -171,6 +189,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", default="deepseek_v3", choices=sorted(CONFIGS))
     ap.add_argument("--chunk", type=int, default=0, help="experts per step (0 = config default)")
+    ap.add_argument("--split", type=int, default=1,
+                    help="sub-batches of a step's experts solved concurrently (one HIP stream each "
+                         "for their gate/up and their down groups)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -189,7 +210,7 @@ def main():
     chunk = a.chunk or cfg["chunk"]
     wl = make_workload(cfg, chunk)
     mse = not a.no_mse
-    STREAMS.extend([torch.cuda.Stream(), torch.cuda.Stream()])      # default priority
+    STREAMS.extend(torch.cuda.Stream() for _ in range(2 * a.split))   # default priority
 
     if a.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
@@ -225,7 +246,8 @@ def main():
     dom = next(iter(breakdown))
     bound, peak_key, unit = KERNEL_BOUND.get(dom, ("hbm", "hbm", "GB/s"))
     roofline = dict(kernel=dom, bound=bound, achieved=breakdown[dom]["rate"], peak=PEAK[peak_key],
-                    unit=unit, frac=round(breakdown[dom]["rate"] / PEAK[peak_key], 4), traffic=None,
+                    unit=unit, frac=round(breakdown[dom]["rate"] / PEAK[peak_key], 4),
+                    traffic=MEASURED_TRAFFIC.get((a.config, chunk, dom)) if a.split == 1 else None,
                     avg_launch_us=breakdown[dom]["avg_us"], launches=breakdown[dom]["launches"])
 
     out = {
