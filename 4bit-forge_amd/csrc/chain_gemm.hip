@@ -11,10 +11,15 @@
 // quadrant = 2x2 MFMA tiles (64 accumulator registers).  Operands are K-major in memory,
 // so a half-wavefront reads 32 consecutive floats of one k row: global loads are
 // coalesced float4, LDS reads are conflict-free ds_read_b32, and no transpose is needed.
-// K advances TK rows per stage: the next stage's rows are fetched into registers while
-// the current stage's 32 MFMAs per wavefront run, all LDS operands of a stage are read
-// before its first MFMA so the matrix pipe is fed back to back, and the register budget
-// leaves room for two workgroups per CU to cover the barrier between stages.
+// K advances 32 rows per LDS stage, as two sub-stages of 16 rows (32 MFMAs each).
+//
+// Two kernels share this layout.  chain_gemm_fast_kernel handles full, aligned tiles and
+// is a software pipeline: while the MFMAs of one sub-stage run, the wavefront issues the
+// LDS reads of the next sub-stage, the LDS writes of the next stage and the global loads
+// of the stage after that, one memory instruction between two MFMAs (a wavefront issues
+// in order, so memory instructions issued in a block of their own leave the matrix pipe
+// idle for their whole issue time).  chain_gemm_kernel<EDGE> is the simple, bounds-checked
+// form for ragged shapes.
 #include "chain_gemm.h"
 
 namespace forge {
@@ -28,8 +33,9 @@ constexpr int TM = 128, TN = 128;
 constexpr int TK = FORGE_GEMM_TK;   // k rows per LDS stage
 constexpr int NH = TK / 8;          // float4 loads per thread, operand and stage
 
-// EDGE: bounds-checked loads/stores for tiles that stick out of [m0,m1) x [n0,n1) or a K
-// range that is not a multiple of 16.  CHUNK > 0: every CHUNK k values the running
+// The simple form.  EDGE: bounds-checked loads/stores for tiles that stick out of
+// [m0,m1) x [n0,n1), a K range that is not a multiple of 32, or rows that are not 16-byte
+// aligned (the launcher only uses EDGE = true; full tiles go to chain_gemm_fast_kernel).  CHUNK > 0: every CHUNK k values the running
 // accumulators are folded into a second set and restarted from zero (blocked summation:
 // the rounding error of each fma is then relative to a short partial sum instead of the
 // whole accumulated value).  Used where only accuracy matters; CHUNK == 0 is the single
@@ -127,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
                     if (nt + lcol + 3 < g.n1) vb.w = qb[3];
                 }
             }
-            ra[h] = make_float4(sign * va.x, sign * va.y, sign * va.z, sign * va.w);
+            ra[h] = va;
             rb[h] = vb;
         }
         pa += NH * a_step8;
@@ -136,7 +142,10 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
     auto stage = [&](int buf) {
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
-            *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
+            // the sign is applied here, not in fetch(): a use right after the loads would
+            // make the wavefront wait out their latency before its first MFMA
+            *reinterpret_cast<float4*>(&As[buf][lrow + 8 * h][lcol]) =
+                make_float4(sign * ra[h].x, sign * ra[h].y, sign * ra[h].z, sign * ra[h].w);
             *reinterpret_cast<float4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
         }
     };
@@ -212,6 +221,217 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
             }
 }
 
+
+// Full 128x128 tiles, 16-byte aligned rows, K range a multiple of 32 (after triangular
+// clipping).  One stage s of the K loop:
+//   region A   32 MFMAs on operand set 0 (sub-stage 0 of stage s)
+//              | 16 LDS reads: operand set 1 (sub-stage 1 of stage s)
+//              | 8 LDS writes: stage s+1 from registers into the other LDS buffer
+//   barrier
+//   region B   32 MFMAs on operand set 1
+//              | 8 global loads: stage s+2 into registers
+//              | 16 LDS reads: operand set 0 of stage s+1
+// A negated A operand is folded into the sign of the accumulator on the way in and out:
+// fma(-a, b, x) == -fma(a, b, -x) exactly, so the result is the same chain bit for bit.
+template <int CHUNK>
+__global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmArgs g) {
+    static_assert(TK == 32, "two 16-row sub-stages per stage");
+    __shared__ __attribute__((aligned(16))) float As[2][TK][TM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TK][TN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int per_matrix = g.n_tiles * g.m_tiles;
+    int bz, tile;
+    if (g.xcd_map) {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        bz = xcd + 8 * (slot / per_matrix);
+        tile = slot % per_matrix;
+    } else {
+        bz = blockIdx.x / per_matrix;
+        tile = blockIdx.x % per_matrix;
+    }
+    float* __restrict__ X = g.X + (int64_t)bz * g.xs;
+    const float* __restrict__ At = g.At + (int64_t)bz * g.as;
+    const float* __restrict__ Bm = g.Bm + (int64_t)bz * g.bs;
+    const int mt = g.m0 + (tile / g.n_tiles) * TM;
+    const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile % g.n_tiles : tile % g.n_tiles;
+    const int nt = g.n0 + tn * TN;
+    int k0 = g.k0, k1 = g.k1;
+    if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
+    if (g.b_lower_tri && k0 < nt) k0 = nt;
+
+    const int m_base = mt + wm * 64 + (lane >> 5) * 4;
+    const int n_base = nt + wn * 64 + (lane & 31);
+    float* __restrict__ Xw = X + (int64_t)m_base * g.ldx + n_base;
+    const float sgn = g.negate_a ? -1.0f : 1.0f;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                float x = 0.0f;
+                if (!g.init_zero) x = sgn * Xw[(int64_t)dm * g.ldx + dn];
+                acc[mi][ni][v] = x;
+            }
+    f32x16 tot[2][2];
+    if constexpr (CHUNK > 0) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                tot[mi][ni] = acc[mi][ni];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+            }
+    }
+
+    if (k0 < k1) {  // uniform over the workgroup
+        // global -> LDS staging: thread loads k rows (tid>>5) + 8h, 4 columns each.  The
+        // eight float4 are named scalars on purpose: as an array captured by a lambda the
+        // compiler kept part of them in memory.
+        const int lrow = tid >> 5, lcol = (tid & 31) * 4;
+        const float* pa = At + (int64_t)(k0 + lrow) * g.lda + mt + lcol;
+        const float* pb = Bm + (int64_t)(k0 + lrow) * g.ldb + nt + lcol;
+        const int64_t a_step8 = 8 * g.lda, b_step8 = 8 * g.ldb;
+        float4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+#define FORGE_GEMM_FETCH()                                              \
+    do {                                                                \
+        ra0 = *reinterpret_cast<const float4*>(pa);                     \
+        rb0 = *reinterpret_cast<const float4*>(pb);                     \
+        ra1 = *reinterpret_cast<const float4*>(pa + a_step8);           \
+        rb1 = *reinterpret_cast<const float4*>(pb + b_step8);           \
+        ra2 = *reinterpret_cast<const float4*>(pa + 2 * a_step8);       \
+        rb2 = *reinterpret_cast<const float4*>(pb + 2 * b_step8);       \
+        ra3 = *reinterpret_cast<const float4*>(pa + 3 * a_step8);       \
+        rb3 = *reinterpret_cast<const float4*>(pb + 3 * b_step8);       \
+        pa += a_adv;                                                    \
+        pb += b_adv;                                                    \
+    } while (0)
+#define FORGE_GEMM_STAGE(buf)                                           \
+    do {                                                                \
+        *reinterpret_cast<float4*>(&As[buf][lrow][lcol]) = ra0;         \
+        *reinterpret_cast<float4*>(&Bs[buf][lrow][lcol]) = rb0;         \
+        *reinterpret_cast<float4*>(&As[buf][lrow + 8][lcol]) = ra1;     \
+        *reinterpret_cast<float4*>(&Bs[buf][lrow + 8][lcol]) = rb1;     \
+        *reinterpret_cast<float4*>(&As[buf][lrow + 16][lcol]) = ra2;    \
+        *reinterpret_cast<float4*>(&Bs[buf][lrow + 16][lcol]) = rb2;    \
+        *reinterpret_cast<float4*>(&As[buf][lrow + 24][lcol]) = ra3;    \
+        *reinterpret_cast<float4*>(&Bs[buf][lrow + 24][lcol]) = rb3;    \
+    } while (0)
+
+        const int a_off = wm * 64 + (lane & 31), b_off = wn * 64 + (lane & 31), kr0 = lane >> 5;
+        float av0[8][2], bv0[8][2], av1[8][2], bv1[8][2];
+        auto read_ops = [&](int buf, int sub, float (&av)[8][2], float (&bv)[8][2]) {
+#pragma unroll
+            for (int kp = 0; kp < 8; ++kp)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    av[kp][i] = As[buf][sub * 16 + 2 * kp + kr0][a_off + i * 32];
+                    bv[kp][i] = Bs[buf][sub * 16 + 2 * kp + kr0][b_off + i * 32];
+                }
+        };
+        auto mfmas = [&](const float (&av)[8][2], const float (&bv)[8][2]) {
+#pragma unroll
+            for (int kp = 0; kp < 8; ++kp)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[kp][mi], bv[kp][ni],
+                                                                           acc[mi][ni], 0, 0, 0);
+        };
+
+        // Every fetch reads rows below k1: the pointers advance only while a further stage
+        // exists; past the end the last stage is fetched again and never used.
+        const int64_t a_full = 4 * a_step8, b_full = 4 * b_step8;
+        int64_t a_adv = (k0 + TK < k1) ? a_full : 0, b_adv = (k0 + TK < k1) ? b_full : 0;
+        FORGE_GEMM_FETCH();
+        FORGE_GEMM_STAGE(0);
+        __syncthreads();
+        read_ops(0, 0, av0, bv0);
+        if (k0 + 2 * TK >= k1) { a_adv = 0; b_adv = 0; }
+        FORGE_GEMM_FETCH();
+
+        int buf = 0, stage_no = 0;
+        for (int kk = k0; kk < k1; kk += TK) {
+            // ---- region A.  The group barriers give the order "MFMA, memory instruction,
+            // MFMA, ..."; the plain barriers keep instructions from leaving their region.
+            read_ops(buf, 1, av1, bv1);
+            mfmas(av0, bv0);
+            FORGE_GEMM_STAGE(buf ^ 1);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- region B
+            read_ops(buf ^ 1, 0, av0, bv0);
+            if (kk + 3 * TK >= k1) { a_adv = 0; b_adv = 0; }
+            mfmas(av1, bv1);
+            FORGE_GEMM_FETCH();
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 1);  // one global load
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (CHUNK > 0) {
+                if (++stage_no == CHUNK / TK) {
+                    stage_no = 0;
+#pragma unroll
+                    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                        for (int ni = 0; ni < 2; ++ni) {
+                            tot[mi][ni] += acc[mi][ni];
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+                        }
+                }
+            }
+            buf ^= 1;
+        }
+#undef FORGE_GEMM_FETCH
+#undef FORGE_GEMM_STAGE
+    }
+    if constexpr (CHUNK > 0) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = tot[mi][ni] + acc[mi][ni];
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                Xw[(int64_t)dm * g.ldx + dn] = sgn * acc[mi][ni][v];
+            }
+}
+
 }  // namespace
 
 int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
@@ -247,10 +467,10 @@ int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
                         2.0 * (g.m1 - g.m0) * kn * (double)batch, WORK_FLOPS);
     if (g.blocked_sum) {
         if (edge) chain_gemm_kernel<true, 128><<<grid, dim3(256), 0, st>>>(g);
-        else chain_gemm_kernel<false, 128><<<grid, dim3(256), 0, st>>>(g);
+        else chain_gemm_fast_kernel<128><<<grid, dim3(256), 0, st>>>(g);
     } else {
         if (edge) chain_gemm_kernel<true, 0><<<grid, dim3(256), 0, st>>>(g);
-        else chain_gemm_kernel<false, 0><<<grid, dim3(256), 0, st>>>(g);
+        else chain_gemm_fast_kernel<0><<<grid, dim3(256), 0, st>>>(g);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
