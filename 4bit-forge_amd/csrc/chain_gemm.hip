@@ -267,18 +267,31 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmArgs g) {
     float* __restrict__ Xw = X + (int64_t)m_base * g.ldx + n_base;
     const float sgn = g.negate_a ? -1.0f : 1.0f;
 
+    // One branch around all 64 loads: tested per element, every load would be followed by
+    // its own wait and the tile would start 64 memory latencies late.
     f32x16 acc[2][2];
+    if (g.init_zero) {
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+        for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+            for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
-                float x = 0.0f;
-                if (!g.init_zero) x = sgn * Xw[(int64_t)dm * g.ldx + dn];
-                acc[mi][ni][v] = x;
-            }
+                for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                    acc[mi][ni][v] = Xw[(int64_t)dm * g.ldx + dn];
+                }
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) acc[mi][ni] *= sgn;
+    }
     f32x16 tot[2][2];
     if constexpr (CHUNK > 0) {
 #pragma unroll
