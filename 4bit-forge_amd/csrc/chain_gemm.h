@@ -27,6 +27,19 @@ struct GemmArgs {
     bool xcd_map;
 };
 
+// Two problems for one grid (see launch_chain_gemm_pair).
+struct GemmPair {
+    GemmArgs first, second;
+    int first_wgs;  // workgroups [0, first_wgs) belong to `first`
+};
+
 int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);
+
+// Runs two problems that do not depend on each other (neither writes what the other reads
+// or writes).  When both are full-tile problems of the same kind they share one launch, the
+// first problem's tiles ahead of the second's; otherwise they are launched one after the
+// other.  Either may be empty.
+int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
+                           hipStream_t st);
 
 }  // namespace forge

@@ -233,9 +233,15 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
 //              | 16 LDS reads: operand set 0 of stage s+1
 // A negated A operand is folded into the sign of the accumulator on the way in and out:
 // fma(-a, b, x) == -fma(a, b, -x) exactly, so the result is the same chain bit for bit.
+// A launch carries one or two independent problems (GemmPair): workgroups below
+// first_wgs work on `first`, the rest on `second`, so that two under-filled or ragged-ended
+// problems share one grid.
 template <int CHUNK>
-__global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) {
     static_assert(TK == 32, "two 16-row sub-stages per stage");
+    const bool in_first = blockIdx.x < (unsigned)pair.first_wgs;
+    const GemmArgs& g = in_first ? pair.first : pair.second;
+    const int wg = in_first ? (int)blockIdx.x : (int)blockIdx.x - pair.first_wgs;
     __shared__ __attribute__((aligned(16))) float As[2][TK][TM];
     __shared__ __attribute__((aligned(16))) float Bs[2][TK][TN];
 
@@ -244,13 +250,13 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
     const int per_matrix = g.n_tiles * g.m_tiles;
     int bz, tile;
-    if (g.xcd_map) {
-        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    if (g.xcd_map) {  // first_wgs is then a multiple of 8, so wg & 7 is still the XCD
+        const int xcd = wg & 7, slot = wg >> 3;
         bz = xcd + 8 * (slot / per_matrix);
         tile = slot % per_matrix;
     } else {
-        bz = blockIdx.x / per_matrix;
-        tile = blockIdx.x % per_matrix;
+        bz = wg / per_matrix;
+        tile = wg % per_matrix;
     }
     float* __restrict__ X = g.X + (int64_t)bz * g.xs;
     const float* __restrict__ At = g.At + (int64_t)bz * g.as;
@@ -447,10 +453,22 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmArgs g) {
 
 }  // namespace
 
-int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
-    GemmArgs g = g_in;
-    if (g.m1 <= g.m0 || g.n1 <= g.n0 || batch <= 0) return FORGE_OK;
-    if (g.k1 <= g.k0 && !g.init_zero) return FORGE_OK;
+namespace {
+
+struct Prepared {
+    GemmArgs g;
+    bool empty, edge;
+    int64_t n_wg;
+    double flops;
+};
+
+// Fills in the tile counts and decides which kernel a problem needs.
+Prepared prepare(const GemmArgs& g_in, int64_t batch) {
+    Prepared p{};
+    GemmArgs& g = p.g;
+    g = g_in;
+    p.empty = g.m1 <= g.m0 || g.n1 <= g.n0 || batch <= 0 || (g.k1 <= g.k0 && !g.init_zero);
+    if (p.empty) return p;
     // float4 loads need 16-byte aligned rows; anything else takes the scalar EDGE path
     const bool aligned = (g.lda % 4) == 0 && (g.ldb % 4) == 0 && (g.m0 % 4) == 0 &&
                          (g.n0 % 4) == 0 && (g.as % 4) == 0 && (g.bs % 4) == 0 &&
@@ -459,14 +477,12 @@ int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
     g.n_tiles = (int)ceil_div(g.n1 - g.n0, TN);
     g.m_tiles = (int)ceil_div(g.m1 - g.m0, TM);
     g.xcd_map = (batch % 8) == 0;
-    const int64_t n_wg = (int64_t)g.n_tiles * g.m_tiles * batch;
-    FORGE_REQUIRE(n_wg < (1LL << 31), "chain_gemm: grid too large");
-    dim3 grid((unsigned)n_wg);
-    // the triangular K clipping keeps multiples of 16 only when tiles and K origin line up
+    p.n_wg = (int64_t)g.n_tiles * g.m_tiles * batch;
+    // the triangular K clipping keeps multiples of TK only when tiles and K origin line up
     const bool tri_ok = (!g.b_upper_tri || ((g.n0 + TN - g.k0) % TK) == 0) &&
                         (!g.b_lower_tri || ((g.n0 - g.k0) % TK) == 0);
-    const bool edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
-                      ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned;
+    p.edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
+             ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned;
     // useful flops: 2*M*N*K with K clipped per n-tile for the triangular variants
     double kn = 0.0;
     for (int nt = g.n0; nt < g.n1; nt += TN) {
@@ -476,17 +492,52 @@ int launch_chain_gemm(const GemmArgs& g_in, int64_t batch, hipStream_t st) {
         const int ncols = (g.n1 - nt) < TN ? (g.n1 - nt) : TN;
         if (k1 > k0) kn += (double)(k1 - k0) * ncols;
     }
-    KernelTiming timing(g.blocked_sum ? "chain_gemm_blocked_sum" : "chain_gemm", st,
-                        2.0 * (g.m1 - g.m0) * kn * (double)batch, WORK_FLOPS);
-    if (g.blocked_sum) {
-        if (edge) chain_gemm_kernel<true, 128><<<grid, dim3(256), 0, st>>>(g);
-        else chain_gemm_fast_kernel<128><<<grid, dim3(256), 0, st>>>(g);
+    p.flops = 2.0 * (g.m1 - g.m0) * kn * (double)batch;
+    return p;
+}
+
+int launch_prepared(const Prepared& a, const Prepared* b, hipStream_t st) {
+    const int64_t n_wg = a.n_wg + (b ? b->n_wg : 0);
+    FORGE_REQUIRE(n_wg < (1LL << 31), "chain_gemm: grid too large");
+    dim3 grid((unsigned)n_wg);
+    KernelTiming timing(a.g.blocked_sum ? "chain_gemm_blocked_sum" : "chain_gemm", st,
+                        a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
+    if (a.edge) {
+        if (a.g.blocked_sum) chain_gemm_kernel<true, 128><<<grid, dim3(256), 0, st>>>(a.g);
+        else chain_gemm_kernel<true, 0><<<grid, dim3(256), 0, st>>>(a.g);
     } else {
-        if (edge) chain_gemm_kernel<true, 0><<<grid, dim3(256), 0, st>>>(g);
-        else chain_gemm_fast_kernel<0><<<grid, dim3(256), 0, st>>>(g);
+        GemmPair pair{};
+        pair.first = a.g;
+        pair.second = b ? b->g : a.g;
+        pair.first_wgs = (int)a.n_wg;
+        if (a.g.blocked_sum) chain_gemm_fast_kernel<128><<<grid, dim3(256), 0, st>>>(pair);
+        else chain_gemm_fast_kernel<0><<<grid, dim3(256), 0, st>>>(pair);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
+}
+
+}  // namespace
+
+int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
+    const Prepared p = prepare(g, batch);
+    if (p.empty) return FORGE_OK;
+    return launch_prepared(p, nullptr, st);
+}
+
+int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
+                           hipStream_t st) {
+    const Prepared a = prepare(first, batch), b = prepare(second, batch);
+    if (a.empty && b.empty) return FORGE_OK;
+    if (a.empty) return launch_prepared(b, nullptr, st);
+    if (b.empty) return launch_prepared(a, nullptr, st);
+    // one grid needs the same kernel for both; a grid split at a multiple of 8 keeps the
+    // workgroup -> XCD map of the second problem
+    const bool fusable = !a.edge && !b.edge && a.g.blocked_sum == b.g.blocked_sum &&
+                         (!b.g.xcd_map || a.n_wg % 8 == 0);
+    if (fusable) return launch_prepared(a, &b, st);
+    if (int e = launch_prepared(a, nullptr, st)) return e;
+    return launch_prepared(b, nullptr, st);
 }
 
 }  // namespace forge

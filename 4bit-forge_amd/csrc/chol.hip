@@ -211,12 +211,19 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
     for (int a = nblk - 1; a >= 0; --a) {
         const int m0 = a * NB;
         const int m1 = (int)(C < (int64_t)m0 + NB ? C : m0 + NB);
-        forge::GemmArgs g{};
-        if (m1 < C) {  // 1a
-            g = forge::GemmArgs{};
-            g.X = H; g.At = H; g.Bm = H; g.ldx = g.lda = g.ldb = C; g.xs = g.as = g.bs = C * C;
-            g.m0 = m0; g.m1 = m1; g.n0 = 0; g.n1 = m1; g.k0 = m1; g.k1 = (int)C; g.negate_a = true; g.blocked_sum = true;
-            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        // 1a and 2a of this step do not depend on each other (2a needs rows > a only), and
+        // their tile counts are complementary, (a+1) and (nblk-1-a) per matrix: one grid
+        forge::GemmArgs g1a{}, g2a{};   // left empty (m1 == m0) when there is nothing below
+        if (m1 < C) {
+            g1a.X = H; g1a.At = H; g1a.Bm = H; g1a.ldx = g1a.lda = g1a.ldb = C;
+            g1a.xs = g1a.as = g1a.bs = C * C;
+            g1a.m0 = m0; g1a.m1 = m1; g1a.n0 = 0; g1a.n1 = m1; g1a.k0 = m1; g1a.k1 = (int)C;
+            g1a.negate_a = true; g1a.blocked_sum = true;
+            g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
+            g2a.xs = g2a.as = g2a.bs = C * C;
+            g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
+            g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
+            if (int e = forge::launch_chain_gemm_pair(g1a, g2a, batch, st)) return e;
         }
         {
             forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,
@@ -228,26 +235,22 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
         // Dinv blocks addressed with global (k, m) indices: shift the base so that
         // element (m0 + k', m0 + m') lands on block entry (k', m').
         const int64_t shift = (int64_t)m0 * NB + m0;
-        if (a > 0) {  // 1c
-            g = forge::GemmArgs{};
-            g.X = H; g.Bm = H; g.ldx = g.ldb = C; g.xs = g.bs = C * C;
-            g.At = Dinv + (int64_t)a * NB * NB - shift; g.lda = NB; g.as = (int64_t)nblk * NB * NB;
-            g.m0 = m0; g.m1 = m1; g.n0 = 0; g.n1 = m0; g.k0 = m0; g.k1 = m1; g.init_zero = true;
-            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        // 1c (rows of L2 left of the diagonal block) and 2b (rows of U0 right of it) both
+        // multiply by Dinv^T and touch different matrices: one grid again
+        forge::GemmArgs g1c{}, g2b{};
+        if (a > 0) {
+            g1c.X = H; g1c.Bm = H; g1c.ldx = g1c.ldb = C; g1c.xs = g1c.bs = C * C;
+            g1c.At = Dinv + (int64_t)a * NB * NB - shift; g1c.lda = NB; g1c.as = (int64_t)nblk * NB * NB;
+            g1c.m0 = m0; g1c.m1 = m1; g1c.n0 = 0; g1c.n1 = m0; g1c.k0 = m0; g1c.k1 = m1;
+            g1c.init_zero = true;
         }
-        if (m1 < C) {  // 2a, 2b
-            g = forge::GemmArgs{};
-            g.X = U; g.At = H; g.Bm = U; g.ldx = g.lda = g.ldb = C; g.xs = g.as = g.bs = C * C;
-            g.m0 = m0; g.m1 = m1; g.n0 = m1; g.n1 = (int)C; g.k0 = m1; g.k1 = (int)C;
-            g.init_zero = true; g.b_upper_tri = true; g.blocked_sum = true;
-            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
-            g = forge::GemmArgs{};
-            g.X = U; g.Bm = U; g.ldx = g.ldb = C; g.xs = g.bs = C * C;
-            g.At = Dinv + (int64_t)a * NB * NB - shift; g.lda = NB; g.as = (int64_t)nblk * NB * NB;
-            g.m0 = m0; g.m1 = m1; g.n0 = m1; g.n1 = (int)C; g.k0 = m0; g.k1 = m1;
-            g.init_zero = true; g.negate_a = true;
-            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        if (m1 < C) {
+            g2b.X = U; g2b.Bm = U; g2b.ldx = g2b.ldb = C; g2b.xs = g2b.bs = C * C;
+            g2b.At = Dinv + (int64_t)a * NB * NB - shift; g2b.lda = NB; g2b.as = (int64_t)nblk * NB * NB;
+            g2b.m0 = m0; g2b.m1 = m1; g2b.n0 = m1; g2b.n1 = (int)C; g2b.k0 = m0; g2b.k1 = m1;
+            g2b.init_zero = true; g2b.negate_a = true;
         }
+        if (int e = forge::launch_chain_gemm_pair(g1c, g2b, batch, st)) return e;
     }
     forge::KernelTiming timing("chol_finish_rows", st, 4.0 * C * C * (double)batch, forge::WORK_BYTES);
     finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(U, udiag, info, C,
