@@ -155,8 +155,9 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     if (tid == 0 && s_fail != 0 && info[b] == 0) info[b] = (int32_t)(m0 + s_fail);
 }
 
-// Last pass over the rows of U0: divide by the diagonal when asked to (gptq.py:164); a
-// failed factorisation hands back the identity instead, as gptq.py:172-175 does.
+// Last pass over the rows of U0: zero what lies left of the diagonal (the GEMMs only write
+// the blocks on and right of it), and divide by the diagonal when asked to (gptq.py:164).
+// A failed factorisation hands back the identity instead, as gptq.py:172-175 does.
 __global__ void finish_rows_kernel(float* __restrict__ U, float* __restrict__ udiag,
                                    const int32_t* __restrict__ info, int64_t C, bool normalise) {
     const int64_t b = blockIdx.y;
@@ -167,6 +168,9 @@ __global__ void finish_rows_kernel(float* __restrict__ U, float* __restrict__ ud
         if (threadIdx.x == 0) udiag[b * C + row] = 1.0f;
         return;
     }
+    // the diagonal block kernel wrote its whole tile, zeros below the diagonal included
+    const int64_t left = row / NB * NB;
+    for (int64_t j = threadIdx.x; j < left; j += blockDim.x) Ur[j] = 0.0f;
     if (!normalise) return;
     const float d = udiag[b * C + row];
     for (int64_t j = row + threadIdx.x; j < C; j += blockDim.x) Ur[j] = Ur[j] / d;
@@ -198,10 +202,6 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
     FORGE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(diag_block_kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDiagLds));
     FORGE_HIP_CHECK(hipMemsetAsync(info, 0, batch * sizeof(int32_t), st));
-    {
-        forge::KernelTiming timing("chol_clear_u", st, 4.0 * C * C * (double)batch, forge::WORK_BYTES);
-        FORGE_HIP_CHECK(hipMemsetAsync(U, 0, batch * C * C * sizeof(float), st));
-    }
     if (damp) {
         add_damp_kernel<<<dim3((unsigned)forge::ceil_div(C, 256), (unsigned)batch), dim3(256), 0, st>>>(
             H, damp, C);
@@ -252,7 +252,7 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
         }
         if (int e = forge::launch_chain_gemm_pair(g1c, g2b, batch, st)) return e;
     }
-    forge::KernelTiming timing("chol_finish_rows", st, 4.0 * C * C * (double)batch, forge::WORK_BYTES);
+    forge::KernelTiming timing("chol_finish_rows", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
     finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(U, udiag, info, C,
                                                                                normalise != 0);
     FORGE_LAUNCH_CHECK();

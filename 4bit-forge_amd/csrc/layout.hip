@@ -57,9 +57,11 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
 }
 
 // Hp[b][i][j] = H[b][perm[i]][perm[j]], dead rows/columns zeroed with a unit diagonal
-// (forge/gptq.py:100-103,117,145-149).  One workgroup per output row: the source row is
-// streamed into LDS with coalesced loads, gathered from there in permuted order and
-// written out coalesced, so HBM sees one sequential read and one sequential write.
+// (forge/gptq.py:100-103,117,145-149).  The source row is streamed into LDS with coalesced
+// loads, gathered from there in permuted order and written out coalesced, so HBM sees one
+// sequential read and one sequential write.
+//
+// General form: one workgroup per output row, scalar accesses, LDS staging when C fits.
 __global__ __launch_bounds__(256) void hessian_permute_kernel(
     const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
     float* __restrict__ Hp, int64_t C) {
@@ -80,6 +82,86 @@ __global__ __launch_bounds__(256) void hessian_permute_kernel(
         if (dead_i || (db && db[j])) v = (i == j) ? 1.0f : 0.0f;
         dst[j] = v;
     }
+}
+
+// Fast form for C % 4 == 0 and C <= 1024 * NCH: a workgroup produces kPermuteRows
+// consecutive output rows.  Thread t owns the output columns 4*(t + 256u) .. +3 (u < NCH)
+// of every row and keeps their source indices in registers, so the permutation is read
+// once per workgroup instead of once per row; rows move as float4 on both sides and the
+// two LDS row buffers alternate, which leaves one barrier per row.
+constexpr int kPermuteRows = 16;
+template <int NCH>
+__global__ __launch_bounds__(256) void hessian_permute_rows_kernel(
+    const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
+    float* __restrict__ Hp, int C) {
+    extern __shared__ float srow[];                 // 2 * C floats
+    const int64_t b = blockIdx.y;
+    const int i0 = blockIdx.x * kPermuteRows;
+    const int tid = threadIdx.x;
+    const int64_t* __restrict__ pb = perm + b * C;
+    const uint8_t* __restrict__ db = dead ? dead + b * C : nullptr;
+    const float* __restrict__ Hb = H + b * (int64_t)C * C;
+    float* __restrict__ Hpb = Hp + b * (int64_t)C * C;
+
+    // Column chunks past the end are clamped onto the last one: they move the same data a
+    // second time and are not written out.  (Guarding the register arrays instead makes
+    // the compiler keep them in scratch memory.)
+    int col[NCH];
+    int src_col[NCH][4];
+    unsigned dead_cols = 0;                         // bit 4u+k: output column is dead
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+        const int j = 4 * (tid + 256 * u);
+        col[u] = j < C ? j : C - 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            src_col[u][k] = (int)pb[col[u] + k];
+            if (db && db[col[u] + k]) dead_cols |= 1u << (4 * u + k);
+        }
+    }
+    // the row in flight: named registers (as an array the compiler left it in scratch memory)
+    float4 st0, st1, st2, st3, st4, st5, st6, st7;
+#define FORGE_CHUNKS(M)                                  \
+    M(0, st0) M(1, st1)                                  \
+    if constexpr (NCH > 2) { M(2, st2) M(3, st3) }       \
+    if constexpr (NCH > 4) { M(4, st4) M(5, st5) M(6, st6) M(7, st7) }
+#define FORGE_LOAD(u, reg) reg = *reinterpret_cast<const float4*>(src + col[u]);
+#define FORGE_STORE(u, reg) *reinterpret_cast<float4*>(buf + col[u]) = reg;
+    static_assert(NCH == 2 || NCH == 4 || NCH == 8, "chunk counts the macro covers");
+    const int rows = (C - i0) < kPermuteRows ? (C - i0) : kPermuteRows;
+    {
+        const float* __restrict__ src = Hb + pb[i0] * C;
+        FORGE_CHUNKS(FORGE_LOAD)
+    }
+    for (int r = 0; r < rows; ++r) {
+        float* __restrict__ buf = srow + (r & 1) * C;
+        FORGE_CHUNKS(FORGE_STORE)
+        __syncthreads();                            // also fences the buffer used two rows ago
+        // next source row -> registers while this one is gathered (the last row again at the end)
+        const int i_next = i0 + (r + 1 < rows ? r + 1 : r);
+        const float* __restrict__ src = Hb + pb[i_next] * C;
+        FORGE_CHUNKS(FORGE_LOAD)
+        const int i = i0 + r;
+        const bool dead_i = db && db[i];
+        float* __restrict__ dst = Hpb + (int64_t)i * C;
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            float4 v;
+            v.x = buf[src_col[u][0]];
+            v.y = buf[src_col[u][1]];
+            v.z = buf[src_col[u][2]];
+            v.w = buf[src_col[u][3]];
+            const unsigned dc = dead_i ? 0xFu : (dead_cols >> (4 * u)) & 0xFu;
+            if (dc & 1u) v.x = (i == col[u] + 0) ? 1.0f : 0.0f;
+            if (dc & 2u) v.y = (i == col[u] + 1) ? 1.0f : 0.0f;
+            if (dc & 4u) v.z = (i == col[u] + 2) ? 1.0f : 0.0f;
+            if (dc & 8u) v.w = (i == col[u] + 3) ? 1.0f : 0.0f;
+            if (4 * (tid + 256 * u) < C) *reinterpret_cast<float4*>(dst + col[u]) = v;
+        }
+    }
+#undef FORGE_CHUNKS
+#undef FORGE_LOAD
+#undef FORGE_STORE
 }
 
 // damp[b] = rel_damp * mean(diag(Hp[b]))   (forge/gptq.py:152-153); fixed-order tree sum.
@@ -170,9 +252,22 @@ extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const 
     FORGE_REQUIRE(H != Hp, "hessian_permute cannot run in place");
     hipStream_t st = (hipStream_t)stream;
     forge::KernelTiming timing("hessian_permute", st, 8.0 * C * C * (double)batch, forge::WORK_BYTES);
-    const size_t lds = C <= kPermuteLdsFloats ? (size_t)C * sizeof(float) : 0;
-    hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), lds, st>>>(H, perm, dead,
-                                                                                     Hp, C);
+    const bool vec_ok = (C % 4) == 0 && C <= 8192 && (reinterpret_cast<uintptr_t>(H) % 16) == 0 &&
+                        (reinterpret_cast<uintptr_t>(Hp) % 16) == 0;
+    if (vec_ok) {
+        const dim3 grid((unsigned)forge::ceil_div(C, kPermuteRows), (unsigned)batch);
+        const size_t lds = 2 * (size_t)C * sizeof(float);   // <= 64 KB
+        if (C <= 2048)
+            hessian_permute_rows_kernel<2><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+        else if (C <= 4096)
+            hessian_permute_rows_kernel<4><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+        else
+            hessian_permute_rows_kernel<8><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+    } else {
+        const size_t lds = C <= kPermuteLdsFloats ? (size_t)C * sizeof(float) : 0;
+        hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), lds, st>>>(
+            H, perm, dead, Hp, C);
+    }
     FORGE_LAUNCH_CHECK();
     damp_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(Hp, damp, rel_damp, C);
     FORGE_LAUNCH_CHECK();
