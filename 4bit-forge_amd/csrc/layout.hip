@@ -56,6 +56,85 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
     }
 }
 
+// Fast forms of the two transposes for the shapes the batched solve uses (bf16 weights,
+// R % 256 == 0, C % 64 == 0 resp. C % 128 == 0).  Tiles are 256 rows of R tall so that a
+// wavefront moves whole 128..1024-byte runs on both sides, with 4..16 bytes per lane.
+
+// 64 (c) x 256 (r) tile, bf16 in, f32 out.  LDS holds the tile as [c][r] 16-bit words.
+__global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
+    const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw,
+    const int64_t* __restrict__ perm_inv, const uint8_t* __restrict__ dead,
+    float* __restrict__ Xout, int64_t R, int64_t C) {
+    constexpr int TC = 64, TR = 256, PITCH = TR + 4;     // rows stay 8-byte aligned
+    __shared__ __attribute__((aligned(8))) uint16_t tile[TC][PITCH];
+    const int64_t b = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
+    const int tid = threadIdx.x;
+    const uint16_t* __restrict__ Wb = W + b * w_stride;
+    {   // 16 lanes x 8 bytes cover one 128-byte row piece; 16 rows per pass
+        const int rr = tid >> 4, c4 = (tid & 15) * 4;
+        uint32_t keep = 0xF;
+        if (dead) {
+            const uint8_t* d = dead + b * C + c0 + c4;
+            keep = (d[0] ? 0u : 1u) | (d[1] ? 0u : 2u) | (d[2] ? 0u : 4u) | (d[3] ? 0u : 8u);
+        }
+#pragma unroll 4
+        for (int p = 0; p < TR / 16; ++p) {
+            const int r = 16 * p + rr;
+            const uint2 v = *reinterpret_cast<const uint2*>(Wb + (r0 + r) * ldw + c0 + c4);
+            tile[c4 + 0][r] = (keep & 1u) ? (uint16_t)(v.x & 0xFFFFu) : (uint16_t)0;
+            tile[c4 + 1][r] = (keep & 2u) ? (uint16_t)(v.x >> 16) : (uint16_t)0;
+            tile[c4 + 2][r] = (keep & 4u) ? (uint16_t)(v.y & 0xFFFFu) : (uint16_t)0;
+            tile[c4 + 3][r] = (keep & 8u) ? (uint16_t)(v.y >> 16) : (uint16_t)0;
+        }
+    }
+    __syncthreads();
+    {   // a wavefront writes the 256 floats (1 KiB) of one output row per instruction
+        const int cw = tid >> 6, r4 = (tid & 63) * 4;
+#pragma unroll 4
+        for (int cc = 0; cc < TC; cc += 4) {
+            const int c = cc + cw;
+            const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
+            const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
+                                         __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
+            *reinterpret_cast<float4*>(Xout + b * C * R + perm_inv[b * C + c0 + c] * R + r0 + r4) = o;
+        }
+    }
+}
+
+// 128 (c) x 256 (r) byte tile.  LDS holds it as [c][r]; a row of the result is gathered
+// back four bytes (four values of c) per lane.
+__global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
+    const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
+    uint8_t* __restrict__ qout, int64_t R, int64_t C) {
+    constexpr int TC = 128, TR = 256, PITCH = TR + 4;    // 65 words per row: odd
+    __shared__ __attribute__((aligned(4))) uint8_t tile[TC][PITCH];
+    const int64_t b = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
+    const int tid = threadIdx.x;
+    {   // a wavefront reads the 256 bytes of one source row per instruction
+        const int cw = tid >> 6, r4 = (tid & 63) * 4;
+#pragma unroll 4
+        for (int cc = 0; cc < TC; cc += 4) {
+            const int c = cc + cw;
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(
+                qin + b * C * R + perm_inv[b * C + c0 + c] * R + r0 + r4);
+            *reinterpret_cast<uint32_t*>(&tile[c][r4]) = v;
+        }
+    }
+    __syncthreads();
+    {   // 32 lanes x 4 bytes cover one 128-byte row piece; 8 rows per pass
+        const int rr = tid >> 5, c4 = (tid & 31) * 4;
+#pragma unroll 4
+        for (int p = 0; p < TR / 8; ++p) {
+            const int r = 8 * p + rr;
+            const uint32_t v = (uint32_t)tile[c4][r] | ((uint32_t)tile[c4 + 1][r] << 8) |
+                               ((uint32_t)tile[c4 + 2][r] << 16) | ((uint32_t)tile[c4 + 3][r] << 24);
+            *reinterpret_cast<uint32_t*>(qout + b * R * C + (r0 + r) * C + c0 + c4) = v;
+        }
+    }
+}
+
 // Hp[b][i][j] = H[b][perm[i]][perm[j]], dead rows/columns zeroed with a unit diagonal
 // (forge/gptq.py:100-103,117,145-149).  The source row is streamed into LDS with coalesced
 // loads, gathered from there in permuted order and written out coalesced, so HBM sees one
@@ -218,12 +297,20 @@ extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t 
     forge::KernelTiming timing("weight_to_solver_order", (hipStream_t)stream,
                                (double)batch * R * C * (4.0 + (w_dtype == FORGE_F32 ? 4.0 : 2.0)),
                                forge::WORK_BYTES);
-    if (w_dtype == FORGE_F32)
+    const bool fast = w_dtype == FORGE_BF16 && (R % 256) == 0 && (C % 64) == 0 && (ldw % 4) == 0 &&
+                      (w_stride % 4) == 0 && (reinterpret_cast<uintptr_t>(W) % 8) == 0 &&
+                      (reinterpret_cast<uintptr_t>(Xout) % 16) == 0 && R / 256 < 65536;
+    if (fast) {
+        const dim3 tiles((unsigned)(C / 64), (unsigned)(R / 256), (unsigned)batch);
+        to_solver_order_bf16_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(
+            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
+    } else if (w_dtype == FORGE_F32) {
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
             (const float*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
-    else
+    } else {
         to_solver_order_kernel<__hip_bfloat16><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
             (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
+    }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }
@@ -238,7 +325,14 @@ extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* per
     FORGE_REQUIRE(grid.y < 65536, "R too large");
     forge::KernelTiming timing("codes_to_layer_order", (hipStream_t)stream, 2.0 * batch * R * C,
                                forge::WORK_BYTES);
-    to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
+    const bool fast = (R % 256) == 0 && (C % 128) == 0 && (reinterpret_cast<uintptr_t>(qin) % 4) == 0 &&
+                      (reinterpret_cast<uintptr_t>(qout) % 4) == 0;
+    if (fast) {
+        const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
+        to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
+    } else {
+        to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
+    }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

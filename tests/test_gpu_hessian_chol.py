@@ -134,3 +134,44 @@ def test_pack_int4_layout(hip):
     pk8 = hip.pack_int4(codes.to(DEV), None, gs).cpu()                 # symmetric: zero = 8
     sh = torch.nn.functional.pad(codes.to(torch.int64), (0, (-C) % 8)).view(R, -1, 8)
     assert torch.equal(pk8.to(torch.int64) & 0xFFFFFFFF, sum(sh[:, :, k] << (4 * k) for k in range(8)))
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,R,C", [(2, 512, 384), (1, 256, 1152)])
+def test_layout_kernels_tall_tiles(hip, B, R, C):
+    """bf16 weights with R % 256 == 0 and C % 128 == 0 take the tall-tile transposes."""
+    g = torch.Generator().manual_seed(3)
+    W = torch.randn(B, R, C, generator=g).bfloat16()
+    perm = torch.stack([torch.randperm(C, generator=g) for _ in range(B)])
+    pinv = torch.argsort(perm, dim=1)
+    dead = (torch.rand(B, C, generator=g) < 0.05).to(torch.uint8)
+    Xo = hip.weight_to_solver_order(W.to(DEV), pinv.to(DEV), dead.to(DEV))
+    Xn = hip.weight_to_solver_order(W.to(DEV), pinv.to(DEV))
+    q = torch.randint(0, 16, (B, C, R), dtype=torch.uint8, generator=g)
+    qo = hip.codes_to_layer_order(q.to(DEV), pinv.to(DEV))
+    for b in range(B):
+        Wz = W[b].float().clone()
+        assert torch.equal(Xn[b].cpu(), Wz.t()[perm[b]].contiguous())
+        Wz[:, dead[b].bool()] = 0
+        assert torch.equal(Xo[b].cpu(), Wz.t()[perm[b]].contiguous())
+        assert torch.equal(qo[b].cpu(), q[b][pinv[b]].t().contiguous())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("C", [70, 1028, 2564, 4104])
+def test_hessian_permute_sizes(hip, C):
+    """Scalar form (C % 4 != 0) and the 2-, 4- and 8-chunk row forms, with a ragged last
+    group of rows and dead columns."""
+    g = torch.Generator().manual_seed(C)
+    Hh = torch.randn(1, C, C, generator=g)
+    Hh = Hh + Hh.transpose(1, 2)
+    perm = torch.randperm(C, generator=g).view(1, C)
+    dead = (torch.rand(1, C, generator=g) < 0.02).to(torch.uint8)
+    Hp, dmp = hip.hessian_permute(Hh.to(DEV), perm.to(DEV), dead.to(DEV), 0.01)
+    ref = Hh[0][perm[0]][:, perm[0]].clone()
+    d = dead[0].bool()
+    ref[d, :] = 0; ref[:, d] = 0; ref[d, d] = 1
+    assert torch.equal(Hp[0].cpu(), ref)
+    assert dmp[0].item() == pytest.approx(0.01 * ref.diag().mean().item(), rel=1e-5)
+
+
+
