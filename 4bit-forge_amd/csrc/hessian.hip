@@ -99,6 +99,8 @@ __device__ __forceinline__ void store_tile(float* __restrict__ H, int64_t C, int
 
 // ---------------------------------------------------------------- rank-k (bf16 MFMA)
 // grid: (tile pair, group).  128x128 tile, 4 wavefronts, each 64x64 = 2x2 MFMA tiles.
+// BLEND = false: every group has beta == 0 (no old values, fewer registers).
+template <bool BLEND>
 __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict__ pack,
                                                         const GroupDesc* __restrict__ gd,
                                                         float* __restrict__ Hall, int64_t C,
@@ -135,6 +137,24 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
         pa[i] = base + (int64_t)(cta[i] < nct ? cta[i] : 0) * g.nchunk * 64;
         pb[i] = base + (int64_t)(ctb[i] < nct ? ctb[i] : 0) * g.nchunk * 64;
     }
+    // With few token rows per expert the kernel is one pass over H: the old values of a
+    // whole tile are requested before the K loop so that their latency overlaps it (and
+    // each other), instead of one load-wait-store round trip per accumulator register.
+    const bool full = (ti + 1) * 128 <= C && (tj + 1) * 128 <= C;    // uniform
+    const bool blend = BLEND && g.beta != 0.0f;
+    f32x16 old[2][2];
+    if (BLEND && full && blend) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                const float* __restrict__ Ht =
+                    H + (int64_t)(cta[mi] * 32 + (lane >> 5) * 4) * C + ctb[ni] * 32 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    old[mi][ni][v] = Ht[(int64_t)((v >> 2) * 8 + (v & 3)) * C];
+            }
+    }
     for (int kc = 0; kc < g.nchunk; ++kc) {
         bf16x8 a[2], b[2];
 #pragma unroll
@@ -152,12 +172,47 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
                     __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
     }
     const bool mirror = ti != tj;
+    if (full) {
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+        for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-            store_tile(H, C, cta[mi] * 32, ctb[ni] * 32, acc[mi][ni], g.alpha, g.beta, mirror,
-                       tbuf[wave], lane);
+            for (int ni = 0; ni < 2; ++ni) {
+                const int row0 = cta[mi] * 32, col0 = ctb[ni] * 32;
+                f32x16 out;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float o = g.alpha * acc[mi][ni][v];
+                    if (BLEND && blend) o = __builtin_fmaf(g.beta, old[mi][ni][v], o);
+                    out[v] = o;
+                }
+                float* __restrict__ Ht = H + (int64_t)(row0 + (lane >> 5) * 4) * C + col0 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) Ht[(int64_t)((v >> 2) * 8 + (v & 3)) * C] = out[v];
+                if (mirror) {   // the wavefront's own 32x32 staging tile: no workgroup barrier needed
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        tbuf[wave][(v >> 2) * 8 + (lane >> 5) * 4 + (v & 3)][lane & 31] = out[v];
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    float* __restrict__ Hm = H + (int64_t)(col0 + (lane >> 5) * 4) * C + row0 + (lane & 31);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int jj = (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                        Hm[(int64_t)((v >> 2) * 8 + (v & 3)) * C] = tbuf[wave][lane & 31][jj];
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+                store_tile(H, C, cta[mi] * 32, ctb[ni] * 32, acc[mi][ni], g.alpha, g.beta, mirror,
+                           tbuf[wave], lane);
+    }
 }
 
 // ---------------------------------------------------------------- rank-k (f32 MFMA)
@@ -318,8 +373,14 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
         forge::KernelTiming timing("hessian_syrk_bf16", st,
                                    2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
                                    forge::WORK_FLOPS);
-        syrk_bf16_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev, H, C,
-                                                                               NT);
+        bool any_blend = false;
+        for (int e = 0; e < n_groups; ++e) any_blend = any_blend || beta_host[e] != 0.0f;
+        if (any_blend)
+            syrk_bf16_kernel<true><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev,
+                                                                                         H, C, NT);
+        else
+            syrk_bf16_kernel<false><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev,
+                                                                                          H, C, NT);
         FORGE_LAUNCH_CHECK();
     } else {
         forge::KernelTiming timing("hessian_syrk_f32", st,
