@@ -39,15 +39,6 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
 // thread (ty,tx) owns the 8x8 sub-block P[8ty.., 8tx..] in registers.  Each elimination
 // step publishes the (unscaled) pivot row through LDS and costs one barrier:
 //   P[i][j] -= (row[i] / piv) * row[j],   D[c][j] = row[j] / sqrt(piv) afterwards.
-__device__ __forceinline__ void select_row(const float (&P)[8][8], int which, float (&out)[8]) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) out[j] = P[0][j];
-#pragma unroll
-    for (int i = 1; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = (which == i) ? P[i][j] : out[j];
-}
-
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
     float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
@@ -63,27 +54,42 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     const int n = (int)((C - m0) < NB ? (C - m0) : NB);
     const float* __restrict__ Ab = A + b * C * C;
 
+    // symmetric tile: both halves were produced by the same GEMM; read the lower one.
+    // (Full blocks load without per-element tests so that the 64 loads are in flight together.)
     float P[8][8];
+    if (n == NB) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int r = 8 * ty + i, c = 8 * tx + j;
-            // symmetric tile: both halves were produced by the same GEMM; read the lower one
-            const int rr = r > c ? r : c, cc = r > c ? c : r;
-            float v = (r == c) ? 1.0f : 0.0f;
-            if (rr < n) v = Ab[(m0 + rr) * C + m0 + cc];
-            P[i][j] = v;
-        }
+            for (int j = 0; j < 8; ++j) {
+                const int r = 8 * ty + i, c = 8 * tx + j;
+                const int rr = r > c ? r : c, cc = r > c ? c : r;
+                P[i][j] = Ab[(m0 + rr) * C + m0 + cc];
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int r = 8 * ty + i, c = 8 * tx + j;
+                const int rr = r > c ? r : c, cc = r > c ? c : r;
+                float v = (r == c) ? 1.0f : 0.0f;
+                if (rr < n) v = Ab[(m0 + rr) * C + m0 + cc];
+                P[i][j] = v;
+            }
+    }
     if (tid == 0) s_fail = 0;
 
     // ---- P = D^T D, eliminating from the last row upwards
-    for (int c = NB - 1; c >= 0; --c) {
-        if (ty == (c >> 3)) {
-            float row[8];
-            select_row(P, c & 7, row);
+    // (outer loop over the 16 row groups, inner 8 steps unrolled: P[c & 7] is then a fixed
+    // register row instead of a select over all eight)
+    for (int cb = NB / 8 - 1; cb >= 0; --cb)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) Dm[c][8 * tx + j] = row[j];
+    for (int ci = 7; ci >= 0; --ci) {
+        const int c = 8 * cb + ci;
+        if (ty == cb) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) Dm[c][8 * tx + j] = P[ci][j];
         }
         __syncthreads();
         const float piv = Dm[c][c];
@@ -119,15 +125,16 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
-    for (int k = 0; k < NB; ++k) {
-        if (ty == (k >> 3)) {
-            float row[8];
-            select_row(P, k & 7, row);
+    for (int kb = 0; kb < NB / 8; ++kb)
+#pragma unroll
+    for (int ki = 0; ki < 8; ++ki) {
+        const int k = 8 * kb + ki;
+        if (ty == kb) {
             const float rc = drc[k];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int col = 8 * tx + j;
-                Zm[k][col] = col <= k ? ((col == k ? 1.0f : 0.0f) - row[j]) * rc : 0.0f;
+                Zm[k][col] = col <= k ? ((col == k ? 1.0f : 0.0f) - P[ki][j]) * rc : 0.0f;
             }
         }
         __syncthreads();
