@@ -55,6 +55,23 @@ __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, floa
     err = x - deq;
 }
 
+// x + (-u_K) * e as ONE fused multiply-add, where u_K is the `u` register of lane K of this
+// lane's row of 16 lanes (DPP row broadcast): sixteen U values sit in one VGPR, spread over
+// the lanes of a row, instead of each being broadcast to every lane through LDS.  Same
+// arithmetic as fmaf(-u, e, x).  The leading s_nop covers the two wait states a DPP read
+// needs after a VALU write of its source, which the compiler cannot see inside the asm.
+template <int K>
+__device__ __forceinline__ void fnma_row_bcast(float& x, float u, float e) {
+    asm("v_fmac_f32_dpp %0, -%1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(x)
+        : "v"(u), "v"(e), "n"(K));
+}
+__device__ __forceinline__ float dpp_source(float u) {
+    asm volatile("s_nop 1" : "+v"(u));
+    return u;
+}
+#define FORGE_FOR_16(M) M(0) M(1) M(2) M(3) M(4) M(5) M(6) M(7) M(8) M(9) M(10) M(11) M(12) M(13) M(14) M(15)
+
 #ifndef FORGE_SWEEP_RING
 #define FORGE_SWEEP_RING 3
 #endif
@@ -110,13 +127,35 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
         __syncthreads();
     }
 
+    // Scale and zero of a column do not depend on the sweep: all 32 pairs of a sub-block
+    // are requested together, one sub-block ahead (while the previous sub-block's errors are
+    // pushed), so that the serial chain never waits on them column by column.
+    float sv[TAIL ? 1 : SB], qv[TAIL ? 1 : SB];
+    auto load_meta = [&](int64_t c_first) {
+        if constexpr (!TAIL) {
+#pragma unroll
+            for (int t = 0; t < SB; ++t) {
+                const int64_t c = c_first + t;
+                if constexpr (PER_ELEM) {
+                    sv[t] = sc[c * R];
+                    qv[t] = qz[c * R];
+                } else {
+                    const int64_t g = gi[c];
+                    sv[t] = sc[g * R];
+                    qv[t] = qz[g * R];
+                }
+            }
+        }
+    };
+    load_meta(a.c0);
+
     for (int sb = 0; sb < nsub; ++sb) {
         const int64_t cs = a.c0 + (int64_t)sb * SB;   // first column of this sub-block
         const int rem = bw - sb * SB;                 // block columns from cs on
         float err[SB];
         uint32_t mask = 0u;
 
-        auto select_and_quantize = [&](int t, int64_t c) {
+        auto select_and_quantize = [&](int t, int64_t c, float s, float q0) {
             bool keep = true;
             if constexpr (SPARSE) {
                 if ((t & 3) == 0) {
@@ -132,15 +171,6 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                     if (best_k > -1) mask |= 1u << (t + best_k);
                 }
                 keep = (mask >> t) & 1u;
-            }
-            float s, q0;
-            if constexpr (PER_ELEM) {
-                s = sc[c * R];
-                q0 = qz[c * R];
-            } else {
-                const int64_t g = gi[c];
-                s = sc[g * R];
-                q0 = qz[g * R];
             }
             float e, deq, qf;
             quantize_scalar(x[t], s, q0, maxq, qf, deq, e);
@@ -180,60 +210,46 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             // alone the scheduler hoists hundreds of reads and spills the x registers).
             // serial chain inside the sub-block: step = (row t, half h) -> 2*SB steps
             {
-                float4 ring[RING][4];
-                auto rd = [&](int step, float4 (&dst)[4]) {
-                    const float4* p = reinterpret_cast<const float4*>(&Up[buf][step >> 1][(step & 1) * 16]);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) dst[j] = p[j];
-                };
-                rd(0, ring[0]);
-                if (RING > 2) rd(1, ring[1]);
+                const int l16 = threadIdx.x & 15;
+                float ring[RING];
+                auto rd = [&](int step) { return Up[buf][step >> 1][(step & 1) * 16 + l16]; };
+                ring[0] = rd(0);
+                if (RING > 2) ring[1] = rd(1);
 #pragma unroll
                 for (int step = 0; step < 2 * SB; ++step) {
                     const int t = step >> 1, h = step & 1;
-                    if (step + RING - 1 < 2 * SB) rd(step + RING - 1, ring[(step + RING - 1) % RING]);
-                    if (h == 0) select_and_quantize(t, cs + t);
+                    if (step + RING - 1 < 2 * SB) ring[(step + RING - 1) % RING] = rd(step + RING - 1);
+                    if (h == 0) select_and_quantize(t, cs + t, sv[t], qv[t]);
                     __builtin_amdgcn_sched_barrier(0);
-                    const float4(&u4)[4] = ring[step % RING];
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) {
-                        const int col = h * 16 + k;
-                        if (col > t) {
-                            const float4 q4 = u4[k >> 2];
-                            const float uv = (k & 3) == 0 ? q4.x : (k & 3) == 1 ? q4.y : (k & 3) == 2 ? q4.z : q4.w;
-                            x[col] = __builtin_fmaf(-uv, err[t], x[col]);
-                        }
-                    }
+                    const float u16 = dpp_source(ring[step % RING]);
+                    const float e = err[t];
+#define FORGE_DIAG_FMA(k) if (h * 16 + k > t) fnma_row_bcast<k>(x[h * 16 + k], u16, e);
+                    FORGE_FOR_16(FORGE_DIAG_FMA)
+#undef FORGE_DIAG_FMA
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
             if constexpr (SPARSE) Mw[(cs >> 5) * R] = mask;
+            if (more) load_meta(cs + SB);
             // push the 32 errors into the rest of the block
 #pragma unroll
             for (int u = 1; u < NSB; ++u) {
                 if (sb + u < nsub) {
-                    float4 ring[RING][4];
-                    auto rd = [&](int step, float4 (&dst)[4]) {
-                        const float4* p = reinterpret_cast<const float4*>(
-                            &Up[buf][step >> 1][u * SB + (step & 1) * 16]);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) dst[j] = p[j];
-                    };
-                    rd(0, ring[0]);
-                    if (RING > 2) rd(1, ring[1]);
+                    const int l16 = threadIdx.x & 15;
+                    float ring[RING];
+                    auto rd = [&](int step) { return Up[buf][step >> 1][u * SB + (step & 1) * 16 + l16]; };
+                    ring[0] = rd(0);
+                    if (RING > 2) ring[1] = rd(1);
 #pragma unroll
                     for (int step = 0; step < 2 * SB; ++step) {
                         const int t = step >> 1, h = step & 1;
-                        if (step + RING - 1 < 2 * SB) rd(step + RING - 1, ring[(step + RING - 1) % RING]);
+                        if (step + RING - 1 < 2 * SB) ring[(step + RING - 1) % RING] = rd(step + RING - 1);
                         __builtin_amdgcn_sched_barrier(0);
-                        const float4(&u4)[4] = ring[step % RING];
-#pragma unroll
-                        for (int k = 0; k < 16; ++k) {
-                            const int col = u * SB + h * 16 + k;
-                            const float4 q4 = u4[k >> 2];
-                            const float uv = (k & 3) == 0 ? q4.x : (k & 3) == 1 ? q4.y : (k & 3) == 2 ? q4.z : q4.w;
-                            x[col] = __builtin_fmaf(-uv, err[t], x[col]);
-                        }
+                        const float u16 = dpp_source(ring[step % RING]);
+                        const float e = err[t];
+#define FORGE_PUSH_FMA(k) fnma_row_bcast<k>(x[u * SB + h * 16 + k], u16, e);
+                        FORGE_FOR_16(FORGE_PUSH_FMA)
+#undef FORGE_PUSH_FMA
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -256,7 +272,16 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             for (int t = 0; t < SB; ++t) {
                 err[t] = 0.0f;
                 if (t < rem) {
-                    select_and_quantize(t, cs + t);
+                    float s_t, q0_t;
+                    if constexpr (PER_ELEM) {
+                        s_t = sc[(cs + t) * R];
+                        q0_t = qz[(cs + t) * R];
+                    } else {
+                        const int64_t g = gi[cs + t];
+                        s_t = sc[g * R];
+                        q0_t = qz[g * R];
+                    }
+                    select_and_quantize(t, cs + t, s_t, q0_t);
                     const float* __restrict__ Urow = U + (cs + t) * C + cs;
                     for (int k = t + 1; k < rem; ++k)
                         x[k] = __builtin_fmaf(-Urow[k], err[t], x[k]);
