@@ -35,9 +35,10 @@ PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, T
 # HBM bytes per launch of the factorisation GEMM on the default workload (64 experts per
 # step), from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each
 # scaled by what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and
-# x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  Algorithmic bytes per
-# launch (operands + accumulator tile once) are ~1.8e9.
-MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 2.14e9}
+# x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  The operand data a
+# launch has to read once (rows below the current block of the factor and of its inverse)
+# averages ~4.4e9 bytes over the 55 launches of a C=7168 factorisation: no wasted re-reads.
+MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 4.40e9}
 
 KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit)
     "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s"),
