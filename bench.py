@@ -201,7 +201,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-              "(experts would shard across GPUs without any exchange, see DESIGN.md)", file=sys.stderr)
+              "(experts are independent and would shard across GPUs without any exchange)", file=sys.stderr)
         sys.exit(2)
 
     import torch
