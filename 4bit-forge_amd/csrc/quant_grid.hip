@@ -23,7 +23,8 @@ __device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
 }
 
 __device__ __forceinline__ float clampf(float v, float lo, float hi) {
-    return fminf(fmaxf(v, lo), hi);
+    // one v_med3_f32; equal to fminf(fmaxf(v, lo), hi) for lo <= hi (a NaN gives lo in both)
+    return __builtin_amdgcn_fmed3f(v, lo, hi);
 }
 
 // Scale and zero of one group from its extrema (quant_grid.cu:74-97).

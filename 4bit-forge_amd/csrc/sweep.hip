@@ -50,7 +50,8 @@ struct SweepArgs {
 __device__ __forceinline__ void quantize_scalar(float x, float s, float q0, float maxq, float& qf,
                                                 float& deq, float& err) {
     const float inv_s = 1.0f / (s + kEps);
-    qf = fminf(fmaxf(__builtin_rintf(__builtin_fmaf(x, inv_s, q0)), 0.0f), maxq);
+    // v_med3_f32: same value as fminf(fmaxf(., 0), maxq)
+    qf = __builtin_amdgcn_fmed3f(__builtin_rintf(__builtin_fmaf(x, inv_s, q0)), 0.0f, maxq);
     deq = __builtin_fmaf(qf, s, -(q0 * s));
     err = x - deq;
 }
