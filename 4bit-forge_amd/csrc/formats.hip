@@ -1,5 +1,7 @@
 // Data formats either side of the solve: the fp8 block-scaled checkpoint weights that
-// come in, and the 1:4 sparse int4 words that go out.  Both are HBM-bound byte movers.
+// come in, the 1:4 sparse int4 words that go out, the dequantised weight written back into
+// the layer and the gather of routed rows in front of the Hessian update.  All HBM-bound
+// byte movers.
 #include "common.h"
 
 namespace {
@@ -96,6 +98,110 @@ __global__ __launch_bounds__(256) void pack_sparse14_kernel(
     out[(g2 * R + r) * 2 + 1] = word[1];
 }
 
+// (q - q0) * s per group -> bf16/f32; 16 codes per thread (forge/utils/engine.py:71-97).
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void dequantize_groups_kernel(
+    const uint8_t* __restrict__ q, const float* __restrict__ scales,
+    const float* __restrict__ qzeros, void* __restrict__ out, int64_t R, int64_t C, int64_t gs,
+    int64_t G, int64_t batch) {
+    const int64_t per_row = (C + 15) / 16;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= batch * R * per_row) return;
+    const int64_t br = idx / per_row;                      // b * R + r
+    const int64_t c0 = (idx - br * per_row) * 16;
+    const uint8_t* __restrict__ src = q + br * C + c0;
+    const float* __restrict__ s = scales + br * G;
+    const float* __restrict__ z = qzeros + br * G;
+    const bool vec = c0 + 16 <= C && ((reinterpret_cast<uintptr_t>(src) & 15u) == 0);
+    uint8_t code[16];
+    if (vec) {
+        const uint4 v = *reinterpret_cast<const uint4*>(src);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 16; ++k) code[k] = (uint8_t)(w[k >> 2] >> (8 * (k & 3)));
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) code[k] = c0 + k < C ? src[k] : (uint8_t)0;
+    }
+    float val[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        const int64_t g = (c0 + k < C ? c0 + k : C - 1) / gs;
+        val[k] = ((float)code[k] - z[g]) * s[g];
+    }
+    if constexpr (OUT_BF16) {
+        uint16_t* __restrict__ dst = reinterpret_cast<uint16_t*>(out) + br * C + c0;
+        if (c0 + 16 <= C && ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0)) {
+            uint32_t pk[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                pk[k] = (uint32_t)f32_to_bf16_rne(val[2 * k]) | ((uint32_t)f32_to_bf16_rne(val[2 * k + 1]) << 16);
+            reinterpret_cast<uint4*>(dst)[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            reinterpret_cast<uint4*>(dst)[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                if (c0 + k < C) dst[k] = f32_to_bf16_rne(val[k]);
+        }
+    } else {
+        float* __restrict__ dst = reinterpret_cast<float*>(out) + br * C + c0;
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+            if (c0 + k < C) dst[k] = val[k];
+    }
+}
+
+// out[i][:] = X[row_idx[i]][:] * weight[i]; one workgroup per output row, 8 bytes per lane.
+template <typename T, bool SCALE>
+__global__ __launch_bounds__(256) void gather_scaled_rows_kernel(
+    const T* __restrict__ X, int64_t ldx, int64_t C, const int64_t* __restrict__ row_idx,
+    const T* __restrict__ weight, T* __restrict__ out) {
+    const int64_t i = blockIdx.x;
+    const T* __restrict__ src = X + row_idx[i] * ldx;
+    T* __restrict__ dst = out + i * C;
+    float w = 1.0f;
+    if constexpr (SCALE) {
+        if constexpr (sizeof(T) == 2) w = __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(weight)[i] << 16);
+        else w = reinterpret_cast<const float*>(weight)[i];
+    }
+    constexpr int PER = 8 / sizeof(T);                      // elements per 8-byte access
+    const bool vec = (C % PER) == 0 && ((reinterpret_cast<uintptr_t>(src) & 7u) == 0) &&
+                     ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0);
+    if (vec) {
+        for (int64_t j = threadIdx.x; j < C / PER; j += blockDim.x) {
+            uint2 v = reinterpret_cast<const uint2*>(src)[j];
+            if constexpr (SCALE) {
+                if constexpr (sizeof(T) == 2) {
+                    const uint32_t in[2] = {v.x, v.y};
+                    uint32_t o[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const float a = __uint_as_float(in[h] << 16) * w;
+                        const float b = __uint_as_float(in[h] & 0xFFFF0000u) * w;
+                        o[h] = (uint32_t)f32_to_bf16_rne(a) | ((uint32_t)f32_to_bf16_rne(b) << 16);
+                    }
+                    v = make_uint2(o[0], o[1]);
+                } else {
+                    v = make_uint2(__float_as_uint(__uint_as_float(v.x) * w),
+                                   __float_as_uint(__uint_as_float(v.y) * w));
+                }
+            }
+            reinterpret_cast<uint2*>(dst)[j] = v;
+        }
+    } else {
+        for (int64_t j = threadIdx.x; j < C; j += blockDim.x) {
+            if constexpr (sizeof(T) == 2) {
+                const uint16_t x = reinterpret_cast<const uint16_t*>(src)[j];
+                reinterpret_cast<uint16_t*>(dst)[j] =
+                    SCALE ? f32_to_bf16_rne(__uint_as_float((uint32_t)x << 16) * w) : x;
+            } else {
+                const float x = reinterpret_cast<const float*>(src)[j];
+                reinterpret_cast<float*>(dst)[j] = SCALE ? x * w : x;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int forge_fp8_e4m3_block_dequant(const uint8_t* w, const float* scale_inv, void* out,
@@ -132,6 +238,60 @@ extern "C" int forge_pack_sparsegptq14_to_u64x2(const uint8_t* qweight_rc, const
                                (double)R * C / 4.0 + 8.0 * G32 * R + 16.0 * G2 * R, forge::WORK_BYTES);
     pack_sparse14_kernel<<<dim3((unsigned)forge::ceil_div(G2 * R, 256)), dim3(256), 0,
                            (hipStream_t)stream>>>(qweight_rc, M, scales, out, C, R, G32);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_dequantize_groups(const uint8_t* q, const float* scales, const float* qzeros,
+                                       void* out, int out_dtype, int64_t batch, int64_t R,
+                                       int64_t C, int64_t gs, forge_stream_t stream) {
+    FORGE_REQUIRE(out_dtype == FORGE_F32 || out_dtype == FORGE_BF16, "out_dtype=%d", out_dtype);
+    FORGE_REQUIRE(batch >= 0 && R >= 0 && C >= 0 && gs >= 1, "bad shape");
+    if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
+    FORGE_REQUIRE(q && scales && qzeros && out, "null pointer");
+    const int64_t G = forge::ceil_div(C, gs);
+    const int64_t n = batch * R * forge::ceil_div(C, 16);
+    forge::KernelTiming timing("dequantize_groups", (hipStream_t)stream,
+                               (double)batch * R * (C * (out_dtype == FORGE_BF16 ? 3.0 : 5.0) + 8.0 * G),
+                               forge::WORK_BYTES);
+    const dim3 grid((unsigned)forge::ceil_div(n, 256));
+    if (out_dtype == FORGE_BF16)
+        dequantize_groups_kernel<true><<<grid, dim3(256), 0, (hipStream_t)stream>>>(q, scales, qzeros, out,
+                                                                                  R, C, gs, G, batch);
+    else
+        dequantize_groups_kernel<false><<<grid, dim3(256), 0, (hipStream_t)stream>>>(q, scales, qzeros, out,
+                                                                                   R, C, gs, G, batch);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_gather_scaled_rows(const void* X, int x_dtype, int64_t ldx, int64_t T, int64_t C,
+                                        const int64_t* row_idx, const void* weight, void* out,
+                                        int64_t N, forge_stream_t stream) {
+    FORGE_REQUIRE(x_dtype == FORGE_F32 || x_dtype == FORGE_BF16, "x_dtype=%d", x_dtype);
+    FORGE_REQUIRE(N >= 0 && N < (1LL << 31) && T >= 0 && C >= 0 && ldx >= C, "bad shape");
+    if (N == 0 || C == 0) return FORGE_OK;
+    FORGE_REQUIRE(T > 0, "rows requested from an empty matrix");
+    FORGE_REQUIRE(X && row_idx && out, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    forge::KernelTiming timing("gather_scaled_rows", st,
+                               2.0 * N * C * (x_dtype == FORGE_BF16 ? 2.0 : 4.0), forge::WORK_BYTES);
+    const dim3 grid((unsigned)N), block(256);
+    if (x_dtype == FORGE_BF16) {
+        if (weight)
+            gather_scaled_rows_kernel<uint16_t, true><<<grid, block, 0, st>>>(
+                (const uint16_t*)X, ldx, C, row_idx, (const uint16_t*)weight, (uint16_t*)out);
+        else
+            gather_scaled_rows_kernel<uint16_t, false><<<grid, block, 0, st>>>(
+                (const uint16_t*)X, ldx, C, row_idx, nullptr, (uint16_t*)out);
+    } else {
+        if (weight)
+            gather_scaled_rows_kernel<float, true><<<grid, block, 0, st>>>(
+                (const float*)X, ldx, C, row_idx, (const float*)weight, (float*)out);
+        else
+            gather_scaled_rows_kernel<float, false><<<grid, block, 0, st>>>(
+                (const float*)X, ldx, C, row_idx, nullptr, (float*)out);
+    }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

@@ -57,6 +57,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_pack_int4": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_fp8_e4m3_block_dequant": ([vp, vp, vp, i32, i64, i64, i64, i64, i64, vp], i32),
         "forge_pack_sparsegptq14_to_u64x2": ([vp, vp, vp, vp, i64, i64, vp], i32),
+        "forge_dequantize_groups": ([vp, vp, vp, vp, i32, i64, i64, i64, i64, vp], i32),
+        "forge_gather_scaled_rows": ([vp, i32, i64, i64, i64, vp, vp, vp, i64, vp], i32),
     }
     for name, (args, res) in sigs.items():
         fn = getattr(lib, name)          # AttributeError here = library/header mismatch
@@ -73,6 +75,7 @@ EXPORTED_SYMBOLS = (
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
+    "forge_dequantize_groups", "forge_gather_scaled_rows",
 )
 
 
@@ -366,6 +369,43 @@ class _HipKernels:
         with torch.cuda.device(qweight_rc.device):
             self._check(self._lib.forge_pack_sparsegptq14_to_u64x2(
                 _ptr(qweight_rc), _ptr(M), _ptr(scales.float()), _ptr(out), R, C, _stream()))
+        return out
+
+    def dequantize_groups(self, qweight, scales, qzeros, group_size, dtype=torch.bfloat16):
+        """qweight [R,C] or [B,R,C] u8, scales/qzeros [.., R*G] f32 -> (q - q0) * s in `dtype`
+        (forge/utils/engine.py:71-97)."""
+        _need_cuda(qweight, scales, qzeros)
+        squeeze = qweight.dim() == 2
+        q3 = (qweight.unsqueeze(0) if squeeze else qweight).contiguous()
+        B, R, C = q3.shape
+        G = (C + group_size - 1) // group_size
+        s2 = scales.reshape(B, -1).float().contiguous()
+        z2 = qzeros.reshape(B, -1).float().contiguous()
+        if q3.dtype != torch.uint8 or s2.shape[1] != R * G or z2.shape[1] != R * G:
+            raise ValueError(f"Expected uint8 codes and scales/qzeros numel == R*G ({R * G})")
+        out = torch.empty((B, R, C), dtype=dtype, device=q3.device)
+        with torch.cuda.device(q3.device):
+            self._check(self._lib.forge_dequantize_groups(
+                _ptr(q3), _ptr(s2), _ptr(z2), _ptr(out), _dtype_code(out), B, R, C, group_size,
+                _stream()))
+        return out[0] if squeeze else out
+
+    def gather_scaled_rows(self, X, row_idx, weight=None):
+        """out[i] = X[row_idx[i]] * weight[i] in X's dtype (weight None: plain gather);
+        X [T,C] bf16/f32 with unit column stride, row_idx [N] int64."""
+        _need_cuda(X, row_idx, weight)
+        assert X.dim() == 2 and X.stride(1) == 1 and row_idx.dtype == torch.int64
+        row_idx = row_idx.contiguous()
+        if weight is not None:
+            weight = weight.to(X.dtype).contiguous()
+            assert weight.numel() == row_idx.numel()
+        T, C = X.shape
+        N = row_idx.numel()
+        out = torch.empty((N, C), dtype=X.dtype, device=X.device)
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_gather_scaled_rows(
+                _ptr(X), _dtype_code(X), X.stride(0), T, C, _ptr(row_idx), _ptr(weight), _ptr(out),
+                N, _stream()))
         return out
 
 

@@ -182,6 +182,25 @@ int forge_pack_sparsegptq14_to_u64x2(const uint8_t* qweight_rc, const uint32_t* 
                                      const float* scales, uint64_t* out, int64_t R, int64_t C,
                                      forge_stream_t stream);
 
+/* Quantised weight back to the layer's dtype, for the re-forward that feeds the next
+ * block's calibration (dequantize_forge_full, forge/utils/engine.py:71-97):
+ * out[b][r][c] = ((f32) q[b][r][c] - qzeros[b][r*G + c/gs]) * scales[b][r*G + c/gs], a
+ * subtraction and a multiplication in f32, then rounded to out_dtype (FORGE_BF16: nearest
+ * even, or FORGE_F32).  q [batch, R, C] u8, scales/qzeros [batch, R*G] f32, G = ceil(C/gs). */
+int forge_dequantize_groups(const uint8_t* q, const float* scales, const float* qzeros, void* out,
+                            int out_dtype, int64_t batch, int64_t R, int64_t C, int64_t gs,
+                            forge_stream_t stream);
+
+/* The front of the Hessian update for fused-expert layers (the per-expert gather of
+ * forge/utils/engine.py:229-238: x_e = x[tok_idx]; x_e_w = x_e * w[:, None]):
+ * out[i][:] = X[row_idx[i]][:] * weight[i], the product rounded to x_dtype (weight NULL =
+ * plain gather).  X [T, C] with row pitch ldx, row_idx [N] int64 (rows already grouped by
+ * expert by the caller), weight [N] in x_dtype, out [N, C] contiguous.  Indices outside
+ * [0, T) are an error of the caller; they are not checked on the device. */
+int forge_gather_scaled_rows(const void* X, int x_dtype, int64_t ldx, int64_t T, int64_t C,
+                             const int64_t* row_idx, const void* weight, void* out, int64_t N,
+                             forge_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

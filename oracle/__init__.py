@@ -362,3 +362,28 @@ def dequantize(qweight, scales, qzeros, group_size):
     s = scales.reshape(R, G).repeat_interleave(group_size, dim=1)[:, :C]
     z = qzeros.reshape(R, G).repeat_interleave(group_size, dim=1)[:, :C]
     return (qweight.to(torch.float32) - z.to(torch.float32)) * s.to(torch.float32)
+
+
+def gather_scaled_rows(X, row_idx, weight=None):
+    """x_e = x[tok_idx]; x_e_w = x_e * w.unsqueeze(-1) with w in x's dtype
+    (forge/utils/engine.py:229-238)."""
+    rows = X[row_idx]
+    if weight is None:
+        return rows
+    return rows * weight.to(X.dtype).unsqueeze(-1)
+
+
+def routed_rows(x, router_indices, routing_weights, num_experts):
+    """The per-expert loop of the fused-expert hook (forge/utils/engine.py:224-238), its
+    scaled rows concatenated in expert order with their offsets."""
+    ri2 = router_indices.reshape(-1, router_indices.shape[-1] if router_indices.ndim > 1 else 1)
+    rw2 = None if routing_weights is None else routing_weights.reshape(ri2.shape)
+    parts, offsets = [], [0]
+    for e in range(num_experts):
+        tok_idx, k_idx = (ri2 == e).nonzero(as_tuple=True)
+        x_e = x[tok_idx]
+        if rw2 is not None:
+            x_e = x_e * rw2[tok_idx, k_idx].to(x.dtype).unsqueeze(-1)
+        parts.append(x_e)
+        offsets.append(offsets[-1] + int(tok_idx.numel()))
+    return torch.cat(parts, 0), offsets
