@@ -42,10 +42,10 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
     float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
-    extern __shared__ float smem[];                      // 2 * NB * LDP floats (135 KB)
+    extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 * NB * LDP floats (135 KB)
     float (*Dm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem);
     float (*Zm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem + NB * LDP);
-    __shared__ float dsq[NB], drc[NB];
+    __shared__ float dsq[NB], drc[NB], s_inv[NB];
     __shared__ int s_fail;
 
     const int64_t b = blockIdx.x;
@@ -79,6 +79,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
             }
     }
     if (tid == 0) s_fail = 0;
+    __syncthreads();   // the pivot owners below test it
 
     // ---- P = D^T D, eliminating from the last row upwards
     // (outer loop over the 16 row groups, inner 8 steps unrolled: P[c & 7] is then a fixed
@@ -88,19 +89,25 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     for (int ci = 7; ci >= 0; --ci) {
         const int c = 8 * cb + ci;
         if (ty == cb) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) Dm[c][8 * tx + j] = P[ci][j];
+            *reinterpret_cast<float4*>(&Dm[c][8 * tx]) = make_float4(P[ci][0], P[ci][1], P[ci][2], P[ci][3]);
+            *reinterpret_cast<float4*>(&Dm[c][8 * tx + 4]) = make_float4(P[ci][4], P[ci][5], P[ci][6], P[ci][7]);
+            // the owner of the pivot divides once for everybody (the division is the longest
+            // dependent chain of a step)
+            if (tx == cb) {
+                const float piv = P[ci][ci];
+                s_inv[c] = piv > 0.0f ? 1.0f / piv : 0.0f;
+                if (!(piv > 0.0f) && s_fail == 0) s_fail = c + 1;
+            }
         }
         __syncthreads();
-        const float piv = Dm[c][c];
-        const bool ok = piv > 0.0f;
-        if (!ok && tid == 0 && s_fail == 0) s_fail = c + 1;
-        const float inv = ok ? 1.0f / piv : 0.0f;
-        float ri[8], rj[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) ri[i] = Dm[c][8 * ty + i] * inv;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) rj[j] = Dm[c][8 * tx + j];
+        const float inv = s_inv[c];
+        const float4 a0 = *reinterpret_cast<const float4*>(&Dm[c][8 * ty]);
+        const float4 a1 = *reinterpret_cast<const float4*>(&Dm[c][8 * ty + 4]);
+        const float4 b0 = *reinterpret_cast<const float4*>(&Dm[c][8 * tx]);
+        const float4 b1 = *reinterpret_cast<const float4*>(&Dm[c][8 * tx + 4]);
+        const float ri[8] = {a0.x * inv, a0.y * inv, a0.z * inv, a0.w * inv,
+                             a1.x * inv, a1.y * inv, a1.z * inv, a1.w * inv};
+        const float rj[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
@@ -125,28 +132,40 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
-    for (int kb = 0; kb < NB / 8; ++kb)
+    for (int kb = 0; kb < NB / 8; ++kb) {
+        // D does not change any more: the 8x8 block of it that these 8 steps multiply by is
+        // fetched once, row-wise, outside the serial chain
+        float Dblk[8][8];
 #pragma unroll
-    for (int ki = 0; ki < 8; ++ki) {
-        const int k = 8 * kb + ki;
-        if (ty == kb) {
-            const float rc = drc[k];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int col = 8 * tx + j;
-                Zm[k][col] = col <= k ? ((col == k ? 1.0f : 0.0f) - P[ki][j]) * rc : 0.0f;
-            }
+        for (int i = 0; i < 8; ++i) {
+            const float4 d0 = *reinterpret_cast<const float4*>(&Dm[8 * ty + i][8 * kb]);
+            const float4 d1 = *reinterpret_cast<const float4*>(&Dm[8 * ty + i][8 * kb + 4]);
+            Dblk[i][0] = d0.x; Dblk[i][1] = d0.y; Dblk[i][2] = d0.z; Dblk[i][3] = d0.w;
+            Dblk[i][4] = d1.x; Dblk[i][5] = d1.y; Dblk[i][6] = d1.z; Dblk[i][7] = d1.w;
         }
-        __syncthreads();
-        float di[8], zj[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) di[i] = Dm[8 * ty + i][k];
+        for (int ki = 0; ki < 8; ++ki) {
+            const int k = 8 * kb + ki;
+            if (ty == kb) {
+                const float rc = drc[k];
+                float z[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) zj[j] = Zm[k][8 * tx + j];
+                for (int j = 0; j < 8; ++j) {
+                    const int col = 8 * tx + j;
+                    z[j] = col <= k ? ((col == k ? 1.0f : 0.0f) - P[ki][j]) * rc : 0.0f;
+                }
+                *reinterpret_cast<float4*>(&Zm[k][8 * tx]) = make_float4(z[0], z[1], z[2], z[3]);
+                *reinterpret_cast<float4*>(&Zm[k][8 * tx + 4]) = make_float4(z[4], z[5], z[6], z[7]);
+            }
+            __syncthreads();
+            const float4 z0 = *reinterpret_cast<const float4*>(&Zm[k][8 * tx]);
+            const float4 z1 = *reinterpret_cast<const float4*>(&Zm[k][8 * tx + 4]);
+            const float zj[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) P[i][j] = __builtin_fmaf(di[i], zj[j], P[i][j]);
+                for (int j = 0; j < 8; ++j) P[i][j] = __builtin_fmaf(Dblk[i][ki], zj[j], P[i][j]);
+        }
     }
     __syncthreads();
 
