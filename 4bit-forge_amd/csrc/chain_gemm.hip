@@ -26,6 +26,7 @@ namespace forge {
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int TM = 128, TN = 128;
 #ifndef FORGE_GEMM_TK
 #define FORGE_GEMM_TK 32
@@ -268,8 +269,8 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
     if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
     if (g.b_lower_tri && k0 < nt) k0 = nt;
 
-    const int m_base = mt + wm * 64 + (lane >> 5) * 4;
-    const int n_base = nt + wn * 64 + (lane & 31);
+    const int m_base = mt + wm * 32 + (lane >> 5) * 4;
+    const int n_base = nt + wn * 32 + (lane & 31);
     float* __restrict__ Xw = X + (int64_t)m_base * g.ldx + n_base;
     const float sgn = g.negate_a ? -1.0f : 1.0f;
 
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
             for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                    const int dm = mi * 64 + (v >> 2) * 8 + (v & 3), dn = ni * 64;
                     acc[mi][ni][v] = Xw[(int64_t)dm * g.ldx + dn];
                 }
 #pragma unroll
@@ -311,48 +312,67 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
     }
 
     if (k0 < k1) {  // uniform over the workgroup
-        // global -> LDS staging: thread loads k rows (tid>>5) + 8h, 4 columns each.  The
-        // eight float4 are named scalars on purpose: as an array captured by a lambda the
-        // compiler kept part of them in memory.
+        // global -> LDS staging: thread loads k rows (tid>>5) + 8h, 4 columns each, as
+        // buffer loads: one resource descriptor per operand (scalar registers), per-thread
+        // byte offsets that never change and a scalar offset that advances with k.  The
+        // fp32 MFMA executes on the vector ALU's multipliers, so every vector instruction in
+        // this loop (address arithmetic included) takes time from it; with this addressing
+        // and the LDS reads below the loop has six of them per 64 MFMAs.
+        // (The eight 16-byte registers are named scalars on purpose: as an array captured
+        // by a lambda the compiler kept part of them in memory.)
         const int lrow = tid >> 5, lcol = (tid & 31) * 4;
-        const float* pa = At + (int64_t)(k0 + lrow) * g.lda + mt + lcol;
-        const float* pb = Bm + (int64_t)(k0 + lrow) * g.ldb + nt + lcol;
-        const int64_t a_step8 = 8 * g.lda, b_step8 = 8 * g.ldb;
-        float4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
-#define FORGE_GEMM_FETCH()                                              \
-    do {                                                                \
-        ra0 = *reinterpret_cast<const float4*>(pa);                     \
-        rb0 = *reinterpret_cast<const float4*>(pb);                     \
-        ra1 = *reinterpret_cast<const float4*>(pa + a_step8);           \
-        rb1 = *reinterpret_cast<const float4*>(pb + b_step8);           \
-        ra2 = *reinterpret_cast<const float4*>(pa + 2 * a_step8);       \
-        rb2 = *reinterpret_cast<const float4*>(pb + 2 * b_step8);       \
-        ra3 = *reinterpret_cast<const float4*>(pa + 3 * a_step8);       \
-        rb3 = *reinterpret_cast<const float4*>(pb + 3 * b_step8);       \
-        pa += a_adv;                                                    \
-        pb += b_adv;                                                    \
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(At + (int64_t)k0 * g.lda + mt), 0, 0x7FFFFFFF, 0x00027000);
+        const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(Bm + (int64_t)k0 * g.ldb + nt), 0, 0x7FFFFFFF, 0x00027000);
+        const int a8 = (int)(8 * g.lda * 4), b8 = (int)(8 * g.ldb * 4);
+        const int ao0 = (int)(((int64_t)lrow * g.lda + lcol) * 4), ao1 = ao0 + a8, ao2 = ao0 + 2 * a8,
+                  ao3 = ao0 + 3 * a8;
+        const int bo0 = (int)(((int64_t)lrow * g.ldb + lcol) * 4), bo1 = bo0 + b8, bo2 = bo0 + 2 * b8,
+                  bo3 = bo0 + 3 * b8;
+        int a_soff = 0, b_soff = 0;
+        u32x4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+#define FORGE_GEMM_FETCH()                                                      \
+    do {                                                                        \
+        ra0 = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, ao0, a_soff, 0);    \
+        rb0 = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, bo0, b_soff, 0);    \
+        ra1 = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, ao1, a_soff, 0);    \
+        rb1 = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, bo1, b_soff, 0);    \
+        ra2 = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, ao2, a_soff, 0);    \
+        rb2 = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, bo2, b_soff, 0);    \
+        ra3 = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, ao3, a_soff, 0);    \
+        rb3 = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, bo3, b_soff, 0);    \
+        a_soff += a_adv;                                                        \
+        b_soff += b_adv;                                                        \
     } while (0)
 #define FORGE_GEMM_STAGE(buf)                                           \
     do {                                                                \
-        *reinterpret_cast<float4*>(&As[buf][lrow][lcol]) = ra0;         \
-        *reinterpret_cast<float4*>(&Bs[buf][lrow][lcol]) = rb0;         \
-        *reinterpret_cast<float4*>(&As[buf][lrow + 8][lcol]) = ra1;     \
-        *reinterpret_cast<float4*>(&Bs[buf][lrow + 8][lcol]) = rb1;     \
-        *reinterpret_cast<float4*>(&As[buf][lrow + 16][lcol]) = ra2;    \
-        *reinterpret_cast<float4*>(&Bs[buf][lrow + 16][lcol]) = rb2;    \
-        *reinterpret_cast<float4*>(&As[buf][lrow + 24][lcol]) = ra3;    \
-        *reinterpret_cast<float4*>(&Bs[buf][lrow + 24][lcol]) = rb3;    \
+        *reinterpret_cast<u32x4*>(&As[buf][lrow][lcol]) = ra0;         \
+        *reinterpret_cast<u32x4*>(&Bs[buf][lrow][lcol]) = rb0;         \
+        *reinterpret_cast<u32x4*>(&As[buf][lrow + 8][lcol]) = ra1;     \
+        *reinterpret_cast<u32x4*>(&Bs[buf][lrow + 8][lcol]) = rb1;     \
+        *reinterpret_cast<u32x4*>(&As[buf][lrow + 16][lcol]) = ra2;    \
+        *reinterpret_cast<u32x4*>(&Bs[buf][lrow + 16][lcol]) = rb2;    \
+        *reinterpret_cast<u32x4*>(&As[buf][lrow + 24][lcol]) = ra3;    \
+        *reinterpret_cast<u32x4*>(&Bs[buf][lrow + 24][lcol]) = rb3;    \
     } while (0)
 
-        const int a_off = wm * 64 + (lane & 31), b_off = wn * 64 + (lane & 31), kr0 = lane >> 5;
+        // The two MFMA tiles of a wavefront sit 64 columns apart (rows wm*32.. and 64+wm*32..
+        // of the tile), so both values of a k-pair are one ds_read2st64_b32 and every read of
+        // a stage is the lane's base address plus an immediate offset.
+        const int kr0 = lane >> 5;
+        const float* a_lane = &As[0][kr0][wm * 32 + (lane & 31)];
+        const float* b_lane = &Bs[0][kr0][wn * 32 + (lane & 31)];
         float av0[8][2], bv0[8][2], av1[8][2], bv1[8][2];
         auto read_ops = [&](int buf, int sub, float (&av)[8][2], float (&bv)[8][2]) {
+            const float* ap = a_lane + buf * (TK * TM);
+            const float* bp = b_lane + buf * (TK * TN);
 #pragma unroll
             for (int kp = 0; kp < 8; ++kp)
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    av[kp][i] = As[buf][sub * 16 + 2 * kp + kr0][a_off + i * 32];
-                    bv[kp][i] = Bs[buf][sub * 16 + 2 * kp + kr0][b_off + i * 32];
+                    av[kp][i] = ap[(sub * 16 + 2 * kp) * TM + i * 64];
+                    bv[kp][i] = bp[(sub * 16 + 2 * kp) * TN + i * 64];
                 }
         };
         auto mfmas = [&](const float (&av)[8][2], const float (&bv)[8][2]) {
@@ -368,8 +388,8 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 
         // Every fetch reads rows below k1: the pointers advance only while a further stage
         // exists; past the end the last stage is fetched again and never used.
-        const int64_t a_full = 4 * a_step8, b_full = 4 * b_step8;
-        int64_t a_adv = (k0 + TK < k1) ? a_full : 0, b_adv = (k0 + TK < k1) ? b_full : 0;
+        const int a_full = 4 * a8, b_full = 4 * b8;                  // 32 rows, in bytes
+        int a_adv = (k0 + TK < k1) ? a_full : 0, b_adv = (k0 + TK < k1) ? b_full : 0;
         FORGE_GEMM_FETCH();
         FORGE_GEMM_STAGE(0);
         __syncthreads();
@@ -446,7 +466,7 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int dm = mi * 32 + (v >> 2) * 8 + (v & 3), dn = ni * 32;
+                const int dm = mi * 64 + (v >> 2) * 8 + (v & 3), dn = ni * 64;
                 Xw[(int64_t)dm * g.ldx + dn] = sgn * acc[mi][ni][v];
             }
 }
@@ -481,8 +501,11 @@ Prepared prepare(const GemmArgs& g_in, int64_t batch) {
     // the triangular K clipping keeps multiples of TK only when tiles and K origin line up
     const bool tri_ok = (!g.b_upper_tri || ((g.n0 + TN - g.k0) % TK) == 0) &&
                         (!g.b_lower_tri || ((g.n0 - g.k0) % TK) == 0);
+    // the full-tile kernel addresses its operands with 32-bit byte offsets from row k0
+    const int64_t ldmax = g.lda > g.ldb ? g.lda : g.ldb;
+    const bool offsets_fit = ((int64_t)(g.k1 - g.k0) + TK) * ldmax * 4 + TM * 4 < (1LL << 31);
     p.edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
-             ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned;
+             ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned || !offsets_fit;
     // useful flops: 2*M*N*K with K clipped per n-tile for the triangular variants
     double kn = 0.0;
     for (int nt = g.n0; nt < g.n1; nt += TN) {
