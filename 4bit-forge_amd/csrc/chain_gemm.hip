@@ -21,6 +21,7 @@
 // idle for their whole issue time).  chain_gemm_kernel<EDGE> is the simple, bounds-checked
 // form for ragged shapes.
 #include "chain_gemm.h"
+#include <type_traits>
 
 namespace forge {
 namespace {
@@ -237,9 +238,15 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
 // A launch carries one or two independent problems (GemmPair): workgroups below
 // first_wgs work on `first`, the rest on `second`, so that two under-filled or ragged-ended
 // problems share one grid.
-template <int CHUNK>
+// SPI = stages per loop iteration.  4 (K a multiple of 128): the LDS buffer of every stage
+// is a compile-time constant, so no address is computed in the loop at all, and with CHUNK =
+// 128 the first MFMAs of a chunk take C = 0 (no registers to clear) and the chunk is folded
+// into the totals once per iteration.  1: any K that is a multiple of 32 (CHUNK = 0 only).
+template <int CHUNK, int SPI>
 __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) {
     static_assert(TK == 32, "two 16-row sub-stages per stage");
+    static_assert(SPI == 1 || SPI == 4, "one stage or one 128-row chunk per iteration");
+    static_assert(CHUNK == 0 || (CHUNK == SPI * TK), "a chunk is one loop iteration");
     const bool in_first = blockIdx.x < (unsigned)pair.first_wgs;
     const GemmArgs& g = in_first ? pair.first : pair.second;
     const int wg = in_first ? (int)blockIdx.x : (int)blockIdx.x - pair.first_wgs;
@@ -299,16 +306,12 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni) acc[mi][ni] *= sgn;
     }
-    f32x16 tot[2][2];
+    f32x16 tot[2][2];   // CHUNK > 0: running totals; acc then holds one chunk at a time
     if constexpr (CHUNK > 0) {
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) {
-                tot[mi][ni] = acc[mi][ni];
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
-            }
+            for (int ni = 0; ni < 2; ++ni) tot[mi][ni] = acc[mi][ni];
     }
 
     if (k0 < k1) {  // uniform over the workgroup
@@ -375,15 +378,18 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
                     bv[kp][i] = bp[(sub * 16 + 2 * kp) * TN + i * 64];
                 }
         };
-        auto mfmas = [&](const float (&av)[8][2], const float (&bv)[8][2]) {
+        // fresh: the accumulators start a new chunk, the first k-pair takes C = 0
+        auto mfmas = [&](const float (&av)[8][2], const float (&bv)[8][2], auto fresh) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kp = 0; kp < 8; ++kp)
 #pragma unroll
                 for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[kp][mi], bv[kp][ni],
-                                                                           acc[mi][ni], 0, 0, 0);
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            av[kp][mi], bv[kp][ni],
+                            (decltype(fresh)::value && kp == 0) ? zero : acc[mi][ni], 0, 0, 0);
         };
 
         // Every fetch reads rows below k1: the pointers advance only while a further stage
@@ -397,12 +403,12 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
         if (k0 + 2 * TK >= k1) { a_adv = 0; b_adv = 0; }
         FORGE_GEMM_FETCH();
 
-        int buf = 0, stage_no = 0;
-        for (int kk = k0; kk < k1; kk += TK) {
+        // One stage; `buf` is a compile-time constant when the caller passes one.
+        auto stage_body = [&](auto buf, int kk, auto fresh) {
             // ---- region A.  The group barriers give the order "MFMA, memory instruction,
             // MFMA, ..."; the plain barriers keep instructions from leaving their region.
             read_ops(buf, 1, av1, bv1);
-            mfmas(av0, bv0);
+            mfmas(av0, bv0, fresh);
             FORGE_GEMM_STAGE(buf ^ 1);
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -421,7 +427,7 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
             // ---- region B
             read_ops(buf ^ 1, 0, av0, bv0);
             if (kk + 3 * TK >= k1) { a_adv = 0; b_adv = 0; }
-            mfmas(av1, bv1);
+            mfmas(av1, bv1, std::false_type{});
             FORGE_GEMM_FETCH();
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -435,29 +441,37 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (CHUNK > 0) {
-                if (++stage_no == CHUNK / TK) {
-                    stage_no = 0;
+        };
+        if constexpr (SPI == 1) {
+            int buf = 0;
+            for (int kk = k0; kk < k1; kk += TK) {
+                stage_body(buf, kk, std::false_type{});
+                buf ^= 1;
+            }
+        } else {
+            using B0 = std::integral_constant<int, 0>;
+            using B1 = std::integral_constant<int, 1>;
+            for (int kk = k0; kk < k1; kk += 4 * TK) {
+                stage_body(B0{}, kk, std::integral_constant<bool, (CHUNK > 0)>{});
+                stage_body(B1{}, kk + TK, std::false_type{});
+                stage_body(B0{}, kk + 2 * TK, std::false_type{});
+                stage_body(B1{}, kk + 3 * TK, std::false_type{});
+                if constexpr (CHUNK > 0) {
 #pragma unroll
                     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-                        for (int ni = 0; ni < 2; ++ni) {
-                            tot[mi][ni] += acc[mi][ni];
-#pragma unroll
-                            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
-                        }
+                        for (int ni = 0; ni < 2; ++ni) tot[mi][ni] += acc[mi][ni];
                 }
             }
-            buf ^= 1;
         }
 #undef FORGE_GEMM_FETCH
 #undef FORGE_GEMM_STAGE
     }
-    if constexpr (CHUNK > 0) {
+    if constexpr (CHUNK > 0) {   // every chunk has been folded already
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = tot[mi][ni] + acc[mi][ni];
+            for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = tot[mi][ni];
     }
 
 #pragma unroll
@@ -478,6 +492,7 @@ namespace {
 struct Prepared {
     GemmArgs g;
     bool empty, edge;
+    bool k128;   // every tile's K range is a whole number of 128-row chunks
     int64_t n_wg;
     double flops;
 };
@@ -506,6 +521,10 @@ Prepared prepare(const GemmArgs& g_in, int64_t batch) {
     const bool offsets_fit = ((int64_t)(g.k1 - g.k0) + TK) * ldmax * 4 + TM * 4 < (1LL << 31);
     p.edge = ((g.m1 - g.m0) % TM) != 0 || ((g.n1 - g.n0) % TN) != 0 ||
              ((g.k1 - g.k0) % TK) != 0 || !tri_ok || !aligned || !offsets_fit;
+    p.k128 = ((g.k1 - g.k0) % 128) == 0 && (!g.b_upper_tri || ((g.n0 + TN - g.k0) % 128) == 0) &&
+             (!g.b_lower_tri || ((g.n0 - g.k0) % 128) == 0);
+    // blocked summation exists for whole chunks only (full tiles) or bounds-checked
+    if (g.blocked_sum && !p.k128) p.edge = true;
     // useful flops: 2*M*N*K with K clipped per n-tile for the triangular variants
     double kn = 0.0;
     for (int nt = g.n0; nt < g.n1; nt += TN) {
@@ -533,8 +552,10 @@ int launch_prepared(const Prepared& a, const Prepared* b, hipStream_t st) {
         pair.first = a.g;
         pair.second = b ? b->g : a.g;
         pair.first_wgs = (int)a.n_wg;
-        if (a.g.blocked_sum) chain_gemm_fast_kernel<128><<<grid, dim3(256), 0, st>>>(pair);
-        else chain_gemm_fast_kernel<0><<<grid, dim3(256), 0, st>>>(pair);
+        const bool k128 = a.k128 && (!b || b->k128);
+        if (a.g.blocked_sum) chain_gemm_fast_kernel<128, 4><<<grid, dim3(256), 0, st>>>(pair);
+        else if (k128) chain_gemm_fast_kernel<0, 4><<<grid, dim3(256), 0, st>>>(pair);
+        else chain_gemm_fast_kernel<0, 1><<<grid, dim3(256), 0, st>>>(pair);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
