@@ -32,13 +32,16 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
 
 PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, TFLOP/s, GB/s
-# HBM bytes per launch of the factorisation GEMM on the default workload (64 experts per
+# HBM bytes per launch of the two GEMM kernels on the default workload (64 experts per
 # step), from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each
 # scaled by what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and
 # x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  The operand data a
-# launch has to read once (rows below the current block of the factor and of its inverse)
-# averages ~4.4e9 bytes over the 55 launches of a C=7168 factorisation: no wasted re-reads.
-MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 4.40e9}
+# launch of the factorisation GEMM has to read once (rows below the current block of the
+# factor and of its inverse) averages ~4.4e9 bytes over the 55 launches of a C=7168
+# factorisation; the sweep update reads the earlier error rows once (~1.9e9 bytes on
+# average): no wasted re-reads in either.
+MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 4.67e9,
+                    ("deepseek_v3", 64, "chain_gemm"): 2.06e9}
 
 KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit)
     "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s"),
