@@ -85,18 +85,22 @@ __device__ __forceinline__ float pow_abs(float e, float norm) {
     return __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(e) * norm);
 }
 
-// Loss of one element for one candidate (quant_grid.cu:159-167).
+// Loss of one element for one candidate (quant_grid.cu:159-167).  FLOOR = false drops the
+// max(|diff|, 1e-20): for norm >= 2.3 the floor's own loss 1e-20^norm is below the smallest
+// fp32 denormal, i.e. 0, which is also what |diff| = 0 gives without it (log2 0 = -inf,
+// exp2 -inf = 0); the launcher chooses.
+template <bool FLOOR>
 __device__ __forceinline__ float element_loss(float x, float s, float rcp, float q0, float maxq,
                                               float norm) {
     const float q = clampf(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq);
     const float diff = __builtin_fmaf(q - q0, s, -x);
-    return pow_abs(fmaxf(fabsf(diff), 1e-20f), norm);
+    return pow_abs(FLOOR ? fmaxf(fabsf(diff), 1e-20f) : fabsf(diff), norm);
 }
 
 // Sum over the 8 "reference lanes" l = Q, Q+4, ..., Q+28 (each the in-order sum of its
 // GS/32 elements), combined exactly as the reference's halving tree combines them:
 // ((p[Q] + p[Q+16]) + (p[Q+8] + p[Q+24])) + ((p[Q+4] + p[Q+20]) + (p[Q+12] + p[Q+28])).
-template <int GS, int Q>
+template <int GS, int Q, bool FLOOR>
 __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, float rcp, float q0,
                                               float maxq, float norm) {
     constexpr int VPL = GS / 32;
@@ -106,7 +110,7 @@ __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, flo
         const int l = Q + 4 * j;
         float loss = 0.0f;
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) loss += element_loss(v[l + 32 * i], s, rcp, q0, maxq, norm);
+        for (int i = 0; i < VPL; ++i) loss += element_loss<FLOOR>(v[l + 32 * i], s, rcp, q0, maxq, norm);
         p[j] = loss;
     }
     return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
@@ -118,23 +122,23 @@ __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, flo
 // once it reaches `bound` for every group of the wavefront the candidate cannot be a new
 // strict minimum and the rest of its evaluation is skipped (returns +inf for it).  The
 // selected candidate and its loss are exactly those of the full evaluation.
-template <int GS>
+template <int GS, bool FLOOR>
 __device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, float rcp,
                                                 float q0, float maxq, float norm, float bound) {
     constexpr float kInf = __builtin_inff();
-    const float a0 = quarter_loss<GS, 0>(v, s, rcp, q0, maxq, norm);
+    const float a0 = quarter_loss<GS, 0, FLOOR>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(a0 < bound) == 0) return kInf;
-    const float h0 = a0 + quarter_loss<GS, 2>(v, s, rcp, q0, maxq, norm);
+    const float h0 = a0 + quarter_loss<GS, 2, FLOOR>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(h0 < bound) == 0) return kInf;
-    const float a1 = quarter_loss<GS, 1>(v, s, rcp, q0, maxq, norm);
+    const float a1 = quarter_loss<GS, 1, FLOOR>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(h0 + a1 < bound) == 0) return kInf;
-    const float h1 = a1 + quarter_loss<GS, 3>(v, s, rcp, q0, maxq, norm);
+    const float h1 = a1 + quarter_loss<GS, 3, FLOOR>(v, s, rcp, q0, maxq, norm);
     return h0 + h1;
 }
 
 // One lane per group.  FUSED: derive (sg, q0g) from the group's own extrema first;
 // otherwise read them from scales/qzeros (the reference's two-call protocol).
-template <typename T, int GS, bool FUSED>
+template <typename T, int GS, bool FUSED, bool FLOOR>
 __global__ __launch_bounds__(64) void mse_grid_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t G,
     int64_t n_groups, const float* __restrict__ cand, int P, float maxq, float norm,
@@ -202,10 +206,10 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
             // them first.  A single summand is a lower bound of the (monotone, non-negative)
             // fp32 sum, so once it reaches the best loss for every group of the wavefront
             // the candidate is out without touching the other gs-2 elements.
-            const float clip = fmaxf(element_loss(lo, s, rcp, q0, maxq, norm),
-                                     element_loss(hi, s, rcp, q0, maxq, norm));
+            const float clip = fmaxf(element_loss<FLOOR>(lo, s, rcp, q0, maxq, norm),
+                                     element_loss<FLOOR>(hi, s, rcp, q0, maxq, norm));
             if (__builtin_amdgcn_ballot_w64(clip < best_loss) == 0) continue;
-            const float loss = candidate_loss<GS>(v, s, rcp, q0, maxq, norm, best_loss);
+            const float loss = candidate_loss<GS, FLOOR>(v, s, rcp, q0, maxq, norm, best_loss);
             if (loss < best_loss) {
                 best_loss = loss;
                 best_s = s;
@@ -227,12 +231,17 @@ int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, 
     forge::KernelTiming timing(search ? "mse_grid" : "minmax_grid_lane", st,
                                (double)n_groups * (gs * sizeof(T) + 8.0 + (FUSED ? 0.0 : 8.0)),
                                forge::WORK_BYTES);
+    const bool floor_needed = !(norm >= 2.3f);
 #define FORGE_MSE_CASE(GS)                                                                    \
     case GS:                                                                                  \
-        mse_grid_kernel<T, GS, FUSED><<<grid, block, 0, st>>>(W, w_stride, R, C, ldw, G,      \
-                                                              n_groups, cand, (int)P, maxq,   \
-                                                              norm, symmetric, search, scales, \
-                                                              qzeros);                        \
+        if (floor_needed)                                                                     \
+            mse_grid_kernel<T, GS, FUSED, true><<<grid, block, 0, st>>>(                      \
+                W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric,     \
+                search, scales, qzeros);                                                      \
+        else                                                                                  \
+            mse_grid_kernel<T, GS, FUSED, false><<<grid, block, 0, st>>>(                     \
+                W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric,     \
+                search, scales, qzeros);                                                      \
         break;
     switch (gs) {
         FORGE_MSE_CASE(32)

@@ -63,6 +63,22 @@ def test_mse_search_matches_oracle(hip, sym, gs):
     _check_mse(s0, z0, L, s1, z1, p, s_mm)
 
 
+@pytest.mark.parametrize("norm", [1.0, 2.0, 3.0])
+def test_mse_search_other_norms(hip, norm):
+    """Norms below 2.3 keep the reference's max(|diff|, 1e-20) floor (its loss 1e-20^norm is a
+    nonzero fp32 there), norms above drop it; groups with exact zeros exercise |diff| = 0."""
+    X = _data(2048, 128, 77)
+    X[::7] = 0.0                                   # all-zero groups: every diff is exactly 0
+    X[1::7, ::3] = 0.0
+    p = torch.linspace(1.0, 0.2, 100)
+    s_mm, z_mm = oracle.build_group_meta_packed(X, 4, True)
+    s0, z0, L = oracle.mse_scale_groups_packed(X, s_mm.clone(), z_mm.clone(), p, norm, 4, True,
+                                               return_losses=True)
+    s1, z1 = hip.mse_scale_groups_packed(X.to(DEV), s_mm.clone().to(DEV), z_mm.clone().to(DEV),
+                                         p.to(DEV), norm, 4, True)
+    _check_mse(s0, z0, L, s1, z1, p, s_mm)
+
+
 def test_mse_rejects_unsupported_group_size(hip):
     X = torch.zeros(8, 48, device=DEV)
     with pytest.raises(RuntimeError, match="group_size=48"):
