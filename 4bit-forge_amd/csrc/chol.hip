@@ -29,6 +29,13 @@ namespace {
 constexpr int NB = 128;       // block size
 constexpr int LDP = NB + 4;   // LDS pitch
 
+// (a fill kernel rather than hipMemsetAsync, so that a caller may capture the whole call
+// into a HIP graph)
+__global__ void clear_info_kernel(int32_t* __restrict__ info, int64_t batch) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < batch) info[i] = 0;
+}
+
 __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__ damp, int64_t C) {
     const int64_t b = blockIdx.y;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -227,7 +234,8 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
     constexpr size_t kDiagLds = 2 * NB * LDP * sizeof(float);
     FORGE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(diag_block_kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDiagLds));
-    FORGE_HIP_CHECK(hipMemsetAsync(info, 0, batch * sizeof(int32_t), st));
+    clear_info_kernel<<<dim3((unsigned)forge::ceil_div(batch, 256)), dim3(256), 0, st>>>(info, batch);
+    FORGE_LAUNCH_CHECK();
     if (damp) {
         add_damp_kernel<<<dim3((unsigned)forge::ceil_div(C, 256), (unsigned)batch), dim3(256), 0, st>>>(
             H, damp, C);
