@@ -39,7 +39,12 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);
 // or writes).  When both are full-tile problems of the same kind they share one launch, the
 // first problem's tiles ahead of the second's; otherwise they are launched one after the
 // other.  Either may be empty.
+// With a workspace of split_gemm_workspace_bytes(batch, k1 - k0), two blocked-sum problems
+// of full tiles that share their A panel (same At, pitch, m0 and k0) run on the bf16 matrix
+// pipe instead (three-piece split of every operand, fp32-grade accuracy, different
+// rounding); FORGE_FP32_BLOCKED_SUM=1 in the environment keeps them on the fp32 kernel.
 int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
-                           hipStream_t st);
+                           hipStream_t st, void* split_ws = nullptr, int64_t split_ws_bytes = 0);
+int64_t split_gemm_workspace_bytes(int64_t batch, int64_t k_rows);
 
 }  // namespace forge

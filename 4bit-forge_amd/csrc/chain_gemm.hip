@@ -21,6 +21,7 @@
 // idle for their whole issue time).  chain_gemm_kernel<EDGE> is the simple, bounds-checked
 // form for ragged shapes.
 #include "chain_gemm.h"
+#include <cstdlib>
 #include <type_traits>
 
 namespace forge {
@@ -485,6 +486,281 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
             }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Blocked-sum GEMM on the bf16 matrix pipe ("bf16x3").  Used where only fp32 ACCURACY is
+// needed (the factorisation's trailing updates), never for the sweep's bit-exact chain.
+//
+// Every fp32 operand is cut, by truncation, into three bf16 pieces a = a1 + a2 + a3 (exact:
+// 8 + 8 + 8 significant bits), and a*b is summed from the six piece products of weight
+// >= 2^-16, smallest first: (3,1) (1,3) (2,2) (2,1) (1,2) (1,1), accumulated in fp32 by
+// v_mfma_f32_32x32x16_bf16.  The dropped products are below 2^-24 |a b|, and the accumulators
+// are folded into running totals every 128 k like the fp32 blocked sum, so the error is that
+// of an fp32 dot product.  Six bf16 MFMAs do the work of sixteen fp32 ones.
+//
+// The fp32 matrix instruction shares the vector ALU, the bf16 one does not, so here the
+// split arithmetic has somewhere to run; but a wavefront that holds 128 accumulators and the
+// operands of the next step has no registers left for it.  Hence 8 wavefronts with two roles:
+//   wavefronts 0..3  multiply: LDS reads and MFMAs only, 64x64 outputs each
+//   wavefronts 4..7  produce: global loads, the split of B, LDS writes
+// A stage is 32 rows of K in two LDS buffers, with one barrier per stage placed in the middle
+// of the multipliers' stage:
+//   multipliers, stage s:  MFMAs of k-step 0 | reads of k-step 1;  barrier s;
+//                          MFMAs of k-step 1 | reads of (stage s+1, k-step 0)
+//   producers, between barriers s-1 and s: stage s+1 into buffer (s+1)&1, then the global
+//                          loads of stage s+5 into the registers just consumed
+// The A panel is the same for every workgroup of a matrix, so it is split once by
+// split_a_panel_kernel into the exact LDS image of each stage and the producers only copy it.
+//
+// LDS image of one operand and stage: [piece 3][k group of eight 4][position 128] 16-byte
+// words, a word = 8 consecutive k as bf16.  Column c of the 128-wide tile sits at position
+// (c & 3) * 32 + (c >> 2): a producer thread loads 4 consecutive columns with one 16-byte
+// load and the writes of a wavefront are then contiguous in LDS.  A multiplier's MFMA tile
+// at positions [32 e, 32 e + 32) therefore covers the columns 4 j + e, j = 0..31.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int SPLIT_TK = 32;                       // k rows per stage
+constexpr int SPLIT_STAGE_WORDS = 3 * 4 * 128;     // 16-byte words per operand and stage
+constexpr int SPLIT_SETS = 4;                      // producer register sets = stages in flight
+
+// N fp32 values (consecutive k of one column) -> N/2 packed words of each piece.
+template <int N, typename W>
+__device__ __forceinline__ void split_pieces(const float (&x)[N], W& p1, W& p2, W& p3) {
+    unsigned h1[N], h2[N], h3[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const unsigned a1 = __float_as_uint(x[j]) & 0xFFFF0000u;
+        const float r1 = x[j] - __uint_as_float(a1);                 // exact
+        const unsigned a2 = __float_as_uint(r1) & 0xFFFF0000u;
+        const float r2 = r1 - __uint_as_float(a2);                   // exact, <= 8 bits
+        h1[j] = a1; h2[j] = a2; h3[j] = __float_as_uint(r2);
+    }
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w) {   // upper halves of (k, k+1) -> one word, k in the low half
+        p1[w] = __builtin_amdgcn_perm(h1[2 * w + 1], h1[2 * w], 0x07060302u);
+        p2[w] = __builtin_amdgcn_perm(h2[2 * w + 1], h2[2 * w], 0x07060302u);
+        p3[w] = __builtin_amdgcn_perm(h3[2 * w + 1], h3[2 * w], 0x07060302u);
+    }
+}
+
+// Rows [k0, k1) x columns [m0, m0+128) of At -> the LDS images of its stages, stage after
+// stage (SPLIT_STAGE_WORDS words each).  One workgroup of 128 threads per matrix and stage.
+__global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restrict__ At, int64_t lda,
+                                                            int64_t as, int m0, int k0, int n_stage,
+                                                            u32x4* __restrict__ Ap, int64_t aps) {
+    const int bz = blockIdx.x / n_stage, st = blockIdx.x % n_stage;
+    const int t = threadIdx.x, kg = t >> 5, cq = t & 31;
+    const float* src = At + (int64_t)bz * as + (int64_t)(k0 + SPLIT_TK * st + 8 * kg) * lda + m0 + 4 * cq;
+    f32x4 x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = *reinterpret_cast<const f32x4*>(src + (int64_t)j * lda);
+    u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * SPLIT_STAGE_WORDS + kg * 128 + cq;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float col[8];
+        u32x4 p1, p2, p3;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) col[j] = x[j][e];
+        split_pieces<8>(col, p1, p2, p3);
+        dst[32 * e] = p1;
+        dst[512 + 32 * e] = p2;
+        dst[1024 + 32 * e] = p3;
+    }
+}
+
+struct SplitPair {
+    GemmPair pair;
+    const u32x4* Ap;   // split A panel of both problems (same At, m0, k0)
+    int64_t aps;       // words per matrix
+};
+
+// Both problems: full 128x128 tiles, one m tile, 16-byte aligned rows, every tile's K range
+// a whole number of 128-row chunks starting at k0.
+__global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
+    const bool in_first = blockIdx.x < (unsigned)sp.pair.first_wgs;
+    const GemmArgs& g = in_first ? sp.pair.first : sp.pair.second;
+    const int wg = in_first ? (int)blockIdx.x : (int)blockIdx.x - sp.pair.first_wgs;
+    // [buffer][operand][piece][k group][position]
+    __shared__ __attribute__((aligned(16))) u32x4 L[2][2][3][4][128];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bz, tile;
+    if (g.xcd_map) {
+        const int xcd = wg & 7, slot = wg >> 3;
+        bz = xcd + 8 * (slot / g.n_tiles);
+        tile = slot % g.n_tiles;
+    } else {
+        bz = wg / g.n_tiles;
+        tile = wg % g.n_tiles;
+    }
+    const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile : tile;
+    const int nt = g.n0 + tn * TN;
+    const int k0 = g.k0;
+    int k1 = g.k1;
+    if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
+    const int n_stage = (k1 - k0) / SPLIT_TK;     // a multiple of 4
+
+    if (wave >= 4) {
+        // ---------------- producers ----------------
+        // B: thread = rows 4 kh .. 4 kh + 3 of the stage x columns 4 cq .. 4 cq + 3
+        const int pt = tid - 256, kh = pt >> 5, cq = pt & 31;
+        const float* Bm = g.Bm + (int64_t)bz * g.bs;
+        const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(Bm + (int64_t)k0 * g.ldb + nt), 0, 0x7FFFFFFF, 0x00027000);
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<u32x4*>(sp.Ap + (int64_t)bz * sp.aps), 0, 0x7FFFFFFF, 0x00027000);
+        int ob[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ob[j] = (int)(((int64_t)(4 * kh + j) * g.ldb + 4 * cq) * 4);
+        const int oa = pt * 16;
+        // Every fetch stays inside [k0, k1): the offsets advance only while a further stage
+        // exists; past the end the last stage is fetched again and never used.
+        int b_soff = 0, a_soff = 0, fetched = 0;
+        int b_adv = (int)(SPLIT_TK * g.ldb * 4), a_adv = SPLIT_STAGE_WORDS * 16;
+        f32x4 xb[SPLIT_SETS][4];
+        u32x4 xa[SPLIT_SETS][6];
+#define FORGE_SPLIT_FETCH(q)                                                                       \
+    do {                                                                                           \
+        ++fetched;                                                                                 \
+        if (fetched >= n_stage) { b_adv = 0; a_adv = 0; }                                          \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) xb[q][j] = __builtin_bit_cast(               \
+            f32x4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ob[j], b_soff, 0));               \
+        _Pragma("unroll") for (int j = 0; j < 6; ++j)                                              \
+            xa[q][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, oa + j * 4096, a_soff, 0);    \
+        b_soff += b_adv;                                                                           \
+        a_soff += a_adv;                                                                           \
+    } while (0)
+        // B word (piece, k group kh >> 1, position 32 e + cq), half kh & 1; A: plain copy
+        u32x2* const Lb = reinterpret_cast<u32x2*>(&L[0][1][0][kh >> 1][cq]) + (kh & 1);
+        u32x4* const La = &L[0][0][0][0][0] + pt;
+        constexpr int BUF = 2 * SPLIT_STAGE_WORDS;   // words per buffer (both operands)
+#define FORGE_SPLIT_STAGE(buf, q)                                                                  \
+    do {                                                                                           \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
+            float col[4];                                                                          \
+            u32x2 p1, p2, p3;                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) col[j] = xb[q][j][e];                    \
+            split_pieces<4>(col, p1, p2, p3);                                                      \
+            Lb[((buf) * BUF + 32 * e) * 2] = p1;                                                   \
+            Lb[((buf) * BUF + 512 + 32 * e) * 2] = p2;                                             \
+            Lb[((buf) * BUF + 1024 + 32 * e) * 2] = p3;                                            \
+        }                                                                                          \
+        _Pragma("unroll") for (int j = 0; j < 6; ++j) La[(buf) * BUF + j * 256] = xa[q][j];        \
+    } while (0)
+        FORGE_SPLIT_FETCH(0);
+        FORGE_SPLIT_FETCH(1);
+        FORGE_SPLIT_FETCH(2);
+        FORGE_SPLIT_FETCH(3);
+        FORGE_SPLIT_STAGE(0, 0);
+        FORGE_SPLIT_FETCH(0);
+        __syncthreads();
+        for (int s0 = 0; s0 < n_stage; s0 += 4) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                FORGE_SPLIT_STAGE((s + 1) & 1, (s + 1) & 3);
+                FORGE_SPLIT_FETCH((s + 1) & 3);
+                __syncthreads();
+            }
+        }
+#undef FORGE_SPLIT_FETCH
+#undef FORGE_SPLIT_STAGE
+        return;
+    }
+
+    // ---------------- multipliers ----------------
+    const int wm = wave >> 1, wn = wave & 1;
+    // MFMA tile (mi, ni) of this wavefront: positions 32 (wm + 2 mi) .. of A, 32 (wn + 2 ni) ..
+    // of B, i.e. output rows m0 + 4 j + wm + 2 mi and columns nt + 4 j' + wn + 2 ni.  Lane
+    // element v of the accumulator is MFMA row (lane >> 5) * 4 + (v >> 2) * 8 + (v & 3),
+    // column lane & 31.
+    const int jrow = (lane >> 5) * 4, jcol = lane & 31;
+    float* __restrict__ Xw = g.X + (int64_t)bz * g.xs + (int64_t)(g.m0 + wm) * g.ldx + nt + wn + 4 * jcol;
+    auto x_off = [&](int mi, int ni, int v) {
+        return (int64_t)(4 * (jrow + (v >> 2) * 8 + (v & 3)) + 2 * mi) * g.ldx + 2 * ni;
+    };
+    const float sgn = g.negate_a ? -1.0f : 1.0f;   // fma(-a, b, x) = -fma(a, b, -x)
+    f32x16 acc[2][2], tot[2][2];
+    if (g.init_zero) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) tot[mi][ni][v] = 0.0f;
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) tot[mi][ni][v] = Xw[x_off(mi, ni, v)];
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) tot[mi][ni] *= sgn;
+    }
+    const int rk = lane >> 5, ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    bf16x8 A0[3][2], B0[3][2], A1[3][2], B1[3][2];   // operands of k-step 0 / 1
+#define FORGE_SPLIT_READ(buf, u, A, B)                                                             \
+    do {                                                                                           \
+        _Pragma("unroll") for (int p = 0; p < 3; ++p) _Pragma("unroll") for (int i = 0; i < 2; ++i) { \
+            A[p][i] = __builtin_bit_cast(bf16x8, L[buf][0][p][2 * (u) + rk][ra + 64 * i]);         \
+            B[p][i] = __builtin_bit_cast(bf16x8, L[buf][1][p][2 * (u) + rk][rb + 64 * i]);         \
+        }                                                                                          \
+    } while (0)
+    // piece products smallest first; the four tiles innermost so that consecutive MFMAs use
+    // different accumulators; `fresh`: the first product of a chunk takes C = 0
+#define FORGE_SPLIT_MFMAS(A, B, fresh)                                                             \
+    do {                                                                                           \
+        constexpr int PA[6] = {2, 0, 1, 1, 0, 0}, PB[6] = {0, 2, 1, 0, 1, 0};                      \
+        _Pragma("unroll") for (int t = 0; t < 6; ++t) _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) \
+            _Pragma("unroll") for (int ni = 0; ni < 2; ++ni)                                       \
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                             \
+                    A[PA[t]][mi], B[PB[t]][ni], ((fresh) && t == 0) ? zero : acc[mi][ni], 0, 0, 0);\
+    } while (0)
+    // 24 MFMAs and 12 LDS reads per k-step: one read after every other MFMA
+#define FORGE_SPLIT_SCHED()                                                                        \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < 12; ++i) {                                           \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                     \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+        }                                                                                          \
+    } while (0)
+    __syncthreads();
+    FORGE_SPLIT_READ(0, 0, A0, B0);
+    for (int s0 = 0; s0 < n_stage; s0 += 4) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            FORGE_SPLIT_READ(s & 1, 1, A1, B1);
+            FORGE_SPLIT_MFMAS(A0, B0, s == 0);
+            FORGE_SPLIT_SCHED();
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            FORGE_SPLIT_READ((s + 1) & 1, 0, A0, B0);
+            FORGE_SPLIT_MFMAS(A1, B1, false);
+            FORGE_SPLIT_SCHED();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) tot[mi][ni] += acc[mi][ni];
+    }
+#undef FORGE_SPLIT_READ
+#undef FORGE_SPLIT_MFMAS
+#undef FORGE_SPLIT_SCHED
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) Xw[x_off(mi, ni, v)] = sgn * tot[mi][ni][v];
+}
+
 }  // namespace
 
 namespace {
@@ -569,12 +845,71 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st) {
     return launch_prepared(p, nullptr, st);
 }
 
+namespace {
+
+// The bf16x3 path: both problems blocked-sum, full tiles, whole 128-row chunks, and the same
+// A panel (At, pitch, m0, k0), which is split once for both.
+bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t ws_bytes,
+                    int* n_stage_out) {
+    const char* forced_fp32 = getenv("FORGE_FP32_BLOCKED_SUM");   // read per call: tests flip it
+    if (forced_fp32 && forced_fp32[0] == '1') return false;
+    auto ok = [](const Prepared& p) {
+        return !p.edge && p.k128 && p.g.blocked_sum && p.g.m_tiles == 1 && !p.g.b_lower_tri &&
+               p.g.k1 - p.g.k0 >= 128 && (!p.g.b_upper_tri || p.g.n0 + TN - p.g.k0 >= 128);
+    };
+    if (!ok(a) || (b && !ok(*b))) return false;
+    int k1 = a.g.k1;
+    if (b) {
+        const GemmArgs &x = a.g, &y = b->g;
+        if (x.At != y.At || x.lda != y.lda || x.as != y.as || x.m0 != y.m0 || x.k0 != y.k0) return false;
+        if (b->g.xcd_map && a.n_wg % 8 != 0) return false;
+        if (y.k1 > k1) k1 = y.k1;
+    }
+    const int n_stage = (k1 - a.g.k0) / SPLIT_TK;
+    if (ws_bytes < split_gemm_workspace_bytes(batch, k1 - a.g.k0)) return false;
+    *n_stage_out = n_stage;
+    return true;
+}
+
+int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stage, void* ws,
+                 hipStream_t st) {
+    const int64_t n_wg = a.n_wg + (b ? b->n_wg : 0);
+    FORGE_REQUIRE(n_wg < (1LL << 31) && batch * n_stage < (1LL << 31), "split_gemm: grid too large");
+    SplitPair sp{};
+    sp.pair.first = a.g;
+    sp.pair.second = b ? b->g : a.g;
+    sp.pair.first_wgs = (int)a.n_wg;
+    sp.Ap = static_cast<const u32x4*>(ws);
+    sp.aps = (int64_t)n_stage * SPLIT_STAGE_WORDS;
+    {
+        KernelTiming timing("split_a_panel", st, 10.0 * n_stage * SPLIT_TK * TM * (double)batch, WORK_BYTES);
+        split_a_panel_kernel<<<dim3((unsigned)(batch * n_stage)), dim3(128), 0, st>>>(
+            a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0, n_stage, static_cast<u32x4*>(ws), sp.aps);
+        FORGE_LAUNCH_CHECK();
+    }
+    KernelTiming timing("split_gemm_bf16x3", st, a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
+    split_gemm_kernel<<<dim3((unsigned)n_wg), dim3(512), 0, st>>>(sp);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+}  // namespace
+
+int64_t split_gemm_workspace_bytes(int64_t batch, int64_t k_rows) {
+    if (batch <= 0 || k_rows <= 0) return 0;
+    return batch * ceil_div(k_rows, (int64_t)SPLIT_TK) * SPLIT_STAGE_WORDS * 16;
+}
+
 int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
-                           hipStream_t st) {
+                           hipStream_t st, void* split_ws, int64_t split_ws_bytes) {
     const Prepared a = prepare(first, batch), b = prepare(second, batch);
     if (a.empty && b.empty) return FORGE_OK;
-    if (a.empty) return launch_prepared(b, nullptr, st);
-    if (b.empty) return launch_prepared(a, nullptr, st);
+    const Prepared* pa = a.empty ? &b : &a;
+    const Prepared* pb = (a.empty || b.empty) ? nullptr : &b;
+    int n_stage = 0;
+    if (split_ws && split_eligible(*pa, pb, batch, split_ws_bytes, &n_stage))
+        return launch_split(*pa, pb, batch, n_stage, split_ws, st);
+    if (!pb) return launch_prepared(*pa, nullptr, st);
     // one grid needs the same kernel for both; a grid split at a multiple of 8 keeps the
     // workgroup -> XCD map of the second problem
     const bool fusable = !a.edge && !b.edge && a.g.blocked_sum == b.g.blocked_sum &&

@@ -214,7 +214,8 @@ __global__ void finish_rows_kernel(float* __restrict__ U, float* __restrict__ ud
 extern "C" int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C) {
     if (batch <= 0 || C <= 0) return 0;
     const int64_t nblk = forge::ceil_div(C, NB);
-    return batch * nblk * NB * NB * (int64_t)sizeof(float);
+    // inverse diagonal blocks, then the split A panel of the trailing updates
+    return batch * nblk * NB * NB * (int64_t)sizeof(float) + forge::split_gemm_workspace_bytes(batch, C);
 }
 
 extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
@@ -229,6 +230,9 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
     hipStream_t st = (hipStream_t)stream;
     const int nblk = (int)forge::ceil_div(C, NB);
     float* Dinv = (float*)ws;
+    const int64_t dinv_bytes = batch * nblk * NB * NB * (int64_t)sizeof(float);
+    void* split_ws = (char*)ws + dinv_bytes;
+    const int64_t split_ws_bytes = ws_bytes - dinv_bytes;
 
     // the diagonal-block kernel keeps two 128x132 fp32 tiles in LDS (gfx950 has 160 KB/CU)
     constexpr size_t kDiagLds = 2 * NB * LDP * sizeof(float);
@@ -257,7 +261,7 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
             g2a.xs = g2a.as = g2a.bs = C * C;
             g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
             g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
-            if (int e = forge::launch_chain_gemm_pair(g1a, g2a, batch, st)) return e;
+            if (int e = forge::launch_chain_gemm_pair(g1a, g2a, batch, st, split_ws, split_ws_bytes)) return e;
         }
         {
             forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,

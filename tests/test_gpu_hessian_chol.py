@@ -77,6 +77,33 @@ def test_factor_matches_float64(hip, C, normalise):
             assert bool((U[b].diagonal() == 1).all())
 
 
+@pytest.mark.parametrize("B,C", [(8, 1536), (3, 640)])
+def test_factor_bf16_split_and_fp32_updates_agree(hip, monkeypatch, B, C):
+    """C a multiple of 128: the trailing updates run as three-piece bf16 products by default
+    and as fp32 blocked sums with FORGE_FP32_BLOCKED_SUM=1; both are fp32-accurate."""
+    g = torch.Generator().manual_seed(C)
+    X = torch.randn(B, 2 * C, C, generator=g, dtype=torch.float64)
+    X[:, :, :5] *= 6
+    H = ((2.0 / X.shape[1]) * X.transpose(1, 2) @ X).float()
+    H[B - 1, 7, 7] = float("nan")                       # one failing matrix among the good ones
+    damp = (0.01 * torch.diagonal(H[:B - 1], dim1=1, dim2=2).mean()).repeat(B).float()
+    monkeypatch.delenv("FORGE_FP32_BLOCKED_SUM", raising=False)
+    Us, uds, infos = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
+    monkeypatch.setenv("FORGE_FP32_BLOCKED_SUM", "1")
+    Uf, udf, infof = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
+    assert infos.tolist()[:B - 1] == [0] * (B - 1) and infos[B - 1].item() > 0
+    assert infof.tolist() == infos.tolist()
+    assert torch.equal(Us[B - 1].cpu(), torch.eye(C))
+    for b in range(B - 1):
+        Hd = H[b].double().numpy().copy()
+        Hd[np.diag_indices(C)] += float(damp[b])
+        U0 = np.linalg.cholesky(np.linalg.inv(Hd)).T
+        ref = U0 / np.diag(U0)[:, None]
+        es, ef = _rel(Us[b], ref), _rel(Uf[b], ref)
+        assert es < 5e-6 and ef < 5e-6 and es < 2 * ef + 1e-7
+        assert int((torch.tril(Us[b], -1) != 0).sum()) == 0
+
+
 def test_factor_failure_gives_identity(hip):
     H = torch.eye(256).repeat(3, 1, 1)
     H[1, 100, 100] = -1.0                               # not positive definite
