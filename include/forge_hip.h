@@ -129,7 +129,12 @@ int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int6
  * factor of inv(A); writes U[b] = U0 / diag(U0)[:,None] (normalise != 0) or U0, upper
  * triangle + zeroed lower; udiag[b] [C] receives diag(U0).  info[b] (int32) is 0 on
  * success or the 1-based index of the first non-positive pivot, in which case U[b] = I.
- * H[b] is destroyed (used as workspace).  ws: workspace of forge_chol_workspace_bytes. */
+ * H[b] is destroyed (used as workspace).  ws: workspace of forge_chol_workspace_bytes
+ * (128x128 inverse diagonal blocks, plus 768 bytes per column and matrix for the bf16
+ * pieces of one panel), 256-byte aligned.
+ * When C is a multiple of 128 the trailing updates are computed from three bf16 pieces per
+ * fp32 operand on the bf16 matrix pipe (fp32-grade accuracy; not bit-identical to the fp32
+ * update).  FORGE_FP32_BLOCKED_SUM=1 in the environment selects the fp32 update. */
 int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
                                  int32_t* info, int64_t batch, int64_t C, int normalise,
                                  void* ws, int64_t ws_bytes, forge_stream_t stream);

@@ -37,7 +37,8 @@ def test_invalid_arguments_are_rejected_without_a_launch():
     rc = lib.forge_quant_grid(None, 7, 1, 0, 4, 128, 128, 128, 4, 1, 0, None, 0, 2.4, None, None, None)
     assert rc == 1 and b"w_dtype" in lib.forge_last_error()
     assert lib.forge_build_group_meta_packed(None, 0, 128, 4, 1, None, None, None) == 0   # empty: no-op
-    assert lib.forge_chol_workspace_bytes(2, 256) == 2 * 2 * 128 * 128 * 4
+    # inverse diagonal blocks (fp32) + the bf16 pieces of one 128-column panel (6 bytes per element)
+    assert lib.forge_chol_workspace_bytes(2, 256) == 2 * 2 * 128 * 128 * 4 + 2 * 256 * 128 * 6
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="CPU-only behaviour")
