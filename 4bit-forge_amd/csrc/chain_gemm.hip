@@ -511,6 +511,9 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 //                          loads of stage s+5 into the registers just consumed
 // The A panel is the same for every workgroup of a matrix, so it is split once by
 // split_a_panel_kernel into the exact LDS image of each stage and the producers only copy it.
+// The multipliers never touch global memory: they start from zero, and at the end hand their
+// sums to the producers through LDS, who add the old X (X + s * sum, s = -1 for a negated A)
+// with coalesced 16-byte accesses.
 //
 // LDS image of one operand and stage: [piece 3][k group of eight 4][position 128] 16-byte
 // words, a word = 8 consecutive k as bf16.  Column c of the 128-wide tile sits at position
@@ -665,6 +668,32 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         }
 #undef FORGE_SPLIT_FETCH
 #undef FORGE_SPLIT_STAGE
+        // Epilogue, on the producers so that it is coalesced: the multipliers leave their
+        // sums in LDS (over the stage buffers, free by then), row r of the tile at
+        // S[r][position]; thread = 16 rows x 4 consecutive columns, X is read and written in
+        // 16-byte pieces of whole 512-byte rows.
+        float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)g.m0 * g.ldx + nt + 4 * cq;
+        const float sgn = g.negate_a ? -1.0f : 1.0f;
+        f32x4 xo[16];
+        if (!g.init_zero) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                xo[i] = *reinterpret_cast<const f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) xo[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        __syncthreads();   // every multiplier has read its last operands
+        __syncthreads();   // the sums are in LDS
+        const float* S = reinterpret_cast<const float*>(&L[0][0][0][0][0]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float* Sr = S + (kh + 8 * i) * TN + cq;
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + sgn * Sr[32 * e];
+            *reinterpret_cast<f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx) = o;
+        }
         return;
     }
 
@@ -675,31 +704,13 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     // element v of the accumulator is MFMA row (lane >> 5) * 4 + (v >> 2) * 8 + (v & 3),
     // column lane & 31.
     const int jrow = (lane >> 5) * 4, jcol = lane & 31;
-    float* __restrict__ Xw = g.X + (int64_t)bz * g.xs + (int64_t)(g.m0 + wm) * g.ldx + nt + wn + 4 * jcol;
-    auto x_off = [&](int mi, int ni, int v) {
-        return (int64_t)(4 * (jrow + (v >> 2) * 8 + (v & 3)) + 2 * mi) * g.ldx + 2 * ni;
-    };
-    const float sgn = g.negate_a ? -1.0f : 1.0f;   // fma(-a, b, x) = -fma(a, b, -x)
-    f32x16 acc[2][2], tot[2][2];
-    if (g.init_zero) {
+    f32x16 acc[2][2], tot[2][2];   // sums of the chunks; X itself is added in the epilogue
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+        for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) tot[mi][ni][v] = 0.0f;
-    } else {
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) tot[mi][ni][v] = Xw[x_off(mi, ni, v)];
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni) tot[mi][ni] *= sgn;
-    }
+            for (int v = 0; v < 16; ++v) tot[mi][ni][v] = 0.0f;
     const int rk = lane >> 5, ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     bf16x8 A0[3][2], B0[3][2], A1[3][2], B1[3][2];   // operands of k-step 0 / 1
@@ -753,12 +764,18 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
 #undef FORGE_SPLIT_READ
 #undef FORGE_SPLIT_MFMAS
 #undef FORGE_SPLIT_SCHED
+    __syncthreads();   // all operand reads done: the stage buffers become the output staging
+    float* S = reinterpret_cast<float*>(&L[0][0][0][0][0]);
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) Xw[x_off(mi, ni, v)] = sgn * tot[mi][ni][v];
+            for (int v = 0; v < 16; ++v) {
+                const int r = 4 * (jrow + (v >> 2) * 8 + (v & 3)) + wm + 2 * mi;
+                S[r * TN + 32 * (wn + 2 * ni) + jcol] = tot[mi][ni][v];
+            }
+    __syncthreads();
 }
 
 }  // namespace

@@ -84,8 +84,11 @@ class ExpertGroupGPTQ:
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
         seen = torch.tensor([n > 0 for n in self.num_samples], device=dev)
         bad = (~seen) | torch.isnan(self.H.diagonal(dim1=1, dim2=2)).any(dim=1)
-        if bool(bad.any()):
-            self.H[bad] = torch.eye(C, device=dev, dtype=torch.float32)
+        # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
+        # fraction of the fill rate)
+        for e in bad.nonzero().flatten().tolist():
+            self.H[e].zero_()
+            self.H[e].diagonal().fill_(1.0)
         failed = []
         side = torch.cuda.Stream(device=dev)          # default priority
 
@@ -112,7 +115,8 @@ class ExpertGroupGPTQ:
             # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149)
             masks = []
             for W in self.W:
-                zero_cols = ((W[e0:e1] == 0) | dead[:, None, :]).all(dim=1)
+                # all_r(W[r, c] == 0 or dead[c]) = all_r(W[r, c] == 0) or dead[c]
+                zero_cols = (W[e0:e1] == 0).all(dim=1) | dead
                 masks.append((dead_perm | zero_cols).to(torch.uint8).contiguous())
             same = torch.stack([(masks[0] == m).all() for m in masks[1:]] + [~dead.any()])
             flags = same.cpu().tolist()                                  # the chunk's one host sync
