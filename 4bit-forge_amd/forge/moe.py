@@ -112,15 +112,30 @@ class ExpertGroupGPTQ:
             dead_u8 = dead.to(torch.uint8).contiguous()
             dead_perm = torch.gather(dead, 1, perm)
             # weights with pruned columns zeroed decide the (unpermuted-index) zero-column
-            # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149)
+            # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149).
+            # A column can only be all zero if its first rows are: one look at 8 rows (fp8- or
+            # int-derived weights do contain single zeros) and at `dead` tells whether the
+            # full pass over the weights is needed at all.
+            first = torch.stack([(W[e0:e1, :8, :] == 0).all(dim=1).any() for W in self.W]
+                                + [dead.any()])
+            flags = first.cpu().tolist()                                 # host sync
+            has_dead = flags[-1]
             masks = []
-            for W in self.W:
-                # all_r(W[r, c] == 0 or dead[c]) = all_r(W[r, c] == 0) or dead[c]
-                zero_cols = (W[e0:e1] == 0).all(dim=1) | dead
-                masks.append((dead_perm | zero_cols).to(torch.uint8).contiguous())
-            same = torch.stack([(masks[0] == m).all() for m in masks[1:]] + [~dead.any()])
-            flags = same.cpu().tolist()                                  # the chunk's one host sync
-            shared, has_dead = all(flags[:-1]), not flags[-1]
+            for W, maybe in zip(self.W, flags[:-1]):
+                if maybe or has_dead:
+                    # all_r(W[r, c] == 0 or dead[c]) = all_r(W[r, c] == 0) or dead[c]
+                    zero_cols = (W[e0:e1] == 0).all(dim=1) | dead
+                    masks.append((dead_perm | zero_cols).to(torch.uint8).contiguous())
+                else:
+                    masks.append(None)
+            if all(m is None for m in masks):
+                shared = True
+                masks = [torch.zeros((B, C), dtype=torch.uint8, device=dev)] * len(self.W)
+            else:
+                zero = torch.zeros((B, C), dtype=torch.uint8, device=dev)
+                masks = [zero if m is None else m for m in masks]
+                shared = all(torch.stack([(masks[0] == m).all() for m in masks[1:]]).cpu().tolist()) \
+                    if len(masks) > 1 else True
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
             for job in jobs:
