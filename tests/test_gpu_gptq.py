@@ -198,6 +198,37 @@ def test_expert_group_matches_per_expert_handles():
     assert worst <= 5e-3, worst
 
 
+@pytest.mark.parametrize("zero_weight_column", [False, True])
+def test_expert_group_dead_and_zero_columns(zero_weight_column):
+    """A feature that one expert never sees (dead column: zero Hessian diagonal) and, in the
+    second case, an all-zero weight column in gate_proj only, which gives gate and up
+    different pruning masks: they no longer share a factor."""
+    from forge.moe import ExpertGroupGPTQ
+    moe = synth.qwen3_moe(experts=3, n_experts=24, hidden=256, inter=128, tokens=768, seed=11)
+    E = 3
+    xs = [moe.expert_inputs(e)[0].clone() for e in range(E)]
+    xs[1][:, 37] = 0
+    xs[1][:, 200] = 0
+    Wg, Wu = moe.Wg[:E].clone(), moe.Wu[:E].clone()
+    if zero_weight_column:
+        Wg[2, :, 5] = 0
+    offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
+              quantization_order="activation")
+    gu = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, **kw)
+    gu.update(torch.cat(xs).to(DEV), offs)
+    (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=4)
+    for e in range(E):
+        for W, (q, s, z) in ((Wg[e], (qg, sg, zg)), (Wu[e], (qu, su, zu))):
+            o = oracle.GPTQ(linear(W), **kw)
+            o.update(xs[e])
+            qo, so, zo = o.quantize()
+            assert float((so != s[e].cpu()).float().mean()) <= 2e-3
+            assert flip_rate(qo, q[e]) <= 5e-3
+            if e == 1:      # dead columns are pruned: weight 0 -> the code of zero
+                assert torch.equal(qo[:, [37, 200]], q[e].cpu()[:, [37, 200]])
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _e2e(W, X, kw, tol_flips, gs=128):
     o, g, H = _run_pair(W, X, chunks=1, **kw)
