@@ -38,9 +38,9 @@ PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, T
 # x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  The operand data a
 # launch of the factorisation GEMM has to read once (rows below the current block of the
 # factor and of its inverse) averages ~4.4e9 bytes over the 55 launches of a C=7168
-# factorisation; the sweep update reads the earlier error rows once (~1.9e9 bytes on
-# average): no wasted re-reads in either.
-MEASURED_TRAFFIC = {("deepseek_v3", 64, "chain_gemm_blocked_sum"): 4.67e9,
+# factorisation (the 15 launches of the C=2048 one are small: ~3.5e9 on average over all
+# 70); the sweep update reads the earlier error rows once (~1.9e9 bytes on average).
+MEASURED_TRAFFIC = {("deepseek_v3", 64, "split_gemm_bf16x3"): 4.48e9,
                     ("deepseek_v3", 64, "chain_gemm"): 2.06e9}
 
 KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit, executed / counted work)
