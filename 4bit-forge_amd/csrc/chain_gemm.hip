@@ -13,7 +13,9 @@
 // coalesced float4, LDS reads are conflict-free ds_read_b32, and no transpose is needed.
 // K advances 32 rows per LDS stage, as two sub-stages of 16 rows (32 MFMAs each).
 //
-// Two kernels share this layout.  chain_gemm_fast_kernel handles full, aligned tiles and
+// Two kernels share this layout (a third, split_gemm_kernel further down, does the
+// factorisation's blocked sums on the bf16 matrix pipe and has its own layout).
+// chain_gemm_fast_kernel handles full, aligned tiles and
 // is a software pipeline: while the MFMAs of one sub-stage run, the wavefront issues the
 // LDS reads of the next sub-stage, the LDS writes of the next stage and the global loads
 // of the stage after that, one memory instruction between two MFMAs (a wavefront issues
