@@ -98,8 +98,9 @@ def make_workload(cfg, chunk, seed=0):
 STREAMS = []
 
 
-def run_step(wl, cfg, chunk, step, mse=True):
-    """Hot path for experts [step*chunk, (step+1)*chunk) of the layer."""
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True):
+    """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
+    jobs one after the other (per-kernel event times are then exclusive)."""
     from forge.moe import ExpertGroupGPTQ
     E = cfg["n_experts"]
     e0 = (step * chunk) % E
@@ -143,8 +144,13 @@ def run_step(wl, cfg, chunk, step, mse=True):
                     grp.update(rows[offs[a]:offs[b]], sub_offs)
                     return grp.quantize(chunk=b - a)
 
-            jobs.append(pool.submit(solve_sub, [wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]))
-            jobs.append(pool.submit(solve_sub, [wl["Wd"]], hs, STREAMS[2 * j + 1]))
+            for weights, rows, stream in (([wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]),
+                                          ([wl["Wd"]], hs, STREAMS[2 * j + 1])):
+                job = pool.submit(solve_sub, weights, rows, stream)
+                if not overlap:
+                    job.result()
+                    stream.synchronize()
+                jobs.append(job)
         results = [j.result() for j in jobs]
     out_gu, out_dn = results[0::2], results[1::2]
     for s in STREAMS:
@@ -235,9 +241,10 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
-    # one more step with per-kernel HIP-event timing (on the stream the kernels run on)
+    # one more step with per-kernel HIP-event timing (on the stream the kernels run on); its
+    # jobs run one after the other so that no kernel's time includes another stream's work
     kernels.timing_enable(True)
-    run_step(wl, cfg, chunk, a.warmup + a.steps, mse)
+    run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False)
     torch.cuda.synchronize()
     stats = kernels.timing_collect()
     kernels.timing_enable(False)
