@@ -23,6 +23,7 @@
 // H.div_(H.diag()[:, None]) of gptq.py:164); diag(U0) is returned separately.  Flops:
 // C^3/3 for phase 1 and C^3/3 for phase 2 against 4/3 C^3 for the three-call route.
 #include "chain_gemm.h"
+#include <type_traits>
 
 namespace {
 
@@ -42,10 +43,16 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
     if (i < C) H[b * C * C + i * C + i] += damp[b];
 }
 
-// 1b for one diagonal block of every matrix in the batch.  256 threads as a 16x16 grid,
-// thread (ty,tx) owns the 8x8 sub-block P[8ty.., 8tx..] in registers.  Each elimination
-// step publishes the (unscaled) pivot row through LDS and costs one barrier:
-//   P[i][j] -= (row[i] / piv) * row[j],   D[c][j] = row[j] / sqrt(piv) afterwards.
+// 1b for one diagonal block of every matrix in the batch.  256 threads as a 16x16 grid;
+// thread (ty, tx) owns the elements (ty + 16 i, tx + 16 j), i, j < 8, of the block in
+// registers (cyclic ownership: at every step of either phase the live part of the block is
+// spread evenly over the threads, so a step costs (cb+1)^2 resp. (8-kb)(kb+1) fmas per
+// thread instead of 64).  Each step publishes one row through LDS and costs one barrier;
+// the row of the NEXT step is published as soon as the fmas that complete it are done, ahead
+// of the rest of the step's fmas, so that its LDS write and the pivot's division are off the
+// barrier-to-barrier path.
+//   phase 1:  P[i][j] -= (row[i] / piv) * row[j],   D[c][j] = row[j] / sqrt(piv) afterwards
+//   phase 2:  Z = D^-1 row by row, P accumulating D[i,k] Z[k,j]
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
     float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
@@ -69,7 +76,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int r = 8 * ty + i, c = 8 * tx + j;
+                const int r = ty + 16 * i, c = tx + 16 * j;
                 const int rr = r > c ? r : c, cc = r > c ? c : r;
                 P[i][j] = Ab[(m0 + rr) * C + m0 + cc];
             }
@@ -78,7 +85,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int r = 8 * ty + i, c = 8 * tx + j;
+                const int r = ty + 16 * i, c = tx + 16 * j;
                 const int rr = r > c ? r : c, cc = r > c ? c : r;
                 float v = (r == c) ? 1.0f : 0.0f;
                 if (rr < n) v = Ab[(m0 + rr) * C + m0 + cc];
@@ -88,38 +95,57 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     if (tid == 0) s_fail = 0;
     __syncthreads();   // the pivot owners below test it
 
-    // ---- P = D^T D, eliminating from the last row upwards
-    // (outer loop over the 16 row groups, inner 8 steps unrolled: P[c & 7] is then a fixed
-    // register row instead of a select over all eight)
-    for (int cb = NB / 8 - 1; cb >= 0; --cb)
+    // ---- P = D^T D, eliminating from the last row upwards.  Row c = 16 cb + r lives in
+    // register row cb of the threads with ty == r; only rows and columns <= c are still
+    // needed, i.e. register rows / columns <= cb.
+    auto publish_row = [&](auto cb_tag, int r) {
+        constexpr int cb = decltype(cb_tag)::value;
+        if (ty == r) {
+            const int c = 16 * cb + r;
 #pragma unroll
-    for (int ci = 7; ci >= 0; --ci) {
-        const int c = 8 * cb + ci;
-        if (ty == cb) {
-            *reinterpret_cast<float4*>(&Dm[c][8 * tx]) = make_float4(P[ci][0], P[ci][1], P[ci][2], P[ci][3]);
-            *reinterpret_cast<float4*>(&Dm[c][8 * tx + 4]) = make_float4(P[ci][4], P[ci][5], P[ci][6], P[ci][7]);
-            // the owner of the pivot divides once for everybody (the division is the longest
-            // dependent chain of a step)
-            if (tx == cb) {
-                const float piv = P[ci][ci];
+            for (int j = 0; j <= cb; ++j) Dm[c][tx + 16 * j] = P[cb][j];
+            // the owner of the pivot divides once for everybody
+            if (tx == r) {
+                const float piv = P[cb][cb];
                 s_inv[c] = piv > 0.0f ? 1.0f / piv : 0.0f;
                 if (!(piv > 0.0f) && s_fail == 0) s_fail = c + 1;
             }
         }
-        __syncthreads();
-        const float inv = s_inv[c];
-        const float4 a0 = *reinterpret_cast<const float4*>(&Dm[c][8 * ty]);
-        const float4 a1 = *reinterpret_cast<const float4*>(&Dm[c][8 * ty + 4]);
-        const float4 b0 = *reinterpret_cast<const float4*>(&Dm[c][8 * tx]);
-        const float4 b1 = *reinterpret_cast<const float4*>(&Dm[c][8 * tx + 4]);
-        const float ri[8] = {a0.x * inv, a0.y * inv, a0.z * inv, a0.w * inv,
-                             a1.x * inv, a1.y * inv, a1.z * inv, a1.w * inv};
-        const float rj[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    };
+    auto eliminate = [&](auto cb_tag) {
+        constexpr int cb = decltype(cb_tag)::value;
+        for (int r = 15; r >= 0; --r) {
+            const int c = 16 * cb + r;
+            __syncthreads();
+            const float inv = s_inv[c];
+            float ri[cb + 1], rj[cb + 1];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+            for (int i = 0; i <= cb; ++i) {
+                ri[i] = Dm[c][ty + 16 * i] * inv;
+                rj[i] = Dm[c][tx + 16 * i];
+            }
+            // the two register rows that can hold the next pivot row first
 #pragma unroll
-            for (int j = 0; j < 8; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
-    }
+            for (int i = cb; i >= (cb > 0 ? cb - 1 : 0); --i)
+#pragma unroll
+                for (int j = 0; j <= cb; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
+            if (r > 0) publish_row(std::integral_constant<int, cb>{}, r - 1);
+            else if constexpr (cb > 0) publish_row(std::integral_constant<int, cb - 1>{}, 15);
+#pragma unroll
+            for (int i = cb - 2; i >= 0; --i)
+#pragma unroll
+                for (int j = 0; j <= cb; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
+        }
+    };
+    publish_row(std::integral_constant<int, 7>{}, 15);
+    eliminate(std::integral_constant<int, 7>{});
+    eliminate(std::integral_constant<int, 6>{});
+    eliminate(std::integral_constant<int, 5>{});
+    eliminate(std::integral_constant<int, 4>{});
+    eliminate(std::integral_constant<int, 3>{});
+    eliminate(std::integral_constant<int, 2>{});
+    eliminate(std::integral_constant<int, 1>{});
+    eliminate(std::integral_constant<int, 0>{});
     __syncthreads();
     if (tid < NB) {
         const float piv = Dm[tid][tid];
@@ -134,46 +160,60 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     }
     __syncthreads();
 
-    // ---- Z = D^-1 (lower), row by row from the top; P now accumulates D[i,k] Z[k,j]
+    // ---- Z = D^-1 (lower), row by row from the top; P accumulates D[i,k] Z[k,j].  Row
+    // k = 16 kb + r: only rows > k (register rows >= kb) and columns <= k (register columns
+    // <= kb) are touched.
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
-    for (int kb = 0; kb < NB / 8; ++kb) {
-        // D does not change any more: the 8x8 block of it that these 8 steps multiply by is
-        // fetched once, row-wise, outside the serial chain
-        float Dblk[8][8];
+    auto publish_z = [&](auto kb_tag, int r) {
+        constexpr int kb = decltype(kb_tag)::value;
+        if (ty == r) {
+            const int k = 16 * kb + r;
+            const float rc = drc[k];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float4 d0 = *reinterpret_cast<const float4*>(&Dm[8 * ty + i][8 * kb]);
-            const float4 d1 = *reinterpret_cast<const float4*>(&Dm[8 * ty + i][8 * kb + 4]);
-            Dblk[i][0] = d0.x; Dblk[i][1] = d0.y; Dblk[i][2] = d0.z; Dblk[i][3] = d0.w;
-            Dblk[i][4] = d1.x; Dblk[i][5] = d1.y; Dblk[i][6] = d1.z; Dblk[i][7] = d1.w;
-        }
-#pragma unroll
-        for (int ki = 0; ki < 8; ++ki) {
-            const int k = 8 * kb + ki;
-            if (ty == kb) {
-                const float rc = drc[k];
-                float z[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int col = 8 * tx + j;
-                    z[j] = col <= k ? ((col == k ? 1.0f : 0.0f) - P[ki][j]) * rc : 0.0f;
-                }
-                *reinterpret_cast<float4*>(&Zm[k][8 * tx]) = make_float4(z[0], z[1], z[2], z[3]);
-                *reinterpret_cast<float4*>(&Zm[k][8 * tx + 4]) = make_float4(z[4], z[5], z[6], z[7]);
+            for (int j = 0; j < 8; ++j) {
+                const int col = tx + 16 * j;
+                float z = 0.0f;
+                if (j <= kb && col <= k) z = ((col == k ? 1.0f : 0.0f) - P[kb][j]) * rc;
+                Zm[k][col] = z;
             }
-            __syncthreads();
-            const float4 z0 = *reinterpret_cast<const float4*>(&Zm[k][8 * tx]);
-            const float4 z1 = *reinterpret_cast<const float4*>(&Zm[k][8 * tx + 4]);
-            const float zj[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) P[i][j] = __builtin_fmaf(Dblk[i][ki], zj[j], P[i][j]);
         }
-    }
+    };
+    auto invert = [&](auto kb_tag) {
+        constexpr int kb = decltype(kb_tag)::value;
+        for (int r = 0; r < 16; ++r) {
+            const int k = 16 * kb + r;
+            // D does not change any more: its column k is read ahead of the barrier
+            float d[8 - kb];
+#pragma unroll
+            for (int i = kb; i < 8; ++i) d[i - kb] = Dm[ty + 16 * i][k];
+            __syncthreads();
+            float zj[kb + 1];
+#pragma unroll
+            for (int j = 0; j <= kb; ++j) zj[j] = Zm[k][tx + 16 * j];
+#pragma unroll
+            for (int i = kb; i <= (kb < 7 ? kb + 1 : 7); ++i)
+#pragma unroll
+                for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
+            if (r < 15) publish_z(std::integral_constant<int, kb>{}, r + 1);
+            else if constexpr (kb < 7) publish_z(std::integral_constant<int, kb + 1>{}, 0);
+#pragma unroll
+            for (int i = kb + 2; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
+        }
+    };
+    publish_z(std::integral_constant<int, 0>{}, 0);
+    invert(std::integral_constant<int, 0>{});
+    invert(std::integral_constant<int, 1>{});
+    invert(std::integral_constant<int, 2>{});
+    invert(std::integral_constant<int, 3>{});
+    invert(std::integral_constant<int, 4>{});
+    invert(std::integral_constant<int, 5>{});
+    invert(std::integral_constant<int, 6>{});
+    invert(std::integral_constant<int, 7>{});
     __syncthreads();
 
     // ---- outputs
