@@ -98,6 +98,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     // ---- P = D^T D, eliminating from the last row upwards.  Row c = 16 cb + r lives in
     // register row cb of the threads with ty == r; only rows and columns <= c are still
     // needed, i.e. register rows / columns <= cb.
+    int my_fail = 0;   // first non-positive pivot this thread owned (1-based), in elimination order
     auto publish_row = [&](auto cb_tag, int r) {
         constexpr int cb = decltype(cb_tag)::value;
         if (ty == r) {
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
             if (tx == r) {
                 const float piv = P[cb][cb];
                 s_inv[c] = piv > 0.0f ? 1.0f / piv : 0.0f;
-                if (!(piv > 0.0f) && s_fail == 0) s_fail = c + 1;
+                if (!(piv > 0.0f) && my_fail == 0) my_fail = c + 1;
             }
         }
     };
@@ -167,11 +168,10 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
-    auto publish_z = [&](auto kb_tag, int r) {
+    auto publish_z = [&](auto kb_tag, int r, float rc) {
         constexpr int kb = decltype(kb_tag)::value;
         if (ty == r) {
             const int k = 16 * kb + r;
-            const float rc = drc[k];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int col = tx + 16 * j;
@@ -185,10 +185,12 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         constexpr int kb = decltype(kb_tag)::value;
         for (int r = 0; r < 16; ++r) {
             const int k = 16 * kb + r;
-            // D does not change any more: its column k is read ahead of the barrier
+            // D does not change any more: its column k (and the next row's 1/d) are read
+            // ahead of the barrier
             float d[8 - kb];
 #pragma unroll
             for (int i = kb; i < 8; ++i) d[i - kb] = Dm[ty + 16 * i][k];
+            const float rc_next = drc[k + 1 < NB ? k + 1 : k];
             __syncthreads();
             float zj[kb + 1];
 #pragma unroll
@@ -197,15 +199,15 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
             for (int i = kb; i <= (kb < 7 ? kb + 1 : 7); ++i)
 #pragma unroll
                 for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
-            if (r < 15) publish_z(std::integral_constant<int, kb>{}, r + 1);
-            else if constexpr (kb < 7) publish_z(std::integral_constant<int, kb + 1>{}, 0);
+            if (r < 15) publish_z(std::integral_constant<int, kb>{}, r + 1, rc_next);
+            else if constexpr (kb < 7) publish_z(std::integral_constant<int, kb + 1>{}, 0, rc_next);
 #pragma unroll
             for (int i = kb + 2; i < 8; ++i)
 #pragma unroll
                 for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
         }
     };
-    publish_z(std::integral_constant<int, 0>{}, 0);
+    publish_z(std::integral_constant<int, 0>{}, 0, drc[0]);
     invert(std::integral_constant<int, 0>{});
     invert(std::integral_constant<int, 1>{});
     invert(std::integral_constant<int, 2>{});
@@ -225,6 +227,8 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         if (m < n && k < n) Ub[(m0 + m) * C + m0 + k] = Zm[k][m];
     }
     if (tid < n) udiag[b * C + m0 + tid] = Zm[tid][tid];
+    if (my_fail != 0) atomicMax(&s_fail, my_fail);   // the first failure = the largest row
+    __syncthreads();
     if (tid == 0 && s_fail != 0 && info[b] == 0) info[b] = (int32_t)(m0 + s_fail);
 }
 
