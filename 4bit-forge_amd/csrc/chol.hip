@@ -236,7 +236,8 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
 // the blocks on and right of it), and divide by the diagonal when asked to (gptq.py:164).
 // A failed factorisation hands back the identity instead, as gptq.py:172-175 does.
 __global__ void finish_rows_kernel(float* __restrict__ U, float* __restrict__ udiag,
-                                   const int32_t* __restrict__ info, int64_t C, bool normalise) {
+                                   const int32_t* __restrict__ info, int64_t C, bool normalise,
+                                   bool zero_left) {
     const int64_t b = blockIdx.y;
     const int64_t row = blockIdx.x;
     float* __restrict__ Ur = U + b * C * C + row * C;
@@ -246,7 +247,7 @@ __global__ void finish_rows_kernel(float* __restrict__ U, float* __restrict__ ud
         return;
     }
     // the diagonal block kernel wrote its whole tile, zeros below the diagonal included
-    const int64_t left = row / NB * NB;
+    const int64_t left = zero_left ? row / NB * NB : 0;
     for (int64_t j = threadIdx.x; j < left; j += blockDim.x) Ur[j] = 0.0f;
     if (!normalise) return;
     const float d = udiag[b * C + row];
@@ -334,9 +335,10 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
         }
         if (int e = forge::launch_chain_gemm_pair(g1c, g2b, batch, st)) return e;
     }
-    forge::KernelTiming timing("chol_finish_rows", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
-    finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(U, udiag, info, C,
-                                                                               normalise != 0);
+    forge::KernelTiming timing("chol_finish_rows", st,
+                               ((normalise & 2) ? 4.0 : 6.0) * C * C * (double)batch, forge::WORK_BYTES);
+    finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(
+        U, udiag, info, C, (normalise & 1) != 0, (normalise & 2) == 0);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

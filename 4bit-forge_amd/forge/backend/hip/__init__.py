@@ -267,8 +267,9 @@ class _HipKernels:
                 nbytes, _stream()))
         return H
 
-    def chol_inv_upper_batched(self, H, damp, normalise=True):
-        """H [B,C,C] f32 (destroyed); damp [B] f32 or None -> U [B,C,C], udiag [B,C], info [B]."""
+    def chol_inv_upper_batched(self, H, damp, normalise=True, upper_only=False):
+        """H [B,C,C] f32 (destroyed); damp [B] f32 or None -> U [B,C,C], udiag [B,C], info [B].
+        upper_only: U is only valid on and above the diagonal blocks (what the sweeps read)."""
         _need_cuda(H, damp)
         B, C, _ = H.shape
         assert H.is_contiguous() and H.dtype == torch.float32
@@ -281,7 +282,7 @@ class _HipKernels:
         with torch.cuda.device(H.device):
             self._check(self._lib.forge_chol_inv_upper_batched(
                 _ptr(H), _ptr(damp), _ptr(U), _ptr(udiag), _ptr(info), B, C,
-                int(bool(normalise)), _ptr(ws), nbytes, _stream()))
+                int(bool(normalise)) | (2 if upper_only else 0), _ptr(ws), nbytes, _stream()))
         return U, udiag, info
 
     def hessian_permute(self, H, perm, dead, rel_damp):

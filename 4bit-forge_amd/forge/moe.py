@@ -156,7 +156,7 @@ class ExpertGroupGPTQ:
                     Wsrc.record_stream(side)
                     del Wsrc
                 Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
-                U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True)
+                U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
                 failed.append((e0, info))
                 X = kernels.weight_to_solver_order(Wc, perm_inv, dead_u8)

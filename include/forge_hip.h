@@ -126,8 +126,10 @@ int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int6
 
 /* Batched form of GPTQ._h_factor's torch.linalg calls (gptq.py:152-175):
  * for each b: A = H[b] + damp[b]*I (lower triangle of H[b] read), U0 = upper Cholesky
- * factor of inv(A); writes U[b] = U0 / diag(U0)[:,None] (normalise != 0) or U0, upper
- * triangle + zeroed lower; udiag[b] [C] receives diag(U0).  info[b] (int32) is 0 on
+ * factor of inv(A); writes U[b] = U0 / diag(U0)[:,None] (normalise & 1) or U0, upper
+ * triangle + zeroed lower; udiag[b] [C] receives diag(U0).  normalise & 2: the caller reads
+ * the upper triangle only (the sweeps do) and the part of U[b] left of the 128x128 diagonal
+ * blocks is left unwritten.  info[b] (int32) is 0 on
  * success or the 1-based index of the first non-positive pivot, in which case U[b] = I.
  * H[b] is destroyed (used as workspace).  ws: workspace of forge_chol_workspace_bytes
  * (128x128 inverse diagonal blocks, plus 768 bytes per column and matrix for the bf16

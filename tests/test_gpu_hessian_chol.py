@@ -91,6 +91,9 @@ def test_factor_bf16_split_and_fp32_updates_agree(hip, monkeypatch, B, C):
     Us, uds, infos = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
     monkeypatch.setenv("FORGE_FP32_BLOCKED_SUM", "1")
     Uf, udf, infof = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
+    # upper_only: same values on and above the diagonal blocks, nothing promised left of them
+    Uu, _, _ = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV), upper_only=True)
+    assert torch.equal(torch.triu(Uu), torch.triu(Uf))
     assert infos.tolist()[:B - 1] == [0] * (B - 1) and infos[B - 1].item() > 0
     assert infof.tolist() == infos.tolist()
     assert torch.equal(Us[B - 1].cpu(), torch.eye(C))
