@@ -43,23 +43,55 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
     if (i < C) H[b * C * C + i * C + i] += damp[b];
 }
 
-// 1b for one diagonal block of every matrix in the batch.  256 threads as a 16x16 grid;
-// thread (ty, tx) owns the elements (ty + 16 i, tx + 16 j), i, j < 8, of the block in
-// registers (cyclic ownership: at every step of either phase the live part of the block is
-// spread evenly over the threads, so a step costs (cb+1)^2 resp. (8-kb)(kb+1) fmas per
-// thread instead of 64).  Each step publishes one row through LDS and costs one barrier;
-// the row of the NEXT step is published as soon as the fmas that complete it are done, ahead
-// of the rest of the step's fmas, so that its LDS write and the pivot's division are off the
-// barrier-to-barrier path.
-//   phase 1:  P[i][j] -= (row[i] / piv) * row[j],   D[c][j] = row[j] / sqrt(piv) afterwards
-//   phase 2:  Z = D^-1 row by row, P accumulating D[i,k] Z[k,j]
+// 1b for one diagonal block of every matrix in the batch: P = D^T D (D lower triangular,
+// elimination from the last row upwards) and Z = D^-1, in one workgroup, blocked by 16 so
+// that a phase is 8 block steps with a handful of barriers each rather than 128
+// barrier-to-barrier pivot steps.
+//   phase 1, block b = 7..0 (rows/columns 16b..16b+15), P = [[P11, P12], [P21, P22]]:
+//     D22^T D22 = P22 by 16 lanes of ONE wavefront, a row of the 16x16 block per lane, the
+//       pivot row taken through DPP row broadcasts: no LDS, no barrier inside
+//     D22^T D21 = P21 by back substitution, a column per thread; P11 -= D21^T D21 (all
+//       threads, P in registers)
+//   W = D22^-1 of the eight diagonal blocks, all at once (16 lanes per block, DPP again)
+//   phase 2, block kb = 0..7:  Z[kb, <kb] = -W (D[kb, <kb] Z[<kb, <kb]); the product in the
+//     brackets is accumulated in registers by rank-16 updates as the rows of Z appear.
+// Thread (ty, tx) of the 16x16 grid owns the elements (ty + 16 i, tx + 16 j), i, j < 8, in
+// registers (cyclic ownership: the live part of the matrix stays spread over all threads).
+template <int K>
+__device__ __forceinline__ float row_bcast(float v) {   // lane K of this lane's row of 16
+    float r;
+    asm volatile("v_mov_b32_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v), "n"(K));
+    return r;
+}
+// x -= bcast_K(u) * f   /   x += bcast_K(u) * f, one fused multiply-add each
+template <int K>
+__device__ __forceinline__ void fnma_bcast(float& x, float u, float f) {
+    asm volatile("v_fmac_f32_dpp %0, -%1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(x) : "v"(u), "v"(f), "n"(K));
+}
+template <int K>
+__device__ __forceinline__ void fma_bcast(float& x, float u, float f) {
+    asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(x) : "v"(u), "v"(f), "n"(K));
+}
+// two wait states between a VALU write of a register and a DPP read of it
+__device__ __forceinline__ void dpp_settle() { asm volatile("s_nop 1"); }
+// the same, placed after whatever wrote these sixteen registers (they pass through the
+// statement, so the compiler can move neither their producers below it nor their DPP
+// readers above it)
+__device__ __forceinline__ void dpp_settle16(float (&v)[16]) {
+    asm volatile("s_nop 1"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]),
+                   "+v"(v[7]), "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]),
+                   "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
+}
+
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
     float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
     extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 * NB * LDP floats (135 KB)
     float (*Dm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem);
     float (*Zm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem + NB * LDP);
-    __shared__ float dsq[NB], drc[NB], s_inv[NB];
+    __shared__ float Pp[16][LDP];   // the 16 rows of the current block, published by their owners
+    __shared__ float s_rc[NB];      // 1 / D[k][k]
     __shared__ int s_fail;
 
     const int64_t b = blockIdx.x;
@@ -68,8 +100,6 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
     const int n = (int)((C - m0) < NB ? (C - m0) : NB);
     const float* __restrict__ Ab = A + b * C * C;
 
-    // symmetric tile: both halves were produced by the same GEMM; read the lower one.
-    // (Full blocks load without per-element tests so that the 64 loads are in flight together.)
     float P[8][8];
     if (n == NB) {
 #pragma unroll
@@ -93,142 +123,194 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
             }
     }
     if (tid == 0) s_fail = 0;
-    __syncthreads();   // the pivot owners below test it
 
-    // ---- P = D^T D, eliminating from the last row upwards.  Row c = 16 cb + r lives in
-    // register row cb of the threads with ty == r; only rows and columns <= c are still
-    // needed, i.e. register rows / columns <= cb.
-    int my_fail = 0;   // first non-positive pivot this thread owned (1-based), in elimination order
-    auto publish_row = [&](auto cb_tag, int r) {
-        constexpr int cb = decltype(cb_tag)::value;
-        if (ty == r) {
-            const int c = 16 * cb + r;
+    // ---- phase 1
+    auto factor_block = [&](auto b_tag) {
+        constexpr int bb = decltype(b_tag)::value;
+        // 1. the owners publish rows 16 bb .. 16 bb + 15, columns < 16 (bb + 1)
 #pragma unroll
-            for (int j = 0; j <= cb; ++j) Dm[c][tx + 16 * j] = P[cb][j];
-            // the owner of the pivot divides once for everybody
-            if (tx == r) {
-                const float piv = P[cb][cb];
-                s_inv[c] = piv > 0.0f ? 1.0f / piv : 0.0f;
-                if (!(piv > 0.0f) && my_fail == 0) my_fail = c + 1;
-            }
+        for (int j = 0; j <= bb; ++j) Pp[ty][tx + 16 * j] = P[bb][j];
+        __syncthreads();
+        // 2. one row of the 16x16 diagonal block per lane
+        if (tid < 16) {
+            const int li = tid;
+            float p[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) p[j] = Pp[li][16 * bb + j];
+            float mypiv = 1.0f;
+            int fail = 0;
+            dpp_settle16(p);
+#define FORGE_ELIM(c)                                                                         \
+    {                                                                                         \
+        const float piv = row_bcast<c>(p[c]);                                                 \
+        const bool ok = piv > 0.0f;                                                           \
+        if (!ok && fail == 0) fail = 16 * bb + c + 1;                                         \
+        mypiv = li == c ? piv : mypiv;                                                        \
+        float inv = __builtin_amdgcn_rcpf(piv);                                               \
+        inv = __builtin_fmaf(__builtin_fmaf(-piv, inv, 1.0f), inv, inv);                      \
+        const float f = (ok && li < c) ? p[c] * inv : 0.0f;                                   \
+        _Pragma("unroll") for (int j = 0; j < c; ++j) fnma_bcast<c>(p[j], p[j], f);          \
+        dpp_settle();                                                                         \
+    }
+            FORGE_ELIM(15) FORGE_ELIM(14) FORGE_ELIM(13) FORGE_ELIM(12) FORGE_ELIM(11) FORGE_ELIM(10)
+            FORGE_ELIM(9) FORGE_ELIM(8) FORGE_ELIM(7) FORGE_ELIM(6) FORGE_ELIM(5) FORGE_ELIM(4)
+            FORGE_ELIM(3) FORGE_ELIM(2) FORGE_ELIM(1) FORGE_ELIM(0)
+#undef FORGE_ELIM
+            // lane li now holds row li of the unscaled factor in p[0..li]
+            const float d = mypiv > 0.0f ? sqrtf(mypiv) : 1.0f;
+            const float rc = 1.0f / d;
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                Dm[16 * bb + li][16 * bb + j] = j < li ? p[j] * rc : (j == li ? d : 0.0f);
+            s_rc[16 * bb + li] = rc;
+            if (li == 0 && fail != 0) atomicMax(&s_fail, fail);
         }
-    };
-    auto eliminate = [&](auto cb_tag) {
-        constexpr int cb = decltype(cb_tag)::value;
-        for (int r = 15; r >= 0; --r) {
-            const int c = 16 * cb + r;
+        __syncthreads();
+        if constexpr (bb > 0) {
+            // 3. D21 from D22^T D21 = P21, one column per thread, last row first
+            if (tid < 16 * bb) {
+                // (column form: once x[i] is known, the fmas that remove it from the rows
+                // above are independent of each other)
+                float x[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[i] = Pp[i][tid];
+#pragma unroll
+                for (int i = 15; i >= 0; --i) {
+                    x[i] = x[i] * s_rc[16 * bb + i];
+#pragma unroll
+                    for (int k = 0; k < i; ++k)
+                        x[k] = __builtin_fmaf(-Dm[16 * bb + i][16 * bb + k], x[i], x[k]);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) Dm[16 * bb + i][tid] = x[i];
+            }
             __syncthreads();
-            const float inv = s_inv[c];
-            float ri[cb + 1], rj[cb + 1];
+            // 4. P11 -= D21^T D21
+#pragma unroll 4
+            for (int m = 0; m < 16; ++m) {
+                float di[bb], dj2[bb];
 #pragma unroll
-            for (int i = 0; i <= cb; ++i) {
-                ri[i] = Dm[c][ty + 16 * i] * inv;
-                rj[i] = Dm[c][tx + 16 * i];
+                for (int i = 0; i < bb; ++i) {
+                    di[i] = Dm[16 * bb + m][ty + 16 * i];
+                    dj2[i] = Dm[16 * bb + m][tx + 16 * i];
+                }
+                // (blocks above the diagonal are never read again)
+#pragma unroll
+                for (int i = 0; i < bb; ++i)
+#pragma unroll
+                    for (int j = 0; j <= i; ++j) P[i][j] = __builtin_fmaf(-di[i], dj2[j], P[i][j]);
             }
-            // the two register rows that can hold the next pivot row first
-#pragma unroll
-            for (int i = cb; i >= (cb > 0 ? cb - 1 : 0); --i)
-#pragma unroll
-                for (int j = 0; j <= cb; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
-            if (r > 0) publish_row(std::integral_constant<int, cb>{}, r - 1);
-            else if constexpr (cb > 0) publish_row(std::integral_constant<int, cb - 1>{}, 15);
-#pragma unroll
-            for (int i = cb - 2; i >= 0; --i)
-#pragma unroll
-                for (int j = 0; j <= cb; ++j) P[i][j] = __builtin_fmaf(-ri[i], rj[j], P[i][j]);
         }
     };
-    publish_row(std::integral_constant<int, 7>{}, 15);
-    eliminate(std::integral_constant<int, 7>{});
-    eliminate(std::integral_constant<int, 6>{});
-    eliminate(std::integral_constant<int, 5>{});
-    eliminate(std::integral_constant<int, 4>{});
-    eliminate(std::integral_constant<int, 3>{});
-    eliminate(std::integral_constant<int, 2>{});
-    eliminate(std::integral_constant<int, 1>{});
-    eliminate(std::integral_constant<int, 0>{});
+    factor_block(std::integral_constant<int, 7>{});
+    factor_block(std::integral_constant<int, 6>{});
+    factor_block(std::integral_constant<int, 5>{});
+    factor_block(std::integral_constant<int, 4>{});
+    factor_block(std::integral_constant<int, 3>{});
+    factor_block(std::integral_constant<int, 2>{});
+    factor_block(std::integral_constant<int, 1>{});
+    factor_block(std::integral_constant<int, 0>{});
+
+    // ---- W = D22^-1 of all eight diagonal blocks at once: lanes 16 g .. 16 g + 15 take block g,
+    // a row per lane, rows in lockstep: row m is finished by lane m at step m, then every
+    // later row adds D[k][m] W[m][j] to its running sums
     __syncthreads();
-    if (tid < NB) {
-        const float piv = Dm[tid][tid];
-        const float d = piv > 0.0f ? sqrtf(piv) : 1.0f;
-        dsq[tid] = d;
-        drc[tid] = 1.0f / d;
+    if (tid < 128) {
+        const int g = tid >> 4, li = tid & 15;
+        float dj[16], acc[16], w[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            dj[j] = Dm[16 * g + li][16 * g + j];
+            acc[j] = 0.0f;
+            w[j] = 0.0f;
+        }
+        const float rc = s_rc[16 * g + li];
+#define FORGE_INV(m)                                                                          \
+    {                                                                                         \
+        _Pragma("unroll") for (int j = 0; j <= m; ++j) {                                      \
+            const float val = ((j == m ? 1.0f : 0.0f) - acc[j]) * rc;                         \
+            w[j] = li == m ? val : w[j];                                                      \
+        }                                                                                     \
+        dpp_settle16(w);                                                                      \
+        _Pragma("unroll") for (int j = 0; j <= m; ++j) fma_bcast<m>(acc[j], w[j], dj[m]);     \
     }
-    __syncthreads();
-    for (int e = tid; e < NB * NB; e += 256) {
-        const int c = e >> 7, j = e & (NB - 1);
-        Dm[c][j] = j < c ? Dm[c][j] * drc[c] : (j == c ? dsq[c] : 0.0f);
+        FORGE_INV(0) FORGE_INV(1) FORGE_INV(2) FORGE_INV(3) FORGE_INV(4) FORGE_INV(5) FORGE_INV(6)
+        FORGE_INV(7) FORGE_INV(8) FORGE_INV(9) FORGE_INV(10) FORGE_INV(11) FORGE_INV(12)
+        FORGE_INV(13) FORGE_INV(14) FORGE_INV(15)
+#undef FORGE_INV
+#pragma unroll
+        for (int j = 0; j < 16; ++j) Zm[16 * g + li][16 * g + j] = j <= li ? w[j] : 0.0f;
     }
     __syncthreads();
 
-    // ---- Z = D^-1 (lower), row by row from the top; P accumulates D[i,k] Z[k,j].  Row
-    // k = 16 kb + r: only rows > k (register rows >= kb) and columns <= k (register columns
-    // <= kb) are touched.
+    // ---- phase 2: P accumulates S = D[rows, < 16 kb] Z[< 16 kb, columns]
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) P[i][j] = 0.0f;
-    auto publish_z = [&](auto kb_tag, int r, float rc) {
+    auto invert_block = [&](auto kb_tag) {
         constexpr int kb = decltype(kb_tag)::value;
-        if (ty == r) {
-            const int k = 16 * kb + r;
+        if constexpr (kb > 0) {
+            // 1. the owners publish S for the rows of block kb
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int col = tx + 16 * j;
-                float z = 0.0f;
-                if (j <= kb && col <= k) z = ((col == k ? 1.0f : 0.0f) - P[kb][j]) * rc;
-                Zm[k][col] = z;
+            for (int j = 0; j < kb; ++j) Pp[ty][tx + 16 * j] = P[kb][j];
+            __syncthreads();
+            // 2. Z[kb, < kb] = -W S: row ty, columns tx + 16 j
+            float wr[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) wr[k] = Zm[16 * kb + ty][16 * kb + k];   // W[ty][k], 0 for k > ty
+            float z[kb];
+#pragma unroll
+            for (int j = 0; j < kb; ++j) z[j] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+#pragma unroll
+                for (int j = 0; j < kb; ++j) z[j] = __builtin_fmaf(-wr[k], Pp[k][tx + 16 * j], z[j]);
+#pragma unroll
+            for (int j = 0; j < kb; ++j) Zm[16 * kb + ty][tx + 16 * j] = z[j];
+        }
+        // columns right of the diagonal block are zero
+#pragma unroll
+        for (int j = kb + 1; j < 8; ++j) Zm[16 * kb + ty][tx + 16 * j] = 0.0f;
+        __syncthreads();
+        if constexpr (kb < 7) {
+            // 3. rows below: S += D[rows, block kb] Z[block kb, columns <= 16 kb + 15]
+#pragma unroll 4
+            for (int m = 0; m < 16; ++m) {
+                float dcol[7 - kb], zrow[kb + 1];
+#pragma unroll
+                for (int i = kb + 1; i < 8; ++i) dcol[i - kb - 1] = Dm[ty + 16 * i][16 * kb + m];
+#pragma unroll
+                for (int j = 0; j <= kb; ++j) zrow[j] = Zm[16 * kb + m][tx + 16 * j];
+#pragma unroll
+                for (int i = kb + 1; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(dcol[i - kb - 1], zrow[j], P[i][j]);
             }
         }
     };
-    auto invert = [&](auto kb_tag) {
-        constexpr int kb = decltype(kb_tag)::value;
-        for (int r = 0; r < 16; ++r) {
-            const int k = 16 * kb + r;
-            // D does not change any more: its column k (and the next row's 1/d) are read
-            // ahead of the barrier
-            float d[8 - kb];
-#pragma unroll
-            for (int i = kb; i < 8; ++i) d[i - kb] = Dm[ty + 16 * i][k];
-            const float rc_next = drc[k + 1 < NB ? k + 1 : k];
-            __syncthreads();
-            float zj[kb + 1];
-#pragma unroll
-            for (int j = 0; j <= kb; ++j) zj[j] = Zm[k][tx + 16 * j];
-#pragma unroll
-            for (int i = kb; i <= (kb < 7 ? kb + 1 : 7); ++i)
-#pragma unroll
-                for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
-            if (r < 15) publish_z(std::integral_constant<int, kb>{}, r + 1, rc_next);
-            else if constexpr (kb < 7) publish_z(std::integral_constant<int, kb + 1>{}, 0, rc_next);
-#pragma unroll
-            for (int i = kb + 2; i < 8; ++i)
-#pragma unroll
-                for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(d[i - kb], zj[j], P[i][j]);
-        }
-    };
-    publish_z(std::integral_constant<int, 0>{}, 0, drc[0]);
-    invert(std::integral_constant<int, 0>{});
-    invert(std::integral_constant<int, 1>{});
-    invert(std::integral_constant<int, 2>{});
-    invert(std::integral_constant<int, 3>{});
-    invert(std::integral_constant<int, 4>{});
-    invert(std::integral_constant<int, 5>{});
-    invert(std::integral_constant<int, 6>{});
-    invert(std::integral_constant<int, 7>{});
+    invert_block(std::integral_constant<int, 0>{});
+    invert_block(std::integral_constant<int, 1>{});
+    invert_block(std::integral_constant<int, 2>{});
+    invert_block(std::integral_constant<int, 3>{});
+    invert_block(std::integral_constant<int, 4>{});
+    invert_block(std::integral_constant<int, 5>{});
+    invert_block(std::integral_constant<int, 6>{});
+    invert_block(std::integral_constant<int, 7>{});
     __syncthreads();
 
     // ---- outputs
     float* __restrict__ Di = Dinv + (b * nblk + a) * NB * NB;
-    for (int e = tid; e < NB * NB; e += 256) Di[e] = Zm[e >> 7][e & (NB - 1)];
+    for (int e = tid; e < NB * NB / 4; e += 256) {
+        const int k = e >> 5, m4 = (e & 31) * 4;
+        *reinterpret_cast<float4*>(Di + k * NB + m4) = *reinterpret_cast<const float4*>(&Zm[k][m4]);
+    }
     float* __restrict__ Ub = U + b * C * C;
     for (int e = tid; e < NB * NB; e += 256) {
         const int m = e >> 7, k = e & (NB - 1);   // U0[a-block row m, column k] = Z[k, m]
         if (m < n && k < n) Ub[(m0 + m) * C + m0 + k] = Zm[k][m];
     }
     if (tid < n) udiag[b * C + m0 + tid] = Zm[tid][tid];
-    if (my_fail != 0) atomicMax(&s_fail, my_fail);   // the first failure = the largest row
-    __syncthreads();
     if (tid == 0 && s_fail != 0 && info[b] == 0) info[b] = (int32_t)(m0 + s_fail);
 }
 
