@@ -177,9 +177,15 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
 #pragma unroll
                 for (int i = 15; i >= 0; --i) {
                     x[i] = x[i] * s_rc[16 * bb + i];
+                    // row i of D22, the same for every thread: 16-byte broadcast reads
+                    float drow[16];
 #pragma unroll
-                    for (int k = 0; k < i; ++k)
-                        x[k] = __builtin_fmaf(-Dm[16 * bb + i][16 * bb + k], x[i], x[k]);
+                    for (int q = 0; 4 * q < i; ++q) {
+                        const float4 v = *reinterpret_cast<const float4*>(&Dm[16 * bb + i][16 * bb + 4 * q]);
+                        drow[4 * q] = v.x; drow[4 * q + 1] = v.y; drow[4 * q + 2] = v.z; drow[4 * q + 3] = v.w;
+                    }
+#pragma unroll
+                    for (int k = 0; k < i; ++k) x[k] = __builtin_fmaf(-drow[k], x[i], x[k]);
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) Dm[16 * bb + i][tid] = x[i];
@@ -275,17 +281,27 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         __syncthreads();
         if constexpr (kb < 7) {
             // 3. rows below: S += D[rows, block kb] Z[block kb, columns <= 16 kb + 15]
-#pragma unroll 4
-            for (int m = 0; m < 16; ++m) {
-                float dcol[7 - kb], zrow[kb + 1];
+            // (the 16 values of D that a register row needs are consecutive in LDS: 16-byte reads)
 #pragma unroll
-                for (int i = kb + 1; i < 8; ++i) dcol[i - kb - 1] = Dm[ty + 16 * i][16 * kb + m];
-#pragma unroll
-                for (int j = 0; j <= kb; ++j) zrow[j] = Zm[16 * kb + m][tx + 16 * j];
+            for (int q = 0; q < 4; ++q) {
+                float4 dq[7 - kb];
 #pragma unroll
                 for (int i = kb + 1; i < 8; ++i)
+                    dq[i - kb - 1] = *reinterpret_cast<const float4*>(&Dm[ty + 16 * i][16 * kb + 4 * q]);
 #pragma unroll
-                    for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(dcol[i - kb - 1], zrow[j], P[i][j]);
+                for (int mm = 0; mm < 4; ++mm) {
+                    const int m = 4 * q + mm;
+                    float zrow[kb + 1];
+#pragma unroll
+                    for (int j = 0; j <= kb; ++j) zrow[j] = Zm[16 * kb + m][tx + 16 * j];
+#pragma unroll
+                    for (int i = kb + 1; i < 8; ++i) {
+                        const float4 v = dq[i - kb - 1];
+                        const float dv = mm == 0 ? v.x : (mm == 1 ? v.y : (mm == 2 ? v.z : v.w));
+#pragma unroll
+                        for (int j = 0; j <= kb; ++j) P[i][j] = __builtin_fmaf(dv, zrow[j], P[i][j]);
+                    }
+                }
             }
         }
     };
