@@ -86,7 +86,10 @@ __device__ __forceinline__ void dpp_settle16(float (&v)[16]) {
 
 __global__ __launch_bounds__(256) void diag_block_kernel(
     const float* __restrict__ A, float* __restrict__ U, float* __restrict__ Dinv,
-    float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk) {
+    float* __restrict__ udiag, int32_t* __restrict__ info, int64_t C, int a, int nblk,
+    float* __restrict__ Lout) {
+    // U/udiag may be null (factor-only call); Lout, when given, receives D (the diagonal block
+    // of the lower factor) in the lower triangle of its tile.
     extern __shared__ __attribute__((aligned(16))) float smem[];   // 2 * NB * LDP floats (135 KB)
     float (*Dm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem);
     float (*Zm)[LDP] = reinterpret_cast<float (*)[LDP]>(smem + NB * LDP);
@@ -321,12 +324,21 @@ __global__ __launch_bounds__(256) void diag_block_kernel(
         const int k = e >> 5, m4 = (e & 31) * 4;
         *reinterpret_cast<float4*>(Di + k * NB + m4) = *reinterpret_cast<const float4*>(&Zm[k][m4]);
     }
-    float* __restrict__ Ub = U + b * C * C;
-    for (int e = tid; e < NB * NB; e += 256) {
-        const int m = e >> 7, k = e & (NB - 1);   // U0[a-block row m, column k] = Z[k, m]
-        if (m < n && k < n) Ub[(m0 + m) * C + m0 + k] = Zm[k][m];
+    if (U != nullptr) {
+        float* __restrict__ Ub = U + b * C * C;
+        for (int e = tid; e < NB * NB; e += 256) {
+            const int m = e >> 7, k = e & (NB - 1);   // U0[a-block row m, column k] = Z[k, m]
+            if (m < n && k < n) Ub[(m0 + m) * C + m0 + k] = Zm[k][m];
+        }
+        if (tid < n) udiag[b * C + m0 + tid] = Zm[tid][tid];
     }
-    if (tid < n) udiag[b * C + m0 + tid] = Zm[tid][tid];
+    if (Lout != nullptr) {
+        float* __restrict__ Lb = Lout + b * C * C;
+        for (int e = tid; e < NB * NB; e += 256) {
+            const int r = e >> 7, c = e & (NB - 1);
+            if (r < n && c <= r) Lb[(m0 + r) * C + m0 + c] = Dm[r][c];
+        }
+    }
     if (tid == 0 && s_fail != 0 && info[b] == 0) info[b] = (int32_t)(m0 + s_fail);
 }
 
@@ -361,16 +373,12 @@ extern "C" int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C) {
     return batch * nblk * NB * NB * (int64_t)sizeof(float) + forge::split_gemm_workspace_bytes(batch, C);
 }
 
-extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
-                                            int32_t* info, int64_t batch, int64_t C,
-                                            int normalise, void* ws, int64_t ws_bytes,
-                                            forge_stream_t stream) {
-    FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1 << 30), "bad shape batch=%lld C=%lld",
-                  (long long)batch, (long long)C);
-    if (batch == 0) return FORGE_OK;
-    FORGE_REQUIRE(H && U && udiag && info && ws, "null pointer");
-    FORGE_REQUIRE(ws_bytes >= forge_chol_workspace_bytes(batch, C), "workspace too small");
-    hipStream_t st = (hipStream_t)stream;
+namespace {
+
+// U0^T-route factorisation (factor_only = false) or only its first phase: H = L2^T L2 with L2
+// lower, left in the lower triangle of H (factor_only = true; U and udiag are not touched).
+int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info, int64_t batch,
+             int64_t C, int normalise, bool factor_only, void* ws, int64_t ws_bytes, hipStream_t st) {
     const int nblk = (int)forge::ceil_div(C, NB);
     float* Dinv = (float*)ws;
     const int64_t dinv_bytes = batch * nblk * NB * NB * (int64_t)sizeof(float);
@@ -400,17 +408,20 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
             g1a.xs = g1a.as = g1a.bs = C * C;
             g1a.m0 = m0; g1a.m1 = m1; g1a.n0 = 0; g1a.n1 = m1; g1a.k0 = m1; g1a.k1 = (int)C;
             g1a.negate_a = true; g1a.blocked_sum = true;
-            g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
-            g2a.xs = g2a.as = g2a.bs = C * C;
-            g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
-            g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
+            if (!factor_only) {
+                g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
+                g2a.xs = g2a.as = g2a.bs = C * C;
+                g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
+                g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
+            }
             if (int e = forge::launch_chain_gemm_pair(g1a, g2a, batch, st, split_ws, split_ws_bytes)) return e;
         }
         {
             forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,
                                        forge::WORK_FLOPS);
             diag_block_kernel<<<dim3((unsigned)batch), dim3(256), kDiagLds, st>>>(
-                H, U, Dinv, udiag, info, C, a, nblk);
+                H, factor_only ? nullptr : U, Dinv, factor_only ? nullptr : udiag, info, C, a, nblk,
+                factor_only ? H : nullptr);
             FORGE_LAUNCH_CHECK();
         }
         // Dinv blocks addressed with global (k, m) indices: shift the base so that
@@ -425,7 +436,7 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
             g1c.m0 = m0; g1c.m1 = m1; g1c.n0 = 0; g1c.n1 = m0; g1c.k0 = m0; g1c.k1 = m1;
             g1c.init_zero = true;
         }
-        if (m1 < C) {
+        if (m1 < C && !factor_only) {
             g2b.X = U; g2b.Bm = U; g2b.ldx = g2b.ldb = C; g2b.xs = g2b.bs = C * C;
             g2b.At = Dinv + (int64_t)a * NB * NB - shift; g2b.lda = NB; g2b.as = (int64_t)nblk * NB * NB;
             g2b.m0 = m0; g2b.m1 = m1; g2b.n0 = m1; g2b.n1 = (int)C; g2b.k0 = m0; g2b.k1 = m1;
@@ -433,10 +444,93 @@ extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* 
         }
         if (int e = forge::launch_chain_gemm_pair(g1c, g2b, batch, st)) return e;
     }
+    if (factor_only) return FORGE_OK;
     forge::KernelTiming timing("chol_finish_rows", st,
                                ((normalise & 2) ? 4.0 : 6.0) * C * C * (double)batch, forge::WORK_BYTES);
     finish_rows_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), 0, st>>>(
         U, udiag, info, C, (normalise & 1) != 0, (normalise & 2) == 0);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+// U[t][k] = L[k][t] / L[k][k] for k > t (as a multiplication by the rounded reciprocal, the
+// way solver_babai.cu:133-141 forms its coefficients), 1 on the diagonal, 0 below; identity
+// where info says that the factorisation failed.  FLIP: L is given as an UPPER factor A with
+// both index orders reversed, L[k][t] = A[C-1-k][C-1-t].  32x32 tiles through LDS so that
+// both sides are accessed along rows.
+template <bool FLIP>
+__global__ __launch_bounds__(256) void unit_upper_from_lower_kernel(
+    const float* __restrict__ L, const int32_t* __restrict__ info, float* __restrict__ U, int64_t C) {
+    __shared__ float tile[32][33];
+    const int64_t b = blockIdx.z;
+    const float* __restrict__ Lb = L + b * C * C;
+    float* __restrict__ Ub = U + b * C * C;
+    const int64_t t0 = (int64_t)blockIdx.y * 32, k0 = (int64_t)blockIdx.x * 32;   // U tile rows t, columns k
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;                      // 32 x 8
+    const bool failed = info != nullptr && info[b] != 0;
+    if (!failed && k0 + 31 >= t0) {
+        // L rows k0.., columns t0..: tile[kk][tt] = L[k0 + kk][t0 + tt] * rcp(L[k0+kk][k0+kk])
+        for (int kk = ty; kk < 32; kk += 8) {
+            const int64_t k = k0 + kk, t = t0 + tx;
+            float v = 0.0f;
+            if (k < C && t < C) {
+                const float a = FLIP ? Lb[(C - 1 - k) * C + (C - 1 - t)] : Lb[k * C + t];
+                const float d = FLIP ? Lb[(C - 1 - k) * (C + 1)] : Lb[k * (C + 1)];
+                v = a * (1.0f / d);
+            }
+            tile[kk][tx] = v;
+        }
+    }
+    __syncthreads();
+    for (int tt = ty; tt < 32; tt += 8) {
+        const int64_t t = t0 + tt, k = k0 + tx;
+        if (t < C && k < C) {
+            float v = (k == t) ? 1.0f : 0.0f;
+            if (!failed && k > t) v = tile[tx][tt];
+            Ub[t * C + k] = v;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
+                                            int32_t* info, int64_t batch, int64_t C,
+                                            int normalise, void* ws, int64_t ws_bytes,
+                                            forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1 << 30), "bad shape batch=%lld C=%lld",
+                  (long long)batch, (long long)C);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(H && U && udiag && info && ws, "null pointer");
+    FORGE_REQUIRE(ws_bytes >= forge_chol_workspace_bytes(batch, C), "workspace too small");
+    return chol_run(H, damp, U, udiag, info, batch, C, normalise, false, ws, ws_bytes, (hipStream_t)stream);
+}
+
+extern "C" int forge_chol_reverse_lower_batched(float* H, const float* damp, int32_t* info,
+                                                int64_t batch, int64_t C, void* ws, int64_t ws_bytes,
+                                                forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1 << 30), "bad shape batch=%lld C=%lld",
+                  (long long)batch, (long long)C);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(H && info && ws, "null pointer");
+    FORGE_REQUIRE(ws_bytes >= forge_chol_workspace_bytes(batch, C), "workspace too small");
+    return chol_run(H, damp, nullptr, nullptr, info, batch, C, 0, true, ws, ws_bytes, (hipStream_t)stream);
+}
+
+extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U,
+                                           int64_t batch, int64_t C, int flipped_upper,
+                                           forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1 << 30), "bad shape batch=%lld C=%lld",
+                  (long long)batch, (long long)C);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(L && U && L != U, "null or aliased pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned nt = (unsigned)forge::ceil_div(C, 32);
+    forge::KernelTiming timing("unit_upper_from_lower", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
+    if (flipped_upper)
+        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C);
+    else
+        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

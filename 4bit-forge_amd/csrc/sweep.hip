@@ -415,3 +415,85 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
     }
     return FORGE_OK;
 }
+
+// ------------------------------------------------------------------ Babai (nearest plane)
+// solver_babai.cu:123-322 walks the columns from the last to the first and, after
+// quantising column t, removes err_t * A[i,t] / A[i,i] from every earlier column i, A being
+// the upper Cholesky factor of H.  With both index orders reversed (t' = C-1-t) this is the
+// forward sweep above with the unit upper matrix U'[t',k'] = A[C-1-k', C-1-t'] / A[C-1-k', C-1-k']:
+// same quantiser, same fused multiply-adds, one chain per element in the same order.  So the
+// operator is a few index-reversing copies around gptq_sweep_batched.
+namespace {
+
+template <typename T>
+__global__ void reverse_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, int64_t C, int64_t R) {
+    const int64_t c = blockIdx.y;
+    for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < R; r += (int64_t)gridDim.x * blockDim.x)
+        dst[c * R + r] = src[(C - 1 - c) * R + r];
+}
+
+// scales/qzeros [R*G] (index r*G + g) -> [G, R]; g_idx reversed and clamped to G-1
+// (solver_babai.cu:196-197)
+__global__ void babai_meta_kernel(const float* __restrict__ scales, const float* __restrict__ qzeros,
+                                  const int32_t* __restrict__ g_idx, float* __restrict__ sT,
+                                  float* __restrict__ zT, int32_t* __restrict__ g_rev, int64_t C,
+                                  int64_t R, int64_t G, int64_t group_size) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < R * G) {
+        const int64_t g = i / R, r = i - g * R;
+        sT[i] = scales[r * G + g];
+        zT[i] = qzeros[r * G + g];
+    }
+    if (i < C) {
+        const int64_t row = C - 1 - i;
+        int64_t g = g_idx ? (int64_t)g_idx[row] : row / group_size;
+        if (g >= G) g = G - 1;
+        if (g < 0) g = 0;
+        g_rev[i] = (int32_t)g;
+    }
+}
+
+int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+
+extern "C" int64_t forge_babai_workspace_bytes(int64_t C, int64_t R, int64_t G) {
+    if (C <= 0 || R <= 0 || G <= 0) return 0;
+    return align256(C * C * 4) + align256(C * R * 4) + 2 * align256(G * R * 4) + align256(C * 4) +
+           align256(C * R);
+}
+
+extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U,
+                                           int64_t batch, int64_t C, int flipped_upper,
+                                           forge_stream_t stream);
+
+extern "C" int forge_babai_solver(const float* W, const float* A, const float* scales,
+                                  const float* qzeros, const int32_t* g_idx, int64_t group_size,
+                                  int bits, int64_t C, int64_t R, int64_t G, uint8_t* qweight,
+                                  void* ws, int64_t ws_bytes, forge_stream_t stream) {
+    if (int e = check_sweep_shape(C, R, bits)) return e;
+    FORGE_REQUIRE(G >= 1 && group_size >= 1, "bad G=%lld group_size=%lld", (long long)G, (long long)group_size);
+    FORGE_REQUIRE(W && A && scales && qzeros && qweight && ws, "null pointer");
+    FORGE_REQUIRE(ws_bytes >= forge_babai_workspace_bytes(C, R, G), "workspace too small");
+    hipStream_t st = (hipStream_t)stream;
+    char* p = (char*)ws;
+    float* Ur = (float*)p; p += align256(C * C * 4);
+    float* Xr = (float*)p; p += align256(C * R * 4);
+    float* sT = (float*)p; p += align256(G * R * 4);
+    float* zT = (float*)p; p += align256(G * R * 4);
+    int32_t* g_rev = (int32_t*)p; p += align256(C * 4);
+    uint8_t* qr = (uint8_t*)p;
+    if (int e = forge_unit_upper_from_lower(A, nullptr, Ur, 1, C, 1, stream)) return e;
+    const unsigned gx = (unsigned)forge::ceil_div(R, 256);
+    reverse_rows_kernel<float><<<dim3(gx, (unsigned)C), dim3(256), 0, st>>>(W, Xr, C, R);
+    FORGE_LAUNCH_CHECK();
+    const int64_t nmeta = R * G > C ? R * G : C;
+    babai_meta_kernel<<<dim3((unsigned)forge::ceil_div(nmeta, 256)), dim3(256), 0, st>>>(
+        scales, qzeros, g_idx, sT, zT, g_rev, C, R, G, group_size);
+    FORGE_LAUNCH_CHECK();
+    if (int e = forge_gptq_sweep_batched(Xr, Ur, sT, zT, g_rev, qr, nullptr, nullptr, 1, C, R, G, bits, 0, stream))
+        return e;
+    reverse_rows_kernel<uint8_t><<<dim3(gx, (unsigned)C), dim3(256), 0, st>>>(qr, qweight, C, R);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}

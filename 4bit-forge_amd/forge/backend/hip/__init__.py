@@ -51,6 +51,10 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
         "forge_chol_workspace_bytes": ([i64, i64], i64),
+        "forge_chol_reverse_lower_batched": ([vp, vp, vp, i64, i64, vp, i64, vp], i32),
+        "forge_unit_upper_from_lower": ([vp, vp, vp, i64, i64, i32, vp], i32),
+        "forge_babai_solver": ([vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp, vp, i64, vp], i32),
+        "forge_babai_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_permute": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
         "forge_weight_to_solver_order": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
@@ -76,6 +80,8 @@ EXPORTED_SYMBOLS = (
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
     "forge_dequantize_groups", "forge_gather_scaled_rows",
+    "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
+    "forge_babai_workspace_bytes",
 )
 
 
@@ -284,6 +290,57 @@ class _HipKernels:
                 _ptr(H), _ptr(damp), _ptr(U), _ptr(udiag), _ptr(info), B, C,
                 int(bool(normalise)) | (2 if upper_only else 0), _ptr(ws), nbytes, _stream()))
         return U, udiag, info
+
+    def chol_reverse_lower_batched(self, H, damp):
+        """H [B,C,C] f32: H + damp I = L^T L with L lower, left in H's lower triangle (the
+        strict upper triangle is destroyed).  Returns (H, info [B])."""
+        _need_cuda(H, damp)
+        B, C, _ = H.shape
+        assert H.is_contiguous() and H.dtype == torch.float32
+        assert damp is None or (damp.dtype == torch.float32 and damp.numel() == B)
+        info = torch.empty(B, dtype=torch.int32, device=H.device)
+        nbytes = int(self._lib.forge_chol_workspace_bytes(B, C))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=H.device)
+        with torch.cuda.device(H.device):
+            self._check(self._lib.forge_chol_reverse_lower_batched(
+                _ptr(H), _ptr(damp), _ptr(info), B, C, _ptr(ws), nbytes, _stream()))
+        return H, info
+
+    def unit_upper_from_lower(self, L, info=None, flipped_upper=False):
+        """U [B,C,C]: U[t,k] = L[k,t] / L[k,k] (k > t), unit diagonal, zero below; identity
+        where info != 0.  flipped_upper: L is the upper factor A with both orders reversed."""
+        _need_cuda(L, info)
+        B, C, _ = L.shape
+        assert L.is_contiguous() and L.dtype == torch.float32
+        U = torch.empty_like(L)
+        with torch.cuda.device(L.device):
+            self._check(self._lib.forge_unit_upper_from_lower(
+                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)), _stream()))
+        return U
+
+    def babai_solver(self, W, A, scales, qzeros, group_size, bits, block_size, g_idx, G):
+        """Reference operator (kernels.cpp:46-56): W [C,R] f32, A [C,C] upper factor,
+        scales/qzeros [R*G], g_idx [C] int32 -> qweight [C,R] u8.  block_size is accepted for
+        signature compatibility; the result does not depend on it."""
+        _need_cuda(W, A, scales, qzeros, g_idx)
+        C, R = W.shape
+        W = W.to(torch.float32).contiguous()
+        A = A.to(torch.float32).contiguous()
+        scales, qzeros = scales.contiguous(), qzeros.contiguous()
+        g_idx = None if g_idx is None else g_idx.to(torch.int32).contiguous()
+        gs = min(int(group_size), C)
+        if gs <= 0 or gs % 32 != 0:
+            raise RuntimeError("group_size must be a positive multiple of 32 (effective group_size)")
+        if (C + gs - 1) // gs != int(G):
+            raise RuntimeError(f"qmeta G mismatch: got G={G} expected ceil(C/group_size)={(C + gs - 1) // gs}")
+        q = torch.empty((C, R), dtype=torch.uint8, device=W.device)
+        nbytes = int(self._lib.forge_babai_workspace_bytes(C, R, int(G)))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=W.device)
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_babai_solver(
+                _ptr(W), _ptr(A), _ptr(scales), _ptr(qzeros), _ptr(g_idx), gs, int(bits), C, R,
+                int(G), _ptr(q), _ptr(ws), nbytes, _stream()))
+        return q
 
     def hessian_permute(self, H, perm, dead, rel_damp):
         _need_cuda(H, perm, dead)

@@ -41,9 +41,8 @@ class GPTQ(object):
     def __init__(self, layer, bits: int = 4, group_size: int = 128, symmetric: bool = False,
                  quantization_scale: str = "mse", quantization_order: str = "activation",
                  rel_damp: float = 1e-2, algorithm: str = "gptq", owner=None, device=None):
-        if algorithm not in ("gptq", "sparsegptq"):
-            raise NotImplementedError(f"algorithm={algorithm!r}: only 'gptq' and 'sparsegptq' "
-                                      "run on the HIP backend")
+        if algorithm not in ("gptq", "sparsegptq", "babai"):
+            raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         self.layer = layer
         self.device = torch.device(device) if device is not None else layer.weight.device
         if self.device.type != "cuda":
@@ -134,7 +133,8 @@ class GPTQ(object):
         o.pruned_ids = dead
         if o.quantization_order == "activation":
             diag = torch.where(dead, torch.ones_like(torch.diag(o.H)), torch.diag(o.H))
-            o.perm = torch.argsort(diag, descending=True)
+            # Babai walks the columns back to front: ascending order (forge/gptq.py:107-108)
+            o.perm = torch.argsort(diag, descending=o.algorithm != "babai")
         else:
             o.perm = torch.arange(C, device=o.device)
         o.perm_inv = torch.argsort(o.perm)
@@ -175,6 +175,14 @@ class GPTQ(object):
             H[:, zero_cols] = 0
             H[zero_cols, zero_cols] = 1.0
         H.diagonal().add_(float(self.rel_damp) * torch.diag(H).mean())
+        if self.algorithm == "babai":
+            # The reference factors H = A^T A (A upper, forge/gptq.py:157-158) and sweeps from
+            # the last column to the first.  With both index orders reversed that is a forward
+            # sweep whose unit upper matrix comes from the LOWER factor of the reversed H.
+            L, info = kernels.chol_reverse_lower_batched(H.flip(0, 1).contiguous().view(1, C, C), None)
+            if int(info.item()) > 0:
+                self.issue_non_invertible = True
+            return kernels.unit_upper_from_lower(L, info)[0]
         U, _, info = kernels.chol_inv_upper_batched(H.clone().view(1, C, C), None,
                                                     normalise=self.algorithm == "gptq")
         if int(info.item()) > 0:
@@ -189,6 +197,16 @@ class GPTQ(object):
         R, C = self.W.shape
         G, gs = self.G, self.group_size
         W = self.W if self.W.dtype in (torch.float32, torch.bfloat16) else self.W.float()
+        if self.algorithm == "babai":
+            # solver order = the reference's permuted order reversed (see _h_factor)
+            perm_r = self.perm.flip(0)
+            perm_r_inv = torch.argsort(perm_r)
+            X = kernels.weight_to_solver_order(W.view(1, R, C), perm_r_inv.view(1, C))
+            g_idx = (perm_r // gs).to(torch.int32).view(1, C)
+            sT = scales.view(R, G).t().contiguous().view(1, G, R)
+            zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
+            q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
+            return kernels.codes_to_layer_order(q, perm_r_inv.view(1, C))[0], scales, qzeros
         X = kernels.weight_to_solver_order(W.view(1, R, C), self.perm_inv.view(1, C))
         if self.algorithm == "sparsegptq":
             s_e = scales.view(R, G).repeat_interleave(gs, dim=1)[:, :C].t()[self.perm].contiguous()

@@ -104,6 +104,21 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
                              int64_t R, int64_t G, int bits, int sparse14,
                              forge_stream_t stream);
 
+/* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
+ * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private
+ * copy with the dequantised values), A [C, C] f32 upper Cholesky factor of H (H = A^T A),
+ * scales/qzeros [R*G] f32 (index r*G + g), g_idx [C] int32 group of solver column c (null:
+ * c / group_size), qweight [C, R] u8.  Columns are quantised from the last to the first with
+ * the reference's quantiser and fused multiply-adds; every element receives its updates as
+ * one fma chain in that order (the reference applies those of other 32-column blocks
+ * through an SGEMM whose summation order is not defined).  The block_size argument of the
+ * reference has no effect on such a chain and is not taken.  ws: forge_babai_workspace_bytes. */
+int forge_babai_solver(const float* W, const float* A, const float* scales, const float* qzeros,
+                       const int32_t* g_idx, int64_t group_size, int bits, int64_t C, int64_t R,
+                       int64_t G, uint8_t* qweight, void* ws, int64_t ws_bytes,
+                       forge_stream_t stream);
+int64_t forge_babai_workspace_bytes(int64_t C, int64_t R, int64_t G);
+
 /* ------------------------------------------------------------------ Hessian */
 
 /* Grouped ragged rank-k update, the batched form of GPTQ.update (gptq.py:61-80):
@@ -141,6 +156,24 @@ int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* u
                                  int32_t* info, int64_t batch, int64_t C, int normalise,
                                  void* ws, int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C);
+
+/* The factor that the Babai branch of GPTQ._h_factor needs (gptq.py:157-158,
+ * torch.linalg.cholesky_ex(H, upper=True)), in the index order of the sweep that consumes it:
+ * for each b, A = H[b] + damp[b]*I is factored as A = L^T L with L LOWER triangular
+ * (elimination from the last row upwards), and L is left in the lower triangle of H[b]
+ * (the strict upper triangle of H[b] is destroyed).  Reversing both index orders of H gives
+ * the reference's upper factor: chol(H_ref, upper)[i][j] = L[C-1-i][C-1-j] for
+ * H[i][j] = H_ref[C-1-i][C-1-j].  info and ws as for forge_chol_inv_upper_batched. */
+int forge_chol_reverse_lower_batched(float* H, const float* damp, int32_t* info, int64_t batch,
+                                     int64_t C, void* ws, int64_t ws_bytes, forge_stream_t stream);
+
+/* U[b][t][k] = L[b][k][t] * (1 / L[b][k][k]) for k > t, 1 on the diagonal, 0 below it: the
+ * coefficients alpha = A[i][t] * invD[i] of solver_babai.cu:133-141,232-236 arranged as the unit
+ * upper matrix of a forward sweep.  U[b] = I where info[b] != 0 (info may be null).
+ * flipped_upper != 0: L is given as the reference's upper factor A instead,
+ * L[k][t] = A[C-1-k][C-1-t].  L and U must not overlap. */
+int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U, int64_t batch,
+                                int64_t C, int flipped_upper, forge_stream_t stream);
 
 /* Fused gather for GPTQ._prep/_h_factor (gptq.py:100-117,145-154): for each b builds
  * Hp[b][i][j] = H[b][perm[i]][perm[j]] with rows/cols flagged in dead[b] (u8, in PERMUTED

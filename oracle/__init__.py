@@ -62,6 +62,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_gptq_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, i32, i64]
         L.oracle_sparsegptq14_solver.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32]
         L.oracle_gptq_inblock.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i64, vp, vp]
+        L.oracle_babai_solver.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp, i32, i64]
+        L.oracle_babai_solver.restype = None
         L.oracle_pack_sparsegptq14.argtypes = [vp, vp, vp, vp, i64, i64]
         L.oracle_pack_sparsegptq14.restype = None
         for f in (L.oracle_build_group_meta, L.oracle_mse_scale_groups, L.oracle_gptq_solver,
@@ -130,6 +132,32 @@ def gptq_solver(W, U, scales, qzeros, bits, trail_mode: int = TRAIL_CHAIN, block
                                  qzeros.data_ptr(), int(bits), C, R, q.data_ptr(),
                                  int(trail_mode), int(block))
     gptq_solver.last_W = W
+    return q
+
+
+def babai_solver(W, A, scales, qzeros, group_size, bits, block_size, g_idx, G,
+                 trail_mode: int = TRAIL_CHAIN):
+    """kernels.cpp:46-56 -> solver_babai.cu:217-322.  W [C,R] f32 (the contiguous copy
+    receives the dequantised weights), A [C,C] upper factor of H, scales/qzeros [R*G],
+    g_idx [C] int32.  Returns qweight [C,R] u8.  The host checks are the reference's."""
+    W = W.contiguous() if W.dtype == torch.float32 else W.to(torch.float32).contiguous()
+    A = _f32c(A); scales = _f32c(scales); qzeros = _f32c(qzeros)
+    C, R = W.shape
+    gs = min(int(group_size), C)
+    if gs <= 0 or gs % 32 != 0:
+        raise RuntimeError("group_size must be multiple of 32 (effective group_size)")
+    if (C + gs - 1) // gs != int(G):
+        raise RuntimeError("qmeta G mismatch")
+    block = int(block_size)
+    if block <= 0 or block > 32:
+        block = 32
+    block = min(block, C)
+    gi = None if g_idx is None else g_idx.to(torch.int32).contiguous()
+    q = torch.zeros((C, R), dtype=torch.uint8)
+    lib().oracle_babai_solver(W.data_ptr(), A.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+                              None if gi is None else gi.data_ptr(), gs, int(bits), C, R, int(G),
+                              q.data_ptr(), int(trail_mode), block)
+    babai_solver.last_W = W
     return q
 
 
@@ -316,7 +344,11 @@ class GPTQ:
         idx = torch.arange(C)
         H[idx, idx] += damp
         if self.algorithm == "babai":
-            raise NotImplementedError("babai is outside the restated path")
+            A, info = torch.linalg.cholesky_ex(H, upper=True)      # gptq.py:157-158: H = A^T A
+            if int(info.item()) > 0:
+                self.issue_non_invertible = True
+                A = torch.eye(C, dtype=torch.float32)
+            return A
         L, info = torch.linalg.cholesky_ex(H, upper=False)
         try:
             Hinv = torch.cholesky_inverse(L, upper=False)
@@ -346,6 +378,12 @@ class GPTQ:
         U = self._h_factor()
         W = self.W.clone().transpose(-2, -1)[self.perm]
         C, R = W.shape
+        if self.algorithm == "babai":
+            # gptq.py:231-246
+            g_idx = (self.perm // self.group_size).to(torch.int32)
+            q = babai_solver(W.to(torch.float32), U, scales, qzeros, self.group_size, self.bits,
+                             self.group_size // 4, g_idx, self.G, trail_mode=self.trail_mode)
+            return q[self.perm_inv].transpose(-2, -1).contiguous(), scales, qzeros
         s_e, z_e = self._expand(scales, C, R), self._expand(qzeros, C, R)
         if self.algorithm == "sparsegptq":
             q, M = sparsegptq14_solver(W.to(torch.float32), U.contiguous(), s_e, z_e, self.bits,

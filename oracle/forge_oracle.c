@@ -16,6 +16,7 @@
  *   oracle_gptq_solver           forge/backend/cuda/solver.cu:9-154
  *   oracle_sparsegptq14_solver   forge/backend/cuda/solver_sparsegptq14.cu:12-200
  *   oracle_pack_sparsegptq14     forge/backend/cuda/bitpacking_sparsegptq14.cu:58-107
+ *   oracle_babai_solver          forge/backend/cuda/solver_babai.cu:123-322
  *
  * Where the reference leaves fp32 bits undefined, the oracle fixes them as follows
  * (each choice is within the reference's own numerical freedom):
@@ -271,6 +272,72 @@ void oracle_sparsegptq14_solver(float* W, float* U, const float* scales, const f
 
 /* bitpacking_sparsegptq14.cu:58-107.  q_rc [R,C] codes, M [G32,R], scales [G32,R] ->
  * out [G2,R,2] u64 = bf16(scale) << 48 | idx16 << 32 | qw32. */
+/* solver_babai.cu:123-322.  W [C,R] fp32 (updated in place to the dequantised weights),
+ * A [C,C] upper Cholesky factor of H (H = A^T A), scales/qzeros [R*G] (index r*G + g),
+ * g_idx [C] (group of solver column; NULL: c / group_size), B the block width (reference:
+ * at most 32).  Blocks and the columns of a block are walked from the last to the first;
+ * after column t every earlier column i receives x_i = fmaf(-A[i,t] * (1/A[i,i]), err_t, x_i).
+ * For the rows above a block the reference does this with an SGEMM (`addmm_`, :313-316)
+ * whose summation order is not defined: TRAIL_CHAIN continues the in-block chain (t
+ * descending), TRAIL_GEMM accumulates the block's sum from zero (k ascending) and subtracts. */
+void oracle_babai_solver(float* W, const float* A, const float* scales, const float* qzeros,
+                         const int32_t* g_idx, int64_t group_size, int bits, int64_t C, int64_t R,
+                         int64_t G, uint8_t* qweight, int trail_mode, int64_t B) {
+    const int maxq_i = (1 << bits) - 1;
+    float* invD = (float*)malloc((size_t)C * sizeof(float));
+    for (int64_t i = 0; i < C; ++i) invD[i] = 1.0f / A[i * C + i];
+    float* E = (float*)malloc((size_t)(B * R) * sizeof(float));
+    for (int64_t block_end = C; block_end > 0; block_end -= B) {
+        const int64_t start = block_end - B > 0 ? block_end - B : 0;
+        const int64_t Bc = block_end - start;
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < R; ++r) {
+            float x[256];
+            for (int64_t i = 0; i < Bc; ++i) x[i] = W[(start + i) * R + r];
+            for (int64_t t = Bc - 1; t >= 0; --t) {
+                const int64_t row = start + t;
+                int64_t g = g_idx ? (int64_t)g_idx[row] : row / group_size;
+                if (g >= G) g = G - 1;
+                const float s = scales[r * G + g], q0 = qzeros[r * G + g];
+                const float inv_s = 1.0f / (s + ORACLE_EPS);
+                float err, deq; uint8_t qb;
+                quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+                qweight[row * R + r] = qb;
+                W[row * R + r] = deq;
+                E[t * R + r] = err;
+                for (int64_t i = 0; i < t; ++i) {
+                    const float alpha = A[(start + i) * C + row] * invD[start + i];
+                    x[i] = fmaf(-alpha, err, x[i]);
+                }
+            }
+        }
+        if (start > 0) {
+#pragma omp parallel for schedule(static)
+            for (int64_t i = 0; i < start; ++i) {
+                float* wi = W + i * R;
+                if (trail_mode == TRAIL_CHAIN) {
+                    for (int64_t t = Bc - 1; t >= 0; --t) {
+                        const float alpha = A[i * C + start + t] * invD[i];
+                        const float* e = E + t * R;
+                        for (int64_t r = 0; r < R; ++r) wi[r] = fmaf(-alpha, e[r], wi[r]);
+                    }
+                } else {
+                    float* acc = (float*)calloc((size_t)R, sizeof(float));
+                    for (int64_t t = 0; t < Bc; ++t) {
+                        const float alpha = A[i * C + start + t] * invD[i];
+                        const float* e = E + t * R;
+                        for (int64_t r = 0; r < R; ++r) acc[r] = fmaf(alpha, e[r], acc[r]);
+                    }
+                    for (int64_t r = 0; r < R; ++r) wi[r] = wi[r] - acc[r];
+                    free(acc);
+                }
+            }
+        }
+    }
+    free(E);
+    free(invD);
+}
+
 static uint16_t bf16_rne_bits(float x) {
     uint32_t u; memcpy(&u, &x, 4);
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
