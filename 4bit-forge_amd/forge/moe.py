@@ -22,8 +22,12 @@ class ExpertGroupGPTQ:
     def __init__(self, weights: Sequence[torch.Tensor], bits: int = 4, group_size: int = 128,
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
-                 device=None):
-        """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C."""
+                 algorithm: str = "gptq", device=None):
+        """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
+        algorithm: "gptq" or "babai" (the 1:4 joint solve is offered per layer only)."""
+        if algorithm not in ("gptq", "babai"):
+            raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq' or 'babai'")
+        self.algorithm = algorithm
         self.device = torch.device(device) if device is not None else weights[0].device
         if self.device.type != "cuda":
             raise RuntimeError("ExpertGroupGPTQ runs on the GPU only; there is no CPU fallback")
@@ -102,15 +106,20 @@ class ExpertGroupGPTQ:
             H = self.H[e0:e1]
             diag = H.diagonal(dim1=1, dim2=2)
             dead = diag == 0                                             # [B, C]
+            babai = self.algorithm == "babai"
             if self.quantization_order == "activation":
+                # Babai walks back to front: ascending order (forge/gptq.py:107-108)
                 perm = torch.argsort(torch.where(dead, torch.ones_like(diag), diag), dim=1,
-                                     descending=True)
+                                     descending=not babai)
             else:
                 perm = torch.arange(C, device=dev).expand(B, C).contiguous()
+            dead_perm = torch.gather(dead, 1, perm)
+            if babai:
+                # the solve runs as a forward sweep over the reversed order (see forge/gptq.py)
+                perm = perm.flip(1).contiguous()
             perm_inv = torch.argsort(perm, dim=1)
             g_idx = (perm // gs).to(torch.int32).contiguous()
             dead_u8 = dead.to(torch.uint8).contiguous()
-            dead_perm = torch.gather(dead, 1, perm)
             # weights with pruned columns zeroed decide the (unpermuted-index) zero-column
             # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149).
             # A column can only be all zero if its first rows are: one look at 8 rows (fp8- or
@@ -136,6 +145,8 @@ class ExpertGroupGPTQ:
                 masks = [zero if m is None else m for m in masks]
                 shared = all(torch.stack([(masks[0] == m).all() for m in masks[1:]]).cpu().tolist()) \
                     if len(masks) > 1 else True
+                if babai:   # positions of the reference's order -> positions of the reversed one
+                    masks = [m.flip(1).contiguous() for m in masks]
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
             for job in jobs:
@@ -156,7 +167,12 @@ class ExpertGroupGPTQ:
                     Wsrc.record_stream(side)
                     del Wsrc
                 Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
-                U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
+                if babai:
+                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
+                    U = kernels.unit_upper_from_lower(L, info)
+                    del L
+                else:
+                    U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
                 failed.append((e0, info))
                 X = kernels.weight_to_solver_order(Wc, perm_inv, dead_u8)

@@ -103,3 +103,31 @@ def test_class_end_to_end_against_the_oracle(order):
     same = so == sg
     assert torch.equal(zo[same], zg[same])
     assert flip_rate(qo, qg) <= 5e-3
+
+
+def test_expert_group_babai_matches_per_expert_oracle():
+    """The batched front end with algorithm="babai": gate/up share Hessian and factor; one
+    expert never saw a token (H = I: plain round-to-nearest, exact)."""
+    from forge.moe import ExpertGroupGPTQ
+    g = torch.Generator().manual_seed(21)
+    E, R, C = 3, 96, 256
+    Wg = 0.02 * torch.randn(E, R, C, generator=g)
+    Wu = 0.02 * torch.randn(E, R, C, generator=g)
+    col = torch.linspace(0.5, 3.0, C)[torch.randperm(C, generator=g)]
+    xs = [torch.randn(n, C, generator=g) * col for n in (400, 0, 700)]
+    offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
+              quantization_order="activation", algorithm="babai")
+    grp = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, **kw)
+    grp.update(torch.cat(xs).to(DEV), offs)
+    (qg, sg, zg), (qu, su, zu) = grp.quantize(chunk=4)
+    for e in range(E):
+        for W, (q, s, z) in ((Wg[e], (qg, sg, zg)), (Wu[e], (qu, su, zu))):
+            o = oracle.GPTQ(linear(W), **kw)
+            o.update(xs[e])
+            qo, so, zo = o.quantize()
+            assert float((so != s[e].cpu()).float().mean()) <= 2e-3
+            if xs[e].shape[0] == 0:
+                assert torch.equal(qo, q[e].cpu())
+            else:
+                assert flip_rate(qo, q[e]) <= 5e-3
