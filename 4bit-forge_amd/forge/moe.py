@@ -24,9 +24,10 @@ class ExpertGroupGPTQ:
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
                  algorithm: str = "gptq", device=None):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
-        algorithm: "gptq" or "babai" (the 1:4 joint solve is offered per layer only)."""
-        if algorithm not in ("gptq", "babai"):
-            raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq' or 'babai'")
+        algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
+        keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai"."""
+        if algorithm not in ("gptq", "sparsegptq", "babai"):
+            raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         self.algorithm = algorithm
         self.device = torch.device(device) if device is not None else weights[0].device
         if self.device.type != "cuda":
@@ -78,7 +79,9 @@ class ExpertGroupGPTQ:
     @torch.no_grad()
     def quantize(self, chunk: int = 32, max_shrink: float = 0.2, n_grid: int = 100,
                  norm: float = 2.4):
-        """Returns one (qweight [E,R,C] u8, scales [E,R*G] f32, qzeros [E,R*G] f32) per stack."""
+        """Returns one (qweight [E,R,C] u8, scales [E,R*G] f32, qzeros [E,R*G] f32) per stack;
+        with algorithm="sparsegptq" a fourth element M [E, ceil(C/32), R] u32 (bit i of word w
+        <-> column 32 w + i of the SOLVER order, as the reference returns it)."""
         E, C, gs, dev = self.E, self.C, self.group_size, self.device
         G = (C + gs - 1) // gs
         mse = self.quantization_scale == "mse"
@@ -97,9 +100,12 @@ class ExpertGroupGPTQ:
         side = torch.cuda.Stream(device=dev)          # default priority
 
         sizes = [int(W.shape[1]) for W in self.W]
+        sparse = self.algorithm == "sparsegptq"
         outs = [[torch.empty((E, R, C), dtype=torch.uint8, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev),
-                 torch.empty((E, R * G), dtype=torch.float32, device=dev)] for R in sizes]
+                 torch.empty((E, R * G), dtype=torch.float32, device=dev)]
+                + ([torch.empty((E, (C + 31) // 32, R), dtype=torch.uint32, device=dev)] if sparse else [])
+                for R in sizes]
         for e0 in range(0, E, chunk):
             e1 = min(E, e0 + chunk)
             B = e1 - e0
@@ -171,6 +177,13 @@ class ExpertGroupGPTQ:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                     U = kernels.unit_upper_from_lower(L, info)
                     del L
+                elif sparse:
+                    # un-normalised factor, rows then scaled by the rounded reciprocal of the
+                    # diagonal as solver_sparsegptq14.cu:153-155 does
+                    U, udiag, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=False,
+                                                                   upper_only=True)
+                    uinv = (1.0 / udiag).contiguous()
+                    U.mul_(uinv.unsqueeze(-1))
                 else:
                     U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
@@ -179,7 +192,12 @@ class ExpertGroupGPTQ:
                 main.wait_stream(side)
                 for t in (scales, qzeros, sT, zT):
                     t.record_stream(main)
-                q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
+                M = None
+                if sparse:
+                    q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
+                                                      uinv=uinv)
+                else:
+                    q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
                 del X, U
                 q = kernels.codes_to_layer_order(q, perm_inv)
                 r0 = 0
@@ -188,6 +206,8 @@ class ExpertGroupGPTQ:
                     outs[i][0][e0:e1] = q[:, r0:r0 + Ri]
                     outs[i][1][e0:e1] = scales.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     outs[i][2][e0:e1] = qzeros.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
+                    if sparse:
+                        outs[i][3][e0:e1] = M[:, :, r0:r0 + Ri]
                     r0 += Ri
         for e0, info in failed:
             self.issue_non_invertible[e0:e0 + info.numel()] |= (info > 0).cpu()

@@ -229,6 +229,34 @@ def test_expert_group_dead_and_zero_columns(zero_weight_column):
                 assert torch.equal(qo[:, [37, 200]], q[e].cpu()[:, [37, 200]])
 
 
+def test_expert_group_sparse14_matches_per_expert_oracle():
+    """algorithm="sparsegptq" through the batched front end: codes, keep-masks (solver order)
+    and scales against oracle.GPTQ expert by expert; one kept weight in every group of four."""
+    from forge.moe import ExpertGroupGPTQ
+    g = torch.Generator().manual_seed(31)
+    E, R, C = 3, 64, 256
+    Wg = (0.02 * torch.randn(E, R, C, generator=g)).bfloat16()
+    Wu = (0.02 * torch.randn(E, R, C, generator=g)).bfloat16()
+    xs = [torch.randn(n, C, generator=g).bfloat16() for n in (500, 320, 640)]
+    offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
+              quantization_order="default", algorithm="sparsegptq")
+    grp = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, **kw)
+    grp.update(torch.cat(xs).to(DEV), offs)
+    (qg, sg, zg, Mg), (qu, su, zu, Mu) = grp.quantize(chunk=4)
+    for e in range(E):
+        for W, (q, s, z, M) in ((Wg[e], (qg, sg, zg, Mg)), (Wu[e], (qu, su, zu, Mu))):
+            o = oracle.GPTQ(linear(W), **kw)
+            o.update(xs[e])
+            qo, so, zo, Mo = o.quantize()
+            assert float((so != s[e].cpu()).float().mean()) <= 2e-3
+            bits_o = np.unpackbits(Mo.numpy().view(np.uint8), bitorder="little")
+            bits_g = np.unpackbits(M[e].cpu().numpy().view(np.uint8), bitorder="little")
+            assert bits_g.reshape(-1, 4).sum(1).tolist() == [1] * (bits_g.size // 4)
+            assert (bits_o != bits_g).mean() <= 1e-2
+            assert flip_rate(qo, q[e]) <= 1e-2
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _e2e(W, X, kw, tol_flips, gs=128):
     o, g, H = _run_pair(W, X, chunks=1, **kw)
