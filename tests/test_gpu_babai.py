@@ -32,6 +32,33 @@ def test_babai_solver_bit_exact(hip, C, R, gs, sym):
     assert torch.equal(qo, qg.cpu())
 
 
+def test_full_size_babai_properties(hip):
+    """Config-1 size (2048 x 2048).  An identity factor must give round-to-nearest bit for
+    bit; the back-to-front solve must equal the forward sweep of the index-reversed problem
+    (rows of the unit factor U'[t', k'] = A[k, t] / A[k, k] with k = C-1-k', t = C-1-t')
+    composed from the library's other entry points; and the oracle's chain must agree."""
+    C = R = 2048
+    gs, G = 128, 16
+    pr = random_problem(C=C, R=R, n=1024, seed=9)
+    A = _upper_factor(pr["H"])
+    Wt = pr["W"].t().contiguous()
+    s, z = pr["s"].to(DEV), pr["z"].to(DEV)
+    q_rtn = hip.babai_solver(Wt.to(DEV), torch.eye(C, device=DEV), s, z, gs, 4, 32, None, G)
+    se, ze = pr["se"].to(DEV), pr["ze"].to(DEV)
+    ref = torch.clamp(torch.round(torch.addcmul(ze.double(), Wt.to(DEV).double(),
+                                                (1.0 / (se + 1e-12)).double()).float()), 0, 15)
+    assert torch.equal(q_rtn.float(), ref)
+    q = hip.babai_solver(Wt.to(DEV), A.to(DEV), s, z, gs, 4, 32, None, G)
+    Ur = hip.unit_upper_from_lower(A.view(1, C, C).to(DEV), None, flipped_upper=True)
+    sT = pr["s"].view(R, G).t().contiguous().view(1, G, R).to(DEV)
+    zT = pr["z"].view(R, G).t().contiguous().view(1, G, R).to(DEV)
+    g_rev = (torch.arange(C - 1, -1, -1) // gs).int().view(1, C).to(DEV)
+    q_fwd = hip.gptq_sweep_batched(Wt.flip(0).contiguous().view(1, C, R).to(DEV), Ur, sT, zT, g_rev, 4)
+    assert torch.equal(q, q_fwd[0].flip(0))
+    qo = oracle.babai_solver(Wt.clone(), A, pr["s"], pr["z"], gs, 4, 32, None, G)
+    assert torch.equal(qo, q.cpu())
+
+
 def test_babai_solver_rejects_what_the_reference_rejects(hip):
     W = torch.zeros(64, 8, device=DEV)
     A = torch.eye(64, device=DEV)
