@@ -460,7 +460,8 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
 // both sides are accessed along rows.
 template <bool FLIP>
 __global__ __launch_bounds__(256) void unit_upper_from_lower_kernel(
-    const float* __restrict__ L, const int32_t* __restrict__ info, float* __restrict__ U, int64_t C) {
+    const float* __restrict__ L, const int32_t* __restrict__ info, float* __restrict__ U, int64_t C,
+    float sign) {
     __shared__ float tile[32][33];
     const int64_t b = blockIdx.z;
     const float* __restrict__ Lb = L + b * C * C;
@@ -476,7 +477,7 @@ __global__ __launch_bounds__(256) void unit_upper_from_lower_kernel(
             if (k < C && t < C) {
                 const float a = FLIP ? Lb[(C - 1 - k) * C + (C - 1 - t)] : Lb[k * C + t];
                 const float d = FLIP ? Lb[(C - 1 - k) * (C + 1)] : Lb[k * (C + 1)];
-                v = a * (1.0f / d);
+                v = sign * (a * (1.0f / d));
             }
             tile[kk][tx] = v;
         }
@@ -527,10 +528,11 @@ extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, 
     hipStream_t st = (hipStream_t)stream;
     const unsigned nt = (unsigned)forge::ceil_div(C, 32);
     forge::KernelTiming timing("unit_upper_from_lower", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
-    if (flipped_upper)
-        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C);
+    const float sign = (flipped_upper & 2) ? -1.0f : 1.0f;
+    if (flipped_upper & 1)
+        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign);
     else
-        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C);
+        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

@@ -40,6 +40,7 @@ struct SweepArgs {
     uint8_t* q;            // [C,R] per matrix
     uint32_t* M;           // [ceil(C/32),R] per matrix (sparse only)
     const float* uinv;     // [C] per matrix (sparse only)
+    const float* W0;       // [C,R] per matrix: the untouched weights (displacement form only)
     int64_t C, R, G;
     int64_t c0;            // first column of this block
     int bw;                // columns in this block (<= BW)
@@ -87,7 +88,15 @@ __device__ __forceinline__ float dpp_source(float u) {
 // broadcast ds_read.  TAIL is the guarded, slower variant (U straight from global memory)
 // for blocks that are not a whole number of 32-column sub-blocks or whose U rows are not
 // 16-byte aligned.
-template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL>
+//
+// DISP is the displacement form: what a column hands on is d = w0 - deq (its ORIGINAL
+// weight minus what it was rounded to) instead of err = x - deq, and `U` holds
+// V[t,k] = -M[t,k] / M[k,k] (k > t) of the factor H = M M^T (M upper) instead of the
+// row-normalised factor of the inverse.  With N = I - strict(V) the inverse of the unit
+// matrix the error form uses, err = d N, so the value a column has when it is reached,
+// w0_k + sum_{t<k} d_t N[t,k], is the same number in exact arithmetic; only fp32 rounding
+// differs.  The quantiser, the fused multiply-adds and their order are those of the error form.
+template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false>
 __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
     constexpr int RING = FORGE_SWEEP_RING;   // LDS read-ahead: RING-1 steps of 16 columns
@@ -108,6 +117,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     const float* __restrict__ uinv = SPARSE ? a.uinv + b * C : nullptr;
     uint32_t* __restrict__ Mw = SPARSE ? a.M + b * ((C + 31) / 32) * R + r : nullptr;
     uint8_t* __restrict__ q = a.q + b * C * R + r;
+    const float* __restrict__ W0 = DISP ? a.W0 + b * C * R + r : nullptr;
     const int bw = a.bw;
     const int nsub = (bw + SB - 1) / SB;
     const float maxq = (float)a.maxq;
@@ -175,11 +185,12 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             }
             float e, deq, qf;
             quantize_scalar(x[t], s, q0, maxq, qf, deq, e);
+            if constexpr (DISP) e = err[t] - deq;   // err[t] holds the original weight here
             if constexpr (SPARSE) {
                 // pruned column: code 0, weight 0, the whole value becomes the error
                 qf = keep ? qf : 0.0f;
                 deq = keep ? deq : 0.0f;
-                e = keep ? e : x[t];
+                e = keep ? e : (DISP ? err[t] : x[t]);
             }
             err[t] = e;
             q[c * R] = (uint8_t)qf;
@@ -192,6 +203,10 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
         };
 
         if constexpr (!TAIL) {
+            if constexpr (DISP) {
+#pragma unroll
+                for (int t = 0; t < SB; ++t) err[t] = W0[(cs + t) * R];
+            }
             // fetch the next sub-block's panel (rows cs+32.., columns cs+32..) into registers
             const bool more = sb + 1 < nsub;
             float4 nxt[(NSB - 1) * (256 / NT)];
@@ -273,6 +288,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             for (int t = 0; t < SB; ++t) {
                 err[t] = 0.0f;
                 if (t < rem) {
+                    if constexpr (DISP) err[t] = W0[(cs + t) * R];
                     float s_t, q0_t;
                     if constexpr (PER_ELEM) {
                         s_t = sc[(cs + t) * R];
@@ -303,7 +319,7 @@ __global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ 
     if (threadIdx.x == 0) uinv[i] = inv;
 }
 
-template <bool SPARSE, bool PER_ELEM>
+template <bool SPARSE, bool PER_ELEM, bool DISP = false>
 int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
     constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
     forge::KernelTiming timing(SPARSE ? "sweep_block_sparse14" : "sweep_block", st,
@@ -314,15 +330,15 @@ int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
                       (reinterpret_cast<uintptr_t>(a.U) % 16) == 0;
     if (fast && a.R % 256 == 0) {
         dim3 grid((unsigned)(a.R / 256), (unsigned)batch);
-        sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false>
+        sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false, DISP>
             <<<grid, dim3(256), 0, st>>>(a);
     } else {
         dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
         if (fast)
-            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, false>
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, false, DISP>
                 <<<grid, dim3(64), 0, st>>>(a);
         else
-            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, true>
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, true, DISP>
                 <<<grid, dim3(64), 0, st>>>(a);
     }
     FORGE_LAUNCH_CHECK();
@@ -384,18 +400,20 @@ extern "C" int forge_sparsegptq14_solver(float* W, float* U, const float* scales
     return solve_single<true>(W, U, scales, qzeros, bits, C, R, qweight, M, E, uinv, st);
 }
 
-// Left-looking schedule for a batch of equally shaped matrices, errors kept in X.
-extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
-                                        const float* qzerosT, const int32_t* g_idx,
-                                        uint8_t* qweight, uint32_t* M, const float* uinv,
-                                        int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
-                                        int sparse14, forge_stream_t stream) {
+// Left-looking schedule for a batch of equally shaped matrices, errors (or, with W0, the
+// displacements) kept in X.
+static int sweep_batched(float* X, const float* W0, const float* U, const float* scalesT,
+                         const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
+                         uint32_t* M, const float* uinv, int64_t batch, int64_t C, int64_t R,
+                         int64_t G, int bits, int sparse14, forge_stream_t stream) {
     if (int e = check_sweep_shape(C, R, bits)) return e;
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && G >= 1, "bad batch=%lld G=%lld", (long long)batch,
                   (long long)G);
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(X && U && scalesT && qzerosT && g_idx && qweight, "null pointer");
     FORGE_REQUIRE(!sparse14 || (M && uinv), "sparse14 needs M and uinv");
+    FORGE_REQUIRE(!(W0 && sparse14), "the displacement form has no 1:4 variant");
+    FORGE_REQUIRE(W0 != X, "W0 must be a copy of X, not X itself");
     hipStream_t st = (hipStream_t)stream;
     for (int64_t start = 0; start < C; start += forge::kBW) {
         const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
@@ -408,12 +426,33 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
         SweepArgs a{};
         a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
+        a.W0 = W0;
         a.maxq = (1 << bits) - 1;
         int e = sparse14 ? launch_block<true, false>(a, batch, st)
+                : W0     ? launch_block<false, false, true>(a, batch, st)
                          : launch_block<false, false>(a, batch, st);
         if (e) return e;
     }
     return FORGE_OK;
+}
+
+extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
+                                        const float* qzerosT, const int32_t* g_idx,
+                                        uint8_t* qweight, uint32_t* M, const float* uinv,
+                                        int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
+                                        int sparse14, forge_stream_t stream) {
+    return sweep_batched(X, nullptr, U, scalesT, qzerosT, g_idx, qweight, M, uinv, batch, C, R, G,
+                         bits, sparse14, stream);
+}
+
+extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
+                                               const float* scalesT, const float* qzerosT,
+                                               const int32_t* g_idx, uint8_t* qweight,
+                                               int64_t batch, int64_t C, int64_t R, int64_t G,
+                                               int bits, forge_stream_t stream) {
+    FORGE_REQUIRE(W0 || batch == 0, "null pointer");
+    return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, nullptr, nullptr, batch, C, R,
+                         G, bits, 0, stream);
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

@@ -47,6 +47,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_sparsegptq14_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp, vp, vp], i32),
         "forge_gptq_sweep_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32,
                                       vp], i32),
+        "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
+                                            i32),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
@@ -74,7 +76,8 @@ EXPORTED_SYMBOLS = (
     "forge_hip_abi_version", "forge_last_error", "forge_kernel_timing_enable",
     "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
-    "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_hessian_update_grouped",
+    "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_gptq_sweep_direct_batched",
+    "forge_hessian_update_grouped",
     "forge_hessian_workspace_bytes",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
@@ -254,6 +257,29 @@ class _HipKernels:
                 _ptr(uinv), B, C, R, G, int(bits), int(bool(sparse14)), _stream()))
         return (q, M) if sparse14 else q
 
+    def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None):
+        """The sweep fed by the factor of H itself: V [B,C,C] = -M[t,k]/M[k,k] above the
+        diagonal (``unit_upper_from_lower(L, info, negate=True)``).  X [B,C,R] f32 in/out
+        (displacements w0 - deq on exit); W0: untouched copy of X (made here when None).
+        Returns qweight [B,C,R] u8."""
+        _need_cuda(X, V, scalesT, qzerosT, g_idx, W0)
+        B, C, R = X.shape
+        G = scalesT.shape[1]
+        assert X.is_contiguous() and V.is_contiguous() and scalesT.is_contiguous()
+        assert qzerosT.is_contiguous() and g_idx.is_contiguous() and g_idx.dtype == torch.int32
+        assert tuple(V.shape) == (B, C, C) and tuple(scalesT.shape) == (B, G, R)
+        assert tuple(qzerosT.shape) == (B, G, R) and tuple(g_idx.shape) == (B, C)
+        if W0 is None:
+            W0 = X.clone()
+        assert W0.is_contiguous() and W0.shape == X.shape and W0.dtype == torch.float32
+        assert W0.data_ptr() != X.data_ptr() or X.numel() == 0
+        q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_gptq_sweep_direct_batched(
+                _ptr(X), _ptr(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
+                B, C, R, G, int(bits), _stream()))
+        return q
+
     def hessian_update_grouped(self, X, offsets, H, alpha, beta):
         """X [T,C] (bf16/f32) rows grouped by expert; offsets: host int64 [E+1];
         H [E,C,C] f32; alpha/beta: host float sequences [E]."""
@@ -306,16 +332,18 @@ class _HipKernels:
                 _ptr(H), _ptr(damp), _ptr(info), B, C, _ptr(ws), nbytes, _stream()))
         return H, info
 
-    def unit_upper_from_lower(self, L, info=None, flipped_upper=False):
+    def unit_upper_from_lower(self, L, info=None, flipped_upper=False, negate=False):
         """U [B,C,C]: U[t,k] = L[k,t] / L[k,k] (k > t), unit diagonal, zero below; identity
-        where info != 0.  flipped_upper: L is the upper factor A with both orders reversed."""
+        where info != 0.  flipped_upper: L is the upper factor A with both orders reversed.
+        negate: entries above the diagonal with the opposite sign."""
         _need_cuda(L, info)
         B, C, _ = L.shape
         assert L.is_contiguous() and L.dtype == torch.float32
         U = torch.empty_like(L)
         with torch.cuda.device(L.device):
             self._check(self._lib.forge_unit_upper_from_lower(
-                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)), _stream()))
+                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)) | (2 if negate else 0),
+                _stream()))
         return U
 
     def babai_solver(self, W, A, scales, qzeros, group_size, bits, block_size, g_idx, G):

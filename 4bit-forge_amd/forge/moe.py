@@ -22,13 +22,22 @@ class ExpertGroupGPTQ:
     def __init__(self, weights: Sequence[torch.Tensor], bits: int = 4, group_size: int = 128,
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
-                 algorithm: str = "gptq", device=None):
+                 algorithm: str = "gptq", device=None, factor_route: str = "direct"):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
-        keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai"."""
+        keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
+        factor_route (algorithm="gptq" only): "inverse" computes the reference's factor, the
+        upper Cholesky factor of inv(H) (forge/gptq.py:160-166), and sweeps with the column
+        errors; "direct" stops at the factor of H itself and sweeps with the displacements
+        w0 - deq (``kernels.gptq_sweep_direct_batched``): the same solve in exact arithmetic
+        at half the factorisation work, codes differing only where fp32 rounding decides a
+        near-tie."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
+        if factor_route not in ("direct", "inverse"):
+            raise ValueError(f"factor_route={factor_route!r}: 'direct' or 'inverse'")
         self.algorithm = algorithm
+        self.factor_route = factor_route
         self.device = torch.device(device) if device is not None else weights[0].device
         if self.device.type != "cuda":
             raise RuntimeError("ExpertGroupGPTQ runs on the GPU only; there is no CPU fallback")
@@ -101,6 +110,7 @@ class ExpertGroupGPTQ:
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
+        direct = self.algorithm == "gptq" and self.factor_route == "direct"
         outs = [[torch.empty((E, R, C), dtype=torch.uint8, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev)]
@@ -184,6 +194,10 @@ class ExpertGroupGPTQ:
                                                                    upper_only=True)
                     uinv = (1.0 / udiag).contiguous()
                     U.mul_(uinv.unsqueeze(-1))
+                elif direct:
+                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
+                    U = kernels.unit_upper_from_lower(L, info, negate=True)
+                    del L
                 else:
                     U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
@@ -196,6 +210,8 @@ class ExpertGroupGPTQ:
                 if sparse:
                     q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
                                                       uinv=uinv)
+                elif direct:
+                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits)
                 else:
                     q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
                 del X, U

@@ -104,6 +104,23 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
                              int64_t R, int64_t G, int bits, int sparse14,
                              forge_stream_t stream);
 
+/* The same sweep fed by the factor of H itself instead of the factor of its inverse, so that
+ * the second half of gptq.py:160-166 (cholesky_inverse and the second Cholesky) is never
+ * computed.  With H + damp*I = M M^T (M upper; M = L^T of forge_chol_reverse_lower_batched)
+ * and N[t][k] = M[t][k] / M[k][k], N is the inverse of the unit matrix that
+ * forge_gptq_sweep_batched takes, and the value column k has when solver.cu:85-94 reaches it
+ * equals w0[k] + sum_{t<k} d[t] N[t][k] with d[t] = w0[t] - deq[t], the column's original
+ * weight minus what it was rounded to.  V[b] [C, C] holds -N above the diagonal
+ * (forge_unit_upper_from_lower with flag 2); W0[b] [C, R] is an untouched copy of X[b] as
+ * passed in.  Same quantiser and chain order as forge_gptq_sweep_batched; codes are equal in
+ * exact arithmetic and differ in fp32 only where a value sits within rounding error of a
+ * tie.  X holds the displacements d on exit.  Dense sweep only. */
+int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
+                                    const float* scalesT, const float* qzerosT,
+                                    const int32_t* g_idx, uint8_t* qweight, int64_t batch,
+                                    int64_t C, int64_t R, int64_t G, int bits,
+                                    forge_stream_t stream);
+
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private
  * copy with the dequantised values), A [C, C] f32 upper Cholesky factor of H (H = A^T A),
@@ -170,8 +187,9 @@ int forge_chol_reverse_lower_batched(float* H, const float* damp, int32_t* info,
 /* U[b][t][k] = L[b][k][t] * (1 / L[b][k][k]) for k > t, 1 on the diagonal, 0 below it: the
  * coefficients alpha = A[i][t] * invD[i] of solver_babai.cu:133-141,232-236 arranged as the unit
  * upper matrix of a forward sweep.  U[b] = I where info[b] != 0 (info may be null).
- * flipped_upper != 0: L is given as the reference's upper factor A instead,
- * L[k][t] = A[C-1-k][C-1-t].  L and U must not overlap. */
+ * flipped_upper bit 0: L is given as the reference's upper factor A instead,
+ * L[k][t] = A[C-1-k][C-1-t].  Bit 1: the entries above the diagonal are negated (the matrix V
+ * of forge_gptq_sweep_direct_batched).  L and U must not overlap. */
 int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U, int64_t batch,
                                 int64_t C, int flipped_upper, forge_stream_t stream);
 

@@ -64,6 +64,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_gptq_inblock.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i64, vp, vp]
         L.oracle_babai_solver.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp, i32, i64]
         L.oracle_babai_solver.restype = None
+        L.oracle_gptq_solver_direct.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp]
+        L.oracle_gptq_solver_direct.restype = None
         L.oracle_pack_sparsegptq14.argtypes = [vp, vp, vp, vp, i64, i64]
         L.oracle_pack_sparsegptq14.restype = None
         for f in (L.oracle_build_group_meta, L.oracle_mse_scale_groups, L.oracle_gptq_solver,
@@ -132,6 +134,20 @@ def gptq_solver(W, U, scales, qzeros, bits, trail_mode: int = TRAIL_CHAIN, block
                                  qzeros.data_ptr(), int(bits), C, R, q.data_ptr(),
                                  int(trail_mode), int(block))
     gptq_solver.last_W = W
+    return q
+
+
+def gptq_solver_direct(W, V, scales, qzeros, bits):
+    """Checker for the library's displacement form of the sweep (no reference counterpart):
+    V [C,C] = -M[t,k]/M[k,k] above the diagonal for H + damp I = M M^T, columns hand on
+    d = w0 - deq.  W [C,R], scales/qzeros [C,R] per element; returns qweight [C,R] u8."""
+    W = W.contiguous() if W.dtype == torch.float32 else W.to(torch.float32).contiguous()
+    V = _f32c(V); scales = _f32c(scales); qzeros = _f32c(qzeros)
+    C, R = W.shape
+    q = torch.empty((C, R), dtype=torch.uint8)
+    lib().oracle_gptq_solver_direct(W.data_ptr(), V.data_ptr(), scales.data_ptr(),
+                                    qzeros.data_ptr(), int(bits), C, R, q.data_ptr())
+    gptq_solver_direct.last_W = W
     return q
 
 

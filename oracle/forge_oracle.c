@@ -17,6 +17,8 @@
  *   oracle_sparsegptq14_solver   forge/backend/cuda/solver_sparsegptq14.cu:12-200
  *   oracle_pack_sparsegptq14     forge/backend/cuda/bitpacking_sparsegptq14.cu:58-107
  *   oracle_babai_solver          forge/backend/cuda/solver_babai.cu:123-322
+ *   oracle_gptq_solver_direct    (the library's own displacement form of solver.cu:9-154;
+ *                                checks that kernel's arithmetic, see its comment)
  *
  * Where the reference leaves fp32 bits undefined, the oracle fixes them as follows
  * (each choice is within the reference's own numerical freedom):
@@ -214,6 +216,36 @@ void oracle_gptq_solver(float* W, const float* U, const float* scales, const flo
         if (start + Bc < C) trailing_update(W, U, E, C, R, start, Bc, trail_mode);
     }
     free(E);
+}
+
+/* Checker for the library's displacement form of the same sweep (no counterpart in the
+ * reference): V [C,C] holds -M[t,k]/M[k,k] above the diagonal, M being the upper factor of
+ * H + damp*I = M M^T; a column hands on d = w0 - deq, its original weight minus what it was
+ * rounded to, instead of err = x - deq.  I - strict(V) is the inverse of the unit matrix U
+ * that oracle_gptq_solver takes, so err = d (I - strict(V)) and both forms reach every column
+ * with the same value in exact arithmetic.  Quantiser and chain (one fmaf per earlier column,
+ * ascending) are those of solver.cu:9-23,91-94.  W [C,R] is updated in place to the
+ * dequantised weights. */
+void oracle_gptq_solver_direct(float* W, const float* V, const float* scales,
+                               const float* qzeros, int bits, int64_t C, int64_t R,
+                               uint8_t* qweight) {
+    const int maxq_i = (1 << bits) - 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r) {
+        float* x = (float*)malloc((size_t)C * sizeof(float));
+        for (int64_t c = 0; c < C; ++c) x[c] = W[c * R + r];
+        for (int64_t t = 0; t < C; ++t) {
+            const float s = scales[t * R + r], q0 = qzeros[t * R + r];
+            const float inv_s = 1.0f / (s + ORACLE_EPS);
+            float err, deq; uint8_t qb;
+            quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+            const float d = W[t * R + r] - deq;          /* W[t] is still the original weight */
+            qweight[t * R + r] = qb;
+            W[t * R + r] = deq;
+            for (int64_t k = t + 1; k < C; ++k) x[k] = fmaf(-V[t * C + k], d, x[k]);
+        }
+        free(x);
+    }
 }
 
 /* solver_sparsegptq14.cu:29-200.  U [C,C] holds the un-normalised upper factor on entry

@@ -32,6 +32,20 @@ def factor(H, rel_damp, normalise=True):
     return U0 / np.diag(U0)[:, None] if normalise else U0
 
 
+def direct_factor(H, rel_damp):
+    """V for the displacement form of the sweep: with H + damp*I = M M^T (M upper, the
+    Cholesky factor taken from the last row upwards), V[t,k] = -M[t,k]/M[k,k] above the
+    diagonal and 1 on it.  I - strict(V) is the inverse of ``factor(H, rel_damp)``."""
+    H = np.array(H, dtype=np.float64)
+    H[np.diag_indices_from(H)] += rel_damp * np.mean(np.diag(H))
+    H = 0.5 * (H + H.T)
+    Lr = np.linalg.cholesky(H[::-1, ::-1])
+    M = Lr[::-1, ::-1]
+    V = -(M / np.diag(M)[None, :])
+    V[np.diag_indices_from(V)] = 1.0
+    return np.triu(V)
+
+
 def minmax_grid(Xg, bits, symmetric):
     """Closed form of the per-group scale/zero (forge/backend/cuda/quant_grid.cu:78-93),
     evaluated with numpy float32 scalars."""

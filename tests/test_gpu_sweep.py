@@ -1,4 +1,5 @@
 """HIP column sweep against the oracle: bit-exact codes, weights and masks."""
+import numpy as np
 import pytest
 import torch
 
@@ -79,6 +80,50 @@ def test_batched_sweep_with_group_lookup_and_permutation(hip, C, R):
                                torch.stack(zT).to(DEV), torch.stack(gi).to(DEV), 4)
     for b in range(B):
         assert torch.equal(want[b], q[b].cpu())
+
+
+@pytest.mark.parametrize("C,R", [(512, 256), (384, 192), (200, 70)])
+def test_direct_sweep_bit_exact(hip, C, R):
+    """Displacement form (factor of H itself) against its CPU checker: codes and the
+    displacements left in X, bit for bit; whole-wavefront, 64-row and ragged variants."""
+    B, gs = 3, 128
+    G = (C + gs - 1) // gs
+    Xs, Vs, sT, zT, gi, want, disp = [], [], [], [], [], [], []
+    for b in range(B):
+        pr = random_problem(C=C, R=R, seed=200 + b, sym=bool(b % 2), n=C // 2 if b == 2 else None)
+        perm = torch.randperm(C, generator=torch.Generator().manual_seed(b))
+        Wt = pr["W"].t()[perm].contiguous()
+        se, ze = pr["se"][perm].contiguous(), pr["ze"][perm].contiguous()
+        V = torch.from_numpy(mathref.direct_factor(pr["H"].double().numpy(), 0.01)).float().contiguous()
+        want.append(oracle.gptq_solver_direct(Wt.clone(), V, se, ze, 4))
+        disp.append(Wt - oracle.gptq_solver_direct.last_W)
+        Xs.append(Wt); Vs.append(V)
+        sT.append(pr["s"].view(R, G).t().contiguous()); zT.append(pr["z"].view(R, G).t().contiguous())
+        gi.append((perm // gs).int())
+    X = torch.stack(Xs).to(DEV)
+    q = hip.gptq_sweep_direct_batched(X, torch.stack(Vs).to(DEV), torch.stack(sT).to(DEV),
+                                      torch.stack(zT).to(DEV), torch.stack(gi).to(DEV), 4)
+    for b in range(B):
+        assert torch.equal(want[b], q[b].cpu())
+        assert torch.equal(disp[b], X[b].cpu())
+
+
+def test_direct_factor_on_the_gpu(hip):
+    """chol_reverse_lower_batched + unit_upper_from_lower(negate=True) give the V of the
+    displacement form: against float64, and I - strict(V) inverts the reference's factor."""
+    C = 384
+    pr = random_problem(C=C, R=8, n=200, seed=31)
+    H = pr["H"]
+    damp = (0.01 * torch.diagonal(H).mean()).view(1)
+    L, info = hip.chol_reverse_lower_batched(H.clone().view(1, C, C).to(DEV), damp.to(DEV))
+    assert info.tolist() == [0]
+    V = hip.unit_upper_from_lower(L, info, negate=True)[0].cpu().double().numpy()
+    Up = hip.unit_upper_from_lower(L, info)[0].cpu().double().numpy()
+    assert np.array_equal(V, 2 * np.eye(C) - Up)
+    ref = mathref.direct_factor(H.double().numpy(), 0.01)
+    assert np.linalg.norm(V - ref) / np.linalg.norm(ref) < 2e-5
+    Ut = mathref.factor(H.double().numpy(), 0.01)
+    assert np.abs((2 * np.eye(C) - V) @ Ut - np.eye(C)).max() < 1e-3
 
 
 def test_full_size_sweep_properties(hip):
