@@ -405,7 +405,8 @@ extern "C" int forge_sparsegptq14_solver(float* W, float* U, const float* scales
 static int sweep_batched(float* X, const float* W0, const float* U, const float* scalesT,
                          const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                          uint32_t* M, const float* uinv, int64_t batch, int64_t C, int64_t R,
-                         int64_t G, int bits, int sparse14, forge_stream_t stream) {
+                         int64_t G, int bits, int sparse14, void* ws, int64_t ws_bytes,
+                         forge_stream_t stream) {
     if (int e = check_sweep_shape(C, R, bits)) return e;
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && G >= 1, "bad batch=%lld G=%lld", (long long)batch,
                   (long long)G);
@@ -422,7 +423,14 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         g.xs = C * R; g.as = C * C; g.bs = C * R;
         g.m0 = (int)start; g.m1 = (int)(start + bw); g.n1 = (int)R; g.k0 = 0; g.k1 = (int)start;
         g.negate_a = true;
-        if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        if (ws) {
+            // sums of 128 products each, three bf16 pieces per operand on the bf16 matrix pipe
+            // where the block is a full tile (fp32 matrix pipe otherwise)
+            g.blocked_sum = true;
+            if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, ws_bytes)) return e;
+        } else {
+            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        }
         SweepArgs a{};
         a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
@@ -442,17 +450,26 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
                                         int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
                                         int sparse14, forge_stream_t stream) {
     return sweep_batched(X, nullptr, U, scalesT, qzerosT, g_idx, qweight, M, uinv, batch, C, R, G,
-                         bits, sparse14, stream);
+                         bits, sparse14, nullptr, 0, stream);
+}
+
+extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C) {
+    if (batch <= 0 || C <= forge::kBW) return 0;
+    return forge::split_gemm_workspace_bytes(batch, C - forge::kBW);
 }
 
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                                const float* scalesT, const float* qzerosT,
                                                const int32_t* g_idx, uint8_t* qweight,
                                                int64_t batch, int64_t C, int64_t R, int64_t G,
-                                               int bits, forge_stream_t stream) {
+                                               int bits, void* ws, int64_t ws_bytes,
+                                               forge_stream_t stream) {
     FORGE_REQUIRE(W0 || batch == 0, "null pointer");
+    FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C),
+                  "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
+                  (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C));
     return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, nullptr, nullptr, batch, C, R,
-                         G, bits, 0, stream);
+                         G, bits, 0, ws, ws_bytes, stream);
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

@@ -47,8 +47,9 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_sparsegptq14_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp, vp, vp], i32),
         "forge_gptq_sweep_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32,
                                       vp], i32),
-        "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
-                                            i32),
+        "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp,
+                                             i64, vp], i32),
+        "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
@@ -77,6 +78,7 @@ EXPORTED_SYMBOLS = (
     "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
     "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_gptq_sweep_direct_batched",
+    "forge_gptq_sweep_direct_workspace_bytes",
     "forge_hessian_update_grouped",
     "forge_hessian_workspace_bytes",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
@@ -257,11 +259,13 @@ class _HipKernels:
                 _ptr(uinv), B, C, R, G, int(bits), int(bool(sparse14)), _stream()))
         return (q, M) if sparse14 else q
 
-    def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None):
+    def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None,
+                                  exact_chain=False):
         """The sweep fed by the factor of H itself: V [B,C,C] = -M[t,k]/M[k,k] above the
         diagonal (``unit_upper_from_lower(L, info, negate=True)``).  X [B,C,R] f32 in/out
         (displacements w0 - deq on exit); W0: untouched copy of X (made here when None).
-        Returns qweight [B,C,R] u8."""
+        exact_chain: keep the block updates as one fp32 fma chain per element (reproducible
+        on a CPU) instead of blocked sums on the bf16 matrix pipe.  Returns qweight [B,C,R] u8."""
         _need_cuda(X, V, scalesT, qzerosT, g_idx, W0)
         B, C, R = X.shape
         G = scalesT.shape[1]
@@ -274,10 +278,12 @@ class _HipKernels:
         assert W0.is_contiguous() and W0.shape == X.shape and W0.dtype == torch.float32
         assert W0.data_ptr() != X.data_ptr() or X.numel() == 0
         q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
+        nbytes = 0 if exact_chain else int(self._lib.forge_gptq_sweep_direct_workspace_bytes(B, C))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_gptq_sweep_direct_batched(
                 _ptr(X), _ptr(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
-                B, C, R, G, int(bits), _stream()))
+                B, C, R, G, int(bits), _ptr(ws), nbytes, _stream()))
         return q
 
     def hessian_update_grouped(self, X, offsets, H, alpha, beta):

@@ -32,16 +32,14 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
 
 PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, TFLOP/s, GB/s
-# HBM bytes per launch of the two GEMM kernels on the default workload (64 experts per
-# step), from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each
-# scaled by what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and
-# x1.0); summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  The operand data a
-# launch of the factorisation GEMM has to read once (rows below the current block of the
-# factor and of its inverse) averages ~4.4e9 bytes over the 55 launches of a C=7168
-# factorisation (the 15 launches of the C=2048 one are small: ~3.5e9 on average over all
-# 70); the sweep update reads the earlier error rows once (~1.9e9 bytes on average).
-MEASURED_TRAFFIC = {("deepseek_v3", 64, "split_gemm_bf16x3"): 4.48e9,
-                    ("deepseek_v3", 64, "chain_gemm"): 2.06e9}
+# HBM bytes per launch of the GEMM kernel on the default workload (64 experts per step),
+# from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by
+# what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and x1.0);
+# summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  What a launch has to read once
+# averages ~2.6e9 bytes over the 140 launches of a step: the rows of the factor below the
+# current block (factorisation, C=7168: ~2.2e9 per launch), the displacement rows of all
+# earlier columns (sweep: ~3.8e9 per launch for gate/up, ~1.9e9 for down).
+MEASURED_TRAFFIC = {("deepseek_v3", 64, "split_gemm_bf16x3"): 3.04e9}
 
 KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit, executed / counted work)
     "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s", 1.0),

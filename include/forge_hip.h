@@ -114,12 +114,19 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * (forge_unit_upper_from_lower with flag 2); W0[b] [C, R] is an untouched copy of X[b] as
  * passed in.  Same quantiser and chain order as forge_gptq_sweep_batched; codes are equal in
  * exact arithmetic and differ in fp32 only where a value sits within rounding error of a
- * tie.  X holds the displacements d on exit.  Dense sweep only. */
+ * tie.  X holds the displacements d on exit.  Dense sweep only.
+ * ws == NULL: the update of a column block by all earlier columns is one fp32 fused
+ * multiply-add per earlier column, in ascending order (the chain of solver.cu:91-94 carried
+ * across blocks), reproducible bit for bit on a CPU.  With a workspace of
+ * forge_gptq_sweep_direct_workspace_bytes(batch, C) bytes that update is summed in blocks of
+ * 128 columns from three bf16 pieces per fp32 operand on the bf16 matrix pipe wherever a
+ * block is a full 128 x 128 tile (fp32-grade accuracy, different rounding, faster). */
 int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                     const float* scalesT, const float* qzerosT,
                                     const int32_t* g_idx, uint8_t* qweight, int64_t batch,
-                                    int64_t C, int64_t R, int64_t G, int bits,
-                                    forge_stream_t stream);
+                                    int64_t C, int64_t R, int64_t G, int bits, void* ws,
+                                    int64_t ws_bytes, forge_stream_t stream);
+int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C);
 
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private

@@ -101,11 +101,18 @@ def test_direct_sweep_bit_exact(hip, C, R):
         sT.append(pr["s"].view(R, G).t().contiguous()); zT.append(pr["z"].view(R, G).t().contiguous())
         gi.append((perm // gs).int())
     X = torch.stack(Xs).to(DEV)
-    q = hip.gptq_sweep_direct_batched(X, torch.stack(Vs).to(DEV), torch.stack(sT).to(DEV),
-                                      torch.stack(zT).to(DEV), torch.stack(gi).to(DEV), 4)
+    args = (torch.stack(Vs).to(DEV), torch.stack(sT).to(DEV), torch.stack(zT).to(DEV),
+            torch.stack(gi).to(DEV), 4)
+    q = hip.gptq_sweep_direct_batched(X, *args, exact_chain=True)
     for b in range(B):
         assert torch.equal(want[b], q[b].cpu())
         assert torch.equal(disp[b], X[b].cpu())
+    # default: block updates as blocked sums (bf16 pieces where the tiles are full, fp32
+    # elsewhere): fp32-grade, so codes move only at near-ties
+    X2 = torch.stack(Xs).to(DEV)
+    q2 = hip.gptq_sweep_direct_batched(X2, *args)
+    assert (q2 != q).float().mean().item() <= 1e-3
+    assert (X2 - X).abs().max().item() <= 0.05 * X.abs().max().item()
 
 
 def test_direct_factor_on_the_gpu(hip):
