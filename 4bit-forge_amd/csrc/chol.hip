@@ -461,8 +461,9 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
 template <bool FLIP>
 __global__ __launch_bounds__(256) void unit_upper_from_lower_kernel(
     const float* __restrict__ L, const int32_t* __restrict__ info, float* __restrict__ U, int64_t C,
-    float sign) {
+    float sign, bool upper_tiles_only) {
     __shared__ float tile[32][33];
+    if (upper_tiles_only && blockIdx.y > blockIdx.x) return;   // whole tile below the diagonal
     const int64_t b = blockIdx.z;
     const float* __restrict__ Lb = L + b * C * C;
     float* __restrict__ Ub = U + b * C * C;
@@ -529,10 +530,11 @@ extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, 
     const unsigned nt = (unsigned)forge::ceil_div(C, 32);
     forge::KernelTiming timing("unit_upper_from_lower", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
     const float sign = (flipped_upper & 2) ? -1.0f : 1.0f;
+    const bool skip = (flipped_upper & 4) != 0;
     if (flipped_upper & 1)
-        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign);
+        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign, skip);
     else
-        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign);
+        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign, skip);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

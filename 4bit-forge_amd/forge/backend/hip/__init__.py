@@ -338,17 +338,19 @@ class _HipKernels:
                 _ptr(H), _ptr(damp), _ptr(info), B, C, _ptr(ws), nbytes, _stream()))
         return H, info
 
-    def unit_upper_from_lower(self, L, info=None, flipped_upper=False, negate=False):
+    def unit_upper_from_lower(self, L, info=None, flipped_upper=False, negate=False,
+                              upper_only=False):
         """U [B,C,C]: U[t,k] = L[k,t] / L[k,k] (k > t), unit diagonal, zero below; identity
         where info != 0.  flipped_upper: L is the upper factor A with both orders reversed.
-        negate: entries above the diagonal with the opposite sign."""
+        negate: entries above the diagonal with the opposite sign.  upper_only: 32x32 tiles
+        wholly below the diagonal are left unwritten (uninitialised memory)."""
         _need_cuda(L, info)
         B, C, _ = L.shape
         assert L.is_contiguous() and L.dtype == torch.float32
         U = torch.empty_like(L)
         with torch.cuda.device(L.device):
             self._check(self._lib.forge_unit_upper_from_lower(
-                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)) | (2 if negate else 0),
+                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)) | (2 if negate else 0) | (4 if upper_only else 0),
                 _stream()))
         return U
 

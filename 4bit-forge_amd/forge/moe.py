@@ -185,7 +185,7 @@ class ExpertGroupGPTQ:
                 Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
                 if babai:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    U = kernels.unit_upper_from_lower(L, info)
+                    U = kernels.unit_upper_from_lower(L, info, upper_only=True)
                     del L
                 elif sparse:
                     # un-normalised factor, rows then scaled by the rounded reciprocal of the
@@ -196,7 +196,7 @@ class ExpertGroupGPTQ:
                     U.mul_(uinv.unsqueeze(-1))
                 elif direct:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    U = kernels.unit_upper_from_lower(L, info, negate=True)
+                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)
                     del L
                 else:
                     U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)

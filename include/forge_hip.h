@@ -196,7 +196,8 @@ int forge_chol_reverse_lower_batched(float* H, const float* damp, int32_t* info,
  * upper matrix of a forward sweep.  U[b] = I where info[b] != 0 (info may be null).
  * flipped_upper bit 0: L is given as the reference's upper factor A instead,
  * L[k][t] = A[C-1-k][C-1-t].  Bit 1: the entries above the diagonal are negated (the matrix V
- * of forge_gptq_sweep_direct_batched).  L and U must not overlap. */
+ * of forge_gptq_sweep_direct_batched).  Bit 2: 32 x 32 tiles that lie wholly below the
+ * diagonal are left unwritten (no sweep reads them).  L and U must not overlap. */
 int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U, int64_t batch,
                                 int64_t C, int flipped_upper, forge_stream_t stream);
 
