@@ -55,7 +55,7 @@ CONFIGS = {
     "deepseek_v3": dict(n_experts=256, hidden=7168, inter=2048, tokens=8192, fp8=True,
                         symmetric=True, order="activation", chunk=64),
     "qwen3": dict(n_experts=128, hidden=2048, inter=768, tokens=4096, fp8=False,
-                  symmetric=False, order="default", chunk=64),
+                  symmetric=False, order="default", chunk=128),
 }
 
 
