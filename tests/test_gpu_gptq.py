@@ -202,6 +202,31 @@ def test_expert_group_matches_per_expert_handles(factor_route):
     assert worst <= 5e-3, worst
 
 
+@pytest.mark.parametrize("factor_route", ["direct", "inverse"])
+def test_expert_group_non_positive_definite_falls_back(factor_route):
+    """No damping and fewer tokens than features: the factorisation of that expert fails, it is
+    quantised by plain round-to-nearest and flagged (gptq.py:172-175); its neighbour, with
+    enough tokens, is solved as usual."""
+    from forge.moe import ExpertGroupGPTQ
+    g0 = torch.Generator().manual_seed(8)
+    E, R, C = 2, 64, 256
+    W = 0.02 * torch.randn(E, R, C, generator=g0)
+    xs = [torch.randn(4, C, generator=g0) + 0.5, torch.randn(600, C, generator=g0)]
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="absmax",
+              quantization_order="default", rel_damp=0.0)
+    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, factor_route=factor_route, **kw)
+    grp.update(torch.cat(xs).to(DEV), [0, 4, 604])
+    (q, s, z), = grp.quantize(chunk=2)
+    assert grp.issue_non_invertible.tolist() == [True, False]
+    se = expand_meta(s[0].cpu(), R, C, 128).t()
+    ze = expand_meta(z[0].cpu(), R, C, 128).t()
+    assert np.array_equal(q[0].cpu().numpy(), mathref.rtn(W[0].numpy(), se.numpy(), ze.numpy(), 4))
+    o = oracle.GPTQ(linear(W[1]), **kw)
+    o.update(xs[1])
+    qo, so, zo = o.quantize()
+    assert torch.equal(so, s[1].cpu()) and flip_rate(qo, q[1]) <= 5e-3
+
+
 @pytest.mark.parametrize("zero_weight_column", [False, True])
 def test_expert_group_dead_and_zero_columns(zero_weight_column):
     """A feature that one expert never sees (dead column: zero Hessian diagonal) and, in the
