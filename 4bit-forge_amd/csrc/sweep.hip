@@ -96,6 +96,8 @@ __device__ __forceinline__ float dpp_source(float u) {
 // matrix the error form uses, err = d N, so the value a column has when it is reached,
 // w0_k + sum_{t<k} d_t N[t,k], is the same number in exact arithmetic; only fp32 rounding
 // differs.  The quantiser, the fused multiply-adds and their order are those of the error form.
+// Values of columns that are NOT yet reached differ between the forms, so the 1:4 mask score,
+// which looks three columns ahead, has no displacement form here (the host refuses it).
 template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false>
 __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
