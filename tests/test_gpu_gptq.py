@@ -407,6 +407,45 @@ def test_config3_factor_routes_agree_at_full_shape():
         assert flips <= 0.06
 
 
+def test_expert_group_few_tokens_routes_agree():
+    """Experts that saw 1 .. 700 tokens of 2048 features (rank-deficient Hessians, damping
+    only): the two routes of the batched front end give the same codes up to near-ties and
+    the same layer output error, far below round-to-nearest's."""
+    from forge.moe import ExpertGroupGPTQ
+    g0 = torch.Generator().manual_seed(3)
+    C, R = 2048, 256
+    ns = (1, 3, 16, 100, 700)
+    E = len(ns)
+    W = (0.02 * torch.randn(E, R, C, generator=g0)).bfloat16()
+    xs = [torch.randn(n, C, generator=g0).bfloat16() for n in ns]
+    offs = np.concatenate([[0], np.cumsum(ns)]).tolist()
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
+              quantization_order="activation", rel_damp=0.01)
+    out = {}
+    for route in ("direct", "inverse"):
+        grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, factor_route=route, **kw)
+        grp.update(torch.cat(xs).to(DEV), offs)
+        (q, s, z), = grp.quantize(chunk=8)
+        assert not grp.issue_non_invertible.any()
+        out[route] = (q.cpu(), s.cpu(), z.cpu())
+    assert torch.equal(out["direct"][1], out["inverse"][1])
+    for e, n in enumerate(ns):
+        X = xs[e].double()
+        H = ((2.0 / n) * X.t() @ X).numpy()
+        Wf = W[e].double().numpy()
+        err = {}
+        for r in out:
+            D = Wf - oracle.dequantize(out[r][0][e], out[r][1][e], out[r][2][e], 128).double().numpy()
+            err[r] = float(((D @ H) * D).sum())
+        se = expand_meta(out["direct"][1][e], R, C, 128).t().double().numpy()
+        ze = expand_meta(out["direct"][2][e], R, C, 128).t().double().numpy()
+        Dr = Wf - (np.clip(np.rint(Wf / (se + 1e-12) + ze), 0, 15) - ze) * se
+        rtn = float(((Dr @ H) * Dr).sum())
+        assert flip_rate(out["direct"][0][e], out["inverse"][0][e]) <= 3e-3
+        assert abs(err["direct"] / err["inverse"] - 1) < 0.01
+        assert err["direct"] < 0.5 * rtn
+
+
 def test_config2_qwen3_experts_at_full_shape():
     """Eight Qwen3-30B-A3B-shaped experts (768x2048 / 2048x768 bf16, asymmetric, MSE) with the
     layer's ragged routing, batched, against per-expert oracle handles."""
