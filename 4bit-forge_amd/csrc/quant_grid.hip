@@ -78,6 +78,64 @@ __global__ __launch_bounds__(256) void minmax_grid_kernel(
     }
 }
 
+// Groups of exactly 128 elements, every group whole and 16-byte aligned: eight lanes per
+// group, 16 consecutive elements per lane as 16-byte loads (two for bf16, four for fp32), so a
+// wavefront has 2-4 KB in flight instead of 128 bytes.  Same extrema, hence the same bits.
+template <typename T>
+__global__ __launch_bounds__(256) void minmax_grid128_kernel(
+    const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t ldw, int64_t G,
+    int64_t n_groups, float maxq, bool symmetric, float* __restrict__ scales,
+    float* __restrict__ qzeros) {
+    const int sub = threadIdx.x & 7;
+    const int64_t g_raw = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int64_t g = g_raw < n_groups ? g_raw : n_groups - 1;   // all lanes take part in the shuffles
+    const int64_t b = g / (R * G);
+    const int64_t rg = g - b * R * G;
+    const int64_t r = rg / G, grp = rg - r * G;
+    const T* src = W + b * w_stride + r * ldw + grp * 128 + sub * 16;
+    float v[16];
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 w = reinterpret_cast<const float4*>(src)[i];
+            v[4 * i + 0] = w.x; v[4 * i + 1] = w.y; v[4 * i + 2] = w.z; v[4 * i + 3] = w.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint4 w = reinterpret_cast<const uint4*>(src)[i];
+            v[8 * i + 0] = __uint_as_float(w.x << 16); v[8 * i + 1] = __uint_as_float(w.x & 0xffff0000u);
+            v[8 * i + 2] = __uint_as_float(w.y << 16); v[8 * i + 3] = __uint_as_float(w.y & 0xffff0000u);
+            v[8 * i + 4] = __uint_as_float(w.z << 16); v[8 * i + 5] = __uint_as_float(w.z & 0xffff0000u);
+            v[8 * i + 6] = __uint_as_float(w.w << 16); v[8 * i + 7] = __uint_as_float(w.w & 0xffff0000u);
+        }
+    }
+    float lo = 1e30f, hi = -1e30f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        hi = fmaxf(hi, v[i]);
+        lo = fminf(lo, v[i]);
+    }
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) {
+        hi = fmaxf(hi, __shfl_xor(hi, off, 8));
+        lo = fminf(lo, __shfl_xor(lo, off, 8));
+    }
+    if (sub == 0 && g_raw < n_groups) {
+        float s, q0;
+        meta_from_extrema(lo, hi, maxq, symmetric, s, q0);
+        scales[g] = s;
+        qzeros[g] = q0;
+    }
+}
+
+template <typename T>
+bool minmax128_ok(const T* W, int64_t w_stride, int64_t C, int64_t ldw, int64_t gs, int64_t n_groups) {
+    constexpr int64_t per16 = 16 / sizeof(T);
+    return gs == 128 && C % 128 == 0 && ldw % per16 == 0 && w_stride % per16 == 0 &&
+           (reinterpret_cast<uintptr_t>(W) % 16) == 0 && n_groups < (1LL << 33);
+}
+
 // ---------------------------------------------------------------- shrink search
 // |diff|^norm as exp2(norm*log2(.)) on the hardware transcendental units (v_log_f32,
 // v_exp_f32: 1 ulp each); mathematically the reference's __expf(__logf(e)*norm).
@@ -276,8 +334,13 @@ extern "C" int forge_build_group_meta_packed(const float* X, int64_t RG, int64_t
     if (blocks > (1 << 20)) blocks = 1 << 20;
     forge::KernelTiming timing("minmax_grid", (hipStream_t)stream, (double)RG * (gs * 4.0 + 8.0),
                                forge::WORK_BYTES);
-    minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-        X, 0, RG, gs, gs, gs, 1, RG, maxq, symmetric != 0, scales, qzeros);
+    if (minmax128_ok(X, 0, gs, gs, gs, RG))
+        minmax_grid128_kernel<float><<<dim3((unsigned)forge::ceil_div(RG, 32)), dim3(256), 0,
+                                       (hipStream_t)stream>>>(X, 0, RG, gs, 1, RG, maxq,
+                                                              symmetric != 0, scales, qzeros);
+    else
+        minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+            X, 0, RG, gs, gs, gs, 1, RG, maxq, symmetric != 0, scales, qzeros);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }
@@ -332,7 +395,16 @@ extern "C" int forge_quant_grid(const void* W, int w_dtype, int64_t batch, int64
                                (double)batch * R * C * (w_dtype == FORGE_F32 ? 4.0 : 2.0) +
                                    8.0 * n_groups,
                                forge::WORK_BYTES);
-    if (w_dtype == FORGE_F32)
+    const dim3 grid128((unsigned)forge::ceil_div(n_groups, 32));
+    if (w_dtype == FORGE_F32 && minmax128_ok((const float*)W, w_stride, C, ldw, gs, n_groups))
+        minmax_grid128_kernel<float><<<grid128, dim3(256), 0, st>>>(
+            (const float*)W, w_stride, R, ldw, G, n_groups, maxq, symmetric != 0, scales, qzeros);
+    else if (w_dtype == FORGE_BF16 &&
+             minmax128_ok((const __hip_bfloat16*)W, w_stride, C, ldw, gs, n_groups))
+        minmax_grid128_kernel<__hip_bfloat16><<<grid128, dim3(256), 0, st>>>(
+            (const __hip_bfloat16*)W, w_stride, R, ldw, G, n_groups, maxq, symmetric != 0, scales,
+            qzeros);
+    else if (w_dtype == FORGE_F32)
         minmax_grid_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(
             (const float*)W, w_stride, R, C, ldw, gs, G, n_groups, maxq, symmetric != 0, scales,
             qzeros);
