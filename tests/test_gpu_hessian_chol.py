@@ -166,6 +166,23 @@ def test_pack_int4_layout(hip):
     assert torch.equal(pk8.to(torch.int64) & 0xFFFFFFFF, sum(sh[:, :, k] << (4 * k) for k in range(8)))
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("gs", [128, 32])
+def test_pack_int4_aligned_rows(hip, gs):
+    """C and the group size multiples of 8: the 8-byte-load form, same words as the general one."""
+    R, C = 96, 1024
+    g = torch.Generator().manual_seed(2)
+    codes = torch.randint(0, 16, (R, C), dtype=torch.uint8, generator=g)
+    G = C // gs
+    z = torch.randint(0, 16, (R * G,), generator=g).float()
+    for zeros in (z, None):
+        pk = hip.pack_int4(codes.to(DEV), None if zeros is None else zeros.to(DEV), gs).cpu()
+        zz = 8 if zeros is None else z.view(R, G).repeat_interleave(gs, 1).to(torch.int64)
+        sh = ((codes.to(torch.int64) - zz + 8) & 0xF).view(R, -1, 8)
+        ref = sum(sh[:, :, k] << (4 * k) for k in range(8))
+        assert torch.equal(pk.to(torch.int64) & 0xFFFFFFFF, ref)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("B,R,C", [(2, 512, 384), (1, 256, 1152)])
 def test_layout_kernels_tall_tiles(hip, B, R, C):
     """bf16 weights with R % 256 == 0 and C % 128 == 0 take the tall-tile transposes."""
