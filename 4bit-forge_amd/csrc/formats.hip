@@ -44,12 +44,34 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(
     const uint8_t* src = w + (b * O + r) * I + c0;
     const float* srow = sinv + (b * nO + r / so) * nI;
     const int n = (int)((I - c0) < 16 ? (I - c0) : 16);
-    uint8_t v[16];
-    if (n == 16 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
-        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(src);
-    } else {
-        for (int i = 0; i < n; ++i) v[i] = src[i];
+    const int64_t o0 = (b * O + r) * I + c0;
+    // whole 16-byte piece inside one scale tile, output piece aligned: one load, one scale,
+    // 32 (bf16) or 64 (f32) bytes out in 16-byte stores
+    const bool out_ok = ((reinterpret_cast<uintptr_t>(out) + (uint64_t)o0 * (OUT_BF16 ? 2 : 4)) & 15u) == 0;
+    if (n == 16 && (si & 15) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && out_ok) {
+        const uint4 q = *reinterpret_cast<const uint4*>(src);
+        const uint32_t wq[4] = {q.x, q.y, q.z, q.w};
+        const float sc = srow[c0 / si];
+        float f[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) f[i] = e4m3fn_to_f32((wq[i >> 2] >> (8 * (i & 3))) & 0xFFu) * sc;
+        if constexpr (OUT_BF16) {
+            uint32_t pk[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                pk[k] = (uint32_t)f32_to_bf16_rne(f[2 * k]) | ((uint32_t)f32_to_bf16_rne(f[2 * k + 1]) << 16);
+            uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out) + o0);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        } else {
+            float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + o0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) dst[k] = make_float4(f[4 * k], f[4 * k + 1], f[4 * k + 2], f[4 * k + 3]);
+        }
+        return;
     }
+    uint8_t v[16];
+    for (int i = 0; i < n; ++i) v[i] = src[i];
     for (int i = 0; i < n; ++i) {
         const float f = e4m3fn_to_f32(v[i]) * srow[(c0 + i) / si];
         const int64_t o = (b * O + r) * I + c0 + i;
@@ -124,10 +146,18 @@ __global__ __launch_bounds__(256) void dequantize_groups_kernel(
         for (int k = 0; k < 16; ++k) code[k] = c0 + k < C ? src[k] : (uint8_t)0;
     }
     float val[16];
+    if (vec && (gs & 15) == 0) {
+        // the 16 columns share a group: one scale, one zero, no per-element division
+        const int64_t g = c0 / gs;
+        const float zz = z[g], ss = s[g];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        const int64_t g = (c0 + k < C ? c0 + k : C - 1) / gs;
-        val[k] = ((float)code[k] - z[g]) * s[g];
+        for (int k = 0; k < 16; ++k) val[k] = ((float)code[k] - zz) * ss;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int64_t g = (c0 + k < C ? c0 + k : C - 1) / gs;
+            val[k] = ((float)code[k] - z[g]) * s[g];
+        }
     }
     if constexpr (OUT_BF16) {
         uint16_t* __restrict__ dst = reinterpret_cast<uint16_t*>(out) + br * C + c0;
