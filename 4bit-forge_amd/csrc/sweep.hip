@@ -96,8 +96,9 @@ __device__ __forceinline__ float dpp_source(float u) {
 // matrix the error form uses, err = d N, so the value a column has when it is reached,
 // w0_k + sum_{t<k} d_t N[t,k], is the same number in exact arithmetic; only fp32 rounding
 // differs.  The quantiser, the fused multiply-adds and their order are those of the error form.
-// Values of columns that are NOT yet reached differ between the forms, so the 1:4 mask score,
-// which looks three columns ahead, has no displacement form here (the host refuses it).
+// Values of columns that are NOT yet reached differ between the forms; the 1:4 mask score,
+// which looks three columns ahead, rebuilds the error form's values from the 4x4 diagonal
+// block of V (see select_and_quantize).
 template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false>
 __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
@@ -172,12 +173,38 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             bool keep = true;
             if constexpr (SPARSE) {
                 if ((t & 3) == 0) {
+                    // the values the score looks at: column t as it is, and the three columns
+                    // after it BEFORE they have received this group's updates
+                    float look[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) look[k] = x[t + k];
+                    if constexpr (DISP) {
+                        // Those three are not the same number in the two forms (only a column
+                        // that has been reached is).  With d_j = x_j - w0_j, what the earlier
+                        // columns have added so far, the error form's value of column k is
+                        // w0_k + sum_{j<=k} d_j A[j,k], A the inverse of the 4x4 unit diagonal
+                        // block of N = I - strict(V).
+                        auto vv = [&](int j, int k) -> float {
+                            if constexpr (TAIL) return (c + k < C) ? U[(c + j) * C + c + k] : 0.0f;
+                            else return Up[buf][t + j][t + k];
+                        };
+                        const float v01 = vv(0, 1), v02 = vv(0, 2), v03 = vv(0, 3);
+                        const float v12 = vv(1, 2), v13 = vv(1, 3), v23 = vv(2, 3);
+                        const float a02 = __builtin_fmaf(v01, v12, v02);
+                        const float a13 = __builtin_fmaf(v12, v23, v13);
+                        const float a03 = __builtin_fmaf(v01, a13, __builtin_fmaf(v02, v23, v03));
+                        const float d0 = x[t] - err[t], d1 = x[t + 1] - err[t + 1];
+                        const float d2 = x[t + 2] - err[t + 2];
+                        look[1] = __builtin_fmaf(d0, v01, x[t + 1]);
+                        look[2] = __builtin_fmaf(d1, v12, __builtin_fmaf(d0, a02, x[t + 2]));
+                        look[3] = __builtin_fmaf(d2, v23, __builtin_fmaf(d1, a13, __builtin_fmaf(d0, a03, x[t + 3])));
+                    }
                     float best = -1e30f;
                     int best_k = -1;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         if (!TAIL || c + k < C) {
-                            const float score = fabsf(x[t + k] * uinv[c + k]);
+                            const float score = fabsf(look[k] * uinv[c + k]);
                             if (best < score) { best = score; best_k = k; }
                         }
                     }
@@ -286,11 +313,14 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             __syncthreads();
             buf ^= 1;
         } else {
+            if constexpr (DISP) {
+#pragma unroll 1
+                for (int t = 0; t < SB; ++t) err[t] = (t < rem) ? W0[(cs + t) * R] : 0.0f;
+            }
 #pragma unroll 1
             for (int t = 0; t < SB; ++t) {
-                err[t] = 0.0f;
+                if constexpr (!DISP) err[t] = 0.0f;
                 if (t < rem) {
-                    if constexpr (DISP) err[t] = W0[(cs + t) * R];
                     float s_t, q0_t;
                     if constexpr (PER_ELEM) {
                         s_t = sc[(cs + t) * R];
@@ -415,7 +445,6 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(X && U && scalesT && qzerosT && g_idx && qweight, "null pointer");
     FORGE_REQUIRE(!sparse14 || (M && uinv), "sparse14 needs M and uinv");
-    FORGE_REQUIRE(!(W0 && sparse14), "the displacement form has no 1:4 variant");
     FORGE_REQUIRE(W0 != X, "W0 must be a copy of X, not X itself");
     hipStream_t st = (hipStream_t)stream;
     for (int64_t start = 0; start < C; start += forge::kBW) {
@@ -438,7 +467,8 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
         a.W0 = W0;
         a.maxq = (1 << bits) - 1;
-        int e = sparse14 ? launch_block<true, false>(a, batch, st)
+        int e = sparse14 ? (W0 ? launch_block<true, false, true>(a, batch, st)
+                               : launch_block<true, false>(a, batch, st))
                 : W0     ? launch_block<false, false, true>(a, batch, st)
                          : launch_block<false, false>(a, batch, st);
         if (e) return e;
@@ -463,15 +493,16 @@ extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                                const float* scalesT, const float* qzerosT,
                                                const int32_t* g_idx, uint8_t* qweight,
+                                               uint32_t* M, const float* mdiag,
                                                int64_t batch, int64_t C, int64_t R, int64_t G,
-                                               int bits, void* ws, int64_t ws_bytes,
+                                               int bits, int sparse14, void* ws, int64_t ws_bytes,
                                                forge_stream_t stream) {
     FORGE_REQUIRE(W0 || batch == 0, "null pointer");
     FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C),
                   "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
                   (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C));
-    return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, nullptr, nullptr, batch, C, R,
-                         G, bits, 0, ws, ws_bytes, stream);
+    return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, M, mdiag, batch, C, R, G, bits,
+                         sparse14, ws, ws_bytes, stream);
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

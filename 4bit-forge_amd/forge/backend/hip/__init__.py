@@ -47,8 +47,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_sparsegptq14_solver": ([vp, vp, vp, vp, i32, i64, i64, vp, vp, vp, vp, vp], i32),
         "forge_gptq_sweep_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32,
                                       vp], i32),
-        "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp,
-                                             i64, vp], i32),
+        "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
+                                             i32, i32, vp, i64, vp], i32),
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
@@ -260,12 +260,14 @@ class _HipKernels:
         return (q, M) if sparse14 else q
 
     def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None,
-                                  exact_chain=False):
+                                  exact_chain=False, sparse14=False, mdiag=None):
         """The sweep fed by the factor of H itself: V [B,C,C] = -M[t,k]/M[k,k] above the
         diagonal (``unit_upper_from_lower(L, info, negate=True)``).  X [B,C,R] f32 in/out
         (displacements w0 - deq on exit); W0: untouched copy of X (made here when None).
         exact_chain: keep the block updates as one fp32 fma chain per element (reproducible
-        on a CPU) instead of blocked sums on the bf16 matrix pipe.  Returns qweight [B,C,R] u8."""
+        on a CPU) instead of blocked sums on the bf16 matrix pipe.  sparse14: the 1:4 joint
+        solve, with mdiag [B,C] = diag(L) (1 where the factorisation failed).
+        Returns qweight [B,C,R] u8 (and M [B, ceil(C/32), R] u32)."""
         _need_cuda(X, V, scalesT, qzerosT, g_idx, W0)
         B, C, R = X.shape
         G = scalesT.shape[1]
@@ -278,13 +280,19 @@ class _HipKernels:
         assert W0.is_contiguous() and W0.shape == X.shape and W0.dtype == torch.float32
         assert W0.data_ptr() != X.data_ptr() or X.numel() == 0
         q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
+        M = None
+        if sparse14:
+            M = torch.empty((B, (C + 31) // 32, R), dtype=torch.uint32, device=X.device)
+            assert mdiag is not None and tuple(mdiag.shape) == (B, C) and mdiag.is_contiguous()
+            assert mdiag.dtype == torch.float32
         nbytes = 0 if exact_chain else int(self._lib.forge_gptq_sweep_direct_workspace_bytes(B, C))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_gptq_sweep_direct_batched(
                 _ptr(X), _ptr(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
-                B, C, R, G, int(bits), _ptr(ws), nbytes, _stream()))
-        return q
+                _ptr(M), _ptr(mdiag), B, C, R, G, int(bits), int(bool(sparse14)), _ptr(ws), nbytes,
+                _stream()))
+        return (q, M) if sparse14 else q
 
     def hessian_update_grouped(self, X, offsets, H, alpha, beta):
         """X [T,C] (bf16/f32) rows grouped by expert; offsets: host int64 [E+1];

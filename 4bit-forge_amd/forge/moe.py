@@ -26,7 +26,7 @@ class ExpertGroupGPTQ:
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
-        factor_route (algorithm="gptq" only): "inverse" computes the reference's factor, the
+        factor_route (algorithms "gptq" and "sparsegptq"): "inverse" computes the reference's factor, the
         upper Cholesky factor of inv(H) (forge/gptq.py:160-166), and sweeps with the column
         errors; "direct" stops at the factor of H itself and sweeps with the displacements
         w0 - deq (``kernels.gptq_sweep_direct_batched``): the same solve in exact arithmetic
@@ -110,7 +110,7 @@ class ExpertGroupGPTQ:
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
-        direct = self.algorithm == "gptq" and self.factor_route == "direct"
+        direct = self.algorithm in ("gptq", "sparsegptq") and self.factor_route == "direct"
         outs = [[torch.empty((E, R, C), dtype=torch.uint8, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev)]
@@ -187,6 +187,15 @@ class ExpertGroupGPTQ:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                     U = kernels.unit_upper_from_lower(L, info, upper_only=True)
                     del L
+                elif direct:
+                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
+                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)
+                    if sparse:
+                        # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the
+                        # diagonal of the factor of H itself; U = I where it failed
+                        uinv = torch.where((info != 0)[:, None], torch.ones((), device=dev),
+                                           L.diagonal(dim1=1, dim2=2)).contiguous()
+                    del L
                 elif sparse:
                     # un-normalised factor, rows then scaled by the rounded reciprocal of the
                     # diagonal as solver_sparsegptq14.cu:153-155 does
@@ -194,10 +203,6 @@ class ExpertGroupGPTQ:
                                                                    upper_only=True)
                     uinv = (1.0 / udiag).contiguous()
                     U.mul_(uinv.unsqueeze(-1))
-                elif direct:
-                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)
-                    del L
                 else:
                     U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
@@ -207,7 +212,10 @@ class ExpertGroupGPTQ:
                 for t in (scales, qzeros, sT, zT):
                     t.record_stream(main)
                 M = None
-                if sparse:
+                if direct and sparse:
+                    q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits,
+                                                             sparse14=True, mdiag=uinv)
+                elif sparse:
                     q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
                                                       uinv=uinv)
                 elif direct:

@@ -114,7 +114,12 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * (forge_unit_upper_from_lower with flag 2); W0[b] [C, R] is an untouched copy of X[b] as
  * passed in.  Same quantiser and chain order as forge_gptq_sweep_batched; codes are equal in
  * exact arithmetic and differ in fp32 only where a value sits within rounding error of a
- * tie.  X holds the displacements d on exit.  Dense sweep only.
+ * tie.  X holds the displacements d on exit.
+ * sparse14 != 0: the 1:4 joint solve (solver_sparsegptq14.cu:29-200) in the same form; then
+ * M[b] [ceil(C/32), R] u32 receives the keep-masks and mdiag[b] [C] must hold the diagonal of
+ * L (= 1/diag(U) of the reference's un-normalised factor, the weight of the mask score;
+ * 1 where the factorisation failed).  A pruned column hands on its whole original weight; the
+ * values of the three columns the score looks ahead at are rebuilt from V's 4 x 4 diagonal block.
  * ws == NULL: the update of a column block by all earlier columns is one fp32 fused
  * multiply-add per earlier column, in ascending order (the chain of solver.cu:91-94 carried
  * across blocks), reproducible bit for bit on a CPU.  With a workspace of
@@ -123,8 +128,9 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * block is a full 128 x 128 tile (fp32-grade accuracy, different rounding, faster). */
 int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                     const float* scalesT, const float* qzerosT,
-                                    const int32_t* g_idx, uint8_t* qweight, int64_t batch,
-                                    int64_t C, int64_t R, int64_t G, int bits, void* ws,
+                                    const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
+                                    const float* mdiag, int64_t batch, int64_t C, int64_t R,
+                                    int64_t G, int bits, int sparse14, void* ws,
                                     int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C);
 

@@ -66,6 +66,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_babai_solver.restype = None
         L.oracle_gptq_solver_direct.argtypes = [vp, vp, vp, vp, i32, i64, i64, vp]
         L.oracle_gptq_solver_direct.restype = None
+        L.oracle_sparsegptq14_solver_direct.argtypes = [vp, vp, vp, vp, vp, i32, i64, i64, vp, vp]
+        L.oracle_sparsegptq14_solver_direct.restype = None
         L.oracle_pack_sparsegptq14.argtypes = [vp, vp, vp, vp, i64, i64]
         L.oracle_pack_sparsegptq14.restype = None
         for f in (L.oracle_build_group_meta, L.oracle_mse_scale_groups, L.oracle_gptq_solver,
@@ -149,6 +151,22 @@ def gptq_solver_direct(W, V, scales, qzeros, bits):
                                     qzeros.data_ptr(), int(bits), C, R, q.data_ptr())
     gptq_solver_direct.last_W = W
     return q
+
+
+def sparsegptq14_solver_direct(W, V, mdiag, scales, qzeros, bits):
+    """Checker for the displacement form of the 1:4 joint solve: V as for gptq_solver_direct,
+    mdiag [C] = diag of the factor M of H + damp I = M M^T.  Returns (qweight [C,R] u8,
+    M [ceil(C/32), R] uint32)."""
+    W = W.contiguous() if W.dtype == torch.float32 else W.to(torch.float32).contiguous()
+    V = _f32c(V); mdiag = _f32c(mdiag); scales = _f32c(scales); qzeros = _f32c(qzeros)
+    C, R = W.shape
+    q = torch.empty((C, R), dtype=torch.uint8)
+    M = torch.zeros(((C + 31) // 32, R), dtype=torch.uint32)
+    lib().oracle_sparsegptq14_solver_direct(W.data_ptr(), V.data_ptr(), mdiag.data_ptr(),
+                                            scales.data_ptr(), qzeros.data_ptr(), int(bits), C, R,
+                                            q.data_ptr(), M.data_ptr())
+    sparsegptq14_solver_direct.last_W = W
+    return q, M
 
 
 def babai_solver(W, A, scales, qzeros, group_size, bits, block_size, g_idx, G,

@@ -19,6 +19,7 @@
  *   oracle_babai_solver          forge/backend/cuda/solver_babai.cu:123-322
  *   oracle_gptq_solver_direct    (the library's own displacement form of solver.cu:9-154;
  *                                checks that kernel's arithmetic, see its comment)
+ *   oracle_sparsegptq14_solver_direct   (the same for solver_sparsegptq14.cu:29-200)
  *
  * Where the reference leaves fp32 bits undefined, the oracle fixes them as follows
  * (each choice is within the reference's own numerical freedom):
@@ -245,6 +246,65 @@ void oracle_gptq_solver_direct(float* W, const float* V, const float* scales,
             for (int64_t k = t + 1; k < C; ++k) x[k] = fmaf(-V[t * C + k], d, x[k]);
         }
         free(x);
+    }
+}
+
+/* The 1:4 joint solve in the displacement form (checker for the library's kernel, no
+ * counterpart in the reference).  mdiag [C] = diagonal of the factor M (= 1/diag(U0) of
+ * solver_sparsegptq14.cu:153).  A pruned column hands on its whole original weight.  The mask
+ * score reads the three columns after t before they have received the group's updates; those
+ * values differ between the forms, so the error form's are rebuilt from d_j = x_j - w0_j and
+ * the inverse A of the 4x4 unit diagonal block of N = I - strict(V):
+ * value_k = w0_k + sum_{j<=k} d_j A[j,k], evaluated with the fused multiply-adds below. */
+void oracle_sparsegptq14_solver_direct(float* W, const float* V, const float* mdiag,
+                                       const float* scales, const float* qzeros, int bits,
+                                       int64_t C, int64_t R, uint8_t* qweight, uint32_t* M) {
+    const int maxq_i = (1 << bits) - 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r) {
+        float* x = (float*)calloc((size_t)C + 4, sizeof(float));
+        float* w0 = (float*)calloc((size_t)C + 4, sizeof(float));
+        for (int64_t c = 0; c < C; ++c) x[c] = w0[c] = W[c * R + r];
+        uint32_t mask = 0u;
+        for (int64_t t = 0; t < C; ++t) {
+            if ((t & 31) == 0) mask = 0u;
+            if (t % 4 == 0) {
+                float v[4][4] = {{0}};
+                for (int j = 0; j < 4; ++j)
+                    for (int k = j + 1; k < 4; ++k)
+                        if (t + k < C) v[j][k] = V[(t + j) * C + t + k];
+                const float a02 = fmaf(v[0][1], v[1][2], v[0][2]);
+                const float a13 = fmaf(v[1][2], v[2][3], v[1][3]);
+                const float a03 = fmaf(v[0][1], a13, fmaf(v[0][2], v[2][3], v[0][3]));
+                const float d0 = x[t] - w0[t], d1 = x[t + 1] - w0[t + 1], d2 = x[t + 2] - w0[t + 2];
+                float look[4];
+                look[0] = x[t];
+                look[1] = fmaf(d0, v[0][1], x[t + 1]);
+                look[2] = fmaf(d1, v[1][2], fmaf(d0, a02, x[t + 2]));
+                look[3] = fmaf(d2, v[2][3], fmaf(d1, a13, fmaf(d0, a03, x[t + 3])));
+                float best = -1e30f; int best_k = -1;
+                for (int k = 0; k < 4; ++k) {
+                    if (t + k >= C) continue;
+                    float score = fabsf(look[k] * mdiag[t + k]);
+                    if (best < score) { best = score; best_k = k; }
+                }
+                if (best_k > -1) mask |= (1u << ((t & 31) + best_k));
+            }
+            float err, deq = 0.0f, d; uint8_t qb = 0;
+            if ((mask >> (t & 31)) & 1u) {
+                const float s = scales[t * R + r], q0 = qzeros[t * R + r];
+                const float inv_s = 1.0f / (s + ORACLE_EPS);
+                quantize_scalar(x[t], inv_s, s, q0, maxq_i, &err, &qb, &deq);
+                d = w0[t] - deq;
+            } else {
+                d = w0[t];
+            }
+            qweight[t * R + r] = qb;
+            W[t * R + r] = deq;
+            for (int64_t k = t + 1; k < C; ++k) x[k] = fmaf(-V[t * C + k], d, x[k]);
+            if ((t & 31) == 31 || t == C - 1) M[(t >> 5) * R + r] = mask;
+        }
+        free(x); free(w0);
     }
 }
 

@@ -258,9 +258,11 @@ def test_expert_group_dead_and_zero_columns(zero_weight_column):
                 assert torch.equal(qo[:, [37, 200]], q[e].cpu()[:, [37, 200]])
 
 
-def test_expert_group_sparse14_matches_per_expert_oracle():
+@pytest.mark.parametrize("factor_route", ["direct", "inverse"])
+def test_expert_group_sparse14_matches_per_expert_oracle(factor_route):
     """algorithm="sparsegptq" through the batched front end: codes, keep-masks (solver order)
-    and scales against oracle.GPTQ expert by expert; one kept weight in every group of four."""
+    and scales against oracle.GPTQ expert by expert; one kept weight in every group of four.
+    Both routes to the sweep's matrix."""
     from forge.moe import ExpertGroupGPTQ
     g = torch.Generator().manual_seed(31)
     E, R, C = 3, 64, 256
@@ -270,7 +272,7 @@ def test_expert_group_sparse14_matches_per_expert_oracle():
     offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
     kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
               quantization_order="default", algorithm="sparsegptq")
-    grp = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, **kw)
+    grp = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, factor_route=factor_route, **kw)
     grp.update(torch.cat(xs).to(DEV), offs)
     (qg, sg, zg, Mg), (qu, su, zu, Mu) = grp.quantize(chunk=4)
     for e in range(E):

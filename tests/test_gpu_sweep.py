@@ -115,6 +115,32 @@ def test_direct_sweep_bit_exact(hip, C, R):
     assert (X2 - X).abs().max().item() <= 0.05 * X.abs().max().item()
 
 
+@pytest.mark.parametrize("C,R,n", [(256, 64, 500), (512, 256, 300), (200, 33, 150)])
+def test_direct_sparse14_sweep_bit_exact(hip, C, R, n):
+    """1:4 joint solve in the displacement form against its CPU checker: codes and masks bit
+    for bit with the fp32 chain; with the bf16-piece block updates only near-ties move."""
+    gs = 128
+    G = (C + gs - 1) // gs
+    pr = random_problem(C=C, R=R, n=n, seed=C)
+    H = pr["H"].double().numpy()
+    V = torch.from_numpy(mathref.direct_factor(H, 0.01)).float().contiguous()
+    Hd = 0.5 * (H + H.T)
+    Hd[np.diag_indices(C)] += 0.01 * np.mean(np.diag(H))
+    mdiag = torch.from_numpy(np.diag(np.linalg.cholesky(Hd[::-1, ::-1])[::-1, ::-1]).copy()).float()
+    Wt = pr["W"].t().contiguous()
+    qd, Md = oracle.sparsegptq14_solver_direct(Wt.clone(), V, mdiag, pr["se"], pr["ze"], 4)
+    args = (V.view(1, C, C).to(DEV), pr["s"].view(R, G).t().contiguous().view(1, G, R).to(DEV),
+            pr["z"].view(R, G).t().contiguous().view(1, G, R).to(DEV),
+            (torch.arange(C) // gs).int().view(1, C).to(DEV), 4)
+    kw = dict(sparse14=True, mdiag=mdiag.view(1, C).to(DEV))
+    q, M = hip.gptq_sweep_direct_batched(Wt.clone().view(1, C, R).to(DEV), *args, exact_chain=True, **kw)
+    assert torch.equal(qd, q[0].cpu())
+    assert torch.equal(Md.view(torch.int32), M[0].cpu().view(torch.int32))
+    q2, M2 = hip.gptq_sweep_direct_batched(Wt.clone().view(1, C, R).to(DEV), *args, **kw)
+    assert (q2 != q).float().mean().item() <= 3e-3
+    assert (M2.view(torch.int32) != M.view(torch.int32)).float().mean().item() <= 3e-3
+
+
 def test_direct_factor_on_the_gpu(hip):
     """chol_reverse_lower_batched + unit_upper_from_lower(negate=True) give the V of the
     displacement form: against float64, and I - strict(V) inverts the reference's factor."""

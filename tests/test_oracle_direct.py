@@ -78,3 +78,71 @@ def test_checker_against_the_reference_form():
         D = W - (q.t().double().numpy() - z) * s
         return float(np.einsum("rc,cd,rd->", D, H, D))
     assert abs(loss(qd) / loss(qe) - 1) < 1e-3
+
+
+def _reverse_factor_diag(H, rel_damp):
+    """diag of M for H + damp I = M M^T (M upper), float64."""
+    C = H.shape[0]
+    Hd = 0.5 * (H + H.T)
+    Hd[np.diag_indices(C)] += rel_damp * np.mean(np.diag(H))
+    return np.diag(np.linalg.cholesky(Hd[::-1, ::-1])[::-1, ::-1]).copy()
+
+
+def test_sparse14_look_ahead_in_float64():
+    """The 1:4 mask score reads three columns that have not received all their updates; in
+    the displacement form those hold different numbers.  Rebuilt through the inverse of N's
+    4x4 diagonal block they give the error form's masks and codes exactly; left as they are
+    they do not."""
+    C, R = 128, 32
+    pr = random_problem(C=C, R=R, n=200, seed=5)
+    H = pr["H"].double().numpy()
+    H = 0.5 * (H + H.T)
+    U0 = mathref.factor(H, 0.01, normalise=False)
+    Ut, uinv = U0 / np.diag(U0)[:, None], 1.0 / np.diag(U0)
+    assert np.allclose(uinv, _reverse_factor_diag(H, 0.01), rtol=1e-9)
+    V = mathref.direct_factor(H, 0.01)
+    W = pr["W"].double().numpy()
+    s, z = pr["se"].t().double().numpy(), pr["ze"].t().double().numpy()
+
+    def run(form):
+        X, Q, mask = W.copy(), np.zeros((R, C)), np.zeros((R, C), bool)
+        for t in range(C):
+            if t % 4 == 0:
+                look = X[:, t:t + 4]
+                if form == "d":   # "d-uncorrected" skips this
+                    v = V[t:t + 4, t:t + 4]
+                    A = np.eye(4)
+                    A[0, 1], A[1, 2], A[2, 3] = v[0, 1], v[1, 2], v[2, 3]
+                    A[0, 2] = v[0, 2] + v[0, 1] * v[1, 2]
+                    A[1, 3] = v[1, 3] + v[1, 2] * v[2, 3]
+                    A[0, 3] = v[0, 3] + v[0, 1] * A[1, 3] + v[0, 2] * v[2, 3]
+                    look = W[:, t:t + 4] + (X[:, t:t + 4] - W[:, t:t + 4]) @ A
+                mask[np.arange(R), t + np.abs(look * uinv[None, t:t + 4]).argmax(1)] = True
+            q = np.clip(np.rint(X[:, t] / (s[:, t] + 1e-12) + z[:, t]), 0, 15)
+            deq = np.where(mask[:, t], (q - z[:, t]) * s[:, t], 0.0)
+            Q[:, t] = np.where(mask[:, t], q, 0)
+            if form == "e":
+                X[:, t + 1:] -= np.outer(X[:, t] - deq, Ut[t, t + 1:])
+            else:
+                X[:, t + 1:] -= np.outer(W[:, t] - deq, V[t, t + 1:])
+        return Q, mask
+
+    (Qe, Me), (Qd, Md), (Qn, Mn) = run("e"), run("d"), run("d-uncorrected")
+    assert np.array_equal(Me, Md) and np.array_equal(Qe, Qd)
+    assert not np.array_equal(Me, Mn)
+
+
+def test_sparse14_checker_against_the_reference_form():
+    for C, R, n, seed in ((256, 64, 500, 1), (200, 33, 150, 2), (512, 32, 300, 3)):
+        pr = random_problem(C=C, R=R, n=n, seed=seed)
+        H = pr["H"].double().numpy()
+        U0 = torch.from_numpy(mathref.factor(H, 0.01, normalise=False)).float().contiguous()
+        V = torch.from_numpy(mathref.direct_factor(H, 0.01)).float().contiguous()
+        mdiag = torch.from_numpy(_reverse_factor_diag(H, 0.01)).float()
+        Wt = pr["W"].t().contiguous()
+        qe, Me = oracle.sparsegptq14_solver(Wt.clone(), U0.clone(), pr["se"], pr["ze"], 4)
+        qd, Md = oracle.sparsegptq14_solver_direct(Wt.clone(), V, mdiag, pr["se"], pr["ze"], 4)
+        be = np.unpackbits(Me.numpy().view(np.uint8), bitorder="little")
+        bd = np.unpackbits(Md.numpy().view(np.uint8), bitorder="little")
+        assert bd.reshape(-1, 4).sum(1).max() <= 1          # at most one kept weight per group of four
+        assert (be != bd).mean() <= 1e-3 and flip_rate(qe, qd) <= 3e-3
