@@ -96,7 +96,7 @@ def make_workload(cfg, chunk, seed=0):
 STREAMS = []
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True):
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"):
     """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
     jobs one after the other (per-kernel event times are then exclusive)."""
     from forge.moe import ExpertGroupGPTQ
@@ -118,7 +118,7 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True):
         offs.append(offs[-1] + wl["counts"][e])
     kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"],
               quantization_scale="mse" if mse else "absmax", quantization_order=cfg["order"],
-              rel_damp=0.01, device="cuda")
+              rel_damp=0.01, device="cuda", factor_route=factor_route)
     # gate/up (shared Hessian) and down are independent: one host thread and one HIP stream
     # each, so that the MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale
     # search and the latency-bound diagonal blocks of the other
@@ -204,6 +204,9 @@ def main():
                     help="sub-batches of a step's experts solved concurrently (one HIP stream each "
                          "for their gate/up and their down groups)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--factor-route", default="direct", choices=["direct", "inverse"],
+                    help="direct (default): sweep fed by the factor of H itself; inverse: the "
+                         "reference's factor of inv(H) and fp32-chain sweep")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run of "
@@ -231,18 +234,18 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     for i in range(a.warmup):
-        run_step(wl, cfg, chunk, i, mse)
+        run_step(wl, cfg, chunk, i, mse, factor_route=a.factor_route)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(a.steps):
-        run_step(wl, cfg, chunk, a.warmup + i, mse)
+        run_step(wl, cfg, chunk, a.warmup + i, mse, factor_route=a.factor_route)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
     # one more step with per-kernel HIP-event timing (on the stream the kernels run on); its
     # jobs run one after the other so that no kernel's time includes another stream's work
     kernels.timing_enable(True)
-    run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False)
+    run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False, factor_route=a.factor_route)
     torch.cuda.synchronize()
     stats = kernels.timing_collect()
     kernels.timing_enable(False)
@@ -260,7 +263,8 @@ def main():
     achieved = round(breakdown[dom]["rate"] * executed, 2)
     roofline = dict(kernel=dom, bound=bound, achieved=achieved, peak=PEAK[peak_key],
                     unit=unit, frac=round(achieved / PEAK[peak_key], 4),
-                    traffic=MEASURED_TRAFFIC.get((a.config, chunk, dom)) if a.split == 1 else None,
+                    traffic=MEASURED_TRAFFIC.get((a.config, chunk, dom))
+                    if a.split == 1 and a.factor_route == "direct" and mse else None,
                     avg_launch_us=breakdown[dom]["avg_us"], launches=breakdown[dom]["launches"])
 
     out = {
@@ -276,7 +280,7 @@ def main():
                                f" 4-bit {'sym' if cfg['symmetric'] else 'asym'} g128"
                                f" {'act-order' if cfg['order'] == 'activation' else 'no act-order'}"
                                f" {'mse' if mse else 'absmax'} grid",
-                   "experts_per_step": chunk},
+                   "experts_per_step": chunk, "factor_route": a.factor_route},
         "roofline": roofline,
         "kernels": breakdown,
     }
