@@ -18,6 +18,7 @@
 // The host schedules them left-looking (batched experts: each column block is brought
 // up to date with ONE long-K GEMM over all earlier errors, so the weights stream through
 // HBM once) or right-looking (a single matrix: more tiles in flight per step).
+#include <cstdlib>
 #include "common.h"
 #include "chain_gemm.h"
 
@@ -447,6 +448,15 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
     FORGE_REQUIRE(!sparse14 || (M && uinv), "sparse14 needs M and uinv");
     FORGE_REQUIRE(W0 != X, "W0 must be a copy of X, not X itself");
     hipStream_t st = (hipStream_t)stream;
+    // Few matrices: a left-looking step has only batch * R/128 tiles, far fewer than the GPU
+    // has CUs.  Then every finished block is pushed into ALL later columns at once instead
+    // (K = 128, (C - start)/128 times as many tiles); the weights are re-read per step, which
+    // a batch could not afford.  Same fma chain per element, hence the same bits.
+    bool right_looking = batch * forge::ceil_div(R, 128) < 128;
+    if (const char* forced = getenv("FORGE_SWEEP_SCHEDULE")) {   // read per call: tests flip it
+        if (forced[0] == 'l') right_looking = false;
+        if (forced[0] == 'r') right_looking = true;
+    }
     for (int64_t start = 0; start < C; start += forge::kBW) {
         const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
         forge::GemmArgs g{};
@@ -454,7 +464,9 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         g.xs = C * R; g.as = C * C; g.bs = C * R;
         g.m0 = (int)start; g.m1 = (int)(start + bw); g.n1 = (int)R; g.k0 = 0; g.k1 = (int)start;
         g.negate_a = true;
-        if (ws) {
+        if (right_looking) {
+            // nothing to do here: the earlier blocks have already been pushed into this one
+        } else if (ws) {
             // sums of 128 products each, three bf16 pieces per operand on the bf16 matrix pipe
             // where the block is a full tile (fp32 matrix pipe otherwise)
             g.blocked_sum = true;
@@ -472,6 +484,10 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
                 : W0     ? launch_block<false, false, true>(a, batch, st)
                          : launch_block<false, false>(a, batch, st);
         if (e) return e;
+        if (right_looking && start + bw < C) {
+            g.m0 = (int)(start + bw); g.m1 = (int)C; g.k0 = (int)start; g.k1 = (int)(start + bw);
+            if (int e2 = forge::launch_chain_gemm(g, batch, st)) return e2;
+        }
     }
     return FORGE_OK;
 }

@@ -97,7 +97,12 @@ int forge_sparsegptq14_solver(float* W, float* U, const float* scales, const flo
  * entry and the per-column errors on exit; U[b] [C, C]; scalesT/qzerosT[b] [G, R] f32
  * (group-major); g_idx[b] [C] int32 = group of solver column c; qweight[b] [C, R] u8.
  * sparse14 != 0 selects the 1:4 joint solve (then M[b] [ceil(C/32), R] u32 and
- * uinv[b] [C] must be given and U must already be row-normalised). */
+ * uinv[b] [C] must be given and U must already be row-normalised).
+ * Schedule: with at least 128 tiles of 128 rows (batch * ceil(R/128)) each column block is
+ * brought up to date by one long product over all earlier columns just before it is swept;
+ * with fewer, every finished block is pushed into all later columns at once (more tiles per
+ * launch).  Same fma chain per element either way, identical results.  FORGE_SWEEP_SCHEDULE=left
+ * or =right in the environment forces one of them. */
 int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
                              const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                              uint32_t* M, const float* uinv, int64_t batch, int64_t C,

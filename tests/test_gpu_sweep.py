@@ -141,6 +141,39 @@ def test_direct_sparse14_sweep_bit_exact(hip, C, R, n):
     assert (M2.view(torch.int32) != M.view(torch.int32)).float().mean().item() <= 3e-3
 
 
+def test_sweep_schedules_and_block_update_kernels_agree(hip, monkeypatch):
+    """32 matrices of 512 rows (128 row tiles: the left-looking schedule by default).  The
+    reference-form sweep gives the same codes under both schedules; the displacement form
+    gives the same codes under both schedules with the fp32 chain, and with the bf16-piece
+    block updates (left-looking only) all but near-ties."""
+    B, C, R, gs = 32, 512, 512, 128
+    G = C // gs
+    g = torch.Generator().manual_seed(41)
+    X = (0.02 * torch.randn(B, C, R, generator=g)).to(DEV)
+    A = torch.randn(B, 2 * C, C, generator=g).to(DEV)
+    H = (2.0 / (2 * C)) * A.transpose(1, 2) @ A
+    damp = 0.01 * torch.diagonal(H, dim1=1, dim2=2).mean(1)
+    U, _, info = hip.chol_inv_upper_batched(H.clone(), damp)
+    L, info2 = hip.chol_reverse_lower_batched(H.clone(), damp)
+    assert not info.any() and not info2.any()
+    V = hip.unit_upper_from_lower(L, info2, negate=True, upper_only=True)
+    amax = X.view(B, G, gs, R).abs().amax(2)
+    sT = (2.0 / 15.0 * amax + 1e-12).contiguous()
+    zT = torch.full_like(sT, 8.0)
+    gi = (torch.arange(C) // gs).int().repeat(B, 1).to(DEV)
+    out = {}
+    for sched in ("left", "right"):
+        monkeypatch.setenv("FORGE_SWEEP_SCHEDULE", sched)
+        out["ref", sched] = hip.gptq_sweep_batched(X.clone(), U, sT, zT, gi, 4)
+        out["direct", sched] = hip.gptq_sweep_direct_batched(X.clone(), V, sT, zT, gi, 4, exact_chain=True)
+    monkeypatch.delenv("FORGE_SWEEP_SCHEDULE")
+    assert torch.equal(out["ref", "left"], out["ref", "right"])
+    assert torch.equal(out["direct", "left"], out["direct", "right"])
+    q_bf16 = hip.gptq_sweep_direct_batched(X.clone(), V, sT, zT, gi, 4)
+    assert (q_bf16 != out["direct", "left"]).float().mean().item() <= 1e-3
+    assert (out["ref", "left"] != out["direct", "left"]).float().mean().item() <= 3e-3
+
+
 def test_direct_factor_on_the_gpu(hip):
     """chol_reverse_lower_batched + unit_upper_from_lower(negate=True) give the V of the
     displacement form: against float64, and I - strict(V) inverts the reference's factor."""
