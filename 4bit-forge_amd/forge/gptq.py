@@ -40,9 +40,19 @@ def _as_calibration_rows(X: torch.Tensor, device) -> torch.Tensor:
 class GPTQ(object):
     def __init__(self, layer, bits: int = 4, group_size: int = 128, symmetric: bool = False,
                  quantization_scale: str = "mse", quantization_order: str = "activation",
-                 rel_damp: float = 1e-2, algorithm: str = "gptq", owner=None, device=None):
+                 rel_damp: float = 1e-2, algorithm: str = "gptq", owner=None, device=None,
+                 factor_route: str = "inverse"):
+        """Arguments of the reference's class (forge/gptq.py:11-22) plus ``factor_route``
+        (algorithm="gptq" only): "inverse", the default, follows the reference's
+        factorisation (Cholesky, inverse, Cholesky of the inverse) and its error-propagating
+        sweep; "direct" stops at the factor of H itself and sweeps with the displacements
+        w - deq, which is the same solve in exact arithmetic at half the factorisation work
+        (see ``forge.moe.ExpertGroupGPTQ``)."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
+        if factor_route not in ("direct", "inverse"):
+            raise ValueError(f"factor_route={factor_route!r}: 'direct' or 'inverse'")
+        self.factor_route = factor_route
         self.layer = layer
         self.device = torch.device(device) if device is not None else layer.weight.device
         if self.device.type != "cuda":
@@ -183,6 +193,11 @@ class GPTQ(object):
             if int(info.item()) > 0:
                 self.issue_non_invertible = True
             return kernels.unit_upper_from_lower(L, info)[0]
+        if self.algorithm == "gptq" and self.factor_route == "direct":
+            L, info = kernels.chol_reverse_lower_batched(H.clone().view(1, C, C), None)
+            if int(info.item()) > 0:
+                self.issue_non_invertible = True
+            return kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)[0]
         U, _, info = kernels.chol_inv_upper_batched(H.clone().view(1, C, C), None,
                                                     normalise=self.algorithm == "gptq")
         if int(info.item()) > 0:
@@ -217,6 +232,9 @@ class GPTQ(object):
         g_idx = (self.perm // gs).to(torch.int32).view(1, C)
         sT = scales.view(R, G).t().contiguous().view(1, G, R)
         zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
-        q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
+        if self.factor_route == "direct":
+            q = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
+        else:
+            q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
         qw = kernels.codes_to_layer_order(q, self.perm_inv.view(1, C))[0]
         return qw, scales, qzeros

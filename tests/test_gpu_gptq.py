@@ -79,6 +79,30 @@ def test_dense_layer_end_to_end(kw):
     assert abs(eg / eo - 1) < 0.01
 
 
+def test_dense_layer_direct_route():
+    """The class with factor_route="direct" (factor of H itself, displacement sweep): same
+    tolerances against the reference-form oracle as the default route."""
+    from forge.gptq import GPTQ
+    case = synth.dense_outlier(R=256, C=1024, n=1024, seed=1)
+    kw = dict(bits=4, rel_damp=0.01, group_size=128, symmetric=False, quantization_scale="mse",
+              quantization_order="activation")
+    o = oracle.GPTQ(linear(case.W), **kw)
+    g = GPTQ(linear(case.W).to(DEV), device=DEV, factor_route="direct", **kw)
+    o.update(case.X)
+    g.update(case.X.to(DEV))
+    H = o.H.double().numpy().copy()
+    qo, so, zo = o.quantize()
+    qg, sg, zg = (t.cpu() for t in g.quantize())
+    same = so == sg
+    assert float((~same).float().mean()) <= 1e-3 and torch.equal(zo[same], zg[same])
+    floor = _noise_floor(case.W, o, so, zo)
+    assert flip_rate(qo, qg) <= max(1e-3, 3 * floor)
+    Wf = case.W.numpy()
+    eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H)
+    eg = mathref.layer_error(Wf, oracle.dequantize(qg, sg, zg, 128).numpy(), H)
+    assert abs(eg / eo - 1) < 0.01
+
+
 def test_fallbacks_zero_tokens_nan_dead_column_and_non_pd():
     from forge.gptq import GPTQ
     g0 = torch.Generator().manual_seed(2)
