@@ -15,8 +15,19 @@
 // load per lane and never touches LDS in its K loop.  Tokens are zero padded to a
 // multiple of 16 per group.  fp32 tokens use v_mfma_f32_32x32x2_f32 on K-major tiles
 // staged through LDS (no transpose needed for that instruction's operand layout).
+//
+// The diagonal is not taken from the matrix pipe: H[c][c] decides the activation order
+// (argsort of diag(H), forge/gptq.py:107-110), and with thousands of columns neighbouring
+// diagonal entries lie closer together than the rounding error of an fp32 sum over the
+// tokens, so the order -- and through it a few per cent of the codes -- would depend on the
+// summation order.  A small kernel sums every column's squares in float64 (the squares of
+// bf16 and f32 values are exact there) and the update beta*old + alpha*sum is rounded to
+// fp32 once; the rank-k kernels write that value where row == column.
 #include "common.h"
 #include <hip/hip_bf16.h>
+#include <algorithm>
+#include <cstring>
+#include <mutex>
 #include <vector>
 
 namespace {
@@ -65,11 +76,75 @@ __device__ __forceinline__ void tile_pair(int p, int NT, int& ti, int& tj) {
     tj = i + p;
 }
 
+// ---------------------------------------------------------------- diagonal in float64
+// grid: (128-column slab, group).  Four wavefronts take every fourth token, two adjacent
+// columns per lane; partial sums meet in LDS and are added in wavefront order.
+// dnew[group][c] = (float)(beta * H[c][c] + alpha * sum_t x[t][c]^2).
+template <typename T>
+__device__ __forceinline__ double as_double(T v);
+template <>
+__device__ __forceinline__ double as_double<uint16_t>(uint16_t v) {
+    return (double)__uint_as_float((uint32_t)v << 16);
+}
+template <>
+__device__ __forceinline__ double as_double<float>(float v) { return (double)v; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void diag_float64_kernel(const T* __restrict__ X, int64_t ldx,
+                                                           int64_t C, const GroupDesc* __restrict__ gd,
+                                                           const float* __restrict__ Hall,
+                                                           float* __restrict__ dnew) {
+    __shared__ double part[4][128];
+    const GroupDesc g = gd[blockIdx.y];
+    if (g.n == 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t c0 = (int64_t)blockIdx.x * 128 + 2 * lane;
+    const bool in0 = c0 < C, in1 = c0 + 1 < C;
+    const T* __restrict__ col = X + g.row0 * ldx + (in0 ? c0 : 0);
+    double s0 = 0.0, s1 = 0.0;
+    int t = wave;
+    for (; t + 12 < g.n; t += 16) {             // four rows in flight per wavefront
+        T a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const T* r = col + (int64_t)(t + 4 * u) * ldx;
+            a[u] = in0 ? r[0] : T(0);
+            b[u] = in1 ? r[1] : T(0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const double x = as_double<T>(a[u]), y = as_double<T>(b[u]);
+            s0 = __builtin_fma(x, x, s0);
+            s1 = __builtin_fma(y, y, s1);
+        }
+    }
+    for (; t < g.n; t += 4) {
+        const T* r = col + (int64_t)t * ldx;
+        const double x = as_double<T>(in0 ? r[0] : T(0)), y = as_double<T>(in1 ? r[1] : T(0));
+        s0 = __builtin_fma(x, x, s0);
+        s1 = __builtin_fma(y, y, s1);
+    }
+    part[wave][2 * lane] = s0;
+    part[wave][2 * lane + 1] = s1;
+    __syncthreads();
+    if (threadIdx.x < 128) {
+        const int64_t c = (int64_t)blockIdx.x * 128 + threadIdx.x;
+        if (c < C) {
+            const double s = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) +
+                             part[3][threadIdx.x];
+            double o = (double)g.alpha * s;
+            if (g.beta != 0.0f)
+                o += (double)g.beta * (double)Hall[(int64_t)blockIdx.y * C * C + c * C + c];
+            dnew[(int64_t)blockIdx.y * C + c] = (float)o;
+        }
+    }
+}
+
 // Write one 32x32 accumulator tile (and its mirror image) with out = alpha*acc + beta*H.
 // Called by all four wavefronts of the workgroup together (it synchronises them).
 __device__ __forceinline__ void store_tile(float* __restrict__ H, int64_t C, int row0, int col0,
                                            const f32x16& acc, float alpha, float beta, bool mirror,
-                                           float (*tbuf)[33], int lane) {
+                                           float (*tbuf)[33], int lane, const float* __restrict__ dn) {
     f32x16 out;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -77,7 +152,8 @@ __device__ __forceinline__ void store_tile(float* __restrict__ H, int64_t C, int
         const int j = col0 + (lane & 31);
         float o = alpha * acc[v];
         if (i < C && j < C) {
-            if (beta != 0.0f) o = __builtin_fmaf(beta, H[(int64_t)i * C + j], o);
+            if (i == j) o = dn[i];                     // the float64 diagonal
+            else if (beta != 0.0f) o = __builtin_fmaf(beta, H[(int64_t)i * C + j], o);
             H[(int64_t)i * C + j] = o;
         }
         out[v] = o;
@@ -104,7 +180,7 @@ template <bool BLEND>
 __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict__ pack,
                                                         const GroupDesc* __restrict__ gd,
                                                         float* __restrict__ Hall, int64_t C,
-                                                        int NT) {
+                                                        int NT, const float* __restrict__ dnew) {
     __shared__ float tbuf[4][32][33];
     const GroupDesc g = gd[blockIdx.y];
     if (g.n == 0) return;
@@ -113,6 +189,7 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     float* __restrict__ H = Hall + (int64_t)blockIdx.y * C * C;
+    const float* __restrict__ dn = dnew + (int64_t)blockIdx.y * C;
     const int nct = (int)((C + 31) / 32);
 
     int cta[2], ctb[2];
@@ -185,6 +262,12 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
                     if (BLEND && blend) o = __builtin_fmaf(g.beta, old[mi][ni][v], o);
                     out[v] = o;
                 }
+                if (row0 == col0) {                     // the float64 diagonal
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if ((v >> 2) * 8 + (lane >> 5) * 4 + (v & 3) == (lane & 31))
+                            out[v] = dn[row0 + (lane & 31)];
+                }
                 float* __restrict__ Ht = H + (int64_t)(row0 + (lane >> 5) * 4) * C + col0 + (lane & 31);
 #pragma unroll
                 for (int v = 0; v < 16; ++v) Ht[(int64_t)((v >> 2) * 8 + (v & 3)) * C] = out[v];
@@ -211,7 +294,7 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni)
                 store_tile(H, C, cta[mi] * 32, ctb[ni] * 32, acc[mi][ni], g.alpha, g.beta, mirror,
-                           tbuf[wave], lane);
+                           tbuf[wave], lane, dn);
     }
 }
 
@@ -220,7 +303,8 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
 constexpr int TK = 16;
 __global__ __launch_bounds__(256) void syrk_f32_kernel(const float* __restrict__ X, int64_t ldx,
                                                        const GroupDesc* __restrict__ gd,
-                                                       float* __restrict__ Hall, int64_t C, int NT) {
+                                                       float* __restrict__ Hall, int64_t C, int NT,
+                                                       const float* __restrict__ dnew) {
     __shared__ __attribute__((aligned(16))) float As[2][TK][128];
     __shared__ __attribute__((aligned(16))) float Bs[2][TK][128];
     __shared__ float tbuf[4][32][33];
@@ -301,11 +385,87 @@ __global__ __launch_bounds__(256) void syrk_f32_kernel(const float* __restrict__
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
             store_tile(H, C, mt + wm * 64 + mi * 32, nt + wn * 64 + ni * 32, acc[mi][ni], g.alpha,
-                       g.beta, mirror, tbuf[wave], lane);
+                       g.beta, mirror, tbuf[wave], lane, dnew + (int64_t)blockIdx.y * C);
 }
 
 int64_t pack_units(int64_t n, int64_t C) {  // 16-byte units for one group
     return forge::ceil_div(n, 16) * forge::ceil_div(C, 32) * 64;
+}
+
+int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
+
+// Pinned host blocks through which group tables travel to the device.  A call fills a
+// block whose previous upload has completed (its event says so), enqueues the copy and
+// returns: the host thread never waits for the stream.  Blocks live until the process ends.
+struct UploadBlock {
+    void* host;
+    int64_t bytes;
+    hipEvent_t done;
+    bool used;
+};
+std::mutex g_upload_mu;
+std::vector<UploadBlock> g_upload;
+
+int upload_async(const void* src, int64_t bytes, void* dst, hipStream_t st) {
+    std::lock_guard<std::mutex> lock(g_upload_mu);
+    UploadBlock* blk = nullptr;
+    for (auto& b : g_upload)
+        if (b.bytes >= bytes && (!b.used || hipEventQuery(b.done) == hipSuccess)) {
+            blk = &b;
+            break;
+        }
+    if (!blk) {
+        UploadBlock b{nullptr, std::max<int64_t>(bytes, 16384), nullptr, false};
+        FORGE_HIP_CHECK(hipHostMalloc(&b.host, (size_t)b.bytes, hipHostMallocDefault));
+        FORGE_HIP_CHECK(hipEventCreateWithFlags(&b.done, hipEventDisableTiming));
+        g_upload.push_back(b);
+        blk = &g_upload.back();
+    }
+    memcpy(blk->host, src, (size_t)bytes);
+    FORGE_HIP_CHECK(hipMemcpyAsync(dst, blk->host, (size_t)bytes, hipMemcpyHostToDevice, st));
+    FORGE_HIP_CHECK(hipEventRecord(blk->done, st));
+    blk->used = true;
+    return FORGE_OK;
+}
+
+// The launches of one update; gd_dev already holds the group table.
+int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const GroupDesc* gd_dev,
+                  int64_t n_groups, int64_t total, int max_chunks, bool any_blend, float* H,
+                  float* dnew, uint4* pack, hipStream_t st) {
+    const int NT = (int)forge::ceil_div(C, 128);
+    const unsigned pairs = (unsigned)(NT * (NT + 1) / 2);
+    const dim3 dgrid((unsigned)NT, (unsigned)n_groups);
+    if (x_dtype == FORGE_BF16) {
+        diag_float64_kernel<uint16_t><<<dgrid, dim3(256), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev,
+                                                                   H, dnew);
+        FORGE_LAUNCH_CHECK();
+        const unsigned ychunks = (unsigned)(max_chunks < 64 ? max_chunks : 64);
+        pack_bf16_kernel<<<dim3((unsigned)forge::ceil_div(C, 32), ychunks, (unsigned)n_groups),
+                           dim3(64), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev, pack);
+        FORGE_LAUNCH_CHECK();
+        // executed flops: tiles on and above the diagonal only
+        forge::KernelTiming timing("hessian_syrk_bf16", st,
+                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
+                                   forge::WORK_FLOPS);
+        if (any_blend)
+            syrk_bf16_kernel<true><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
+                pack, gd_dev, H, C, NT, dnew);
+        else
+            syrk_bf16_kernel<false><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
+                pack, gd_dev, H, C, NT, dnew);
+        FORGE_LAUNCH_CHECK();
+    } else {
+        diag_float64_kernel<float><<<dgrid, dim3(256), 0, st>>>((const float*)X, ldx, C, gd_dev, H,
+                                                                dnew);
+        FORGE_LAUNCH_CHECK();
+        forge::KernelTiming timing("hessian_syrk_f32", st,
+                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
+                                   forge::WORK_FLOPS);
+        syrk_f32_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
+            (const float*)X, ldx, gd_dev, H, C, NT, dnew);
+        FORGE_LAUNCH_CHECK();
+    }
+    return FORGE_OK;
 }
 
 }  // namespace
@@ -313,7 +473,7 @@ int64_t pack_units(int64_t n, int64_t C) {  // 16-byte units for one group
 extern "C" int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int64_t C,
                                                  int x_dtype) {
     if (n_groups <= 0 || C <= 0) return 0;
-    int64_t bytes = n_groups * (int64_t)sizeof(GroupDesc) + 256;
+    int64_t bytes = round256(n_groups * (int64_t)sizeof(GroupDesc)) + round256(n_groups * C * 4);
     if (x_dtype == FORGE_BF16) bytes += pack_units(total_rows + 16 * n_groups, C) * 16;
     return bytes;
 }
@@ -339,7 +499,7 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
     std::vector<GroupDesc> gd((size_t)n_groups);
     int64_t off = 0;
     int max_chunks = 0;
-    bool any = false;
+    bool any = false, any_blend = false;
     for (int64_t e = 0; e < n_groups; ++e) {
         const int64_t n = offsets_host[e + 1] - offsets_host[e];
         FORGE_REQUIRE(n >= 0 && n < (1LL << 31), "offsets must be non-decreasing");
@@ -352,43 +512,15 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
         off += pack_units(n, C);
         if (gd[e].nchunk > max_chunks) max_chunks = gd[e].nchunk;
         any |= n > 0;
+        any_blend |= n > 0 && beta_host[e] != 0.0f;
     }
     if (!any) return FORGE_OK;
     GroupDesc* gd_dev = (GroupDesc*)ws;
-    const int64_t desc_bytes = ((n_groups * (int64_t)sizeof(GroupDesc) + 255) / 256) * 256;
-    FORGE_HIP_CHECK(hipMemcpyAsync(gd_dev, gd.data(), n_groups * sizeof(GroupDesc),
-                                   hipMemcpyHostToDevice, st));
-    // the host vector dies with this call: make sure the copy has been consumed
-    FORGE_HIP_CHECK(hipStreamSynchronize(st));
-
-    const int NT = (int)forge::ceil_div(C, 128);
-    const unsigned pairs = (unsigned)(NT * (NT + 1) / 2);
-    if (x_dtype == FORGE_BF16) {
-        uint4* pack = (uint4*)((char*)ws + desc_bytes);
-        const unsigned ychunks = (unsigned)(max_chunks < 64 ? max_chunks : 64);
-        pack_bf16_kernel<<<dim3((unsigned)forge::ceil_div(C, 32), ychunks, (unsigned)n_groups),
-                           dim3(64), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev, pack);
-        FORGE_LAUNCH_CHECK();
-        // executed flops: tiles on and above the diagonal only
-        forge::KernelTiming timing("hessian_syrk_bf16", st,
-                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
-                                   forge::WORK_FLOPS);
-        bool any_blend = false;
-        for (int e = 0; e < n_groups; ++e) any_blend = any_blend || beta_host[e] != 0.0f;
-        if (any_blend)
-            syrk_bf16_kernel<true><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev,
-                                                                                         H, C, NT);
-        else
-            syrk_bf16_kernel<false><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(pack, gd_dev,
-                                                                                          H, C, NT);
-        FORGE_LAUNCH_CHECK();
-    } else {
-        forge::KernelTiming timing("hessian_syrk_f32", st,
-                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
-                                   forge::WORK_FLOPS);
-        syrk_f32_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
-            (const float*)X, ldx, gd_dev, H, C, NT);
-        FORGE_LAUNCH_CHECK();
-    }
-    return FORGE_OK;
+    const int64_t desc_bytes = round256(n_groups * (int64_t)sizeof(GroupDesc));
+    float* dnew = (float*)((char*)ws + desc_bytes);
+    uint4* pack = (uint4*)((char*)ws + desc_bytes + round256(n_groups * C * 4));
+    // through a pinned block of the library's own: the host does not wait for the copy
+    if (int rc = upload_async(gd.data(), n_groups * (int64_t)sizeof(GroupDesc), gd_dev, st)) return rc;
+    return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, any_blend, H, dnew,
+                         pack, st);
 }

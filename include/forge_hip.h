@@ -163,8 +163,11 @@ int64_t forge_babai_workspace_bytes(int64_t C, int64_t R, int64_t G);
  * alpha_host/beta_host [n_groups] are host arrays (the caller owns the running-mean
  * bookkeeping); H[e] is not read when beta[e] == 0.  Groups with zero rows are left
  * untouched.  bf16 inputs use bf16 MFMA with fp32 accumulation (products exact); f32
- * inputs use f32 MFMA.  ws: device workspace of forge_hessian_workspace_bytes(total rows,
- * n_groups, C, x_dtype).  Synchronises `stream` once (after uploading the group table). */
+ * inputs use f32 MFMA.  The diagonal entries, which decide the activation order
+ * (gptq.py:107-110), are summed in float64 and rounded to f32 once per call.  ws: device
+ * workspace of forge_hessian_workspace_bytes(total rows, n_groups, C, x_dtype).  The host
+ * arrays are consumed before the call returns; nothing waits for the stream (the group
+ * table travels through pinned memory that the library keeps). */
 int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_t C,
                                  const int64_t* offsets_host, int64_t n_groups,
                                  const float* alpha_host, const float* beta_host, float* H,
