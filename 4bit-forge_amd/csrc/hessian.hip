@@ -318,13 +318,13 @@ __global__ __launch_bounds__(256) void syrk_f32_kernel(const float* __restrict__
     const float* __restrict__ Xg = X + g.row0 * ldx;
     const int mt = ti * 128, nt = tj * 128;
 
-    f32x16 acc[2][2];
+    f32x16 acc[2][2], tot[2][2];
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = tot[mi][ni][v] = 0.0f;
 
     const int lrow = tid >> 5, lcol = (tid & 31) * 4;
     float4 ra[2], rb[2];
@@ -378,7 +378,27 @@ __global__ __launch_bounds__(256) void syrk_f32_kernel(const float* __restrict__
         if (more) stage(buf ^ 1);
         __syncthreads();
         buf ^= 1;
+        // Blocked summation: the matrix instruction adds its products to the accumulator one
+        // after the other, so a single chain over n tokens carries a rounding error that grows
+        // like sqrt(n).  Every 128 tokens the chain is folded into a second set of sums.
+        if (((kk / TK) & 7) == 7 && more) {
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        tot[mi][ni][v] += acc[mi][ni][v];
+                        acc[mi][ni][v] = 0.0f;
+                    }
+        }
     }
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] += tot[mi][ni][v];
     const bool mirror = ti != tj;
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)

@@ -383,7 +383,17 @@ class GPTQ:
                 self.issue_non_invertible = True
                 A = torch.eye(C, dtype=torch.float32)
             return A
+        U, info = self._factor_upper(H)
+        if int(info) > 0:
+            self.issue_non_invertible = True
+            U = torch.eye(C, dtype=torch.float32)
+        return U
+
+    def _factor_upper(self, H):
+        """gptq.py:160-166: upper Cholesky factor of inv(H) through LAPACK's potrf, potri,
+        potrf in fp32, rows divided by the diagonal for "gptq".  Returns (U, info)."""
         L, info = torch.linalg.cholesky_ex(H, upper=False)
+        U = None
         try:
             Hinv = torch.cholesky_inverse(L, upper=False)
             U, info2 = torch.linalg.cholesky_ex(Hinv, upper=True)
@@ -392,12 +402,9 @@ class GPTQ:
                 U = U / U.diag()[:, None]
         except RuntimeError:
             # torch's CPU potri raises on a singular factor instead of carrying on; the
-            # outcome the reference codes for is the identity fallback below
+            # outcome the reference codes for is the identity fallback of the caller
             info = info + 1
-        if int(info.item()) > 0:
-            self.issue_non_invertible = True
-            U = torch.eye(C, dtype=torch.float32)
-        return U
+        return U, int(info.item())
 
     def _expand(self, v, C, R):
         # gptq.py:251-252: per-element [C,R] meta in solver (permuted) column order.
@@ -410,6 +417,7 @@ class GPTQ:
         self._prep()
         scales, qzeros = self._quant_grid()
         U = self._h_factor()
+        self.last_factor = U            # kept for tests that swap single stages
         W = self.W.clone().transpose(-2, -1)[self.perm]
         C, R = W.shape
         if self.algorithm == "babai":

@@ -38,3 +38,49 @@ def random_problem(C, R, n=None, sym=True, gs=128, seed=0, outliers=3, mse=False
 
 def flip_rate(a, b):
     return (a.cpu() != b.cpu()).float().mean().item()
+
+
+class Float64StagesGPTQ(oracle.GPTQ):
+    """The oracle's per-layer flow with its two fp32 LIBRARY stages -- the SGEMM that sums the
+    Hessian (gptq.py:79) and LAPACK's potrf/potri/potrf (gptq.py:160-164) -- computed in
+    float64 and rounded to fp32 once.  The reference fixes neither library's summation order,
+    so this is as valid a realisation of its arithmetic as the oracle's own, and the most
+    accurate one; everything else (activation order from the fp32 diagonal, damping, grid
+    search, the sweep's fma chain) is the oracle's code unchanged.
+
+    flips(oracle, this) is the FLOOR the end-to-end tests use: how far the reference's codes
+    move when only the rounding inside those two library calls changes."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self._sum64 = None
+
+    def update(self, X):
+        if not self._is_owner():
+            return
+        X = X.reshape(-1, X.shape[-1]).to(device="cpu", dtype=torch.float64)
+        if X.shape[0] == 0:
+            return
+        S = X.T @ X
+        self._sum64 = S if self._sum64 is None else self._sum64 + S
+        self.num_samples.add_(X.shape[0])
+        self.H = ((2.0 / int(self.num_samples.item())) * self._sum64).float()
+
+    add_batch = update
+
+    def _factor_upper(self, H):
+        try:
+            U = mathref.factor(H.double().numpy(), 0.0, normalise=self.algorithm == "gptq")
+        except np.linalg.LinAlgError:
+            return None, 1
+        return torch.from_numpy(U).float().contiguous(), 0
+
+
+def reference_floor(W, batches, qo, **kw):
+    """(floor, q64): q64 = codes of Float64StagesGPTQ on the same inputs, floor = the share
+    of the oracle's codes `qo` that differ from them."""
+    t = Float64StagesGPTQ(linear(W), **kw)
+    for b in batches:
+        t.update(b)
+    out = t.quantize()
+    return flip_rate(qo, out[0]), out

@@ -1,12 +1,17 @@
 """End-to-end: forge.gptq.GPTQ / forge.moe.ExpertGroupGPTQ on the GPU against oracle.GPTQ.
 
 Tolerances.  Scales and zeros: equal (MSE: except candidate ties, <= 0.1 % of groups,
-checked in test_gpu_grid).  Codes: with the SAME factor the sweep is bit-exact
-(test_gpu_sweep); end to end the factor comes from a different fp32 algorithm than
-LAPACK's, and GPTQ's rounding decisions amplify last-bit differences of U, so the oracle
-itself moves by FLOOR = flips(LAPACK fp32 factor vs float64 factor) when only its factor's
-rounding changes.  The GPU result must stay within max(1e-3, 3 * FLOOR) of the oracle and
-its layer output error ||WX - QX||^2 within 1 % of the oracle's.
+checked in test_gpu_grid).  Codes: with the SAME Hessian and factor every integer stage is
+bit-exact at the benchmark shapes (test_gpu_stage_substitution).  End to end the Hessian sum
+and the factorisation are fp32 library calls in the reference (an SGEMM and LAPACK's
+potrf/potri/potrf, gptq.py:79,160-164) whose summation order it does not fix, and GPTQ's
+rounding decisions amplify their last bits: a flipped code changes the error fed to every
+later column of its row.  FLOOR = the share of the oracle's own codes that move when those
+two library stages are computed in float64 and rounded to fp32 once
+(helpers.Float64StagesGPTQ) -- the distance between two valid realisations of the reference.
+The GPU result must stay within max(1e-3, 1.5 * FLOOR) of the oracle, as close to the
+float64-stage result as that, and its layer output error ||WX - QX||^2 within 1 % of the
+oracle's.
 """
 import numpy as np
 import pytest
@@ -15,26 +20,22 @@ import torch
 import oracle
 from oracle import mathref
 from forge import synth
-from helpers import linear, flip_rate, expand_meta
+from helpers import linear, flip_rate, expand_meta, reference_floor
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
+FLOORS = 1.5
 
 
-def _noise_floor(W, o, scales, zeros):
-    """Flips of the oracle's own sweep when its fp32 LAPACK factor is replaced by the
-    float64 factor rounded to fp32 (same prepared Hessian, same grid)."""
-    R, C = W.shape
-    Hd = o.H.double().numpy().copy()                   # damped + permuted (after quantize)
-    U64 = torch.from_numpy(mathref.factor(Hd, 0.0)).float().contiguous()
-    L, _ = torch.linalg.cholesky_ex(o.H)
-    U32 = torch.linalg.cholesky_ex(torch.cholesky_inverse(L), upper=True)[0]
-    U32 = (U32 / U32.diag()[:, None]).contiguous()
-    Wt = o.W.float().t()[o.perm].contiguous()
-    se, ze = o._expand(scales, C, R), o._expand(zeros, C, R)
-    a = oracle.gptq_solver(Wt.clone(), U32, se, ze, 4)
-    b = oracle.gptq_solver(Wt.clone(), U64, se, ze, 4)
-    return flip_rate(a, b)
+def _codes_at_floor(tag, qo, qg, W, batches, kw, owner_batches=None):
+    """flips(GPU, oracle) and flips(GPU, float64-stage realisation) against the floor."""
+    floor, out64 = reference_floor(W, batches, qo, **kw)
+    flips, to64 = flip_rate(qo, qg), flip_rate(out64[0], qg)
+    print(f"{tag}: flips vs oracle {flips:.2e}, vs float64 stages {to64:.2e}, floor {floor:.2e}")
+    bound = max(1e-3, FLOORS * floor)
+    assert flips <= bound, (tag, flips, floor)
+    assert to64 <= bound, (tag, to64, floor)
+    return flips, floor, out64
 
 
 def _run_pair(W, X, chunks=2, **kw):
@@ -69,9 +70,7 @@ def test_dense_layer_end_to_end(kw):
     same = so == sg.cpu()
     assert float((~same).float().mean()) <= 1e-3
     assert torch.equal(zo[same], zg.cpu()[same])
-    floor = _noise_floor(case.W, o, so, zo)
-    flips = flip_rate(qo, qg)
-    assert flips <= max(1e-3, 3 * floor), (flips, floor)
+    _codes_at_floor("dense 256x1024", qo, qg, case.W, torch.chunk(case.X, 2), kw)
     gs = kw["group_size"]
     Wf = case.W.numpy()
     eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, gs).numpy(), H)
@@ -95,8 +94,7 @@ def test_dense_layer_direct_route():
     qg, sg, zg = (t.cpu() for t in g.quantize())
     same = so == sg
     assert float((~same).float().mean()) <= 1e-3 and torch.equal(zo[same], zg[same])
-    floor = _noise_floor(case.W, o, so, zo)
-    assert flip_rate(qo, qg) <= max(1e-3, 3 * floor)
+    _codes_at_floor("dense 256x1024 direct", qo, qg, case.W, [case.X], kw)
     Wf = case.W.numpy()
     eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H)
     eg = mathref.layer_error(Wf, oracle.dequantize(qg, sg, zg, 128).numpy(), H)
@@ -128,7 +126,8 @@ def test_fallbacks_zero_tokens_nan_dead_column_and_non_pd():
     h = GPTQ(linear(W).to(DEV), device=DEV, **kw); h.update(X.to(DEV))
     qo, so, zo = o.quantize(); qg, sg, zg = h.quantize()
     assert bool(h.pruned_ids[9]) and int(h.pruned_ids.sum()) == 1
-    assert torch.equal(so, sg.cpu()) and flip_rate(qo, qg) <= 2e-3
+    assert torch.equal(so, sg.cpu())
+    _codes_at_floor("dead column", qo, qg, W, [X], kw)
     assert torch.equal(qo[:, 9], qg.cpu()[:, 9])
     # not positive definite (rank 4, no damping): identity fallback + flag, like gptq.py:172-175
     h = GPTQ(linear(W).to(DEV), device=DEV, rel_damp=0.0, **kw)
@@ -155,7 +154,8 @@ def test_owner_sharing_reset_and_in_place_damping():
     qg_g, _, _ = hg.quantize(); qg_u, sg_u, _ = hu.quantize()
     assert torch.equal(hu.perm.cpu(), ou.perm) and int(hu.num_samples) == 400
     assert torch.equal(so_u, sg_u.cpu())
-    assert flip_rate(qo_g, qg_g) <= 3e-3 and flip_rate(qo_u, qg_u) <= 3e-3
+    _, floor, _ = _codes_at_floor("owner gate", qo_g, qg_g, Wg, [X], kw)
+    assert flip_rate(qo_u, qg_u) <= max(1e-3, FLOORS * floor) + 1e-3   # 48 x 256 codes: 1e-3 = 12 codes
     ratio = (hu.H.diagonal().cpu() - ou.H.diagonal()).abs().max() / ou.H.diagonal().abs().max()
     assert ratio < 1e-5                      # both damped twice
     hg.reset()
@@ -172,12 +172,13 @@ def test_sparse14_end_to_end():
     qg, sg, zg, Mg = g.quantize()
     assert tuple(Mg.shape) == (16, 192) and Mg.dtype == torch.uint32
     assert float((so != sg.cpu()).float().mean()) <= 1e-3
-    mask_diff = (Mo.view(torch.int32) != Mg.cpu().view(torch.int32)).float().mean().item()
-    assert mask_diff <= 5e-3 and flip_rate(qo, qg) <= 5e-3
+    _, floor, out64 = _codes_at_floor("sparse14 192x512", qo, qg, case.W, torch.chunk(case.X, 2), kw)
     bits = lambda M: ((M.view(torch.int32).cpu().numpy().astype(np.uint32)[np.arange(512) // 32]
                        >> (np.arange(512) % 32)[:, None]) & 1)
     keep = bits(Mg)
     assert np.all(keep.reshape(128, 4, 192).sum(axis=1) == 1)           # exactly 1 of 4 kept
+    mask_floor = float((bits(Mo) != bits(out64[3])).mean())
+    assert float((bits(Mo) != keep).mean()) <= max(1e-3, FLOORS * mask_floor)
     dq = lambda q, s, z, M: (oracle.dequantize(q, s, z, 128) * torch.from_numpy(bits(M).T.copy()).float()).numpy()
     eo = mathref.layer_error(case.W.float().numpy(), dq(qo, so, zo, Mo), H)
     eg = mathref.layer_error(case.W.float().numpy(), dq(qg.cpu(), sg.cpu(), zg.cpu(), Mg), H)
@@ -210,7 +211,6 @@ def test_expert_group_matches_per_expert_handles(factor_route):
         dn.update(torch.cat(ph).to(DEV), o2)
     (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=4)
     (qd, sd, zd), = dn.quantize(chunk=4)
-    worst = 0.0
     for e in range(E):
         for W, X, (q, s, z) in ((moe.Wg[e], xs[e], (qg, sg, zg)), (moe.Wu[e], xs[e], (qu, su, zu)),
                                 (moe.Wd[e], hs[e], (qd, sd, zd))):
@@ -220,10 +220,10 @@ def test_expert_group_matches_per_expert_handles(factor_route):
             assert float((so != s[e].cpu()).float().mean()) <= 2e-3
             same = so == s[e].cpu()
             assert torch.equal(zo[same], z[e].cpu()[same])
-            worst = max(worst, flip_rate(qo, q[e]))
             if X.shape[0] == 0:
                 assert torch.equal(qo, q[e].cpu())                       # H = I: pure RTN, exact
-    assert worst <= 5e-3, worst
+            else:
+                _codes_at_floor(f"expert {e} {tuple(W.shape)} {factor_route}", qo, q[e], W, [X], kw)
 
 
 @pytest.mark.parametrize("factor_route", ["direct", "inverse"])
@@ -248,7 +248,8 @@ def test_expert_group_non_positive_definite_falls_back(factor_route):
     o = oracle.GPTQ(linear(W[1]), **kw)
     o.update(xs[1])
     qo, so, zo = o.quantize()
-    assert torch.equal(so, s[1].cpu()) and flip_rate(qo, q[1]) <= 5e-3
+    assert torch.equal(so, s[1].cpu())
+    _codes_at_floor(f"undamped neighbour {factor_route}", qo, q[1], W[1], [xs[1]], kw)
 
 
 @pytest.mark.parametrize("zero_weight_column", [False, True])
@@ -277,7 +278,7 @@ def test_expert_group_dead_and_zero_columns(zero_weight_column):
             o.update(xs[e])
             qo, so, zo = o.quantize()
             assert float((so != s[e].cpu()).float().mean()) <= 2e-3
-            assert flip_rate(qo, q[e]) <= 5e-3
+            _codes_at_floor(f"dead/zero columns, expert {e}", qo, q[e], W, [xs[e]], kw)
             if e == 1:      # dead columns are pruned: weight 0 -> the code of zero
                 assert torch.equal(qo[:, [37, 200]], q[e].cpu()[:, [37, 200]])
 
@@ -308,12 +309,13 @@ def test_expert_group_sparse14_matches_per_expert_oracle(factor_route):
             bits_o = np.unpackbits(Mo.numpy().view(np.uint8), bitorder="little")
             bits_g = np.unpackbits(M[e].cpu().numpy().view(np.uint8), bitorder="little")
             assert bits_g.reshape(-1, 4).sum(1).tolist() == [1] * (bits_g.size // 4)
-            assert (bits_o != bits_g).mean() <= 1e-2
-            assert flip_rate(qo, q[e]) <= 1e-2
+            _, floor, out64 = _codes_at_floor(f"sparse14 expert {e} {factor_route}", qo, q[e], W, [xs[e]], kw)
+            bits_64 = np.unpackbits(out64[3].numpy().view(np.uint8), bitorder="little")
+            assert (bits_o != bits_g).mean() <= max(1e-3, FLOORS * (bits_o != bits_64).mean())
 
 
 # ---------------------------------------------------------------- benchmark configurations
-def _e2e(W, X, kw, tol_flips, gs=128):
+def _e2e(tag, W, X, kw, gs=128):
     o, g, H = _run_pair(W, X, chunks=1, **kw)
     ro, rg = o.quantize(), g.quantize()
     qo, so, zo = ro[:3]
@@ -326,7 +328,7 @@ def _e2e(W, X, kw, tol_flips, gs=128):
     eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, gs).numpy(), H)
     eg = mathref.layer_error(Wf, oracle.dequantize(qg, sg, zg, gs).numpy(), H)
     assert abs(eg / eo - 1) < 0.01, eg / eo
-    assert flips <= tol_flips, flips
+    _codes_at_floor(tag, qo, qg, W, [X], kw)
     return flips, eg / eo, ro, rg
 
 
@@ -337,7 +339,7 @@ def test_config1_dense_2048_full_size(scale):
     case = synth.dense_outlier()
     kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale=scale,
               quantization_order="default", rel_damp=0.01)
-    flips, ratio, _, _ = _e2e(case.W, case.X, kw, tol_flips=4e-3)
+    flips, ratio, _, _ = _e2e(f"config1 {scale}", case.W, case.X, kw)
     print(f"config1 {scale}: flips {flips:.2e} error ratio {ratio:.5f}")
 
 
@@ -356,7 +358,8 @@ def test_config5_sparse14_full_size():
                          >> (np.arange(C) % 32)[:, None]) & 1).astype(bool)
     ko, kg = unpack(Mo), unpack(Mg)
     assert np.all(kg.reshape(C // 4, 4, R).sum(axis=1) == 1)
-    assert float((ko != kg).mean()) <= 5e-3 and flip_rate(qo, qg) <= 5e-3
+    _, floor, out64 = _codes_at_floor("config5", qo, qg, case.W, [case.X], kw)
+    assert float((ko != kg).mean()) <= max(1e-3, FLOORS * float((ko != unpack(out64[3])).mean()))
     dq = lambda q, s, z, k: (oracle.dequantize(q, s, z, 128) * torch.from_numpy(k.T.copy()).float()).numpy()
     Wf = case.W.float().numpy()
     eo = mathref.layer_error(Wf, dq(qo, so, zo, ko), H)
@@ -370,67 +373,54 @@ def test_config5_sparse14_full_size():
     assert torch.equal(words, want)
 
 
-def test_config3_one_expert_at_full_shape():
+@pytest.mark.parametrize("n_tokens", [1536, 200])
+def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 512 of
-    its 2048 rows, rows being independent, to keep the CPU oracle's three sweeps short)
-    with a heavy expert's worth of tokens.  At C = 7168 (rank-deficient Hessian, act-order)
-    the problem is ill conditioned: the oracle's OWN codes move by ~1 % when only its fp32
-    LAPACK factor is replaced by the float64 one (the floor computed below), although both
-    factors agree to 2.5e-5.  The GPU factor is as accurate as LAPACK's (2.2e-5 vs 2.5e-5
-    against float64) but its Hessian and factor carry independent fp32 rounding, so codes
-    are required to stay within 6 floors of the oracle and the output error within 1 %."""
+    its 2048 rows, rows being independent, to keep the CPU oracle's sweeps short) with a heavy
+    expert's tokens and with 200 (Hessian of rank 200 before damping).  At this size the
+    problem is ill conditioned: the oracle's own codes move by 1-2 % between two valid fp32
+    realisations of its library stages (the floor).  Three GPU routes are held to that floor
+    against the reference-form oracle: the drop-in class (reference's factor of inv(H), fp32
+    chain sweep), the batched front end on the same route, and the batched front end's default
+    -- the route the benchmark times: factor of H itself, displacement sweep, block updates
+    from bf16 pieces."""
+    from forge.gptq import GPTQ
+    from forge.moe import ExpertGroupGPTQ
     g0 = torch.Generator().manual_seed(11)
     W = synth.fp8_block_roundtrip((0.02 * torch.randn(512, 7168, generator=g0)).bfloat16())
-    X = torch.randn(1536, 7168, generator=g0).bfloat16()
+    X = torch.randn(1536, 7168, generator=g0).bfloat16()[:n_tokens].contiguous()
     kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
               quantization_order="activation", rel_damp=0.01)
-    o, g, H = _run_pair(W, X, chunks=1, **kw)
+    o = oracle.GPTQ(linear(W), **kw)
+    o.update(X)
+    H = o.H.double().numpy().copy()
     qo, so, zo = o.quantize()
-    qg, sg, zg = (t.cpu() for t in g.quantize())
-    assert float((so != sg).float().mean()) <= 1e-3
-    floor = _noise_floor(W, o, so, zo)
-    flips = flip_rate(qo, qg)
+    floor, out64 = reference_floor(W, [X], qo, **kw)
+    bound = max(1e-3, FLOORS * floor)
     Wf = W.float().numpy()
     eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H)
-    eg = mathref.layer_error(Wf, oracle.dequantize(qg, sg, zg, 128).numpy(), H)
-    print(f"config3 expert: flips {flips:.2e} oracle noise floor {floor:.2e} error ratio {eg / eo:.5f}")
-    assert abs(eg / eo - 1) < 0.01
-    assert flips <= max(1e-3, 6 * floor)
 
+    def check(tag, q, s, z):
+        q, s, z = q.cpu(), s.cpu(), z.cpu()
+        assert float((so != s).float().mean()) <= 1e-3
+        flips, to64 = flip_rate(qo, q), flip_rate(out64[0], q)
+        eg = mathref.layer_error(Wf, oracle.dequantize(q, s, z, 128).numpy(), H)
+        print(f"config3 n={n_tokens} {tag}: flips vs oracle {flips:.2e}, vs float64 stages {to64:.2e}, "
+              f"floor {floor:.2e}, error ratio {eg / eo:.5f}")
+        assert abs(eg / eo - 1) < 0.01
+        assert flips <= bound and to64 <= bound
 
-def test_config3_factor_routes_agree_at_full_shape():
-    """DeepSeek-V3-shaped experts (C = 7168, act-order, MSE; 512 rows each), one with a heavy
-    expert's tokens and one with 200: the batched front end's two routes to the sweep's matrix
-    are the same solve, so their layer output errors must agree within 1 % and their codes
-    within the spread that fp32 rounding alone causes at this size (the test above measures
-    ~1 % for the oracle's own factor)."""
-    from forge.moe import ExpertGroupGPTQ
-    g0 = torch.Generator().manual_seed(12)
-    W = synth.fp8_block_roundtrip((0.02 * torch.randn(2 * 512, 7168, generator=g0)).bfloat16()).view(2, 512, 7168)
-    xs = [torch.randn(n, 7168, generator=g0).bfloat16() for n in (1536, 200)]
-    offs = [0, 1536, 1736]
-    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
-              quantization_order="activation", rel_damp=0.01)
-    out = {}
-    for route in ("direct", "inverse"):
-        grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, factor_route=route, **kw)
-        grp.update(torch.cat(xs).to(DEV), offs)
-        (q, s, z), = grp.quantize(chunk=2)
-        out[route] = (q.cpu(), s.cpu(), z.cpu())
+    g = GPTQ(linear(W).to(DEV), device=DEV, **kw)
+    g.add_batch(X.to(DEV))
+    check("class", *g.quantize())
+    del g
+    for route in ("inverse", "direct"):
+        grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **kw)
+        grp.update(X.to(DEV), [0, n_tokens])
+        (q, s, z), = grp.quantize(chunk=1)
         assert not grp.issue_non_invertible.any()
-    assert torch.equal(out["direct"][1], out["inverse"][1])              # same grid search
-    for e in range(2):
-        X = xs[e].double()
-        H = ((2.0 / X.shape[0]) * X.t() @ X).numpy()
-        Wf = W[e].float().numpy()
-        err = {}
-        for r in out:
-            D = Wf.astype(np.float64) - oracle.dequantize(out[r][0][e], out[r][1][e], out[r][2][e], 128).double().numpy()
-            err[r] = float(((D @ H) * D).sum())                          # tr(D H D^T)
-        flips = flip_rate(out["direct"][0][e], out["inverse"][0][e])
-        print(f"expert {e}: flips between routes {flips:.2e}, error ratio {err['direct'] / err['inverse']:.5f}")
-        assert abs(err["direct"] / err["inverse"] - 1) < 0.01
-        assert flips <= 0.06
+        check(f"batched {route}", q[0], s[0], z[0])
+        del grp
 
 
 def test_expert_group_few_tokens_routes_agree():
@@ -502,6 +492,8 @@ def test_config2_qwen3_experts_at_full_shape():
             qo, so, zo = o.quantize()
             assert float((so != s[e].cpu()).float().mean()) <= 2e-3
             worst = max(worst, flip_rate(qo, q[e]))
+            if n:
+                _codes_at_floor(f"config2 expert {e} {tuple(W.shape)} n={n}", qo, q[e], W, [X], kw)
             Wf = W.float().numpy()
             eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H) * n / 2
             eg = mathref.layer_error(Wf, oracle.dequantize(q[e].cpu(), s[e].cpu(), z[e].cpu(), 128).numpy(), H) * n / 2
@@ -511,4 +503,4 @@ def test_config2_qwen3_experts_at_full_shape():
                 worst_ratio = max(worst_ratio, abs(eg / eo - 1))
     print(f"config2 experts: worst flips {worst:.2e}, worst per-expert error deviation "
           f"{worst_ratio:.2e}, layer error ratio {sum_g / sum_o:.5f}")
-    assert worst <= 1e-2 and worst_ratio < 0.01 and abs(sum_g / sum_o - 1) < 0.01
+    assert worst_ratio < 0.01 and abs(sum_g / sum_o - 1) < 0.01
