@@ -63,6 +63,7 @@ int summarise() {
 
 KernelTiming::KernelTiming(const char* name, hipStream_t st, double work, WorkKind kind)
     : slot_(-1), st_(st) {
+    if (!name) return;                       // a caller that must not create events
     std::lock_guard<std::mutex> lock(g_mu);
     if (!g_enabled) return;
     TimedLaunch l{name, work, kind, nullptr, nullptr};

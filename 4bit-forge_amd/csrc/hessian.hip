@@ -451,7 +451,7 @@ int upload_async(const void* src, int64_t bytes, void* dst, hipStream_t st) {
 // The launches of one update; gd_dev already holds the group table.
 int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const GroupDesc* gd_dev,
                   int64_t n_groups, int64_t total, int max_chunks, bool any_blend, float* H,
-                  float* dnew, uint4* pack, hipStream_t st) {
+                  float* dnew, uint4* pack, hipStream_t st, bool timed = true) {
     const int NT = (int)forge::ceil_div(C, 128);
     const unsigned pairs = (unsigned)(NT * (NT + 1) / 2);
     const dim3 dgrid((unsigned)NT, (unsigned)n_groups);
@@ -464,7 +464,7 @@ int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const Grou
                            dim3(64), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev, pack);
         FORGE_LAUNCH_CHECK();
         // executed flops: tiles on and above the diagonal only
-        forge::KernelTiming timing("hessian_syrk_bf16", st,
+        forge::KernelTiming timing(timed ? "hessian_syrk_bf16" : nullptr, st,
                                    2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
                                    forge::WORK_FLOPS);
         if (any_blend)
@@ -478,7 +478,7 @@ int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const Grou
         diag_float64_kernel<float><<<dgrid, dim3(256), 0, st>>>((const float*)X, ldx, C, gd_dev, H,
                                                                 dnew);
         FORGE_LAUNCH_CHECK();
-        forge::KernelTiming timing("hessian_syrk_f32", st,
+        forge::KernelTiming timing(timed ? "hessian_syrk_f32" : nullptr, st,
                                    2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
                                    forge::WORK_FLOPS);
         syrk_f32_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
@@ -486,6 +486,41 @@ int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const Grou
         FORGE_LAUNCH_CHECK();
     }
     return FORGE_OK;
+}
+
+// ---------------------------------------------------------------- entry point without allocation
+// Device memory of the library's own for forge_hessian_update_static: one group table entry,
+// the float64-summed diagonal and the bf16 operand panels.  Every GPU the library runs on
+// holds its own copy at its own address until the process ends.
+constexpr int64_t STATIC_MAX_C = 16384;
+constexpr int64_t STATIC_PACK_BYTES = 32ll << 20;
+constexpr int64_t STATIC_DESC_BYTES = 256;
+constexpr int64_t STATIC_BYTES = STATIC_DESC_BYTES + STATIC_MAX_C * 4 + STATIC_PACK_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_static_mu;
+void* g_static_ptr[MAX_DEVICES] = {nullptr};
+
+// Address of `scratch` on the current device (looked up once per device; in host code the
+// array's name is only a handle for this lookup, never an address).
+int static_scratch(unsigned char** out) {
+    int dev = -1;
+    FORGE_HIP_CHECK(hipGetDevice(&dev));
+    FORGE_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "device index %d not supported", dev);
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void* p = nullptr;
+        FORGE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        FORGE_REQUIRE(p != nullptr, "no device address for the static workspace");
+        g_static_ptr[dev] = p;
+    }
+    *out = (unsigned char*)g_static_ptr[dev];
+    return FORGE_OK;
+}
+
+__global__ void write_desc_kernel(GroupDesc* __restrict__ gd, GroupDesc v) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *gd = v;
 }
 
 }  // namespace
@@ -543,4 +578,46 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
     if (int rc = upload_async(gd.data(), n_groups * (int64_t)sizeof(GroupDesc), gd_dev, st)) return rc;
     return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, any_blend, H, dnew,
                          pack, st);
+}
+
+extern "C" int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype) {
+    if (C < 1 || C > STATIC_MAX_C) return 0;
+    if (x_dtype != FORGE_BF16) return (1LL << 31) - 1;
+    const int64_t chunks = STATIC_PACK_BYTES / (forge::ceil_div(C, 32) * 64 * 16);
+    return chunks * 16;
+}
+
+extern "C" int forge_hessian_update_static(const void* X, int x_dtype, int64_t ldx, int64_t n_rows,
+                                           int64_t C, float alpha, float beta, float* H,
+                                           forge_stream_t stream) {
+    FORGE_REQUIRE(x_dtype == FORGE_F32 || x_dtype == FORGE_BF16, "x_dtype=%d", x_dtype);
+    FORGE_REQUIRE(C >= 1 && ldx >= C && n_rows >= 0, "bad shape n_rows=%lld C=%lld ldx=%lld",
+                  (long long)n_rows, (long long)C, (long long)ldx);
+    FORGE_REQUIRE(C <= STATIC_MAX_C, "C=%lld exceeds the static workspace's limit of %lld columns",
+                  (long long)C, (long long)STATIC_MAX_C);
+    FORGE_REQUIRE(n_rows <= forge_hessian_update_static_max_rows(C, x_dtype),
+                  "n_rows=%lld exceeds the static workspace's limit of %lld rows at C=%lld "
+                  "(use forge_hessian_update_grouped with a workspace of the caller's)",
+                  (long long)n_rows, (long long)forge_hessian_update_static_max_rows(C, x_dtype),
+                  (long long)C);
+    if (n_rows == 0) return FORGE_OK;
+    FORGE_REQUIRE(X && H, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char* base = nullptr;
+    if (int rc = static_scratch(&base)) return rc;
+    GroupDesc* gd_dev = (GroupDesc*)base;
+    float* dnew = (float*)(base + STATIC_DESC_BYTES);
+    uint4* pack = (uint4*)(base + STATIC_DESC_BYTES + STATIC_MAX_C * 4);
+    GroupDesc g;
+    g.row0 = 0;
+    g.pack_off = 0;
+    g.n = (int32_t)n_rows;
+    g.nchunk = (int32_t)forge::ceil_div(n_rows, 16);
+    g.alpha = alpha;
+    g.beta = beta;
+    // the table entry travels as a kernel argument: no staging buffer, nothing to allocate
+    write_desc_kernel<<<dim3(1), dim3(64), 0, st>>>(gd_dev, g);
+    FORGE_LAUNCH_CHECK();
+    return launch_update(X, x_dtype, ldx, C, gd_dev, 1, n_rows, g.nchunk, beta != 0.0f, H, dnew, pack,
+                         st, /*timed=*/false);
 }

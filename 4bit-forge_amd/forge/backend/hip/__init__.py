@@ -52,6 +52,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
+        "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
+        "forge_hessian_update_static_max_rows": ([i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
         "forge_chol_workspace_bytes": ([i64, i64], i64),
         "forge_chol_reverse_lower_batched": ([vp, vp, vp, i64, i64, vp, i64, vp], i32),
@@ -81,6 +83,7 @@ EXPORTED_SYMBOLS = (
     "forge_gptq_sweep_direct_workspace_bytes",
     "forge_hessian_update_grouped",
     "forge_hessian_workspace_bytes",
+    "forge_hessian_update_static", "forge_hessian_update_static_max_rows",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
@@ -311,6 +314,20 @@ class _HipKernels:
             self._check(self._lib.forge_hessian_update_grouped(
                 _ptr(X), _dtype_code(X), X.stride(0), C, offs, E, al, be, _ptr(H), _ptr(ws),
                 nbytes, _stream()))
+        return H
+
+    def hessian_update_static(self, X, H, alpha, beta):
+        """H [C,C] f32 <- beta*H + alpha * X^T X for X [n,C] (bf16/f32) through the entry point
+        that allocates nothing (its workspace is a device array of the library's own; see
+        forge_hessian_update_static in forge_hip.h for the size limits)."""
+        _need_cuda(X, H)
+        C = H.shape[-1]
+        assert X.dim() == 2 and X.shape[1] == C and X.stride(1) == 1
+        assert tuple(H.shape) == (C, C) and H.is_contiguous() and H.dtype == torch.float32
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_hessian_update_static(
+                _ptr(X), _dtype_code(X), X.stride(0), X.shape[0], C, float(alpha), float(beta),
+                _ptr(H), _stream()))
         return H
 
     def chol_inv_upper_batched(self, H, damp, normalise=True, upper_only=False):

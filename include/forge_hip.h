@@ -175,6 +175,26 @@ int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_
 int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int64_t C,
                                       int x_dtype);
 
+/* GPTQ.update for ONE matrix without any allocation: H <- beta*H + alpha * X^T X for the
+ * n_rows rows of X ([n_rows, C], pitch ldx, dtype x_dtype), the same kernels and the same
+ * bits as forge_hessian_update_grouped with a single group.  No counterpart in the
+ * reference; it is for callers that cannot allocate or bring a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The group table, the
+ * float64 diagonal and the bf16 operand panels live in a device array of the library's own
+ * (32 MiB + 64.25 KiB per GPU, held until the process ends), which fixes the limits:
+ * C <= 16384 and n_rows <= forge_hessian_update_static_max_rows(C, x_dtype) (bf16: the
+ * panels, ceil(n_rows/16) * ceil(C/32) KiB, must fit in 32 MiB -- 2336 rows at C = 7168,
+ * 8192 at C = 2048; f32: no limit on rows); larger inputs are rejected with
+ * FORGE_ERR_INVALID before any launch.  Calls no hipMalloc/hipFree/hipHostMalloc and creates
+ * no events (its launches never appear in the forge_kernel_timing_* records).  Every call on
+ * a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream are ordered.  Nothing in the array has to be cleared
+ * between calls: every byte a call reads it has written first. */
+int forge_hessian_update_static(const void* X, int x_dtype, int64_t ldx, int64_t n_rows,
+                                int64_t C, float alpha, float beta, float* H,
+                                forge_stream_t stream);
+int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype);
+
 /* ------------------------------------------------------------------ factorisation */
 
 /* Batched form of GPTQ._h_factor's torch.linalg calls (gptq.py:152-175):
