@@ -22,6 +22,7 @@ struct GemmArgs {
     bool b_upper_tri;  // Bm[k, n] == 0 for k > n: stop each tile's K loop at its last column
     bool b_lower_tri;  // Bm[k, n] == 0 for k < n: start each tile's K loop at its first column
     bool blocked_sum;  // sum K in blocks of 128 (more accurate; NOT the sweep's single chain)
+    int products;      // bf16-piece path only: piece products per fp32 product (1, 3, 4; else 6)
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;
@@ -42,7 +43,7 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);
 // With a workspace of split_gemm_workspace_bytes(batch, k1 - k0), two blocked-sum problems
 // of full tiles that share their A panel (same At, pitch, m0 and k0) run on the bf16 matrix
 // pipe instead (three-piece split of every operand, fp32-grade accuracy, different
-// rounding); FORGE_FP32_BLOCKED_SUM=1 in the environment keeps them on the fp32 kernel.
+// rounding); the option fp32_blocked_sum = 1 keeps them on the fp32 kernel.
 int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
                            hipStream_t st, void* split_ws = nullptr, int64_t split_ws_bytes = 0);
 int64_t split_gemm_workspace_bytes(int64_t batch, int64_t k_rows);

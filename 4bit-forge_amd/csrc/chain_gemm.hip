@@ -526,7 +526,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int SPLIT_TK = 32;                       // k rows per stage
-constexpr int SPLIT_STAGE_WORDS = 3 * 4 * 128;     // 16-byte words per operand and stage
+constexpr int SPLIT_STAGE_WORDS = 3 * 4 * 128;     // 16-byte words per operand and stage (three pieces)
+constexpr int split_stage_words(int np) { return np * 4 * 128; }
 constexpr int SPLIT_SETS = 4;                      // producer register sets = stages in flight
 
 // N fp32 values (consecutive k of one column) -> N/2 packed words of each piece.
@@ -549,8 +550,26 @@ __device__ __forceinline__ void split_pieces(const float (&x)[N], W& p1, W& p2, 
     }
 }
 
+// Two pieces, each rounded to nearest even by the hardware's packing conversion
+// (v_cvt_pk_bf16_f32): a = a1 + a2 + r with |r| <= 2^-18 |a|.  Used with the three products
+// (2,1) (1,2) (1,1), whose sum is then within ~2^-17 of a*b with errors of either sign.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+template <int N, typename W>
+__device__ __forceinline__ void split_pieces2(const float (&x)[N], W& p1, W& p2) {
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w) {
+        const f32x2 v = {x[2 * w], x[2 * w + 1]};
+        const unsigned h1 = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+        const f32x2 r = {v[0] - __uint_as_float(h1 << 16), v[1] - __uint_as_float(h1 & 0xFFFF0000u)};
+        p1[w] = h1;                                                  // k in the low half
+        p2[w] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, bf16x2));
+    }
+}
+
 // Rows [k0, k1) x columns [m0, m0+128) of At -> the LDS images of its stages, stage after
 // stage (SPLIT_STAGE_WORDS words each).  One workgroup of 128 threads per matrix and stage.
+template <int NP>
 __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restrict__ At, int64_t lda,
                                                             int64_t as, int m0, int k0, int n_stage,
                                                             u32x4* __restrict__ Ap, int64_t aps) {
@@ -560,17 +579,21 @@ __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restr
     f32x4 x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[j] = *reinterpret_cast<const f32x4*>(src + (int64_t)j * lda);
-    u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * SPLIT_STAGE_WORDS + kg * 128 + cq;
+    u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * split_stage_words(NP) + kg * 128 + cq;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float col[8];
         u32x4 p1, p2, p3;
 #pragma unroll
         for (int j = 0; j < 8; ++j) col[j] = x[j][e];
-        split_pieces<8>(col, p1, p2, p3);
+        if (NP == 3) {
+            split_pieces<8>(col, p1, p2, p3);
+            dst[1024 + 32 * e] = p3;
+        } else {
+            split_pieces2<8>(col, p1, p2);
+        }
         dst[32 * e] = p1;
         dst[512 + 32 * e] = p2;
-        dst[1024 + 32 * e] = p3;
     }
 }
 
@@ -582,12 +605,18 @@ struct SplitPair {
 
 // Both problems: full 128x128 tiles, one m tile, 16-byte aligned rows, every tile's K range
 // a whole number of 128-row chunks starting at k0.
+// NP pieces per operand, NPROD piece products per fp32 product (the largest ones).
+//   NP = 3, NPROD = 6: all products of weight >= 2^-16, fp32-grade (the factorisation).
+//   NP = 2 (pieces rounded to nearest): NPROD = 3: (2,1) (1,2) (1,1), within ~2^-17 of a*b;
+//   NPROD = 4 adds (2,2); NPROD = 1 is (1,1) alone, i.e. plain bf16 operands.  Only where the
+//   caller asks for it (the direct sweep's block updates, option "sweep_update_products").
+template <int NP, int NPROD>
 __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     const bool in_first = blockIdx.x < (unsigned)sp.pair.first_wgs;
     const GemmArgs& g = in_first ? sp.pair.first : sp.pair.second;
     const int wg = in_first ? (int)blockIdx.x : (int)blockIdx.x - sp.pair.first_wgs;
     // [buffer][operand][piece][k group][position]
-    __shared__ __attribute__((aligned(16))) u32x4 L[2][2][3][4][128];
+    __shared__ __attribute__((aligned(16))) u32x4 L[2][2][NP][4][128];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bz, tile;
@@ -622,16 +651,16 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         // Every fetch stays inside [k0, k1): the offsets advance only while a further stage
         // exists; past the end the last stage is fetched again and never used.
         int b_soff = 0, a_soff = 0, fetched = 0;
-        int b_adv = (int)(SPLIT_TK * g.ldb * 4), a_adv = SPLIT_STAGE_WORDS * 16;
+        int b_adv = (int)(SPLIT_TK * g.ldb * 4), a_adv = split_stage_words(NP) * 16;
         f32x4 xb[SPLIT_SETS][4];
-        u32x4 xa[SPLIT_SETS][6];
+        u32x4 xa[SPLIT_SETS][2 * NP];
 #define FORGE_SPLIT_FETCH(q)                                                                       \
     do {                                                                                           \
         ++fetched;                                                                                 \
         if (fetched >= n_stage) { b_adv = 0; a_adv = 0; }                                          \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) xb[q][j] = __builtin_bit_cast(               \
             f32x4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ob[j], b_soff, 0));               \
-        _Pragma("unroll") for (int j = 0; j < 6; ++j)                                              \
+        _Pragma("unroll") for (int j = 0; j < 2 * NP; ++j)                                         \
             xa[q][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, oa + j * 4096, a_soff, 0);    \
         b_soff += b_adv;                                                                           \
         a_soff += a_adv;                                                                           \
@@ -639,19 +668,23 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         // B word (piece, k group kh >> 1, position 32 e + cq), half kh & 1; A: plain copy
         u32x2* const Lb = reinterpret_cast<u32x2*>(&L[0][1][0][kh >> 1][cq]) + (kh & 1);
         u32x4* const La = &L[0][0][0][0][0] + pt;
-        constexpr int BUF = 2 * SPLIT_STAGE_WORDS;   // words per buffer (both operands)
+        constexpr int BUF = 2 * split_stage_words(NP);   // words per buffer (both operands)
 #define FORGE_SPLIT_STAGE(buf, q)                                                                  \
     do {                                                                                           \
         _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
             float col[4];                                                                          \
             u32x2 p1, p2, p3;                                                                      \
             _Pragma("unroll") for (int j = 0; j < 4; ++j) col[j] = xb[q][j][e];                    \
-            split_pieces<4>(col, p1, p2, p3);                                                      \
+            if (NP == 3) {                                                                         \
+                split_pieces<4>(col, p1, p2, p3);                                                  \
+                Lb[((buf) * BUF + (NP - 1) * 512 + 32 * e) * 2] = p3;                              \
+            } else {                                                                               \
+                split_pieces2<4>(col, p1, p2);                                                     \
+            }                                                                                      \
             Lb[((buf) * BUF + 32 * e) * 2] = p1;                                                   \
             Lb[((buf) * BUF + 512 + 32 * e) * 2] = p2;                                             \
-            Lb[((buf) * BUF + 1024 + 32 * e) * 2] = p3;                                            \
         }                                                                                          \
-        _Pragma("unroll") for (int j = 0; j < 6; ++j) La[(buf) * BUF + j * 256] = xa[q][j];        \
+        _Pragma("unroll") for (int j = 0; j < 2 * NP; ++j) La[(buf) * BUF + j * 256] = xa[q][j];   \
     } while (0)
         FORGE_SPLIT_FETCH(0);
         FORGE_SPLIT_FETCH(1);
@@ -715,10 +748,10 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             for (int v = 0; v < 16; ++v) tot[mi][ni][v] = 0.0f;
     const int rk = lane >> 5, ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    bf16x8 A0[3][2], B0[3][2], A1[3][2], B1[3][2];   // operands of k-step 0 / 1
+    bf16x8 A0[NP][2], B0[NP][2], A1[NP][2], B1[NP][2];   // operands of k-step 0 / 1
 #define FORGE_SPLIT_READ(buf, u, A, B)                                                             \
     do {                                                                                           \
-        _Pragma("unroll") for (int p = 0; p < 3; ++p) _Pragma("unroll") for (int i = 0; i < 2; ++i) { \
+        _Pragma("unroll") for (int p = 0; p < NP; ++p) _Pragma("unroll") for (int i = 0; i < 2; ++i) { \
             A[p][i] = __builtin_bit_cast(bf16x8, L[buf][0][p][2 * (u) + rk][ra + 64 * i]);         \
             B[p][i] = __builtin_bit_cast(bf16x8, L[buf][1][p][2 * (u) + rk][rb + 64 * i]);         \
         }                                                                                          \
@@ -727,19 +760,30 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     // different accumulators; `fresh`: the first product of a chunk takes C = 0
 #define FORGE_SPLIT_MFMAS(A, B, fresh)                                                             \
     do {                                                                                           \
-        constexpr int PA[6] = {2, 0, 1, 1, 0, 0}, PB[6] = {0, 2, 1, 0, 1, 0};                      \
-        _Pragma("unroll") for (int t = 0; t < 6; ++t) _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) \
+        constexpr int PA[6] = {NP - 1, 0, 1, 1, 0, 0}, PB[6] = {0, NP - 1, 1, 0, 1, 0};            \
+        _Pragma("unroll") for (int t = 6 - NPROD; t < 6; ++t) _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) \
             _Pragma("unroll") for (int ni = 0; ni < 2; ++ni)                                       \
                 acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                             \
-                    A[PA[t]][mi], B[PB[t]][ni], ((fresh) && t == 0) ? zero : acc[mi][ni], 0, 0, 0);\
+                    A[PA[t]][mi], B[PB[t]][ni], ((fresh) && t == 6 - NPROD) ? zero : acc[mi][ni], 0, 0, 0);\
     } while (0)
-    // 24 MFMAs and 12 LDS reads per k-step: one read after every other MFMA
+    // 4 NPROD MFMAs and 4 NP LDS reads per k-step (24 and 12, or 12 and 8): the reads spread
+    // evenly between the MFMAs
 #define FORGE_SPLIT_SCHED()                                                                        \
     do {                                                                                           \
-        _Pragma("unroll") for (int i = 0; i < 12; ++i) {                                           \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                     \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+        if (NPROD == 6) {                                                                          \
+            _Pragma("unroll") for (int i = 0; i < 12; ++i) {                                       \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+            }                                                                                      \
+        } else if (NPROD == 3) {                                                                   \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                        \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+            }                                                                                      \
         }                                                                                          \
     } while (0)
     __syncthreads();
@@ -870,8 +914,7 @@ namespace {
 // A panel (At, pitch, m0, k0), which is split once for both.
 bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t ws_bytes,
                     int* n_stage_out) {
-    const char* forced_fp32 = getenv("FORGE_FP32_BLOCKED_SUM");   // read per call: tests flip it
-    if (forced_fp32 && forced_fp32[0] == '1') return false;
+    if (option(OPT_FP32_BLOCKED_SUM) == 1) return false;
     auto ok = [](const Prepared& p) {
         return !p.edge && p.k128 && p.g.blocked_sum && p.g.m_tiles == 1 && !p.g.b_lower_tri &&
                p.g.k1 - p.g.k0 >= 128 && (!p.g.b_upper_tri || p.g.n0 + TN - p.g.k0 >= 128);
@@ -899,15 +942,31 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
     sp.pair.second = b ? b->g : a.g;
     sp.pair.first_wgs = (int)a.n_wg;
     sp.Ap = static_cast<const u32x4*>(ws);
-    sp.aps = (int64_t)n_stage * SPLIT_STAGE_WORDS;
+    const int products = a.g.products;
+    const bool two = products == 1 || products == 3 || products == 4;     // two-piece layout
+    const int np = two ? 2 : 3;
+    sp.aps = (int64_t)n_stage * split_stage_words(np);
     {
-        KernelTiming timing("split_a_panel", st, 10.0 * n_stage * SPLIT_TK * TM * (double)batch, WORK_BYTES);
-        split_a_panel_kernel<<<dim3((unsigned)(batch * n_stage)), dim3(128), 0, st>>>(
-            a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0, n_stage, static_cast<u32x4*>(ws), sp.aps);
+        KernelTiming timing("split_a_panel", st, (4.0 + 2.0 * np) * n_stage * SPLIT_TK * TM * (double)batch,
+                            WORK_BYTES);
+        const dim3 pgrid((unsigned)(batch * n_stage)), pblock(128);
+        if (two)
+            split_a_panel_kernel<2><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0,
+                                                              n_stage, static_cast<u32x4*>(ws), sp.aps);
+        else
+            split_a_panel_kernel<3><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0,
+                                                              n_stage, static_cast<u32x4*>(ws), sp.aps);
         FORGE_LAUNCH_CHECK();
     }
-    KernelTiming timing("split_gemm_bf16x3", st, a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
-    split_gemm_kernel<<<dim3((unsigned)n_wg), dim3(512), 0, st>>>(sp);
+    KernelTiming timing(two ? "split_gemm_bf16x2" : "split_gemm_bf16x3", st,
+                        a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
+    const dim3 grid((unsigned)n_wg), block(512);
+    switch (products) {
+        case 1: split_gemm_kernel<2, 1><<<grid, block, 0, st>>>(sp); break;
+        case 3: split_gemm_kernel<2, 3><<<grid, block, 0, st>>>(sp); break;
+        case 4: split_gemm_kernel<2, 4><<<grid, block, 0, st>>>(sp); break;
+        default: split_gemm_kernel<3, 6><<<grid, block, 0, st>>>(sp); break;
+    }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

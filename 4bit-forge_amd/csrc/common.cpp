@@ -1,6 +1,9 @@
 #include "common.h"
 
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -107,6 +110,62 @@ extern "C" int forge_kernel_timing_get(int index, char* name, int name_cap, int6
     if (work) *work = s.work;
     if (work_kind) *work_kind = s.kind;
     return FORGE_OK;
+}
+
+namespace forge {
+namespace {
+struct OptionInfo { const char* name; const char* env; int64_t lo, hi, dflt; };
+const OptionInfo kOptions[OPT_COUNT] = {
+    {"sweep_schedule", "FORGE_SWEEP_SCHEDULE", 0, 2, 0},
+    {"fp32_blocked_sum", "FORGE_FP32_BLOCKED_SUM", 0, 1, 0},
+    {"sweep_update_products", "FORGE_SWEEP_UPDATE_PRODUCTS", 0, 6, 0},
+};
+std::atomic<int64_t> g_options[OPT_COUNT];
+
+bool valid_option(int o, int64_t v) {
+    if (v < kOptions[o].lo || v > kOptions[o].hi) return false;
+    return o != OPT_SWEEP_PRODUCTS || v == 0 || v == 1 || v == 3 || v == 4 || v == 6;
+}
+
+// Runs when the library is loaded: the environment is looked at here and nowhere else.
+struct OptionInit {
+    OptionInit() {
+        for (int o = 0; o < OPT_COUNT; ++o) {
+            int64_t v = kOptions[o].dflt;
+            if (const char* e = getenv(kOptions[o].env)) {
+                int64_t x = v;
+                if (o == OPT_SWEEP_SCHEDULE && (e[0] == 'l' || e[0] == 'r')) x = e[0] == 'l' ? 1 : 2;
+                else if (e[0] >= '0' && e[0] <= '9') x = strtoll(e, nullptr, 10);
+                if (valid_option(o, x)) v = x;
+            }
+            g_options[o].store(v, std::memory_order_relaxed);
+        }
+    }
+} g_option_init;
+}  // namespace
+
+int64_t option(Option o) { return g_options[o].load(std::memory_order_relaxed); }
+}  // namespace forge
+
+extern "C" int forge_set_option(const char* name, int64_t value) {
+    if (!name) return forge::fail(FORGE_ERR_INVALID, "option name is null");
+    for (int o = 0; o < forge::OPT_COUNT; ++o)
+        if (strcmp(name, forge::kOptions[o].name) == 0) {
+            if (!forge::valid_option(o, value))
+                return forge::fail(FORGE_ERR_INVALID, "option %s: value %lld not allowed", name,
+                                   (long long)value);
+            forge::g_options[o].store(value, std::memory_order_relaxed);
+            return FORGE_OK;
+        }
+    return forge::fail(FORGE_ERR_INVALID, "unknown option %s", name);
+}
+
+extern "C" int64_t forge_get_option(const char* name) {
+    if (name)
+        for (int o = 0; o < forge::OPT_COUNT; ++o)
+            if (strcmp(name, forge::kOptions[o].name) == 0) return forge::option((forge::Option)o);
+    forge::fail(FORGE_ERR_INVALID, "unknown option %s", name ? name : "(null)");
+    return -1;
 }
 
 extern "C" int forge_hip_abi_version(void) { return 1; }

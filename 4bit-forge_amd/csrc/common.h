@@ -29,6 +29,17 @@ int fail(int code, const char* fmt, ...);
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Library-wide settings (forge_set_option / forge_get_option in forge_hip.h).  Each starts from
+// an environment variable read ONCE, when the library is loaded; after that only
+// forge_set_option changes it.  Reading one is a relaxed atomic load.
+enum Option {
+    OPT_SWEEP_SCHEDULE = 0,    // 0 = by tile count, 1 = left-looking, 2 = right-looking
+    OPT_FP32_BLOCKED_SUM = 1,  // 1 = blocked sums stay on the fp32 matrix instruction
+    OPT_SWEEP_PRODUCTS = 2,    // piece products per fp32 product in the direct sweep's updates
+    OPT_COUNT
+};
+int64_t option(Option o);
+
 // Optional per-kernel timing (forge_kernel_timing_* in forge_hip.h).  When enabled, a
 // KernelTiming object brackets one launch with two HIP events on the launch stream and
 // files the pair under `name` together with the launch's algorithmic work (flops or HBM

@@ -453,10 +453,15 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
     // (K = 128, (C - start)/128 times as many tiles); the weights are re-read per step, which
     // a batch could not afford.  Same fma chain per element, hence the same bits.
     bool right_looking = batch * forge::ceil_div(R, 128) < 128;
-    if (const char* forced = getenv("FORGE_SWEEP_SCHEDULE")) {   // read per call: tests flip it
-        if (forced[0] == 'l') right_looking = false;
-        if (forced[0] == 'r') right_looking = true;
-    }
+    const int64_t forced = forge::option(forge::OPT_SWEEP_SCHEDULE);
+    if (forced == 1) right_looking = false;
+    if (forced == 2) right_looking = true;
+    // Piece products per fp32 product in the direct route's block updates.  By default three
+    // (two rounded pieces per operand) from 4096 columns on, where the codes' own sensitivity to
+    // fp32 rounding is an order of magnitude above what the shorter sum adds and where the
+    // updates are most of the sweep's time; six (fp32-grade) below.
+    int products = (int)forge::option(forge::OPT_SWEEP_PRODUCTS);
+    if (products == 0) products = C >= 4096 ? 3 : 6;
     for (int64_t start = 0; start < C; start += forge::kBW) {
         const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
         forge::GemmArgs g{};
@@ -470,6 +475,7 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
             // sums of 128 products each, three bf16 pieces per operand on the bf16 matrix pipe
             // where the block is a full tile (fp32 matrix pipe otherwise)
             g.blocked_sum = true;
+            g.products = products;
             if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, ws_bytes)) return e;
         } else {
             if (int e = forge::launch_chain_gemm(g, batch, st)) return e;

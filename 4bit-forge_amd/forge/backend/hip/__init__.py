@@ -39,6 +39,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_kernel_timing_get": ([i32, ctypes.c_char_p, i32, ctypes.POINTER(i64),
                                      ctypes.POINTER(ctypes.c_double),
                                      ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i32)], i32),
+        "forge_set_option": ([ctypes.c_char_p, i64], i32),
+        "forge_get_option": ([ctypes.c_char_p], i64),
         "forge_build_group_meta_packed": ([vp, i64, i64, i32, i32, vp, vp, vp], i32),
         "forge_mse_scale_groups_packed": ([vp, vp, vp, vp, i64, i64, i64, f32, i32, i32, vp], i32),
         "forge_quant_grid": ([vp, i32, i64, i64, i64, i64, i64, i64, i32, i32, i32, vp, i64, f32,
@@ -77,7 +79,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
 
 EXPORTED_SYMBOLS = (
     "forge_hip_abi_version", "forge_last_error", "forge_kernel_timing_enable",
-    "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_build_group_meta_packed",
+    "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_set_option",
+    "forge_get_option", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
     "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_gptq_sweep_direct_batched",
     "forge_gptq_sweep_direct_workspace_bytes",
@@ -136,6 +139,16 @@ class _HipKernels:
             raise RuntimeError(self._lib.forge_last_error().decode())
 
     # -- per-kernel timing (benchmarks) ------------------------------------------------
+    def set_option(self, name: str, value: int):
+        """Library-wide setting ("sweep_schedule", "fp32_blocked_sum", "sweep_update_products";
+        see forge_set_option in forge_hip.h).  Returns the previous value."""
+        old = int(self._lib.forge_get_option(name.encode()))
+        self._check(self._lib.forge_set_option(name.encode(), int(value)))
+        return old
+
+    def get_option(self, name: str) -> int:
+        return int(self._lib.forge_get_option(name.encode()))
+
     def timing_enable(self, on: bool):
         self._check(self._lib.forge_kernel_timing_enable(int(bool(on))))
 

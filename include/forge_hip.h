@@ -48,6 +48,26 @@ int forge_kernel_timing_collect(void);
 int forge_kernel_timing_get(int index, char* name, int name_cap, int64_t* launches,
                             double* total_ms, double* work, int* work_kind);
 
+/* Library-wide settings; no counterpart in the reference.  Each starts from an environment
+ * variable that is read once, when the library is loaded, and is changed afterwards only
+ * through forge_set_option (an atomic store; a launch reads the value it finds).
+ *   "sweep_schedule"        FORGE_SWEEP_SCHEDULE=left|right   0 (default): by tile count,
+ *                           1: left-looking, 2: right-looking -- see forge_gptq_sweep_batched
+ *   "fp32_blocked_sum"      FORGE_FP32_BLOCKED_SUM=1          1: the factorisation's and the direct
+ *                           sweep's blocked sums stay on the fp32 matrix instruction
+ *   "sweep_update_products" FORGE_SWEEP_UPDATE_PRODUCTS=n     bf16 piece products per fp32 product in
+ *                           the block updates of forge_gptq_sweep_direct_batched: 3 (two pieces
+ *                           per operand, each rounded to nearest, products (2,1) (1,2) (1,1),
+ *                           within ~2^-17 of the fp32 product), 4 (adds (2,2)), 6 (three
+ *                           truncated pieces, every product of weight >= 2^-16: fp32-grade), 1
+ *                           (operands rounded to bf16; for measurements: it moves 2-16 % of
+ *                           the codes) or 0 (default): 3 from C = 4096 on, 6 below; the
+ *                           factorisation always uses 6
+ * forge_set_option returns FORGE_ERR_INVALID for an unknown name or a value out of range;
+ * forge_get_option returns -1 for an unknown name. */
+int forge_set_option(const char* name, int64_t value);
+int64_t forge_get_option(const char* name);
+
 /* ------------------------------------------------------------------ quant grid */
 
 /* Replaces kernels.build_group_meta_packed (kernels.cpp:93-97, quant_grid.cu:186-224).
@@ -101,8 +121,8 @@ int forge_sparsegptq14_solver(float* W, float* U, const float* scales, const flo
  * Schedule: with at least 128 tiles of 128 rows (batch * ceil(R/128)) each column block is
  * brought up to date by one long product over all earlier columns just before it is swept;
  * with fewer, every finished block is pushed into all later columns at once (more tiles per
- * launch).  Same fma chain per element either way, identical results.  FORGE_SWEEP_SCHEDULE=left
- * or =right in the environment forces one of them. */
+ * launch).  Same fma chain per element either way, identical results.  The option
+ * "sweep_schedule" forces one of them. */
 int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
                              const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                              uint32_t* M, const float* uinv, int64_t batch, int64_t C,
@@ -129,8 +149,9 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * multiply-add per earlier column, in ascending order (the chain of solver.cu:91-94 carried
  * across blocks), reproducible bit for bit on a CPU.  With a workspace of
  * forge_gptq_sweep_direct_workspace_bytes(batch, C) bytes that update is summed in blocks of
- * 128 columns from three bf16 pieces per fp32 operand on the bf16 matrix pipe wherever a
- * block is a full 128 x 128 tile (fp32-grade accuracy, different rounding, faster). */
+ * 128 columns from bf16 pieces of the fp32 operands on the bf16 matrix pipe wherever a block
+ * is a full 128 x 128 tile and the left-looking schedule applies (see "sweep_update_products"
+ * under forge_set_option: different rounding than the chain, faster). */
 int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                     const float* scalesT, const float* qzerosT,
                                     const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
@@ -209,7 +230,7 @@ int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype);
  * pieces of one panel), 256-byte aligned.
  * When C is a multiple of 128 the trailing updates are computed from three bf16 pieces per
  * fp32 operand on the bf16 matrix pipe (fp32-grade accuracy; not bit-identical to the fp32
- * update).  FORGE_FP32_BLOCKED_SUM=1 in the environment selects the fp32 update. */
+ * update).  The option "fp32_blocked_sum" selects the fp32 update. */
 int forge_chol_inv_upper_batched(float* H, const float* damp, float* U, float* udiag,
                                  int32_t* info, int64_t batch, int64_t C, int normalise,
                                  void* ws, int64_t ws_bytes, forge_stream_t stream);

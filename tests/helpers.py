@@ -41,15 +41,17 @@ def flip_rate(a, b):
 
 
 class Float64StagesGPTQ(oracle.GPTQ):
-    """The oracle's per-layer flow with its two fp32 LIBRARY stages -- the SGEMM that sums the
-    Hessian (gptq.py:79) and LAPACK's potrf/potri/potrf (gptq.py:160-164) -- computed in
-    float64 and rounded to fp32 once.  The reference fixes neither library's summation order,
-    so this is as valid a realisation of its arithmetic as the oracle's own, and the most
-    accurate one; everything else (activation order from the fp32 diagonal, damping, grid
-    search, the sweep's fma chain) is the oracle's code unchanged.
+    """The oracle's per-layer flow with the reference's LIBRARY calls realised differently:
+    the SGEMM that sums the Hessian (gptq.py:79) and LAPACK's potrf/potri/potrf
+    (gptq.py:160-164) are computed in float64 and rounded to fp32 once, and the SGEMM of the
+    trailing update (solver.cu:146-150) sums each block's products from zero and then
+    subtracts (``TRAIL_GEMM``) instead of continuing the in-block fma chain.  The reference
+    fixes none of these libraries' summation orders, so this is as valid a realisation of its
+    arithmetic as the oracle's own; everything else (activation order from the fp32 diagonal,
+    damping, grid search, the in-block kernel) is the oracle's code unchanged.
 
     flips(oracle, this) is the FLOOR the end-to-end tests use: how far the reference's codes
-    move when only the rounding inside those two library calls changes."""
+    move when only the rounding inside its library calls changes."""
 
     def __init__(self, *a, **kw):
         super().__init__(*a, **kw)
@@ -79,7 +81,7 @@ class Float64StagesGPTQ(oracle.GPTQ):
 def reference_floor(W, batches, qo, **kw):
     """(floor, q64): q64 = codes of Float64StagesGPTQ on the same inputs, floor = the share
     of the oracle's codes `qo` that differ from them."""
-    t = Float64StagesGPTQ(linear(W), **kw)
+    t = Float64StagesGPTQ(linear(W), trail_mode=oracle.TRAIL_GEMM, **kw)
     for b in batches:
         t.update(b)
     out = t.quantize()

@@ -41,6 +41,20 @@ def test_invalid_arguments_are_rejected_without_a_launch():
     assert lib.forge_chol_workspace_bytes(2, 256) == 2 * 2 * 128 * 128 * 4 + 2 * 256 * 128 * 6
 
 
+def test_options_are_settings_of_the_library_not_of_the_environment(monkeypatch):
+    from forge.backend.hip import load_library
+    lib = load_library()
+    assert lib.forge_get_option(b"sweep_update_products") == 0
+    assert lib.forge_get_option(b"sweep_schedule") == 0
+    monkeypatch.setenv("FORGE_SWEEP_SCHEDULE", "right")          # read at load time only
+    assert lib.forge_get_option(b"sweep_schedule") == 0
+    assert lib.forge_set_option(b"sweep_schedule", 2) == 0 and lib.forge_get_option(b"sweep_schedule") == 2
+    assert lib.forge_set_option(b"sweep_schedule", 0) == 0
+    assert lib.forge_set_option(b"sweep_update_products", 5) == 1
+    assert b"not allowed" in lib.forge_last_error()
+    assert lib.forge_set_option(b"no_such_option", 1) == 1 and lib.forge_get_option(b"no_such_option") == -1
+
+
 @pytest.mark.skipif(torch.cuda.is_available(), reason="CPU-only behaviour")
 def test_no_cpu_fallback():
     from forge.backend.hip import kernels

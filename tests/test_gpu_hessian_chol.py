@@ -80,19 +80,22 @@ def test_factor_matches_float64(hip, C, normalise):
 @pytest.mark.parametrize("B,C", [(8, 1536), (3, 640)])
 def test_factor_bf16_split_and_fp32_updates_agree(hip, monkeypatch, B, C):
     """C a multiple of 128: the trailing updates run as three-piece bf16 products by default
-    and as fp32 blocked sums with FORGE_FP32_BLOCKED_SUM=1; both are fp32-accurate."""
+    and as fp32 blocked sums with the option fp32_blocked_sum = 1; both are fp32-accurate."""
     g = torch.Generator().manual_seed(C)
     X = torch.randn(B, 2 * C, C, generator=g, dtype=torch.float64)
     X[:, :, :5] *= 6
     H = ((2.0 / X.shape[1]) * X.transpose(1, 2) @ X).float()
     H[B - 1, 7, 7] = float("nan")                       # one failing matrix among the good ones
     damp = (0.01 * torch.diagonal(H[:B - 1], dim1=1, dim2=2).mean()).repeat(B).float()
-    monkeypatch.delenv("FORGE_FP32_BLOCKED_SUM", raising=False)
+    assert hip.get_option("fp32_blocked_sum") == 0
     Us, uds, infos = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
-    monkeypatch.setenv("FORGE_FP32_BLOCKED_SUM", "1")
-    Uf, udf, infof = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
-    # upper_only: same values on and above the diagonal blocks, nothing promised left of them
-    Uu, _, _ = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV), upper_only=True)
+    hip.set_option("fp32_blocked_sum", 1)
+    try:
+        Uf, udf, infof = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV))
+        # upper_only: same values on and above the diagonal blocks, nothing promised left of them
+        Uu, _, _ = hip.chol_inv_upper_batched(H.clone().to(DEV), damp.to(DEV), upper_only=True)
+    finally:
+        hip.set_option("fp32_blocked_sum", 0)
     assert torch.equal(torch.triu(Uu), torch.triu(Uf))
     assert infos.tolist()[:B - 1] == [0] * (B - 1) and infos[B - 1].item() > 0
     assert infof.tolist() == infos.tolist()

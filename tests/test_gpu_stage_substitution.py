@@ -14,7 +14,7 @@ import torch
 
 import oracle
 from forge import synth
-from helpers import linear
+from helpers import linear, reference_floor
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -105,11 +105,16 @@ def test_direct_route_sweep_on_the_oracles_hessian(hip, name):
     """The route the benchmark times.  The oracle's permuted, damped Hessian is factored on
     the GPU (factor of H itself), the matrix V is copied back, and the displacement-form
     sweep runs on both sides with that V: the fp32-chain form equals its CPU checker bit for
-    bit, and the shipped bf16-piece block updates differ from it in <= 0.1 % of the codes."""
+    bit.  The block updates the library ships for batches of experts (left-looking schedule,
+    sums of 128 products from bf16 pieces) are a different fp32-grade summation, not a chain:
+    their codes are compared with the chain's for 6, 3 (the default) and 1 piece products per
+    fp32 product.  6 and 3 must stay within max(0.1 %, a quarter of the floor) -- the floor
+    being what the reference's own codes move by between two fp32 realisations of its
+    library stages; plain bf16 operands (1 product) are reported: they move 2-16 %."""
     W, X, kw = _case(name)
     R, C = W.shape
     sparse = kw.get("algorithm") == "sparsegptq"
-    o, scales, qzeros, _, Wt = _oracle_stages(W, X, kw)
+    o, scales, qzeros, U, Wt = _oracle_stages(W, X, kw)
     se, ze = o._expand(scales, C, R).contiguous(), o._expand(qzeros, C, R).contiguous()
     L, info = hip.chol_reverse_lower_batched(o.H.to(DEV).view(1, C, C).clone(), None)
     assert int(info.item()) == 0
@@ -117,21 +122,42 @@ def test_direct_route_sweep_on_the_oracles_hessian(hip, name):
     Vc = torch.triu(V[0].cpu()).contiguous()          # tiles below the diagonal are unwritten
     sT, zT, g_idx = _batched_meta(o, scales, qzeros, R)
     Xd = Wt.to(DEV).view(1, C, R)
+    mdiag = L[0].diagonal().contiguous().view(1, C) if sparse else None
+
+    def gpu(**k):
+        r = hip.gptq_sweep_direct_batched(Xd.clone(), V, sT, zT, g_idx, 4, sparse14=sparse,
+                                          mdiag=mdiag, **k)
+        return r if sparse else (r, None)
+
     if sparse:
-        mdiag = L[0].diagonal().contiguous().view(1, C)
         q_ref, M_ref = oracle.sparsegptq14_solver_direct(Wt.clone(), Vc, mdiag[0].cpu(), se, ze, 4)
-        q_x, M_x = hip.gptq_sweep_direct_batched(Xd.clone(), V, sT, zT, g_idx, 4, exact_chain=True,
-                                                 sparse14=True, mdiag=mdiag)
-        q_s, M_s = hip.gptq_sweep_direct_batched(Xd.clone(), V, sT, zT, g_idx, 4, sparse14=True,
-                                                 mdiag=mdiag)
-        assert torch.equal(M_ref.view(torch.int32), M_x[0].cpu().view(torch.int32))
-        mask_diff = (M_x.view(torch.int32) != M_s.view(torch.int32)).float().mean().item()
-        assert mask_diff <= 1e-3
+        q_orc, _ = oracle.sparsegptq14_solver(Wt.clone(), U.clone(), se, ze, 4)
     else:
-        q_ref = oracle.gptq_solver_direct(Wt.clone(), Vc, se, ze, 4)
-        q_x = hip.gptq_sweep_direct_batched(Xd.clone(), V, sT, zT, g_idx, 4, exact_chain=True)
-        q_s = hip.gptq_sweep_direct_batched(Xd.clone(), V, sT, zT, g_idx, 4)
+        q_ref, M_ref = oracle.gptq_solver_direct(Wt.clone(), Vc, se, ze, 4), None
+        q_orc = oracle.gptq_solver(Wt.clone(), U, se, ze, 4)
+    q_x, M_x = gpu(exact_chain=True)
     assert torch.equal(q_ref, q_x[0].cpu())
-    flips = (q_x != q_s).float().mean().item()
-    print(f"{name}: bf16-piece block updates vs fp32 chain, flips {flips:.2e}")
-    assert flips <= 1e-3
+    if sparse:
+        assert torch.equal(M_ref.view(torch.int32), M_x[0].cpu().view(torch.int32))
+    # floor: the oracle's own codes against its float64-stage realisation (solver order)
+    floor, out64 = reference_floor(W, [X], q_orc[o.perm_inv].t().contiguous(), **kw)
+    bound = max(1e-3, 0.25 * floor)
+    hip.set_option("sweep_schedule", 1)               # what a batch of experts takes
+    try:
+        for products in (6, 3, 1):
+            old = hip.set_option("sweep_update_products", products)
+            try:
+                q_s, M_s = gpu()
+            finally:
+                hip.set_option("sweep_update_products", old)
+            flips = (q_x != q_s).float().mean().item()
+            print(f"{name}: block updates from {products} piece product(s) vs fp32 chain: flips "
+                  f"{flips:.2e} (floor {floor:.2e})")
+            if products > 1:
+                assert flips <= bound, (products, flips, floor)
+                if sparse:
+                    assert (M_x.view(torch.int32) != M_s.view(torch.int32)).float().mean().item() <= bound
+            else:
+                assert flips > bound                  # why plain bf16 operands are not shipped
+    finally:
+        hip.set_option("sweep_schedule", 0)

@@ -162,11 +162,13 @@ def test_sweep_schedules_and_block_update_kernels_agree(hip, monkeypatch):
     zT = torch.full_like(sT, 8.0)
     gi = (torch.arange(C) // gs).int().repeat(B, 1).to(DEV)
     out = {}
-    for sched in ("left", "right"):
-        monkeypatch.setenv("FORGE_SWEEP_SCHEDULE", sched)
-        out["ref", sched] = hip.gptq_sweep_batched(X.clone(), U, sT, zT, gi, 4)
-        out["direct", sched] = hip.gptq_sweep_direct_batched(X.clone(), V, sT, zT, gi, 4, exact_chain=True)
-    monkeypatch.delenv("FORGE_SWEEP_SCHEDULE")
+    try:
+        for code, sched in ((1, "left"), (2, "right")):
+            hip.set_option("sweep_schedule", code)
+            out["ref", sched] = hip.gptq_sweep_batched(X.clone(), U, sT, zT, gi, 4)
+            out["direct", sched] = hip.gptq_sweep_direct_batched(X.clone(), V, sT, zT, gi, 4, exact_chain=True)
+    finally:
+        hip.set_option("sweep_schedule", 0)
     assert torch.equal(out["ref", "left"], out["ref", "right"])
     assert torch.equal(out["direct", "left"], out["direct", "right"])
     q_bf16 = hip.gptq_sweep_direct_batched(X.clone(), V, sT, zT, gi, 4)
