@@ -5,23 +5,36 @@
 Workload (default): the DeepSeek-V3-style MoE layer of the benchmark definition -- 256
 experts, gate/up 2048x7168 and down 7168x2048 (bf16 after an fp8-e4m3 128x128 block-scale
 round trip), 8192 bf16 tokens routed top-8 with Zipf(1.1) popularity, 4-bit symmetric
-g128, act-order, MSE scale search (the GPTQ class default), damp 0.01.  One STEP = one
-pass of the hot path over one chunk of experts, everything already resident in HBM:
-ragged Hessian accumulation for gate/up and for down, then per expert two factorisations
-(gate and up share theirs), three scale searches and three sweeps.  Successive steps walk
-through the layer's experts chunk by chunk (their routed-token lists differ).
+g128, act-order, MSE scale search (the GPTQ class default), damp 0.01; built by
+forge.synth.deepseek_v3_moe (seed 0) on the GPU.  One STEP = one pass of the hot path over
+one chunk of experts, everything already resident in HBM: ragged Hessian accumulation for
+gate/up and for down, then per expert two factorisations (gate and up share theirs), three
+scale searches and three sweeps.  Successive steps walk through the layer's experts chunk
+by chunk (their routed-token lists differ).
 value = experts quantised per second = steps * chunk / elapsed.
 
-After the timed steps one more step runs with the library's per-kernel event timing
-switched on; its dominant kernel gives the `roofline` object.  `cpu_baseline` times the CPU
-oracle (reference-structured: 32-column C kernel + BLAS SGEMM trailing update, LAPACK
-factorisation, OpenMP grid search) on one expert of the same workload.
+After the timed steps:
+* one more step runs with the library's per-kernel HIP-event timing switched on (events on
+  the stream each kernel is launched on); its dominant kernel gives `roofline`, every
+  kernel a line in `kernels` with its algorithmic rate and the fraction of the peak that
+  bounds it;
+* `reference_route`: the same steps on the reference's route (factor of inv(H), fp32-chain
+  sweep: every integer stage bit-exact against the CPU oracle);
+* `hessian_buckets`: the rank-k kernel alone at 16 / 256 / 1024 / 4096 tokens per expert;
+* `hbm_kernels`: min/max grid, int4 pack, fp8 block dequant at benchmark shapes;
+* `other_configs`: configs 1, 2, 4, 5 of the benchmark definition, end to end;
+* `cpu_baseline`: the CPU oracle in the reference's structure (32-column C kernel + BLAS
+  SGEMM trailing update, LAPACK potrf/potri/potrf, OpenMP grid search) on four experts of
+  the same layer (light, median, heavy, heaviest token count), 1 warm-up + 3 repetitions
+  each, median.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 from concurrent.futures import ThreadPoolExecutor
@@ -31,24 +44,25 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
 
-PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "hbm": 8000.0}      # TFLOP/s, TFLOP/s, GB/s
-# HBM bytes per launch of the GEMM kernel on the default workload (64 experts per step),
-# from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by
-# what the counter reads for the plain 1 GiB copy of --copy-calibration: x2.0 and x1.0);
-# summary in profiles/bench_deepseek_v3_hbm_traffic_pmc.txt.  What a launch has to read once
-# averages ~2.6e9 bytes over the 140 launches of a step: the rows of the factor below the
-# current block (factorisation, C=7168: ~2.2e9 per launch), the displacement rows of all
-# earlier columns (sweep: ~3.8e9 per launch for gate/up, ~1.9e9 for down).
-MEASURED_TRAFFIC = {("deepseek_v3", 64, "split_gemm_bf16x3"): 3.04e9}
+PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "valu_f32": 157.3, "hbm": 8000.0}   # TFLOP/s ... GB/s
+# Transcendental issue rate: v_log_f32 / v_exp_f32 run at a quarter of the fp32 rate, 16 lanes
+# per clock and SIMD: 256 CUs x 4 SIMDs x 4 per clock x 2.4 GHz.
+PEAK_TRANSCENDENTALS = 256 * 4 * 4 * 2.4e9
 
-KERNEL_BOUND = {          # kernel name -> (bound, peak key, unit, executed / counted work)
-    "chain_gemm_blocked_sum": ("mfma", "mfma_f32", "TFLOP/s", 1.0),
-    "chain_gemm": ("mfma", "mfma_f32", "TFLOP/s", 1.0),
-    # the library counts 2*M*N*K per launch; the kernel forms every fp32 product from six
-    # bf16 products on the bf16 matrix pipe, and it is that pipe's peak it is priced against
-    "split_gemm_bf16x3": ("mfma", "mfma_bf16", "TFLOP/s", 6.0),
-    "hessian_syrk_bf16": ("mfma", "mfma_bf16", "TFLOP/s", 1.0),
-    "hessian_syrk_f32": ("mfma", "mfma_f32", "TFLOP/s", 1.0),
+# kernel name (as the library's timing records call it) -> (bound, peak key, executed / counted)
+# The library counts ALGORITHMIC work per launch: 2*M*N*K for the GEMMs whatever the number
+# of bf16 piece products that form an fp32 product (`executed` = that number), executed tiles
+# (on and above the diagonal) for the Hessian, unique bytes for the movers.
+KERNEL_BOUND = {
+    "split_gemm_bf16x2": ("mfma", "mfma_bf16", 3.0),
+    "split_gemm_bf16x3": ("mfma", "mfma_bf16", 6.0),
+    "chain_gemm_blocked_sum": ("mfma", "mfma_f32", 1.0),
+    "chain_gemm": ("mfma", "mfma_f32", 1.0),
+    "hessian_syrk_bf16": ("mfma", "mfma_bf16", 1.0),
+    "hessian_syrk_f32": ("mfma", "mfma_f32", 1.0),
+    "sweep_block": ("valu", "valu_f32", 1.0),
+    "sweep_block_sparse14": ("valu", "valu_f32", 1.0),
+    "chol_diag_block": ("latency", "valu_f32", 1.0),
 }
 
 CONFIGS = {
@@ -59,38 +73,28 @@ CONFIGS = {
 }
 
 
-def make_workload(cfg, chunk, seed=0):
-    """Weights of `chunk` experts (reused by every step: values do not change the work) and
-    the routed, expert-sorted activations of ALL experts, on the GPU."""
+def make_workload(name, cfg, chunk, seed=0):
+    """forge.synth's MoE layer of that configuration, generated on the GPU: weights of `chunk`
+    experts (reused by every step: values do not change the work) and the routed,
+    expert-sorted activations of ALL experts."""
     import torch
     from forge import synth
-    dev = "cuda"
-    g = torch.Generator(device=dev).manual_seed(seed)
-    Hd, I, E = cfg["hidden"], cfg["inter"], cfg["n_experts"]
-    X = torch.randn(cfg["tokens"], Hd, generator=g, device=dev).to(torch.bfloat16)
-    rows = synth.route_topk(cfg["tokens"], E, 8, g, device=dev)
-
-    def w(R, C):
-        t = (0.02 * torch.randn(chunk, R, C, generator=g, device=dev)).to(torch.bfloat16)
-        if cfg["fp8"]:
-            for i in range(chunk):
-                t[i] = synth.fp8_block_roundtrip(t[i])
-        return t
-
-    Wg, Wu, Wd = w(I, Hd), w(I, Hd), w(Hd, I)
-    counts = [int(r.numel()) for r in rows]
-    xs = X[torch.cat(rows)].contiguous()                      # gate/up inputs, grouped by expert
+    make = synth.deepseek_v3_moe if name == "deepseek_v3" else synth.qwen3_moe
+    moe = make(seed=seed, device="cuda", experts=chunk)
+    assert (moe.hidden, moe.inter, moe.n_experts) == (cfg["hidden"], cfg["inter"], cfg["n_experts"])
+    counts = [int(r.numel()) for r in moe.rows]
+    xs = moe.X[torch.cat(moe.rows)].contiguous()              # gate/up inputs, grouped by expert
     # down-proj inputs silu(x Wg^T) * (x Wu^T) with the unquantised weights of the chunk's
     # slot the expert will be solved in (one calibration forward, outside the timed region)
-    hs = torch.empty(xs.shape[0], I, dtype=torch.bfloat16, device=dev)
+    hs = torch.empty(xs.shape[0], cfg["inter"], dtype=torch.bfloat16, device="cuda")
     o = 0
     for e, n in enumerate(counts):
         if n:
             x = xs[o:o + n]
             slot = e % chunk
-            hs[o:o + n] = (torch.nn.functional.silu(x @ Wg[slot].T) * (x @ Wu[slot].T))
+            hs[o:o + n] = torch.nn.functional.silu(x @ moe.Wg[slot].T) * (x @ moe.Wu[slot].T)
         o += n
-    return dict(Wg=Wg, Wu=Wu, Wd=Wd, xs=xs, hs=hs, counts=counts)
+    return dict(Wg=moe.Wg, Wu=moe.Wu, Wd=moe.Wd, xs=xs, hs=hs, counts=counts)
 
 
 STREAMS = []
@@ -99,6 +103,7 @@ STREAMS = []
 def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"):
     """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
     jobs one after the other (per-kernel event times are then exclusive)."""
+    import torch
     from forge.moe import ExpertGroupGPTQ
     E = cfg["n_experts"]
     e0 = (step * chunk) % E
@@ -106,7 +111,6 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
     starts = [0]
     for c in wl["counts"]:
         starts.append(starts[-1] + c)
-    import torch
     if ids == list(range(ids[0], ids[0] + chunk)):
         xs = wl["xs"][starts[ids[0]]:starts[ids[-1] + 1]]
         hs = wl["hs"][starts[ids[0]]:starts[ids[-1] + 1]]
@@ -125,8 +129,7 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
     cur = torch.cuda.current_stream()
     for s in STREAMS:
         s.wait_stream(cur)
-    # SPLIT sub-batches of experts per group, each on its own stream
-    nsub = max(1, len(STREAMS) // 2)
+    nsub = max(1, len(STREAMS) // 2)              # sub-batches of experts, each on its own streams
     per = (chunk + nsub - 1) // nsub
     jobs = []
     with ThreadPoolExecutor(max_workers=len(STREAMS)) as pool:
@@ -150,53 +153,242 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
                     stream.synchronize()
                 jobs.append(job)
         results = [j.result() for j in jobs]
-    out_gu, out_dn = results[0::2], results[1::2]
     for s in STREAMS:
         cur.wait_stream(s)
-    return out_gu, out_dn
+    return results[0::2], results[1::2]
 
 
-def cpu_baseline(wl, cfg, expert_slot=0):
-    """One expert (gate, up, down) on the host cores with the CPU oracle."""
+def timed_steps(wl, cfg, chunk, steps, warmup, first_step=0, **kw):
+    import torch
+    for i in range(warmup):
+        run_step(wl, cfg, chunk, first_step + i, **kw)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        run_step(wl, cfg, chunk, first_step + warmup + i, **kw)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def kernel_table(stats):
+    """Per-kernel lines from the library's timing records: algorithmic rate and the fraction
+    of the peak of the unit that bounds the kernel."""
+    total_ms = sum(s["ms"] for s in stats.values()) or 1.0
+    out = {}
+    for name, s in sorted(stats.items(), key=lambda kv: -kv[1]["ms"]):
+        flop = s["unit"] == "flop"
+        rate = s["work"] / (s["ms"] * 1e-3) / (1e12 if flop else 1e9) if s["ms"] > 0 else 0.0
+        bound, peak_key, executed = KERNEL_BOUND.get(name, ("hbm", "hbm", 1.0))
+        line = dict(launches=s["launches"], ms=round(s["ms"], 3),
+                    avg_us=round(1e3 * s["ms"] / max(s["launches"], 1), 2),
+                    share=round(s["ms"] / total_ms, 4), rate=round(rate, 2),
+                    rate_unit="TFLOP/s" if flop else "GB/s", bound=bound,
+                    frac=round(rate / PEAK[peak_key], 4))
+        if executed != 1.0:
+            line["executed_frac"] = round(rate * executed / PEAK[peak_key], 4)
+        out[name] = line
+    return out
+
+
+def measured_traffic(config, chunk, kernel):
+    """HBM bytes per launch of `kernel`, from the committed rocprofv3 --pmc summary of this
+    file's default command (a line `traffic <config> <chunk> <kernel> <bytes>`), or None."""
+    path = ROOT / "profiles" / f"bench_{config}_hbm_traffic_pmc.txt"
+    if not path.exists():
+        return None
+    for line in path.read_text().splitlines():
+        m = re.match(r"traffic\s+(\S+)\s+(\d+)\s+(\S+)\s+([0-9.eE+]+)", line.strip())
+        if m and m.group(1) == config and int(m.group(2)) == chunk and m.group(3) == kernel:
+            return float(m.group(4))
+    return None
+
+
+def timing_pass(fn):
+    import torch
+    from forge.backend.hip import kernels
+    torch.cuda.synchronize()
+    kernels.timing_enable(True)
+    fn()
+    torch.cuda.synchronize()
+    stats = kernels.timing_collect()
+    kernels.timing_enable(False)
+    return stats
+
+
+# ---------------------------------------------------------------- side measurements
+def hessian_buckets(C=7168, E=64):
+    """The rank-k kernel alone, E experts with the same token count each: algorithmic flops
+    2 n C^2 and bytes 2 n C + 4 C^2 per expert against the kernel's event time."""
+    import torch
+    from forge.backend.hip import kernels
+    out = {}
+    H = torch.empty((E, C, C), dtype=torch.float32, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    for n in (16, 256, 1024, 4096):
+        X = torch.randn(E * n, C, generator=g, device="cuda").to(torch.bfloat16)
+        offs = [i * n for i in range(E + 1)]
+        kernels.hessian_update_grouped(X, offs, H, [2.0 / n] * E, [0.0] * E)      # warm-up
+        stats = timing_pass(lambda: kernels.hessian_update_grouped(X, offs, H, [2.0 / n] * E, [0.0] * E))
+        ms = sum(s["ms"] for k, s in stats.items() if k.startswith("hessian"))
+        flops = 2.0 * n * C * C * E
+        nbytes = (2.0 * n * C + 4.0 * C * C) * E
+        out[str(n)] = dict(ms=round(ms, 3), tflops=round(flops / ms / 1e9, 1),
+                           mfma_frac=round(flops / ms / 1e9 / PEAK["mfma_bf16"], 4),
+                           gbps=round(nbytes / ms / 1e6, 1),
+                           hbm_frac=round(nbytes / ms / 1e6 / PEAK["hbm"], 4))
+        del X
+    return dict(C=C, experts=E, tokens_per_expert=out,
+                note="flops 2nC^2 (the full product the reference's SGEMM executes; the kernel "
+                     "computes the tiles on and above the diagonal), bytes 2nC + 4C^2 per expert")
+
+
+def hbm_kernels(wl):
+    """min/max grid, int4 pack and fp8 block dequant on the chunk's gate_proj stack (64 x 2048 x
+    7168): achieved GB/s of the algorithmic bytes against 8 TB/s."""
+    import torch
+    from forge.backend.hip import kernels
+    Wg = wl["Wg"]
+    B, O, I = Wg.shape
+    g = torch.Generator(device="cuda").manual_seed(2)
+    codes = torch.randint(0, 16, (B * O, I), generator=g, device="cuda", dtype=torch.uint8)
+    zeros = torch.full((B * O * ((I + 127) // 128),), 8.0, device="cuda")
+    w8 = Wg.float().clamp(-0.05, 0.05).mul(448 / 0.05).to(torch.float8_e4m3fn).view(torch.uint8)
+    sinv = torch.full((B, (O + 127) // 128, (I + 127) // 128), 0.05 / 448, device="cuda")
+
+    def work():
+        for _ in range(3):
+            kernels.quant_grid(Wg, 128, 4, False, False)
+            kernels.pack_int4(codes, zeros, 128)
+            kernels.fp8_block_dequant(w8, sinv)
+
+    work()
+    stats = timing_pass(work)
+    return {k: dict(avg_us=v["avg_us"], gbps=v["rate"], hbm_frac=v["frac"])
+            for k, v in kernel_table(stats).items() if v["rate_unit"] == "GB/s"}
+
+
+def other_configs(reps=3):
+    """Configs 1, 4, 5 through forge.gptq.GPTQ (update + quantize, wall clock, median of
+    `reps` after one warm-up) and config 2 (the whole Qwen3-shaped layer in one step)."""
+    import torch
+    from forge import synth
+    from forge.gptq import GPTQ
+    out = {}
+
+    def dense(tag, case, **kw):
+        W, X = case.W.cuda(), case.X.cuda()
+        layer = torch.nn.Linear(W.shape[1], W.shape[0], bias=False, device="cuda", dtype=W.dtype)
+        layer.weight.data = W
+
+        def once():
+            h = GPTQ(layer, device="cuda", **kw)
+            h.update(X)
+            return h.quantize()
+
+        once()
+        times = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            once()
+            torch.cuda.synchronize()
+            times.append(1e3 * (time.perf_counter() - t0))
+        table = kernel_table(timing_pass(once))
+        dom = next(iter(table))
+        out[tag] = dict(ms=round(statistics.median(times), 3), shape=list(W.shape), tokens=X.shape[0],
+                        dominant_kernel=dom, dominant=table[dom])
+
+    base = dict(bits=4, group_size=128, rel_damp=0.01)
+    dense("config1_dense_2048_mse", synth.dense_outlier(), symmetric=True,
+          quantization_scale="mse", quantization_order="default", **base)
+    dense("config1_dense_2048_absmax", synth.dense_outlier(), symmetric=True,
+          quantization_scale="absmax", quantization_order="default", **base)
+    dense("config4_student_t_4096x7168", synth.student_t_weight(), symmetric=False,
+          quantization_scale="mse", quantization_order="default", **base)
+    dense("config5_sparse14_3072x1536", synth.sparse14_down_proj(), symmetric=True,
+          quantization_scale="mse", quantization_order="default", algorithm="sparsegptq", **base)
+    cfg = CONFIGS["qwen3"]
+    wl = make_workload("qwen3", cfg, cfg["chunk"])
+    dt = timed_steps(wl, cfg, cfg["chunk"], reps, 1)
+    table = kernel_table(timing_pass(lambda: run_step(wl, cfg, cfg["chunk"], 0, overlap=False)))
+    dom = next(iter(table))
+    out["config2_qwen3_layer"] = dict(ms=round(1e3 * dt / reps, 3), experts=cfg["chunk"],
+                                      experts_per_s=round(reps * cfg["chunk"] / dt, 1),
+                                      dominant_kernel=dom, dominant=table[dom])
+    return out
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(wl, cfg, reps=3):
+    """Four experts of the same layer (gate, up, down each) on the host cores with the CPU
+    oracle in the reference's structure; 1 warm-up, then `reps` timed repetitions per expert,
+    median per expert; experts/s = 4 / sum of the medians."""
     import torch
     import oracle
     counts = wl["counts"]
-    # an expert with a median token count
-    order = sorted(range(len(counts)), key=lambda e: counts[e])
-    e = order[len(order) // 2]
-    start = sum(counts[:e])
-    x = wl["xs"][start:start + counts[e]].cpu()
-    h = wl["hs"][start:start + counts[e]].cpu()
-    slot = e % wl["Wg"].shape[0]
+    order = sorted((e for e in range(len(counts)) if counts[e] > 0), key=lambda e: counts[e])
+    picks = [order[int(round(q * (len(order) - 1)))] for q in (0.1, 0.5, 0.9, 1.0)]
     kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"], quantization_scale="mse",
               quantization_order=cfg["order"], rel_damp=0.01, trail_mode=oracle.TRAIL_BLAS)
 
     def lin(W):
         layer = torch.nn.Linear(W.shape[1], W.shape[0], bias=False)
-        layer.weight.data = W.cpu().float().to(torch.bfloat16)
+        layer.weight.data = W
         return layer
 
-    t0 = time.perf_counter()
-    gate = oracle.GPTQ(lin(wl["Wg"][slot]), **kw)
-    gate.update(x)
-    gate.quantize()
-    # up_proj is a non-owner of gate_proj's Hessian and re-factorises it, as in the
-    # reference's flow (quant.py:382-397,514-517)
-    up = oracle.GPTQ(lin(wl["Wu"][slot]), owner=gate, **kw)
-    up.quantize()
-    down = oracle.GPTQ(lin(wl["Wd"][slot]), **kw)
-    down.update(h)
-    down.quantize()
-    dt = time.perf_counter() - t0
-    return dict(value=1.0 / dt, unit="experts/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"1 expert (gate+up+down, {counts[e]} routed tokens) of the same layer, "
-                       f"{dt:.1f} s on the host; 3 factorisations as in the reference's flow")
+    def inputs(e):
+        start = sum(counts[:e])
+        slot = e % wl["Wg"].shape[0]
+        return (wl["xs"][start:start + counts[e]].cpu(), wl["hs"][start:start + counts[e]].cpu(),
+                wl["Wg"][slot].cpu(), wl["Wu"][slot].cpu(), wl["Wd"][slot].cpu())
+
+    def solve(x, h, Wg, Wu, Wd):
+        t0 = time.perf_counter()
+        gate = oracle.GPTQ(lin(Wg), **kw)
+        gate.update(x)
+        gate.quantize()
+        # up_proj is a non-owner of gate_proj's Hessian and re-factorises it, as in the
+        # reference's flow (quant.py:382-397,514-517)
+        up = oracle.GPTQ(lin(Wu), owner=gate, **kw)
+        up.quantize()
+        down = oracle.GPTQ(lin(Wd), **kw)
+        down.update(h)
+        down.quantize()
+        return time.perf_counter() - t0
+
+    medians, listed = [], []
+    warm = True
+    for e in picks:
+        args = inputs(e)
+        if warm:
+            solve(*args)
+            warm = False
+        times = [solve(*args) for _ in range(reps)]
+        medians.append(statistics.median(times))
+        listed.append(dict(expert=e, tokens=counts[e], seconds=[round(t, 2) for t in times]))
+    total = sum(medians)
+    return dict(value=round(len(picks) / total, 4), unit="experts/s", cores=torch.get_num_threads(),
+                kind="port", os_cpu_count=os.cpu_count(), torch_num_threads=torch.get_num_threads(),
+                cpu_model=cpu_model(), experts=listed,
+                sample=f"{len(picks)} experts (gate+up+down; token counts "
+                       f"{[counts[e] for e in picks]}: 10 %, median, 90 %, heaviest) of the same layer, "
+                       f"1 warm-up + {reps} repetitions each, median; {total:.1f} s per pass; "
+                       "3 factorisations per expert as in the reference's flow")
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=4)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", default="deepseek_v3", choices=sorted(CONFIGS))
     ap.add_argument("--chunk", type=int, default=0, help="experts per step (0 = config default)")
@@ -204,6 +396,8 @@ def main():
                     help="sub-batches of a step's experts solved concurrently (one HIP stream each "
                          "for their gate/up and their down groups)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip reference_route, hessian_buckets, hbm_kernels and other_configs")
     ap.add_argument("--factor-route", default="direct", choices=["direct", "inverse"],
                     help="direct (default): sweep fed by the factor of H itself; inverse: the "
                          "reference's factor of inv(H) and fp32-chain sweep")
@@ -218,11 +412,10 @@ def main():
         sys.exit(2)
 
     import torch
-    from forge.backend.hip import kernels
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     cfg = CONFIGS[a.config]
     chunk = a.chunk or cfg["chunk"]
-    wl = make_workload(cfg, chunk)
+    wl = make_workload(a.config, cfg, chunk)
     mse = not a.no_mse
     STREAMS.extend(torch.cuda.Stream() for _ in range(2 * a.split))   # default priority
 
@@ -233,39 +426,26 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for i in range(a.warmup):
-        run_step(wl, cfg, chunk, i, mse, factor_route=a.factor_route)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        run_step(wl, cfg, chunk, a.warmup + i, mse, factor_route=a.factor_route)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    elapsed = timed_steps(wl, cfg, chunk, a.steps, a.warmup, mse=mse, factor_route=a.factor_route)
 
     # one more step with per-kernel HIP-event timing (on the stream the kernels run on); its
     # jobs run one after the other so that no kernel's time includes another stream's work
-    kernels.timing_enable(True)
-    run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False, factor_route=a.factor_route)
-    torch.cuda.synchronize()
-    stats = kernels.timing_collect()
-    kernels.timing_enable(False)
-    total_ms = sum(s["ms"] for s in stats.values())
-    breakdown = {}
-    for name, s in sorted(stats.items(), key=lambda kv: -kv[1]["ms"]):
-        rate = s["work"] / (s["ms"] * 1e-3) if s["ms"] > 0 else 0.0
-        breakdown[name] = dict(launches=s["launches"], ms=round(s["ms"], 3),
-                               avg_us=round(1e3 * s["ms"] / max(s["launches"], 1), 2),
-                               share=round(s["ms"] / total_ms, 4),
-                               rate=round(rate / (1e12 if s["unit"] == "flop" else 1e9), 2),
-                               rate_unit="TFLOP/s" if s["unit"] == "flop" else "GB/s")
+    stats = timing_pass(lambda: run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False,
+                                         factor_route=a.factor_route))
+    breakdown = kernel_table(stats)
     dom = next(iter(breakdown))
-    bound, peak_key, unit, executed = KERNEL_BOUND.get(dom, ("hbm", "hbm", "GB/s", 1.0))
-    achieved = round(breakdown[dom]["rate"] * executed, 2)
-    roofline = dict(kernel=dom, bound=bound, achieved=achieved, peak=PEAK[peak_key],
-                    unit=unit, frac=round(achieved / PEAK[peak_key], 4),
-                    traffic=MEASURED_TRAFFIC.get((a.config, chunk, dom))
+    d = breakdown[dom]
+    bound, peak_key, executed = KERNEL_BOUND.get(dom, ("hbm", "hbm", 1.0))
+    roofline = dict(kernel=dom, bound="mfma" if bound == "mfma" else "hbm", achieved=d["rate"],
+                    peak=PEAK[peak_key], unit=d["rate_unit"], frac=d["frac"],
+                    traffic=measured_traffic(a.config, chunk, dom)
                     if a.split == 1 and a.factor_route == "direct" and mse else None,
-                    avg_launch_us=breakdown[dom]["avg_us"], launches=breakdown[dom]["launches"])
+                    avg_launch_us=d["avg_us"], launches=d["launches"],
+                    note="achieved = algorithmic work (2*M*N*K counted once per fp32 product) / event time")
+    if executed != 1.0:
+        roofline["executed_frac"] = d["executed_frac"]
+        roofline["executed_note"] = (f"every fp32 product is formed from {int(executed)} bf16 piece products: "
+                                     f"{executed:.0f} x achieved is what the bf16 matrix pipe executes")
 
     out = {
         "metric": "experts quantized/sec (GPTQ 4-bit g128)",
@@ -274,7 +454,7 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(1e3 * elapsed / a.steps, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic (forge.synth, seed 0, generated on the GPU)",
         "config": {"workload": f"{a.config}: {cfg['n_experts']} experts, gate/up {cfg['inter']}x{cfg['hidden']}"
                                f" + down {cfg['hidden']}x{cfg['inter']}, {cfg['tokens']} tokens top-8 Zipf(1.1),"
                                f" 4-bit {'sym' if cfg['symmetric'] else 'asym'} g128"
@@ -284,6 +464,25 @@ def main():
         "roofline": roofline,
         "kernels": breakdown,
     }
+    if "mse_grid" in breakdown and mse:
+        # nominal candidate evaluations: P = 100 shrink factors for every weight of the step
+        n_w = chunk * 3 * cfg["inter"] * cfg["hidden"]
+        evals = 100.0 * n_w / (breakdown["mse_grid"]["ms"] * 1e-3)
+        out["mse_grid_search"] = dict(
+            candidate_evals_per_s=round(evals, 0),
+            frac_of_transcendental_rate=round(2.0 * evals / PEAK_TRANSCENDENTALS, 4),
+            note="nominal evaluations (100 candidates x weights) per second; each costs two "
+                 "transcendentals (v_log_f32, v_exp_f32); candidates dropped by the exact "
+                 "partial-sum pruning count as evaluated, so the fraction can exceed 1")
+    if not a.no_extras:
+        other = "inverse" if a.factor_route == "direct" else "direct"
+        dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route=other)
+        out["reference_route" if other == "inverse" else "direct_route"] = dict(
+            factor_route=other, ms_per_step=round(1e3 * dt / a.steps, 2),
+            value=round(a.steps * chunk / dt, 3), unit="experts/s")
+        out["hessian_buckets"] = hessian_buckets(cfg["hidden"], min(chunk, 64))
+        out["hbm_kernels"] = hbm_kernels(wl)
+        out["other_configs"] = other_configs()
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, cfg)
         out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)

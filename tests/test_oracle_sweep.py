@@ -139,3 +139,34 @@ def test_sparse_selection_uses_updated_weights_and_saliency():
         x[t + 1:] -= np.outer(Un[t, t + 1:], err)
     assert clear.any()
     assert np.array_equal(keep[:, clear], mine[:, clear])
+
+
+def test_reference_shaped_host_loop_is_pinned():
+    """TRAIL_BLAS: the 32-column kernel alone (oracle_gptq_inblock) followed by one BLAS SGEMM
+    per block, the reference's host loop literally (solver.cu:118-150).  The in-block kernel by
+    itself is the fma chain: with one block spanning the matrix it equals the chained solver
+    bit for bit, and with U = I it is round-to-nearest.  With 32-column blocks the SGEMM's
+    summation order differs from the chain's, so codes may move at ties only, and the
+    Hessian-weighted error stays the same."""
+    pr = random_problem(C=192, R=40)
+    Wt = pr["W"].t().contiguous()
+    one_block = oracle.gptq_solver(Wt.clone(), pr["U"], pr["se"], pr["ze"], 4,
+                                   trail_mode=oracle.TRAIL_BLAS, block=192)
+    chain = oracle.gptq_solver(Wt.clone(), pr["U"], pr["se"], pr["ze"], 4)
+    assert torch.equal(one_block, chain)
+    rtn = oracle.gptq_solver(Wt.clone(), torch.eye(192), pr["se"], pr["ze"], 4,
+                             trail_mode=oracle.TRAIL_BLAS)
+    assert np.array_equal(rtn.numpy(), mathref.rtn(Wt.numpy(), pr["se"].numpy(), pr["ze"].numpy(), 4))
+    pr = random_problem(C=512, R=128)
+    Wt = pr["W"].t().contiguous()
+    a = oracle.gptq_solver(Wt.clone(), pr["U"], pr["se"], pr["ze"], 4, trail_mode=oracle.TRAIL_CHAIN)
+    b = oracle.gptq_solver(Wt.clone(), pr["U"], pr["se"], pr["ze"], 4, trail_mode=oracle.TRAIL_BLAS)
+    Wb = oracle.gptq_solver.last_W                     # dequantised weights of the BLAS run
+    assert flip_rate(a, b) < 5e-3
+    want = (b.double() * pr["se"].double() - (pr["ze"] * pr["se"]).double()).float()
+    assert torch.equal(Wb, want)
+    H = pr["H"].double().numpy()
+    deq = lambda q: ((q.double() - pr["ze"].double()) * pr["se"].double()).t().numpy()
+    ea = mathref.layer_error(pr["W"].numpy(), deq(a), H)
+    eb = mathref.layer_error(pr["W"].numpy(), deq(b), H)
+    assert abs(eb / ea - 1) < 5e-3
