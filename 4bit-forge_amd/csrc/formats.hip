@@ -80,44 +80,93 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(
     }
 }
 
-// One thread per (pair of 32-column words, row): two u64 =
+// 1:4 codes + keep-masks -> the inference layout of bitpacking_sparsegptq14.cu:58-107: for
+// every row and every 32-column word one u64
 //   bf16(scale) << 48 | idx16 << 32 | qw32
-// qw32: eight 4-bit codes (default 8 = zero weight), idx16: eight 2-bit positions of the
-// kept column inside its group of four (bitpacking_sparsegptq14.cu:58-107).
-__global__ __launch_bounds__(256) void pack_sparse14_kernel(
-    const uint8_t* __restrict__ q_rc, const uint32_t* __restrict__ M,
-    const float* __restrict__ scales, uint64_t* __restrict__ out, int64_t C, int64_t R, int64_t G32) {
-    const int64_t G2 = (G32 + 1) >> 1;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t r = tid % R, g2 = tid / R;
-    if (g2 >= G2) return;
-    uint64_t word[2];
+// qw32 = the eight kept 4-bit codes of the word (8, the code of a zero weight, where a group
+// of four kept nothing), idx16 = their 2-bit positions inside their groups; words are stored
+// in pairs, out[pair][row][2].
+//
+// The three inputs want different lane orders: the codes are row-major [R, C] (a word's 32
+// bytes are contiguous, neighbouring words of one row follow each other), while masks,
+// scales and the output are word-major ([word][row]: neighbouring rows are contiguous).  So a
+// workgroup takes a tile of 32 rows x 32 words, brings the tile's codes into LDS with lanes
+// running along the columns (1 KiB contiguous per row, 16 bytes per lane), and then switches
+// to lanes running along the rows for everything else: 128-byte runs of masks and scales,
+// 512-byte runs of output, and byte reads from LDS whose row pitch (1040 bytes) spreads the
+// 32 rows over the banks.
+constexpr int SP_ROWS = 32, SP_WORDS = 32, SP_COLS = SP_WORDS * 32, SP_PITCH = SP_COLS + 16;
+
+__global__ __launch_bounds__(256) void pack_sparse14_tile_kernel(
+    const uint8_t* __restrict__ codes, const uint32_t* __restrict__ keep,
+    const float* __restrict__ scales, uint64_t* __restrict__ out, int64_t C, int64_t R,
+    int64_t n_words, bool vec_ok) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[SP_ROWS * SP_PITCH];
+    const int64_t row0 = (int64_t)blockIdx.y * SP_ROWS;
+    const int64_t word0 = (int64_t)blockIdx.x * SP_WORDS;
+    const int64_t col0 = word0 * 32;
+    const int tid = threadIdx.x;
+    // phase 1: lanes along the columns
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int64_t gid = 2 * g2 + h;
-        uint64_t packed = 0ull;
-        if (gid < G32) {
-            const uint32_t bitmask = M[gid * R + r];
-            uint32_t idx16 = 0, qw32 = 0x88888888u;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const uint32_t sub = (bitmask >> (4 * i)) & 0xFu;
-                if (sub == 0u) continue;
-                const int c = __ffs((int)sub) - 1;
-                idx16 |= (uint32_t)(c & 3) << (2 * i);
-                const int64_t cid = gid * 32 + i * 4 + c;
-                if (cid < C) {
-                    const uint32_t q = q_rc[r * C + cid] & 0xFu;
-                    qw32 = (qw32 & ~(0xFu << (4 * i))) | (q << (4 * i));
-                }
+    for (int j = 0; j < SP_ROWS * (SP_COLS / 16) / 256; ++j) {
+        const int piece = tid + 256 * j;
+        const int lr = piece / (SP_COLS / 16), lc = (piece % (SP_COLS / 16)) * 16;
+        const int64_t r = row0 + lr, c = col0 + lc;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (r < R && c < C) {
+            const uint8_t* src = codes + r * C + c;
+            if (vec_ok && c + 16 <= C) {
+                v = *reinterpret_cast<const uint4*>(src);
+            } else {
+                uint32_t w[4] = {0u, 0u, 0u, 0u};
+                for (int k = 0; k < 16 && c + k < C; ++k) w[k >> 2] |= (uint32_t)src[k] << (8 * (k & 3));
+                v = make_uint4(w[0], w[1], w[2], w[3]);
             }
-            packed = ((uint64_t)f32_to_bf16_rne(scales[gid * R + r]) << 48) |
-                     ((uint64_t)(idx16 & 0xFFFFu) << 32) | (uint64_t)qw32;
         }
-        word[h] = packed;
+        *reinterpret_cast<uint4*>(&tile[lr * SP_PITCH + lc]) = v;
     }
-    out[(g2 * R + r) * 2 + 0] = word[0];
-    out[(g2 * R + r) * 2 + 1] = word[1];
+    __syncthreads();
+    // phase 2: lanes along the rows; a thread builds both words of a pair
+    const int lr = tid & (SP_ROWS - 1);
+    const int64_t r = row0 + lr;
+    if (r >= R) return;
+    const uint8_t* trow = &tile[lr * SP_PITCH];
+#pragma unroll
+    for (int it = 0; it < SP_WORDS / 2 / 8; ++it) {
+        const int lpair = (tid >> 5) + 8 * it;                 // pair of words inside the tile
+        const int64_t pair = word0 / 2 + lpair;
+        if (2 * pair >= n_words) break;
+        uint64_t both[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int64_t word = 2 * pair + h;
+            uint64_t packed = 0ull;
+            if (word < n_words) {
+                const uint32_t mask = keep[word * R + r];
+                const uint8_t* tw = trow + (2 * lpair + h) * 32;
+                uint32_t where = 0u, kept = 0u;
+#pragma unroll
+                for (int grp = 0; grp < 8; ++grp) {
+                    const uint32_t four = (mask >> (4 * grp)) & 0xFu;
+                    uint32_t code = 8u, pos = 0u;
+                    if (four != 0u) {
+                        pos = (uint32_t)__builtin_ctz(four);   // first kept column of the group
+                        // columns past C hold no code: the slot keeps the code of zero
+                        if (word * 32 + 4 * grp + pos < C) code = tw[4 * grp + pos] & 0xFu;
+                    }
+                    where |= pos << (2 * grp);
+                    kept |= code << (4 * grp);
+                }
+                packed = ((uint64_t)f32_to_bf16_rne(scales[word * R + r]) << 48) |
+                         ((uint64_t)where << 32) | (uint64_t)kept;
+            }
+            both[h] = packed;
+        }
+        ulonglong2 o;
+        o.x = both[0];
+        o.y = both[1];
+        *reinterpret_cast<ulonglong2*>(out + (pair * R + r) * 2) = o;
+    }
 }
 
 // (q - q0) * s per group -> bf16/f32; 16 codes per thread (forge/utils/engine.py:71-97).
@@ -265,9 +314,13 @@ extern "C" int forge_pack_sparsegptq14_to_u64x2(const uint8_t* qweight_rc, const
     FORGE_REQUIRE(qweight_rc && M && scales && out, "null pointer");
     const int64_t G32 = forge::ceil_div(C, 32), G2 = (G32 + 1) >> 1;
     forge::KernelTiming timing("pack_sparse14_u64x2", (hipStream_t)stream,
-                               (double)R * C / 4.0 + 8.0 * G32 * R + 16.0 * G2 * R, forge::WORK_BYTES);
-    pack_sparse14_kernel<<<dim3((unsigned)forge::ceil_div(G2 * R, 256)), dim3(256), 0,
-                           (hipStream_t)stream>>>(qweight_rc, M, scales, out, C, R, G32);
+                               (double)R * C + 8.0 * G32 * R + 16.0 * G2 * R, forge::WORK_BYTES);
+    const bool vec_ok = (C % 16) == 0 && (reinterpret_cast<uintptr_t>(qweight_rc) % 16) == 0;
+    FORGE_REQUIRE(forge::ceil_div(R, SP_ROWS) < 65536, "R=%lld too large", (long long)R);
+    pack_sparse14_tile_kernel<<<dim3((unsigned)forge::ceil_div(G32, SP_WORDS),
+                                     (unsigned)forge::ceil_div(R, SP_ROWS)),
+                                dim3(256), 0, (hipStream_t)stream>>>(qweight_rc, M, scales, out, C, R,
+                                                                     G32, vec_ok);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

@@ -538,8 +538,9 @@ namespace {
 
 template <typename T>
 __global__ void reverse_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, int64_t C, int64_t R) {
-    const int64_t c = blockIdx.y;
-    for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < R; r += (int64_t)gridDim.x * blockDim.x)
+    // rows on grid.x (no 65535 limit), row pieces on grid.y
+    const int64_t c = blockIdx.x;
+    for (int64_t r = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; r < R; r += (int64_t)gridDim.y * blockDim.x)
         dst[c * R + r] = src[(C - 1 - c) * R + r];
 }
 
@@ -595,8 +596,9 @@ extern "C" int forge_babai_solver(const float* W, const float* A, const float* s
     int32_t* g_rev = (int32_t*)p; p += align256(C * 4);
     uint8_t* qr = (uint8_t*)p;
     if (int e = forge_unit_upper_from_lower(A, nullptr, Ur, 1, C, 1, stream)) return e;
-    const unsigned gx = (unsigned)forge::ceil_div(R, 256);
-    reverse_rows_kernel<float><<<dim3(gx, (unsigned)C), dim3(256), 0, st>>>(W, Xr, C, R);
+    const int64_t pieces = forge::ceil_div(R, 256);
+    const unsigned gx = (unsigned)(pieces < 65535 ? pieces : 65535);   // the kernel strides over the rest
+    reverse_rows_kernel<float><<<dim3((unsigned)C, gx), dim3(256), 0, st>>>(W, Xr, C, R);
     FORGE_LAUNCH_CHECK();
     const int64_t nmeta = R * G > C ? R * G : C;
     babai_meta_kernel<<<dim3((unsigned)forge::ceil_div(nmeta, 256)), dim3(256), 0, st>>>(
@@ -604,7 +606,7 @@ extern "C" int forge_babai_solver(const float* W, const float* A, const float* s
     FORGE_LAUNCH_CHECK();
     if (int e = forge_gptq_sweep_batched(Xr, Ur, sT, zT, g_rev, qr, nullptr, nullptr, 1, C, R, G, bits, 0, stream))
         return e;
-    reverse_rows_kernel<uint8_t><<<dim3(gx, (unsigned)C), dim3(256), 0, st>>>(qr, qweight, C, R);
+    reverse_rows_kernel<uint8_t><<<dim3((unsigned)C, gx), dim3(256), 0, st>>>(qr, qweight, C, R);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

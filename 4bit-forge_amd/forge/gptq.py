@@ -43,7 +43,7 @@ class GPTQ(object):
                  rel_damp: float = 1e-2, algorithm: str = "gptq", owner=None, device=None,
                  factor_route: str = "inverse"):
         """Arguments of the reference's class (forge/gptq.py:11-22) plus ``factor_route``
-        (algorithm="gptq" only): "inverse", the default, follows the reference's
+        (algorithms "gptq" and "sparsegptq"; Babai has its own factor): "inverse", the default, follows the reference's
         factorisation (Cholesky, inverse, Cholesky of the inverse) and its error-propagating
         sweep; "direct" stops at the factor of H itself and sweeps with the displacements
         w - deq, which is the same solve in exact arithmetic at half the factorisation work
@@ -193,15 +193,26 @@ class GPTQ(object):
             if int(info.item()) > 0:
                 self.issue_non_invertible = True
             return kernels.unit_upper_from_lower(L, info)[0]
-        if self.algorithm == "gptq" and self.factor_route == "direct":
+        sparse = self.algorithm == "sparsegptq"
+        if self.factor_route == "direct":
             L, info = kernels.chol_reverse_lower_batched(H.clone().view(1, C, C), None)
             if int(info.item()) > 0:
                 self.issue_non_invertible = True
+            if sparse:
+                # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the diagonal of
+                # the factor of H itself; 1 where the factorisation failed (U = I)
+                self._score_weight = torch.where(info[:, None] != 0, torch.ones((), device=H.device),
+                                                 L.diagonal(dim1=1, dim2=2)).contiguous()
             return kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)[0]
-        U, _, info = kernels.chol_inv_upper_batched(H.clone().view(1, C, C), None,
-                                                    normalise=self.algorithm == "gptq")
+        U, udiag, info = kernels.chol_inv_upper_batched(H.clone().view(1, C, C), None,
+                                                        normalise=not sparse)
         if int(info.item()) > 0:
             self.issue_non_invertible = True
+        if sparse:
+            # rows scaled by the rounded reciprocal of the diagonal, as
+            # solver_sparsegptq14.cu:153-155 does to its caller's tensor
+            self._score_weight = (1.0 / udiag).contiguous()
+            U.mul_(self._score_weight.unsqueeze(-1))
         return U[0]
 
     @torch.no_grad()
@@ -223,15 +234,20 @@ class GPTQ(object):
             q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
             return kernels.codes_to_layer_order(q, perm_r_inv.view(1, C))[0], scales, qzeros
         X = kernels.weight_to_solver_order(W.view(1, R, C), self.perm_inv.view(1, C))
-        if self.algorithm == "sparsegptq":
-            s_e = scales.view(R, G).repeat_interleave(gs, dim=1)[:, :C].t()[self.perm].contiguous()
-            z_e = qzeros.view(R, G).repeat_interleave(gs, dim=1)[:, :C].t()[self.perm].contiguous()
-            q, M = kernels.sparsegptq14_solver(X[0], U, s_e, z_e, self.bits)
-            qw = kernels.codes_to_layer_order(q.view(1, C, R), self.perm_inv.view(1, C))[0]
-            return qw, scales, qzeros, M
         g_idx = (self.perm // gs).to(torch.int32).view(1, C)
         sT = scales.view(R, G).t().contiguous().view(1, G, R)
         zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
+        # per-group scales and zeros are looked up through g_idx inside the sweep: the two
+        # [C, R] expansions of forge/gptq.py:251-252 are never materialised
+        if self.algorithm == "sparsegptq":
+            if self.factor_route == "direct":
+                q, M = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits,
+                                                         sparse14=True, mdiag=self._score_weight)
+            else:
+                q, M = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits,
+                                                  sparse14=True, uinv=self._score_weight)
+            qw = kernels.codes_to_layer_order(q, self.perm_inv.view(1, C))[0]
+            return qw, scales, qzeros, M[0]
         if self.factor_route == "direct":
             q = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
         else:

@@ -99,10 +99,20 @@ class ExpertGroupGPTQ:
             self.H = torch.empty((E, C, C), dtype=torch.float32, device=dev)
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
         seen = torch.tensor([n > 0 for n in self.num_samples], device=dev)
-        bad = (~seen) | torch.isnan(self.H.diagonal(dim1=1, dim2=2)).any(dim=1)
+        diag_all = self.H.diagonal(dim1=1, dim2=2)                        # [E, C] view
+        bad = (~seen) | torch.isnan(diag_all).any(dim=1)
+        # Weights with pruned columns zeroed decide the (unpermuted-index) zero-column mask
+        # that the reference applies to the permuted Hessian (forge/gptq.py:145-149).  A column
+        # can only be all zero if its first rows are: one look at 8 rows of every expert (fp8-
+        # or int-derived weights do contain single zeros) and at the Hessian diagonals tells
+        # which experts need the full pass over their weights at all.  These flags and `bad`
+        # reach the host in ONE transfer, the only synchronisation before the solve.
+        dead_any = ((diag_all == 0) & ~bad[:, None]).any(dim=1)
+        maybe_zero = [(W[:, :8, :] == 0).all(dim=1).any(dim=1) for W in self.W]
+        host_flags = torch.stack([bad, dead_any] + maybe_zero).cpu()       # [2 + stacks, E]
         # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
         # fraction of the fill rate)
-        for e in bad.nonzero().flatten().tolist():
+        for e in host_flags[0].nonzero().flatten().tolist():
             self.H[e].zero_()
             self.H[e].diagonal().fill_(1.0)
         failed = []
@@ -136,17 +146,10 @@ class ExpertGroupGPTQ:
             perm_inv = torch.argsort(perm, dim=1)
             g_idx = (perm // gs).to(torch.int32).contiguous()
             dead_u8 = dead.to(torch.uint8).contiguous()
-            # weights with pruned columns zeroed decide the (unpermuted-index) zero-column
-            # mask that the reference applies to the permuted Hessian (forge/gptq.py:145-149).
-            # A column can only be all zero if its first rows are: one look at 8 rows (fp8- or
-            # int-derived weights do contain single zeros) and at `dead` tells whether the
-            # full pass over the weights is needed at all.
-            first = torch.stack([(W[e0:e1, :8, :] == 0).all(dim=1).any() for W in self.W]
-                                + [dead.any()])
-            flags = first.cpu().tolist()                                 # host sync
-            has_dead = flags[-1]
+            has_dead = bool(host_flags[1, e0:e1].any())
+            flags = [bool(host_flags[2 + i, e0:e1].any()) for i in range(len(self.W))]
             masks = []
-            for W, maybe in zip(self.W, flags[:-1]):
+            for W, maybe in zip(self.W, flags):
                 if maybe or has_dead:
                     # all_r(W[r, c] == 0 or dead[c]) = all_r(W[r, c] == 0) or dead[c]
                     zero_cols = (W[e0:e1] == 0).all(dim=1) | dead

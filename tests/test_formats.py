@@ -67,7 +67,7 @@ def test_oracle_fp8_dequant_matches_tile_loop():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("R,C", [(64, 256), (17, 200), (130, 96)])
+@pytest.mark.parametrize("R,C", [(64, 256), (17, 200), (130, 96), (100, 1100), (33, 2080), (70, 4100)])
 def test_gpu_sparse_pack_bit_exact(hip, R, C):
     q, M32, scales, _ = _sparse_case(R, C, R + C)
     want = oracle.pack_sparsegptq14_to_u64x2(q, M32, scales)
@@ -104,3 +104,52 @@ def test_gpu_fp8_roundtrip_feeds_the_solver(hip):
     q = (blk / s_inv[:, None, :, None]).to(torch.float8_e4m3fn).reshape(256, 384)
     got = hip.fp8_block_dequant(q.to(DEV), s_inv.to(DEV)).cpu()
     assert torch.equal(got, synth.fp8_block_roundtrip(W))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sym", [True, False])
+def test_layer_record_and_consumer_tensors(hip, sym):
+    """The per-layer dict of quant.py:498-511 and the tensor set of pack_quantized.py:279-313
+    built from a quantize() result: dtypes and shapes as the reference writes them, the record
+    dequantises to the same weights, and weight_packed decodes back to code - zero."""
+    from forge.gptq import GPTQ
+    from forge import export
+    from helpers import linear
+    g = torch.Generator().manual_seed(9)
+    R, C, gs = 96, 328, 128
+    W = 0.02 * torch.randn(R, C, generator=g)
+    h = GPTQ(linear(W).to(DEV), device=DEV, bits=4, group_size=gs, symmetric=sym,
+             quantization_scale="absmax", quantization_order="activation")
+    h.update(torch.randn(512, C, generator=g).to(DEV))
+    q, s, z = h.quantize()
+    G = h.G
+    rec = export.layer_record(q, s, z, gs, 4, W.shape)
+    assert rec["qweight"].dtype == torch.int8 and tuple(rec["qweight"].shape) == (R, C)
+    assert rec["scales"].dtype == torch.float32 and rec["qzeros"].dtype == torch.int32
+    assert rec["scales"].numel() == R * G and rec["group_size"] == gs and rec["bits"] == 4
+    assert rec["shape"] == (R, C)
+    assert torch.equal(rec["qzeros"].float(), z)                      # zeros are whole numbers
+    deq = oracle.dequantize(rec["qweight"].cpu().to(torch.uint8), rec["scales"].cpu(),
+                            rec["qzeros"].cpu().float(), gs)
+    assert torch.equal(deq, oracle.dequantize(q.cpu(), s.cpu(), z.cpu(), gs))
+    out = export.pack_weight(rec, bits=4, sym=sym, group_size=gs)
+    assert set(out) == {"weight_packed", "weight_shape", "weight_scale"} | (set() if sym else {"weight_zero_point"})
+    assert out["weight_shape"].tolist() == [R, C] and out["weight_shape"].dtype == torch.int64
+    assert tuple(out["weight_scale"].shape) == (R, G) and torch.equal(out["weight_scale"].reshape(-1), s)
+    pk = out["weight_packed"].cpu()
+    assert pk.dtype == torch.int32 and tuple(pk.shape) == (R, (C + 7) // 8)
+    nib = torch.stack([(pk.to(torch.int64) >> (4 * k)) & 0xF for k in range(8)], dim=-1).reshape(R, -1)[:, :C]
+    zz = z.cpu().view(R, G).repeat_interleave(gs, 1)[:, :C].to(torch.int64)
+    # offset binary of code - zero; a difference outside [-8, 7] (possible with asymmetric
+    # zeros) wraps in the nibble, as it does in the reference's int8 subtraction + 4-bit pack
+    assert torch.equal(nib, (q.cpu().to(torch.int64) - zz + 8) & 0xF)
+    inside = (q.cpu().to(torch.int64) - zz).abs() < 8
+    assert torch.equal((nib - 8)[inside], (q.cpu().to(torch.int64) - zz)[inside])
+    if not sym:
+        assert torch.equal(out["weight_zero_point"].reshape(-1).float(), z)
+    # the reference's own key names are read too
+    alt = export.pack_weight({"qweight": rec["qweight"], "scale": rec["scales"].view(R, G),
+                              "zero": rec["qzeros"].view(R, G).to(torch.int8)}, 4, sym, gs)
+    assert torch.equal(alt["weight_packed"], out["weight_packed"])
+    with pytest.raises(NotImplementedError):
+        export.pack_weight(rec, bits=3, sym=sym, group_size=gs)
