@@ -601,6 +601,7 @@ struct SplitPair {
     GemmPair pair;
     const u32x4* Ap;   // split A panel of both problems (same At, m0, k0)
     int64_t aps;       // words per matrix
+    int64_t apt;       // words per m tile (all matrices): a problem may have two m tiles
 };
 
 // Both problems: full 128x128 tiles, one m tile, 16-byte aligned rows, every tile's K range
@@ -619,15 +620,20 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     __shared__ __attribute__((aligned(16))) u32x4 L[2][2][NP][4][128];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    int bz, tile;
+    // The m tiles of one (matrix, n tile) follow each other on the same XCD: they read the same
+    // rows of B at about the same time, so the second reading is served by that XCD's L2.
+    const int per_matrix = g.n_tiles * g.m_tiles;
+    int bz, rem;
     if (g.xcd_map) {
         const int xcd = wg & 7, slot = wg >> 3;
-        bz = xcd + 8 * (slot / g.n_tiles);
-        tile = slot % g.n_tiles;
+        bz = xcd + 8 * (slot / per_matrix);
+        rem = slot % per_matrix;
     } else {
-        bz = wg / g.n_tiles;
-        tile = wg % g.n_tiles;
+        bz = wg / per_matrix;
+        rem = wg % per_matrix;
     }
+    const int tile = rem / g.m_tiles, mtile = rem % g.m_tiles;
+    const int m0 = g.m0 + mtile * TM;
     const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile : tile;
     const int nt = g.n0 + tn * TN;
     const int k0 = g.k0;
@@ -643,7 +649,8 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float*>(Bm + (int64_t)k0 * g.ldb + nt), 0, 0x7FFFFFFF, 0x00027000);
         const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<u32x4*>(sp.Ap + (int64_t)bz * sp.aps), 0, 0x7FFFFFFF, 0x00027000);
+            const_cast<u32x4*>(sp.Ap + (int64_t)mtile * sp.apt + (int64_t)bz * sp.aps), 0, 0x7FFFFFFF,
+            0x00027000);
         int ob[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) ob[j] = (int)(((int64_t)(4 * kh + j) * g.ldb + 4 * cq) * 4);
@@ -707,7 +714,7 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         // sums in LDS (over the stage buffers, free by then), row r of the tile at
         // S[r][position]; thread = 16 rows x 4 consecutive columns, X is read and written in
         // 16-byte pieces of whole 512-byte rows.
-        float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)g.m0 * g.ldx + nt + 4 * cq;
+        float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)m0 * g.ldx + nt + 4 * cq;
         const float sgn = g.negate_a ? -1.0f : 1.0f;
         f32x4 xo[16];
         if (!g.init_zero) {
@@ -916,10 +923,12 @@ bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t
                     int* n_stage_out) {
     if (option(OPT_FP32_BLOCKED_SUM) == 1) return false;
     auto ok = [](const Prepared& p) {
-        return !p.edge && p.k128 && p.g.blocked_sum && p.g.m_tiles == 1 && !p.g.b_lower_tri &&
+        return !p.edge && p.k128 && p.g.blocked_sum && !p.g.b_lower_tri &&
+               (p.g.m_tiles == 1 || (p.g.m_tiles == 2 && !p.g.b_upper_tri)) &&
                p.g.k1 - p.g.k0 >= 128 && (!p.g.b_upper_tri || p.g.n0 + TN - p.g.k0 >= 128);
     };
     if (!ok(a) || (b && !ok(*b))) return false;
+    if (b && (a.g.m_tiles != 1 || b->g.m_tiles != 1)) return false;   // two m tiles: alone in its grid
     int k1 = a.g.k1;
     if (b) {
         const GemmArgs &x = a.g, &y = b->g;
@@ -928,7 +937,7 @@ bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t
         if (y.k1 > k1) k1 = y.k1;
     }
     const int n_stage = (k1 - a.g.k0) / SPLIT_TK;
-    if (ws_bytes < split_gemm_workspace_bytes(batch, k1 - a.g.k0)) return false;
+    if (ws_bytes < a.g.m_tiles * split_gemm_workspace_bytes(batch, k1 - a.g.k0)) return false;
     *n_stage_out = n_stage;
     return true;
 }
@@ -946,16 +955,18 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
     const bool two = products == 1 || products == 3 || products == 4;     // two-piece layout
     const int np = two ? 2 : 3;
     sp.aps = (int64_t)n_stage * split_stage_words(np);
-    {
+    sp.apt = sp.aps * batch;
+    for (int mt = 0; mt < a.g.m_tiles; ++mt) {
         KernelTiming timing("split_a_panel", st, (4.0 + 2.0 * np) * n_stage * SPLIT_TK * TM * (double)batch,
                             WORK_BYTES);
         const dim3 pgrid((unsigned)(batch * n_stage)), pblock(128);
+        u32x4* dst = static_cast<u32x4*>(ws) + (int64_t)mt * sp.apt;
         if (two)
-            split_a_panel_kernel<2><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0,
-                                                              n_stage, static_cast<u32x4*>(ws), sp.aps);
+            split_a_panel_kernel<2><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM,
+                                                              a.g.k0, n_stage, dst, sp.aps);
         else
-            split_a_panel_kernel<3><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0, a.g.k0,
-                                                              n_stage, static_cast<u32x4*>(ws), sp.aps);
+            split_a_panel_kernel<3><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM,
+                                                              a.g.k0, n_stage, dst, sp.aps);
         FORGE_LAUNCH_CHECK();
     }
     KernelTiming timing(two ? "split_gemm_bf16x2" : "split_gemm_bf16x3", st,

@@ -472,11 +472,24 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         if (right_looking) {
             // nothing to do here: the earlier blocks have already been pushed into this one
         } else if (ws) {
-            // sums of 128 products each, three bf16 pieces per operand on the bf16 matrix pipe
-            // where the block is a full tile (fp32 matrix pipe otherwise)
-            g.blocked_sum = true;
-            g.products = products;
-            if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, ws_bytes)) return e;
+            // sums of 128 products each from bf16 pieces of the operands on the bf16 matrix pipe
+            // where the block is a full tile (fp32 matrix pipe otherwise).  That product is
+            // bound by reading the displacement rows of all earlier columns from HBM, so full
+            // blocks are brought up to date two at a time: every row read then serves 256
+            // columns (the second block's reading comes from L2), and the odd block only lacks
+            // what its even neighbour adds, a K = 128 product on the fp32 pipe.
+            const bool pairs = C % forge::kBW == 0;
+            const bool odd = pairs && ((start / forge::kBW) & 1) != 0;
+            if (!odd) {
+                g.blocked_sum = true;
+                g.products = products;
+                if (pairs && start + 2 * forge::kBW <= C) g.m1 = (int)(start + 2 * forge::kBW);
+                if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, ws_bytes)) return e;
+                g.m1 = (int)(start + bw);
+            } else {
+                g.k0 = (int)(start - forge::kBW);
+                if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+            }
         } else {
             if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
         }
@@ -509,7 +522,7 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
 
 extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C) {
     if (batch <= 0 || C <= forge::kBW) return 0;
-    return forge::split_gemm_workspace_bytes(batch, C - forge::kBW);
+    return 2 * forge::split_gemm_workspace_bytes(batch, C - forge::kBW);   // two column blocks per product
 }
 
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,

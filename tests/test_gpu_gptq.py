@@ -347,6 +347,35 @@ def test_config1_dense_2048_full_size(scale):
     print(f"config1 {scale}: flips {flips:.2e} error ratio {ratio:.5f}")
 
 
+def test_config4_student_t_full_size_against_a_row_subset():
+    """Config 4 as specified (4096 x 7168 bf16 weight with Student-t(3) rows, 2048 tokens,
+    4-bit asymmetric g128, MSE search with 100 shrink factors and p = 2.4) solved in full on the
+    GPU.  Rows are independent given the Hessian, so the CPU oracle solves the first 256 rows
+    of the same weight with the same tokens and those rows are compared."""
+    from forge.gptq import GPTQ
+    case = synth.student_t_weight()
+    rows = 256
+    kw = dict(bits=4, group_size=128, symmetric=False, quantization_scale="mse",
+              quantization_order="default", rel_damp=0.01)
+    g = GPTQ(linear(case.W).to(DEV), device=DEV, **kw)
+    g.add_batch(case.X.to(DEV))
+    qg, sg, zg = (t.cpu() for t in g.quantize())
+    assert tuple(qg.shape) == (4096, 7168) and g.G == 56
+    Wsub = case.W[:rows].contiguous()
+    o = oracle.GPTQ(linear(Wsub), **kw)
+    o.update(case.X)
+    H = o.H.double().numpy().copy()
+    qo, so, zo = o.quantize()
+    sg, zg, qg = sg[:rows * 56], zg[:rows * 56], qg[:rows]
+    same = so == sg
+    assert float((~same).float().mean()) <= 1e-3 and torch.equal(zo[same], zg[same])
+    _codes_at_floor("config4 rows 0-255", qo, qg, Wsub, [case.X], kw, both=True)
+    Wf = Wsub.float().numpy()
+    eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H)
+    eg = mathref.layer_error(Wf, oracle.dequantize(qg, sg, zg, 128).numpy(), H)
+    assert abs(eg / eo - 1) < 0.01, eg / eo
+
+
 def test_config5_sparse14_full_size():
     """Config 5 as specified: 3072x1536 bf16 down_proj, 2048 bf16 tokens, 1:4 mask + 4-bit
     symmetric g128 on the survivors."""
