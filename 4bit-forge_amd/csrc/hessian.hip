@@ -180,10 +180,11 @@ template <bool BLEND>
 __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict__ pack,
                                                         const GroupDesc* __restrict__ gd,
                                                         float* __restrict__ Hall, int64_t C,
-                                                        int NT, const float* __restrict__ dnew) {
+                                                        int NT, const float* __restrict__ dnew,
+                                                        int n_hi) {
     __shared__ float tbuf[4][32][33];
     const GroupDesc g = gd[blockIdx.y];
-    if (g.n == 0) return;
+    if (g.n == 0 || g.n >= n_hi) return;           // groups with n_hi tokens and more: the kernel below
     int ti, tj;
     tile_pair(blockIdx.x, NT, ti, tj);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -296,6 +297,169 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(const uint4* __restrict_
                 store_tile(H, C, cta[mi] * 32, ctb[ni] * 32, acc[mi][ni], g.alpha, g.beta, mirror,
                            tbuf[wave], lane, dn);
     }
+}
+
+// ---------------------------------------------------------------- rank-k (bf16 MFMA), many tokens
+// For groups with hundreds of tokens and more the kernel above is bound by the path from L2
+// to the registers: every wavefront fetches its own operand panels, 16 KiB per workgroup and
+// 16-token chunk for 2 x 128^3/8 flops.  Here a workgroup of 8 wavefronts owns a 256 x 256
+// tile; per chunk its 16 operand panels (8 column tiles of A, 8 of B, 1 KiB each, already in
+// the lane order of the matrix instruction) go through LDS once, one panel of each per
+// wavefront, and every wavefront reads the 4 + 2 it needs for its 128 x 64 part (8 matrix
+// instructions per 6 LDS reads and 2 global loads).  Two LDS buffers, one barrier per chunk;
+// the loads of chunk k+2 are in flight while chunk k is multiplied.
+// grid: (pair of 256-column tiles, group); only groups with n_lo <= n tokens are taken, C must
+// be a multiple of 256.
+constexpr int BIG = 256;
+constexpr int kBigTokens = 512;   // groups with this many tokens and more take the kernel below
+__global__ __launch_bounds__(512, 1) void syrk_bf16_big_kernel(const uint4* __restrict__ pack,
+                                                               const GroupDesc* __restrict__ gd,
+                                                               float* __restrict__ Hall, int64_t C,
+                                                               int NT2, const float* __restrict__ dnew,
+                                                               int n_lo) {
+    // two stages of KC chunks x 16 panels; reused as per-wavefront 32 x 33 transposition tiles
+    // afterwards
+    constexpr int KC = 4;
+    __shared__ __attribute__((aligned(16))) uint4 stage[2][KC][16][64];
+    const GroupDesc g = gd[blockIdx.y];
+    if (g.n < n_lo) return;
+    int ti, tj;
+    tile_pair(blockIdx.x, NT2, ti, tj);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 2, wn = wave & 3;              // 2 x 4 wavefronts, 128 x 64 each
+    float* __restrict__ H = Hall + (int64_t)blockIdx.y * C * C;
+    const float* __restrict__ dn = dnew + (int64_t)blockIdx.y * C;
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+    // this wavefront brings in panel `wave` of A (column tile ti*8 + wave) and of B, KC chunks
+    // of 16 tokens per stage; chunks past the group's last one are zeros
+    const uint4* __restrict__ srcA = pack + g.pack_off + (int64_t)(ti * 8 + wave) * g.nchunk * 64 + lane;
+    const uint4* __restrict__ srcB = pack + g.pack_off + (int64_t)(tj * 8 + wave) * g.nchunk * 64 + lane;
+    const int nchunk = g.nchunk;
+    const int nstage = (nchunk + KC - 1) / KC;
+    uint4 ra[KC], rb[KC];
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            // (a branch on a wavefront-uniform condition: a select on the loaded value would make
+            // the wavefront wait for the load right here instead of one stage later)
+            const int chunk = st * KC + c;
+            if (chunk < nchunk) {
+                ra[c] = srcA[(int64_t)chunk * 64];
+                rb[c] = srcB[(int64_t)chunk * 64];
+            } else {
+                ra[c] = make_uint4(0u, 0u, 0u, 0u);
+                rb[c] = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    };
+    auto put = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            stage[buf][c][wave][lane] = ra[c];
+            stage[buf][c][8 + wave][lane] = rb[c];
+        }
+    };
+    fetch(0);
+    put(0);
+    if (nstage > 1) fetch(1);
+    // Operands of a chunk are read from LDS while the matrix instructions of the chunk before
+    // run (two register sets, one LDS read slotted in after each of the first six instructions
+    // of a chunk): a wavefront issues in order, so reads issued as a block of their own would
+    // leave the matrix pipe waiting for them.
+    bf16x8 a[2][4], b[2][2];
+#define FORGE_BIG_READ(buf, c, set)                                                             \
+    do {                                                                                        \
+        _Pragma("unroll") for (int mi = 0; mi < 4; ++mi) {                                      \
+            const uint4 u = stage[buf][c][wm * 4 + mi][lane];                                   \
+            a[set][mi] = __builtin_bit_cast(bf16x8, u);                                         \
+        }                                                                                       \
+        _Pragma("unroll") for (int ni = 0; ni < 2; ++ni) {                                      \
+            const uint4 u = stage[buf][c][8 + wn * 2 + ni][lane];                               \
+            b[set][ni] = __builtin_bit_cast(bf16x8, u);                                         \
+        }                                                                                       \
+    } while (0)
+#define FORGE_BIG_MFMAS(set)                                                                    \
+    do {                                                                                        \
+        _Pragma("unroll") for (int mi = 0; mi < 4; ++mi) _Pragma("unroll") for (int ni = 0; ni < 2; ++ni) \
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[set][mi], b[set][ni], acc[mi][ni], \
+                                                                  0, 0, 0);                     \
+    } while (0)
+    for (int st = 0; st < nstage; ++st) {
+        const int cur = st & 1;
+        __syncthreads();                                   // stage `cur` is complete, `cur^1` is free
+        FORGE_BIG_READ(cur, 0, 0);
+        if (st + 1 < nstage) put(cur ^ 1);
+        if (st + 2 < nstage) fetch(st + 2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            if (c + 1 < KC) FORGE_BIG_READ(cur, c + 1, (c + 1) & 1);
+            FORGE_BIG_MFMAS(c & 1);
+            if (c + 1 < KC) {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#undef FORGE_BIG_READ
+#undef FORGE_BIG_MFMAS
+    __syncthreads();                                       // the stages become transposition tiles
+    float (*tbuf)[33] = reinterpret_cast<float (*)[33]>(reinterpret_cast<float*>(&stage[0][0][0][0]) +
+                                                        wave * 32 * 33);
+    const bool blend = g.beta != 0.0f;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+            const int row0 = (ti * 8 + wm * 4 + mi) * 32, col0 = (tj * 8 + wn * 2 + ni) * 32;
+            if (row0 > col0) continue;                     // below the diagonal: its mirror image writes it
+            float* __restrict__ Ht = H + (int64_t)(row0 + (lane >> 5) * 4) * C + col0 + (lane & 31);
+            f32x16 out;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float o = g.alpha * acc[mi][ni][v];
+                if (blend) o = __builtin_fmaf(g.beta, Ht[(int64_t)((v >> 2) * 8 + (v & 3)) * C], o);
+                out[v] = o;
+            }
+            if (row0 == col0) {                            // the float64 diagonal
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if ((v >> 2) * 8 + (lane >> 5) * 4 + (v & 3) == (lane & 31))
+                        out[v] = dn[row0 + (lane & 31)];
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) Ht[(int64_t)((v >> 2) * 8 + (v & 3)) * C] = out[v];
+            if (row0 != col0) {                            // mirror image through the wavefront's own tile
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    tbuf[(v >> 2) * 8 + (lane >> 5) * 4 + (v & 3)][lane & 31] = out[v];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                float* __restrict__ Hm = H + (int64_t)(col0 + (lane >> 5) * 4) * C + row0 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int jj = (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                    Hm[(int64_t)((v >> 2) * 8 + (v & 3)) * C] = tbuf[lane & 31][jj];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
 }
 
 // ---------------------------------------------------------------- rank-k (f32 MFMA)
@@ -450,12 +614,17 @@ int upload_async(const void* src, int64_t bytes, void* dst, hipStream_t st) {
 
 // The launches of one update; gd_dev already holds the group table.
 int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const GroupDesc* gd_dev,
-                  int64_t n_groups, int64_t total, int max_chunks, bool any_blend, float* H,
-                  float* dnew, uint4* pack, hipStream_t st, bool timed = true) {
+                  int64_t n_groups, int64_t total, int max_chunks, int min_tokens, bool any_blend,
+                  float* H, float* dnew, uint4* pack, hipStream_t st, bool timed = true) {
     const int NT = (int)forge::ceil_div(C, 128);
     const unsigned pairs = (unsigned)(NT * (NT + 1) / 2);
     const dim3 dgrid((unsigned)NT, (unsigned)n_groups);
     if (x_dtype == FORGE_BF16) {
+        // one record for the whole update (diagonal, operand panels, rank-k kernels); executed
+        // flops: tiles on and above the diagonal only
+        forge::KernelTiming timing(timed ? "hessian_syrk_bf16" : nullptr, st,
+                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
+                                   forge::WORK_FLOPS);
         diag_float64_kernel<uint16_t><<<dgrid, dim3(256), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev,
                                                                    H, dnew);
         FORGE_LAUNCH_CHECK();
@@ -463,24 +632,32 @@ int launch_update(const void* X, int x_dtype, int64_t ldx, int64_t C, const Grou
         pack_bf16_kernel<<<dim3((unsigned)forge::ceil_div(C, 32), ychunks, (unsigned)n_groups),
                            dim3(64), 0, st>>>((const uint16_t*)X, ldx, C, gd_dev, pack);
         FORGE_LAUNCH_CHECK();
-        // executed flops: tiles on and above the diagonal only
-        forge::KernelTiming timing(timed ? "hessian_syrk_bf16" : nullptr, st,
-                                   2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
-                                   forge::WORK_FLOPS);
-        if (any_blend)
-            syrk_bf16_kernel<true><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
-                pack, gd_dev, H, C, NT, dnew);
-        else
-            syrk_bf16_kernel<false><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
-                pack, gd_dev, H, C, NT, dnew);
-        FORGE_LAUNCH_CHECK();
+        // groups with many tokens take the 256 x 256 workgroup tiles (operands shared through
+        // LDS), the others the one-pass kernel that overlaps the old tile's loads with its K loop
+        const bool big = (C % BIG) == 0 && max_chunks * 16 >= kBigTokens;
+        const int n_split = big ? kBigTokens : (1 << 30);
+        if (max_chunks * 16 < kBigTokens || !big || min_tokens < kBigTokens) {
+            if (any_blend)
+                syrk_bf16_kernel<true><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
+                    pack, gd_dev, H, C, NT, dnew, n_split);
+            else
+                syrk_bf16_kernel<false><<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
+                    pack, gd_dev, H, C, NT, dnew, n_split);
+            FORGE_LAUNCH_CHECK();
+        }
+        if (big) {
+            const int NT2 = (int)(C / BIG);
+            syrk_bf16_big_kernel<<<dim3((unsigned)(NT2 * (NT2 + 1) / 2), (unsigned)n_groups), dim3(512), 0,
+                                   st>>>(pack, gd_dev, H, C, NT2, dnew, n_split);
+            FORGE_LAUNCH_CHECK();
+        }
     } else {
-        diag_float64_kernel<float><<<dgrid, dim3(256), 0, st>>>((const float*)X, ldx, C, gd_dev, H,
-                                                                dnew);
-        FORGE_LAUNCH_CHECK();
         forge::KernelTiming timing(timed ? "hessian_syrk_f32" : nullptr, st,
                                    2.0 * (double)total * 128.0 * 128.0 * (double)pairs,
                                    forge::WORK_FLOPS);
+        diag_float64_kernel<float><<<dgrid, dim3(256), 0, st>>>((const float*)X, ldx, C, gd_dev, H,
+                                                                dnew);
+        FORGE_LAUNCH_CHECK();
         syrk_f32_kernel<<<dim3(pairs, (unsigned)n_groups), dim3(256), 0, st>>>(
             (const float*)X, ldx, gd_dev, H, C, NT, dnew);
         FORGE_LAUNCH_CHECK();
@@ -553,7 +730,7 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
 
     std::vector<GroupDesc> gd((size_t)n_groups);
     int64_t off = 0;
-    int max_chunks = 0;
+    int max_chunks = 0, min_tokens = 1 << 30;
     bool any = false, any_blend = false;
     for (int64_t e = 0; e < n_groups; ++e) {
         const int64_t n = offsets_host[e + 1] - offsets_host[e];
@@ -566,6 +743,7 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
         gd[e].beta = beta_host[e];
         off += pack_units(n, C);
         if (gd[e].nchunk > max_chunks) max_chunks = gd[e].nchunk;
+        if (n > 0 && n < min_tokens) min_tokens = (int)n;
         any |= n > 0;
         any_blend |= n > 0 && beta_host[e] != 0.0f;
     }
@@ -576,8 +754,8 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
     uint4* pack = (uint4*)((char*)ws + desc_bytes + round256(n_groups * C * 4));
     // through a pinned block of the library's own: the host does not wait for the copy
     if (int rc = upload_async(gd.data(), n_groups * (int64_t)sizeof(GroupDesc), gd_dev, st)) return rc;
-    return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, any_blend, H, dnew,
-                         pack, st);
+    return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, min_tokens, any_blend,
+                         H, dnew, pack, st);
 }
 
 extern "C" int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype) {
@@ -618,6 +796,6 @@ extern "C" int forge_hessian_update_static(const void* X, int x_dtype, int64_t l
     // the table entry travels as a kernel argument: no staging buffer, nothing to allocate
     write_desc_kernel<<<dim3(1), dim3(64), 0, st>>>(gd_dev, g);
     FORGE_LAUNCH_CHECK();
-    return launch_update(X, x_dtype, ldx, C, gd_dev, 1, n_rows, g.nchunk, beta != 0.0f, H, dnew, pack,
-                         st, /*timed=*/false);
+    return launch_update(X, x_dtype, ldx, C, gd_dev, 1, n_rows, g.nchunk, (int)n_rows, beta != 0.0f, H,
+                         dnew, pack, st, /*timed=*/false);
 }

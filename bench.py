@@ -230,16 +230,21 @@ def hessian_buckets(C=7168, E=64):
         kernels.hessian_update_grouped(X, offs, H, [2.0 / n] * E, [0.0] * E)      # warm-up
         stats = timing_pass(lambda: kernels.hessian_update_grouped(X, offs, H, [2.0 / n] * E, [0.0] * E))
         ms = sum(s["ms"] for k, s in stats.items() if k.startswith("hessian"))
+        executed = sum(s["work"] for k, s in stats.items() if k.startswith("hessian"))
         flops = 2.0 * n * C * C * E
         nbytes = (2.0 * n * C + 4.0 * C * C) * E
         out[str(n)] = dict(ms=round(ms, 3), tflops=round(flops / ms / 1e9, 1),
                            mfma_frac=round(flops / ms / 1e9 / PEAK["mfma_bf16"], 4),
+                           executed_tflops=round(executed / ms / 1e9, 1),
+                           executed_mfma_frac=round(executed / ms / 1e9 / PEAK["mfma_bf16"], 4),
                            gbps=round(nbytes / ms / 1e6, 1),
                            hbm_frac=round(nbytes / ms / 1e6 / PEAK["hbm"], 4))
         del X
     return dict(C=C, experts=E, tokens_per_expert=out,
-                note="flops 2nC^2 (the full product the reference's SGEMM executes; the kernel "
-                     "computes the tiles on and above the diagonal), bytes 2nC + 4C^2 per expert")
+                note="ms = the whole update (float64 diagonal, operand panels, rank-k kernels); "
+                     "tflops counts 2nC^2, the full product the reference's SGEMM executes; "
+                     "executed_tflops counts the 128 x 128 tiles on and above the diagonal that "
+                     "the kernels compute; bytes 2nC + 4C^2 per expert")
 
 
 def hbm_kernels(wl):

@@ -40,6 +40,39 @@ def test_grouped_ragged_hessian(hip, dtype, C):
         assert _rel(H[e], ref) < 2e-6 and torch.equal(H[e], H[e].t())
 
 
+@pytest.mark.parametrize("C", [256, 768])
+def test_grouped_hessian_heavy_and_light_groups_in_one_call(hip, C):
+    """Groups with 512 tokens and more take the 256 x 256 workgroup tiles with operands staged
+    through LDS, the others (in the same call) the one-pass kernel; token counts that are not
+    multiples of the 64-token stage, an empty group between them, then a running-mean update."""
+    counts = [700, 5, 0, 1030, 513, 511, 64]
+    offs = np.concatenate([[0], np.cumsum(counts)])
+    g = torch.Generator().manual_seed(C + 1)
+    X = torch.randn(int(offs[-1]), C, generator=g).bfloat16()
+    E = len(counts)
+    H = torch.full((E, C, C), float("nan"), device=DEV)
+    hip.hessian_update_grouped(X.to(DEV), offs, H, [2.0 / max(c, 1) for c in counts], [0.0] * E)
+    for e, c in enumerate(counts):
+        if c == 0:
+            assert bool(torch.isnan(H[e]).all())
+            continue
+        ref = mathref.hessian([X[offs[e]:offs[e + 1]].double().numpy()])
+        assert _rel(H[e], ref) < 2e-6, (e, c)
+        assert torch.equal(H[e], H[e].t())
+    X2 = torch.randn(int(offs[-1]), C, generator=g).bfloat16()
+    hip.hessian_update_grouped(X2.to(DEV), offs, H, [2.0 / max(2 * c, 1) for c in counts], [0.5] * E)
+    for e, c in enumerate(counts):
+        if c:
+            ref = mathref.hessian([X[offs[e]:offs[e + 1]].double().numpy(),
+                                   X2[offs[e]:offs[e + 1]].double().numpy()])
+            assert _rel(H[e], ref) < 2e-6 and torch.equal(H[e], H[e].t())
+    # every group heavy: only the big-tile kernel runs
+    Hb = torch.full((2, C, C), float("nan"), device=DEV)
+    hip.hessian_update_grouped(X[:1400].to(DEV), [0, 700, 1400], Hb, [2.0 / 700] * 2, [0.0] * 2)
+    assert torch.equal(Hb[0], H.new_tensor(0) + Hb[0]) and _rel(Hb[0], mathref.hessian([X[:700].double().numpy()])) < 2e-6
+    assert _rel(Hb[1], mathref.hessian([X[700:1400].double().numpy()])) < 2e-6
+
+
 def test_hessian_strided_rows_and_empty_call(hip):
     X = torch.randn(40, 300, device=DEV).bfloat16()[:, :256]          # row pitch 300
     H = torch.zeros((1, 256, 256), device=DEV)
