@@ -18,7 +18,8 @@ __device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
 template <typename T>
 __global__ __launch_bounds__(256) void to_solver_order_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const int64_t* __restrict__ perm_inv,
-    const uint8_t* __restrict__ dead, float* __restrict__ Xout, int64_t R, int64_t C) {
+    const uint8_t* __restrict__ dead, float* __restrict__ Xout, int64_t R, int64_t C,
+    int64_t ldo, int64_t o_stride) {
     __shared__ float tile[64][65];
     const int64_t b = blockIdx.z;
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
@@ -33,21 +34,21 @@ __global__ __launch_bounds__(256) void to_solver_order_kernel(
     __syncthreads();
     for (int j = ty; j < 64; j += 4) {
         const int64_t c = c0 + j, r = r0 + tx;
-        if (c < C && r < R) Xout[b * C * R + perm_inv[b * C + c] * R + r] = tile[tx][j];
+        if (c < C && r < R) Xout[b * o_stride + perm_inv[b * C + c] * ldo + r] = tile[tx][j];
     }
 }
 
 // qout[b][r][c] = qin[b][perm_inv[c]][r]   (qweight[perm_inv].T of forge/gptq.py:139)
 __global__ __launch_bounds__(256) void to_layer_order_kernel(
     const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
-    uint8_t* __restrict__ qout, int64_t R, int64_t C) {
+    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride) {
     __shared__ uint8_t tile[64][65];
     const int64_t b = blockIdx.z;
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int j = ty; j < 64; j += 4) {
         const int64_t c = c0 + j, r = r0 + tx;
-        tile[j][tx] = (c < C && r < R) ? qin[b * C * R + perm_inv[b * C + c] * R + r] : 0;
+        tile[j][tx] = (c < C && r < R) ? qin[b * i_stride + perm_inv[b * C + c] * ldi + r] : 0;
     }
     __syncthreads();
     for (int i = ty; i < 64; i += 4) {
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
 __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw,
     const int64_t* __restrict__ perm_inv, const uint8_t* __restrict__ dead,
-    float* __restrict__ Xout, int64_t R, int64_t C) {
+    float* __restrict__ Xout, int64_t R, int64_t C, int64_t ldo, int64_t o_stride) {
     constexpr int TC = 64, TR = 256, PITCH = TR + 4;     // rows stay 8-byte aligned
     __shared__ __attribute__((aligned(8))) uint16_t tile[TC][PITCH];
     const int64_t b = blockIdx.z;
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
             const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
             const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
                                          __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
-            *reinterpret_cast<float4*>(Xout + b * C * R + perm_inv[b * C + c0 + c] * R + r0 + r4) = o;
+            *reinterpret_cast<float4*>(Xout + b * o_stride + perm_inv[b * C + c0 + c] * ldo + r0 + r4) = o;
         }
     }
 }
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
 // back four bytes (four values of c) per lane.
 __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
     const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
-    uint8_t* __restrict__ qout, int64_t R, int64_t C) {
+    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride) {
     constexpr int TC = 128, TR = 256, PITCH = TR + 4;    // 65 words per row: odd
     __shared__ __attribute__((aligned(4))) uint8_t tile[TC][PITCH];
     const int64_t b = blockIdx.z;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
         for (int cc = 0; cc < TC; cc += 4) {
             const int c = cc + cw;
             const uint32_t v = *reinterpret_cast<const uint32_t*>(
-                qin + b * C * R + perm_inv[b * C + c0 + c] * R + r0 + r4);
+                qin + b * i_stride + perm_inv[b * C + c0 + c] * ldi + r0 + r4);
             *reinterpret_cast<uint32_t*>(&tile[c][r4]) = v;
         }
     }
@@ -306,12 +307,14 @@ __global__ __launch_bounds__(256) void pack_int4_fast_kernel(const uint8_t* __re
 
 }  // namespace
 
-extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride,
-                                            int64_t ldw, const int64_t* perm_inv,
-                                            const uint8_t* dead, float* Xout, int64_t batch,
-                                            int64_t R, int64_t C, forge_stream_t stream) {
+extern "C" int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_stride,
+                                                    int64_t ldw, const int64_t* perm_inv,
+                                                    const uint8_t* dead, float* Xout, int64_t ldo,
+                                                    int64_t o_stride, int64_t batch, int64_t R,
+                                                    int64_t C, forge_stream_t stream) {
     FORGE_REQUIRE(w_dtype == FORGE_F32 || w_dtype == FORGE_BF16, "w_dtype=%d", w_dtype);
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0 && ldw >= C, "bad shape");
+    FORGE_REQUIRE(ldo >= R && o_stride >= (C > 0 ? (C - 1) * ldo + R : 0), "output pitch too small");
     if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
     FORGE_REQUIRE(W && perm_inv && Xout, "null pointer");
     dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
@@ -321,17 +324,52 @@ extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t 
                                forge::WORK_BYTES);
     const bool fast = w_dtype == FORGE_BF16 && (R % 256) == 0 && (C % 64) == 0 && (ldw % 4) == 0 &&
                       (w_stride % 4) == 0 && (reinterpret_cast<uintptr_t>(W) % 8) == 0 &&
-                      (reinterpret_cast<uintptr_t>(Xout) % 16) == 0 && R / 256 < 65536;
+                      (reinterpret_cast<uintptr_t>(Xout) % 16) == 0 && (ldo % 4) == 0 &&
+                      (o_stride % 4) == 0 && R / 256 < 65536;
     if (fast) {
         const dim3 tiles((unsigned)(C / 64), (unsigned)(R / 256), (unsigned)batch);
         to_solver_order_bf16_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(
-            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
+            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
     } else if (w_dtype == FORGE_F32) {
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
-            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
+            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
     } else {
         to_solver_order_kernel<__hip_bfloat16><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
-            (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, R, C);
+            (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
+    }
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride,
+                                            int64_t ldw, const int64_t* perm_inv,
+                                            const uint8_t* dead, float* Xout, int64_t batch,
+                                            int64_t R, int64_t C, forge_stream_t stream) {
+    return forge_weight_to_solver_order_strided(W, w_dtype, w_stride, ldw, perm_inv, dead, Xout, R,
+                                                C * R, batch, R, C, stream);
+}
+
+extern "C" int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
+                                                  const int64_t* perm_inv, uint8_t* qout,
+                                                  int64_t batch, int64_t R, int64_t C,
+                                                  forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0, "bad shape");
+    FORGE_REQUIRE(ldi >= R && i_stride >= (C > 0 ? (C - 1) * ldi + R : 0), "input pitch too small");
+    if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
+    FORGE_REQUIRE(qin && perm_inv && qout, "null pointer");
+    dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
+    FORGE_REQUIRE(grid.y < 65536, "R too large");
+    forge::KernelTiming timing("codes_to_layer_order", (hipStream_t)stream, 2.0 * batch * R * C,
+                               forge::WORK_BYTES);
+    const bool fast = (R % 256) == 0 && (C % 128) == 0 && (reinterpret_cast<uintptr_t>(qin) % 4) == 0 &&
+                      (reinterpret_cast<uintptr_t>(qout) % 4) == 0 && (ldi % 4) == 0 && (i_stride % 4) == 0;
+    if (fast) {
+        const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
+        to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C,
+                                                                                 ldi, i_stride);
+    } else {
+        to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C, ldi,
+                                                                           i_stride);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
@@ -340,23 +378,7 @@ extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t 
 extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm_inv,
                                           uint8_t* qout, int64_t batch, int64_t R, int64_t C,
                                           forge_stream_t stream) {
-    FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0, "bad shape");
-    if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
-    FORGE_REQUIRE(qin && perm_inv && qout, "null pointer");
-    dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
-    FORGE_REQUIRE(grid.y < 65536, "R too large");
-    forge::KernelTiming timing("codes_to_layer_order", (hipStream_t)stream, 2.0 * batch * R * C,
-                               forge::WORK_BYTES);
-    const bool fast = (R % 256) == 0 && (C % 128) == 0 && (reinterpret_cast<uintptr_t>(qin) % 4) == 0 &&
-                      (reinterpret_cast<uintptr_t>(qout) % 4) == 0;
-    if (fast) {
-        const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
-        to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
-    } else {
-        to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C);
-    }
-    FORGE_LAUNCH_CHECK();
-    return FORGE_OK;
+    return forge_codes_to_layer_order_strided(qin, R, C * R, perm_inv, qout, batch, R, C, stream);
 }
 
 extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead,

@@ -65,6 +65,9 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_hessian_permute": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
         "forge_weight_to_solver_order": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_weight_to_solver_order_strided": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, i64, i64,
+                                                  vp], i32),
+        "forge_codes_to_layer_order_strided": ([vp, i64, i64, vp, vp, i64, i64, i64, vp], i32),
         "forge_pack_int4": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_fp8_e4m3_block_dequant": ([vp, vp, vp, i32, i64, i64, i64, i64, i64, vp], i32),
         "forge_pack_sparsegptq14_to_u64x2": ([vp, vp, vp, vp, i64, i64, vp], i32),
@@ -89,6 +92,7 @@ EXPORTED_SYMBOLS = (
     "forge_hessian_update_static", "forge_hessian_update_static_max_rows",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
+    "forge_weight_to_solver_order_strided", "forge_codes_to_layer_order_strided",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
     "forge_dequantize_groups", "forge_gather_scaled_rows",
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
@@ -429,30 +433,43 @@ class _HipKernels:
                 _stream()))
         return Hp, damp
 
-    def weight_to_solver_order(self, W, perm_inv, dead=None):
-        """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c]."""
-        _need_cuda(W, perm_inv, dead)
+    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0):
+        """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c].
+        With ``out`` [B,C,Rtot] (f32, contiguous) the rows land at out[:, :, row0:row0+R]: stacks
+        that share a factor fill one tall matrix without being concatenated first."""
+        _need_cuda(W, perm_inv, dead, out)
         B, R, C = W.shape
         assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
         assert tuple(perm_inv.shape) == (B, C)
         assert dead is None or (dead.dtype == torch.uint8 and dead.is_contiguous())
-        out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
+        if out is None:
+            out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
+            row0 = 0
+        assert out.is_contiguous() and out.dtype == torch.float32 and out.dim() == 3
+        Rtot = out.shape[2]
+        assert tuple(out.shape[:2]) == (B, C) and 0 <= row0 and row0 + R <= Rtot
         with torch.cuda.device(W.device):
-            self._check(self._lib.forge_weight_to_solver_order(
+            self._check(self._lib.forge_weight_to_solver_order_strided(
                 _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
-                _ptr(out), B, R, C, _stream()))
+                out.data_ptr() + 4 * row0, Rtot, C * Rtot, B, R, C, _stream()))
         return out
 
-    def codes_to_layer_order(self, q, perm_inv):
-        """q [B,C,R] u8 (solver order) -> [B,R,C] u8, out[b, r, c] = q[b, perm_inv[b,c], r]."""
-        _need_cuda(q, perm_inv)
-        B, C, R = q.shape
+    def codes_to_layer_order(self, q, perm_inv, out=None, row0=0, rows=None):
+        """q [B,C,R] u8 (solver order) -> [B,R,C] u8, out[b, r, c] = q[b, perm_inv[b,c], r].
+        ``row0``/``rows`` select a band of q's rows (a stack of a tall shared-factor matrix);
+        ``out`` [B,rows,C] (contiguous) receives it."""
+        _need_cuda(q, perm_inv, out)
+        B, C, Rtot = q.shape
+        R = Rtot - row0 if rows is None else int(rows)
         assert q.is_contiguous() and q.dtype == torch.uint8 and perm_inv.is_contiguous()
         assert perm_inv.dtype == torch.int64 and tuple(perm_inv.shape) == (B, C)
-        out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
+        assert 0 <= row0 and R >= 0 and row0 + R <= Rtot
+        if out is None:
+            out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
+        assert out.is_contiguous() and out.dtype == torch.uint8 and tuple(out.shape) == (B, R, C)
         with torch.cuda.device(q.device):
-            self._check(self._lib.forge_codes_to_layer_order(_ptr(q), _ptr(perm_inv), _ptr(out), B,
-                                                             R, C, _stream()))
+            self._check(self._lib.forge_codes_to_layer_order_strided(
+                q.data_ptr() + row0, Rtot, C * Rtot, _ptr(perm_inv), _ptr(out), B, R, C, _stream()))
         return out
 
     def pack_int4(self, codes, qzeros, group_size):

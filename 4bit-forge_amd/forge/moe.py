@@ -169,22 +169,31 @@ class ExpertGroupGPTQ:
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
             for job in jobs:
-                Wc = self.W[job[0]][e0:e1] if len(job) == 1 else torch.cat(
-                    [self.W[i][e0:e1] for i in job], dim=1)
-                R = Wc.shape[1]
+                # the stacks of a job share the factor and are swept as ONE tall matrix, their rows
+                # one after the other; nothing is concatenated: each stack is searched and laid
+                # out from where it is
+                R = sum(sizes[i] for i in job)
                 # the scale search only needs the weights: it runs on a side stream so that
                 # its VALU/transcendental work shares the CUs with the MFMA-bound factorisation
                 main = torch.cuda.current_stream()
                 side.wait_stream(main)
                 with torch.cuda.stream(side):
-                    # pruned columns are zero in the reference's W before the grid is built
-                    Wsrc = Wc.masked_fill(dead[:, None, :], 0) if has_dead else Wc
-                    scales, qzeros = kernels.quant_grid(Wsrc, gs, self.bits, self.symmetric, mse,
-                                                        cand, norm)
+                    parts = []
+                    for i in job:
+                        # pruned columns are zero in the reference's W before the grid is built
+                        Wi = self.W[i][e0:e1]
+                        Wsrc = Wi.masked_fill(dead[:, None, :], 0) if has_dead else Wi
+                        parts.append(kernels.quant_grid(Wsrc, gs, self.bits, self.symmetric, mse,
+                                                        cand, norm))
+                        Wsrc.record_stream(side)
+                        del Wsrc
+                    if len(parts) == 1:
+                        scales, qzeros = parts[0]
+                    else:
+                        scales = torch.cat([p[0].view(B, sizes[i], G) for p, i in zip(parts, job)], dim=1)
+                        qzeros = torch.cat([p[1].view(B, sizes[i], G) for p, i in zip(parts, job)], dim=1)
                     sT = scales.view(B, R, G).transpose(1, 2).contiguous()
                     zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
-                    Wsrc.record_stream(side)
-                    del Wsrc
                 Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
                 if babai:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
@@ -210,7 +219,11 @@ class ExpertGroupGPTQ:
                     U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                 del Hp
                 failed.append((e0, info))
-                X = kernels.weight_to_solver_order(Wc, perm_inv, dead_u8)
+                X = torch.empty((B, C, R), dtype=torch.float32, device=dev)
+                r0 = 0
+                for i in job:
+                    kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0)
+                    r0 += sizes[i]
                 main.wait_stream(side)
                 for t in (scales, qzeros, sT, zT):
                     t.record_stream(main)
@@ -226,11 +239,10 @@ class ExpertGroupGPTQ:
                 else:
                     q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
                 del X, U
-                q = kernels.codes_to_layer_order(q, perm_inv)
                 r0 = 0
                 for i in job:
                     Ri = sizes[i]
-                    outs[i][0][e0:e1] = q[:, r0:r0 + Ri]
+                    kernels.codes_to_layer_order(q, perm_inv, out=outs[i][0][e0:e1], row0=r0, rows=Ri)
                     outs[i][1][e0:e1] = scales.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     outs[i][2][e0:e1] = qzeros.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     if sparse:

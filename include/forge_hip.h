@@ -278,6 +278,20 @@ int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, i
 int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm_inv, uint8_t* qout,
                                int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
 
+/* The two layout passes on a band of rows of a taller solver-order matrix: weight stacks that
+ * share one factor (gate_proj and up_proj, gptq.py:36,84-94) are swept as ONE matrix whose
+ * rows are the stacks' rows one after the other, without first concatenating the stacks.
+ * _strided forms: Xout / qin point at the band's first row inside the tall matrix, ldo / ldi is
+ * the tall matrix's row pitch in elements (>= R) and o_stride / i_stride its batch stride;
+ * everything else as above (the plain forms are the case ldo = R, o_stride = C*R). */
+int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                                         const int64_t* perm_inv, const uint8_t* dead, float* Xout,
+                                         int64_t ldo, int64_t o_stride, int64_t batch, int64_t R,
+                                         int64_t C, forge_stream_t stream);
+int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
+                                       const int64_t* perm_inv, uint8_t* qout, int64_t batch,
+                                       int64_t R, int64_t C, forge_stream_t stream);
+
 /* Nibble packing of [R, C] u8 codes into the compressed-tensors "pack-quantized" int32
  * layout consumed by pack_quantized.py:279-313: value = code - zero + 8 (offset binary of
  * the zero-shifted int4), eight values per int32 along C, lowest nibble first.
