@@ -23,6 +23,11 @@ struct GemmArgs {
     bool b_lower_tri;  // Bm[k, n] == 0 for k < n: start each tile's K loop at its first column
     bool blocked_sum;  // sum K in blocks of 128 (more accurate; NOT the sweep's single chain)
     int products;      // bf16-piece path only: piece products per fp32 product (1, 3, 4; else 6)
+    // piece path only: not null = two fp16 pieces of every operand, column c of At and of Bm
+    // scaled by the power of two scale[matrix * scale_stride + c] (the caller's bound:
+    // |entry| * scale <= 2^14; At and Bm share their column indexing), three products, fp32-grade
+    const float* scale;
+    int64_t scale_stride;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;

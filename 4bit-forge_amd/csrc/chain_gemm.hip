@@ -567,12 +567,39 @@ __device__ __forceinline__ void split_pieces2(const float (&x)[N], W& p1, W& p2)
     }
 }
 
+// Two fp16 pieces of sc * x, each rounded to nearest (v_cvt_pk_f16_f32).  fp16 carries 11
+// significant bits, so a1 = fp16(x), a2 = fp16(x - a1) leave |x - a1 - a2| <= 2^-24 |x|: the pair
+// holds an fp32 value to its own precision, and the three products (2,1) (1,2) (1,1) give a*b
+// to ~2^-23 -- fp32-grade from THREE products of the fp16 matrix instruction instead of six of
+// the bf16 one.  The price is fp16's range: sc is a power of two, one per column of the operand
+// matrix, chosen by the caller so that the column's largest entry lands at or below 2^14 (no
+// overflow; the result is divided by the two columns' factors afterwards, exactly); an entry
+// below 2^-17 of its column's bound loses low bits of its second piece (subnormal or flushed),
+// an absolute error of at most 2^-29 of that bound, far below the fp32 rounding of the sums it
+// enters.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+template <int N, typename W>
+__device__ __forceinline__ void split_pieces2h(const float (&x)[N], float sc, W& p1, W& p2) {
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w) {
+        const f32x2 v = {x[2 * w] * sc, x[2 * w + 1] * sc};
+        const f16x2 h1 = __builtin_convertvector(v, f16x2);
+        const f32x2 back = __builtin_convertvector(h1, f32x2);
+        const f32x2 r = {v[0] - back[0], v[1] - back[1]};
+        p1[w] = __builtin_bit_cast(unsigned, h1);                    // k in the low half
+        p2[w] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, f16x2));
+    }
+}
+
 // Rows [k0, k1) x columns [m0, m0+128) of At -> the LDS images of its stages, stage after
 // stage (SPLIT_STAGE_WORDS words each).  One workgroup of 128 threads per matrix and stage.
-template <int NP>
+template <int NP, bool HALF>
 __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restrict__ At, int64_t lda,
                                                             int64_t as, int m0, int k0, int n_stage,
-                                                            u32x4* __restrict__ Ap, int64_t aps) {
+                                                            u32x4* __restrict__ Ap, int64_t aps,
+                                                            const float* __restrict__ scale,
+                                                            int64_t scale_stride) {
     const int bz = blockIdx.x / n_stage, st = blockIdx.x % n_stage;
     const int t = threadIdx.x, kg = t >> 5, cq = t & 31;
     const float* src = At + (int64_t)bz * as + (int64_t)(k0 + SPLIT_TK * st + 8 * kg) * lda + m0 + 4 * cq;
@@ -580,6 +607,8 @@ __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restr
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[j] = *reinterpret_cast<const f32x4*>(src + (int64_t)j * lda);
     u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * split_stage_words(NP) + kg * 128 + cq;
+    f32x4 sc4 = {1.f, 1.f, 1.f, 1.f};
+    if (HALF) sc4 = *reinterpret_cast<const f32x4*>(scale + (int64_t)bz * scale_stride + m0 + 4 * cq);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float col[8];
@@ -589,6 +618,8 @@ __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restr
         if (NP == 3) {
             split_pieces<8>(col, p1, p2, p3);
             dst[1024 + 32 * e] = p3;
+        } else if (HALF) {
+            split_pieces2h<8>(col, sc4[e], p1, p2);
         } else {
             split_pieces2<8>(col, p1, p2);
         }
@@ -611,7 +642,9 @@ struct SplitPair {
 //   NP = 2 (pieces rounded to nearest): NPROD = 3: (2,1) (1,2) (1,1), within ~2^-17 of a*b;
 //   NPROD = 4 adds (2,2); NPROD = 1 is (1,1) alone, i.e. plain bf16 operands.  Only where the
 //   caller asks for it (the direct sweep's block updates, option "sweep_update_products").
-template <int NP, int NPROD>
+//   HALF (NP = 2, NPROD = 3): the pieces are fp16 halves of operands scaled by the powers of two
+//   g.scale[matrix][column] (split_pieces2h): fp32-grade from three products.
+template <int NP, int NPROD, bool HALF>
 __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     const bool in_first = blockIdx.x < (unsigned)sp.pair.first_wgs;
     const GemmArgs& g = in_first ? sp.pair.first : sp.pair.second;
@@ -654,6 +687,9 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         int ob[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) ob[j] = (int)(((int64_t)(4 * kh + j) * g.ldb + 4 * cq) * 4);
+        // fp16 halves: the power-of-two factors of this thread's four B columns
+        f32x4 scb = {1.f, 1.f, 1.f, 1.f};
+        if (HALF) scb = *reinterpret_cast<const f32x4*>(g.scale + (int64_t)bz * g.scale_stride + nt + 4 * cq);
         const int oa = pt * 16;
         // Every fetch stays inside [k0, k1): the offsets advance only while a further stage
         // exists; past the end the last stage is fetched again and never used.
@@ -685,6 +721,8 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             if (NP == 3) {                                                                         \
                 split_pieces<4>(col, p1, p2, p3);                                                  \
                 Lb[((buf) * BUF + (NP - 1) * 512 + 32 * e) * 2] = p3;                              \
+            } else if (HALF) {                                                                     \
+                split_pieces2h<4>(col, scb[e], p1, p2);                                            \
             } else {                                                                               \
                 split_pieces2<4>(col, p1, p2);                                                     \
             }                                                                                      \
@@ -716,6 +754,17 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         // 16-byte pieces of whole 512-byte rows.
         float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)m0 * g.ldx + nt + 4 * cq;
         const float sgn = g.negate_a ? -1.0f : 1.0f;
+        // fp16 halves: element (row, column) of the sums carries the factors of A's column
+        // m0 + row and of B's column; powers of two, so dividing them out is exact
+        f32x4 ib = {1.f, 1.f, 1.f, 1.f};
+        if (HALF) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ib[e] = sgn / scb[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ib[e] = sgn;
+        }
+        const float* __restrict__ sca = HALF ? g.scale + (int64_t)bz * g.scale_stride + m0 : nullptr;
         f32x4 xo[16];
         if (!g.init_zero) {
 #pragma unroll
@@ -731,9 +780,10 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const float* Sr = S + (kh + 8 * i) * TN + cq;
+            const float ia = HALF ? 1.0f / sca[kh + 8 * i] : 1.0f;
             f32x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + sgn * Sr[32 * e];
+            for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + (ib[e] * ia) * Sr[32 * e];
             *reinterpret_cast<f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx) = o;
         }
         return;
@@ -770,7 +820,10 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         constexpr int PA[6] = {NP - 1, 0, 1, 1, 0, 0}, PB[6] = {0, NP - 1, 1, 0, 1, 0};            \
         _Pragma("unroll") for (int t = 6 - NPROD; t < 6; ++t) _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) \
             _Pragma("unroll") for (int ni = 0; ni < 2; ++ni)                                       \
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                             \
+                acc[mi][ni] = HALF ? __builtin_amdgcn_mfma_f32_32x32x16_f16(                       \
+                    __builtin_bit_cast(f16x8, A[PA[t]][mi]), __builtin_bit_cast(f16x8, B[PB[t]][ni]), \
+                    ((fresh) && t == 6 - NPROD) ? zero : acc[mi][ni], 0, 0, 0)                     \
+                    : __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                     \
                     A[PA[t]][mi], B[PB[t]][ni], ((fresh) && t == 6 - NPROD) ? zero : acc[mi][ni], 0, 0, 0);\
     } while (0)
     // 4 NPROD MFMAs and 4 NP LDS reads per k-step (24 and 12, or 12 and 8): the reads spread
@@ -933,6 +986,7 @@ bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t
     if (b) {
         const GemmArgs &x = a.g, &y = b->g;
         if (x.At != y.At || x.lda != y.lda || x.as != y.as || x.m0 != y.m0 || x.k0 != y.k0) return false;
+        if (x.scale != y.scale || x.scale_stride != y.scale_stride) return false;
         if (b->g.xcd_map && a.n_wg % 8 != 0) return false;
         if (y.k1 > k1) k1 = y.k1;
     }
@@ -951,7 +1005,8 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
     sp.pair.second = b ? b->g : a.g;
     sp.pair.first_wgs = (int)a.n_wg;
     sp.Ap = static_cast<const u32x4*>(ws);
-    const int products = a.g.products;
+    const bool half = a.g.scale != nullptr;                               // fp16 pieces, three products
+    const int products = half ? 3 : a.g.products;
     const bool two = products == 1 || products == 3 || products == 4;     // two-piece layout
     const int np = two ? 2 : 3;
     sp.aps = (int64_t)n_stage * split_stage_words(np);
@@ -961,22 +1016,30 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
                             WORK_BYTES);
         const dim3 pgrid((unsigned)(batch * n_stage)), pblock(128);
         u32x4* dst = static_cast<u32x4*>(ws) + (int64_t)mt * sp.apt;
-        if (two)
-            split_a_panel_kernel<2><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM,
-                                                              a.g.k0, n_stage, dst, sp.aps);
+        if (half)
+            split_a_panel_kernel<2, true><<<pgrid, pblock, 0, st>>>(
+                a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, a.g.scale,
+                a.g.scale_stride);
+        else if (two)
+            split_a_panel_kernel<2, false><<<pgrid, pblock, 0, st>>>(
+                a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, nullptr, 0);
         else
-            split_a_panel_kernel<3><<<pgrid, pblock, 0, st>>>(a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM,
-                                                              a.g.k0, n_stage, dst, sp.aps);
+            split_a_panel_kernel<3, false><<<pgrid, pblock, 0, st>>>(
+                a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, nullptr, 0);
         FORGE_LAUNCH_CHECK();
     }
-    KernelTiming timing(two ? "split_gemm_bf16x2" : "split_gemm_bf16x3", st,
+    KernelTiming timing(half ? "split_gemm_f16x2" : two ? "split_gemm_bf16x2" : "split_gemm_bf16x3", st,
                         a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
     const dim3 grid((unsigned)n_wg), block(512);
-    switch (products) {
-        case 1: split_gemm_kernel<2, 1><<<grid, block, 0, st>>>(sp); break;
-        case 3: split_gemm_kernel<2, 3><<<grid, block, 0, st>>>(sp); break;
-        case 4: split_gemm_kernel<2, 4><<<grid, block, 0, st>>>(sp); break;
-        default: split_gemm_kernel<3, 6><<<grid, block, 0, st>>>(sp); break;
+    if (half) {
+        split_gemm_kernel<2, 3, true><<<grid, block, 0, st>>>(sp);
+    } else {
+        switch (products) {
+            case 1: split_gemm_kernel<2, 1, false><<<grid, block, 0, st>>>(sp); break;
+            case 3: split_gemm_kernel<2, 3, false><<<grid, block, 0, st>>>(sp); break;
+            case 4: split_gemm_kernel<2, 4, false><<<grid, block, 0, st>>>(sp); break;
+            default: split_gemm_kernel<3, 6, false><<<grid, block, 0, st>>>(sp); break;
+        }
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;

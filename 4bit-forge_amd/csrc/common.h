@@ -36,6 +36,7 @@ enum Option {
     OPT_SWEEP_SCHEDULE = 0,    // 0 = by tile count, 1 = left-looking, 2 = right-looking
     OPT_FP32_BLOCKED_SUM = 1,  // 1 = blocked sums stay on the fp32 matrix instruction
     OPT_SWEEP_PRODUCTS = 2,    // piece products per fp32 product in the direct sweep's updates
+    OPT_FACTOR_PIECES = 3,     // 0 = fp16 halves where the operand bound is known, 1 = bf16 thirds
     OPT_COUNT
 };
 int64_t option(Option o);

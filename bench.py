@@ -55,6 +55,7 @@ PEAK_TRANSCENDENTALS = 256 * 4 * 4 * 2.4e9
 # (on and above the diagonal) for the Hessian, unique bytes for the movers.
 KERNEL_BOUND = {
     "split_gemm_bf16x2": ("mfma", "mfma_bf16", 3.0),
+    "split_gemm_f16x2": ("mfma", "mfma_bf16", 3.0),      # fp16 and bf16 share the dense peak
     "split_gemm_bf16x3": ("mfma", "mfma_bf16", 6.0),
     "chain_gemm_blocked_sum": ("mfma", "mfma_f32", 1.0),
     "chain_gemm": ("mfma", "mfma_f32", 1.0),

@@ -63,6 +63,12 @@ int forge_kernel_timing_get(int index, char* name, int name_cap, int64_t* launch
  *                           (operands rounded to bf16; for measurements: it moves 2-16 % of
  *                           the codes) or 0 (default): 3 from C = 4096 on, 6 below; the
  *                           factorisation always uses 6
+ *   "factor_pieces"         FORGE_FACTOR_PIECES=1             0 (default): where only the factor of H is
+ *                           computed (forge_chol_reverse_lower_batched, C a multiple of 128) the
+ *                           trailing updates take two fp16 halves of every operand, each column
+ *                           scaled by a power of two from its diagonal entry, and three
+ *                           products (fp32-grade: the halves hold 22+ bits); 1: three bf16 thirds
+ *                           and six products everywhere, as forge_chol_inv_upper_batched always does
  * forge_set_option returns FORGE_ERR_INVALID for an unknown name or a value out of range;
  * forge_get_option returns -1 for an unknown name. */
 int forge_set_option(const char* name, int64_t value);

@@ -79,10 +79,21 @@ class Float64StagesGPTQ(oracle.GPTQ):
 
 
 def reference_floor(W, batches, qo, **kw):
-    """(floor, q64): q64 = codes of Float64StagesGPTQ on the same inputs, floor = the share
-    of the oracle's codes `qo` that differ from them."""
+    """(floor, out64).  Two other valid realisations of the reference on the same inputs:
+    (a) Float64StagesGPTQ (out64 = what it returns), (b) the oracle itself with every
+    calibration batch fed in three pieces, i.e. the running-mean Hessian of gptq.py:73-79
+    summed in another order by the same fp32 SGEMM.  floor = the larger of the two shares of
+    the oracle's codes `qo` that differ: the codes' own sensitivity is heavy-tailed (one early
+    flip cascades along its row), and a single alternative underestimates it as often as not."""
     t = Float64StagesGPTQ(linear(W), trail_mode=oracle.TRAIL_GEMM, **kw)
     for b in batches:
         t.update(b)
     out = t.quantize()
-    return flip_rate(qo, out[0]), out
+    floor = flip_rate(qo, out[0])
+    if sum(int(b.shape[0]) for b in batches) >= 3:
+        c = oracle.GPTQ(linear(W), **kw)
+        for b in batches:
+            for part in torch.chunk(b, 3):
+                c.update(part)
+        floor = max(floor, flip_rate(qo, c.quantize()[0]))
+    return floor, out

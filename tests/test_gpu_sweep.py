@@ -198,6 +198,44 @@ def test_direct_factor_on_the_gpu(hip):
     assert np.abs((2 * np.eye(C) - V) @ Ut - np.eye(C)).max() < 1e-3
 
 
+@pytest.mark.parametrize("spread", [0.0, 4.0])
+def test_factor_of_h_from_fp16_halves(hip, spread):
+    """Where only the factor of H is needed, the trailing updates form every fp32 product from
+    two fp16 halves of the operands (three products), each column scaled by a power of two
+    taken from its diagonal entry.  Against float64 it must be as accurate as the three-bf16-
+    thirds form (six products), also when the diagonal spans 16 orders of magnitude (feature
+    scales 1e-4 .. 1e4) and the batch mixes differently scaled matrices."""
+    C, B = 640, 3
+    g = torch.Generator().manual_seed(17)
+    Hs = []
+    for b in range(B):
+        X = torch.randn(900, C, generator=g, dtype=torch.float64)
+        X = X * (10.0 ** (spread * (2 * torch.rand(C, generator=g, dtype=torch.float64) - 1))) * 10.0 ** (b - 1)
+        Hs.append((2.0 / 900) * X.T @ X)
+    H = torch.stack(Hs)
+    damp = 1e-4 * torch.diagonal(H, dim1=1, dim2=2).mean(1)       # small: the spread stays in the factor
+    Hd = H + torch.diag_embed(damp[:, None].expand(B, C))
+    errs = {}
+    for tag, opt in (("halves", 0), ("thirds", 1)):
+        old = hip.set_option("factor_pieces", opt)
+        try:
+            L, info = hip.chol_reverse_lower_batched(H.float().to(DEV), damp.float().to(DEV))
+        finally:
+            hip.set_option("factor_pieces", old)
+        assert info.tolist() == [0] * B
+        worst = 0.0
+        for b in range(B):
+            A = Hd[b].float().double().numpy()            # what the GPU was given
+            Lr = np.linalg.cholesky(A[::-1, ::-1])[::-1, ::-1].T    # A = L2^T L2, L2 lower
+            d = 1.0 / np.sqrt(np.diag(A))
+            got = np.tril(L[b].cpu().double().numpy())
+            worst = max(worst, np.linalg.norm((got - Lr) * d[None, :]) / np.linalg.norm(Lr * d[None, :]))
+        errs[tag] = worst
+    print(f"spread 1e+-{spread}: equilibrated factor error halves {errs['halves']:.2e} thirds {errs['thirds']:.2e}")
+    assert errs["halves"] <= 1.5 * errs["thirds"] + 1e-7
+    assert errs["halves"] < (2e-3 if spread else 1e-5)
+
+
 def test_full_size_sweep_properties(hip):
     """Config-1 size (2048 x 2048): U = I must give round-to-nearest bit for bit, and the
     batched (left-looking) and single-matrix (right-looking) schedules must agree."""
