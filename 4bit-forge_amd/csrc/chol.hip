@@ -388,7 +388,9 @@ extern "C" int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C) {
     if (batch <= 0 || C <= 0) return 0;
     const int64_t nblk = forge::ceil_div(C, NB);
     // inverse diagonal blocks, then the split A panel of the trailing updates
-    return batch * nblk * NB * NB * (int64_t)sizeof(float) + forge::split_gemm_workspace_bytes(batch, C) +
+    // inverse diagonal blocks, then the split A panels of the trailing updates (two block rows
+    // per product on the factor-only route)
+    return batch * nblk * NB * NB * (int64_t)sizeof(float) + 2 * forge::split_gemm_workspace_bytes(batch, C) +
            (batch * C * (int64_t)sizeof(float) + 255) / 256 * 256;   // + one scale per column
 }
 
@@ -402,7 +404,7 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
     float* Dinv = (float*)ws;
     const int64_t dinv_bytes = batch * nblk * NB * NB * (int64_t)sizeof(float);
     void* split_ws = (char*)ws + dinv_bytes;
-    const int64_t split_ws_bytes = forge::split_gemm_workspace_bytes(batch, C);
+    const int64_t split_ws_bytes = 2 * forge::split_gemm_workspace_bytes(batch, C);
     float* scale = (float*)((char*)ws + dinv_bytes + split_ws_bytes);   // one per column and matrix
     // Factor only (no triangular inverse follows): every operand of the trailing updates is a
     // finished row of the factor, whose entries are bounded by the diagonal of the matrix, so
@@ -428,26 +430,31 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
             H, C, scale);
         FORGE_LAUNCH_CHECK();
     }
-    for (int a = nblk - 1; a >= 0; --a) {
+    // 1a (+ 2a) for block rows [a_lo, a]: P[rows, 0..a] -= sum_{k > a} L2[k, rows]^T L2[k, 0..a].
+    // 1a and 2a of a step do not depend on each other (2a needs rows > a only), and their tile
+    // counts are complementary, (a+1) and (nblk-1-a) per matrix: one grid.
+    auto trailing_update = [&](int a_lo, int a) -> int {
+        const int m0 = a_lo * NB;
+        const int m1 = (int)(C < (int64_t)(a + 1) * NB ? C : (int64_t)(a + 1) * NB);
+        if (m1 >= C) return FORGE_OK;                       // nothing below
+        forge::GemmArgs g1a{}, g2a{};
+        g1a.X = H; g1a.At = H; g1a.Bm = H; g1a.ldx = g1a.lda = g1a.ldb = C;
+        g1a.xs = g1a.as = g1a.bs = C * C;
+        g1a.m0 = m0; g1a.m1 = m1; g1a.n0 = 0; g1a.n1 = m1; g1a.k0 = m1; g1a.k1 = (int)C;
+        g1a.negate_a = true; g1a.blocked_sum = true;
+        if (halves) { g1a.scale = scale; g1a.scale_stride = C; }
+        if (!factor_only) {
+            g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
+            g2a.xs = g2a.as = g2a.bs = C * C;
+            g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
+            g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
+        }
+        return forge::launch_chain_gemm_pair(g1a, g2a, batch, st, split_ws, split_ws_bytes);
+    };
+    // 1b, 1c (+ 2b) of block row a: diagonal block, then the row's panels times Dinv^T.
+    auto finish_block_row = [&](int a) -> int {
         const int m0 = a * NB;
         const int m1 = (int)(C < (int64_t)m0 + NB ? C : m0 + NB);
-        // 1a and 2a of this step do not depend on each other (2a needs rows > a only), and
-        // their tile counts are complementary, (a+1) and (nblk-1-a) per matrix: one grid
-        forge::GemmArgs g1a{}, g2a{};   // left empty (m1 == m0) when there is nothing below
-        if (m1 < C) {
-            g1a.X = H; g1a.At = H; g1a.Bm = H; g1a.ldx = g1a.lda = g1a.ldb = C;
-            g1a.xs = g1a.as = g1a.bs = C * C;
-            g1a.m0 = m0; g1a.m1 = m1; g1a.n0 = 0; g1a.n1 = m1; g1a.k0 = m1; g1a.k1 = (int)C;
-            g1a.negate_a = true; g1a.blocked_sum = true;
-            if (halves) { g1a.scale = scale; g1a.scale_stride = C; }
-            if (!factor_only) {
-                g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
-                g2a.xs = g2a.as = g2a.bs = C * C;
-                g2a.m0 = m0; g2a.m1 = m1; g2a.n0 = m1; g2a.n1 = (int)C; g2a.k0 = m1; g2a.k1 = (int)C;
-                g2a.init_zero = true; g2a.b_upper_tri = true; g2a.blocked_sum = true;
-            }
-            if (int e = forge::launch_chain_gemm_pair(g1a, g2a, batch, st, split_ws, split_ws_bytes)) return e;
-        }
         {
             forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,
                                        forge::WORK_FLOPS);
@@ -474,7 +481,31 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
             g2b.m0 = m0; g2b.m1 = m1; g2b.n0 = m1; g2b.n1 = (int)C; g2b.k0 = m0; g2b.k1 = m1;
             g2b.init_zero = true; g2b.negate_a = true;
         }
-        if (int e = forge::launch_chain_gemm_pair(g1c, g2b, batch, st)) return e;
+        return forge::launch_chain_gemm_pair(g1c, g2b, batch, st);
+    };
+    // With the fp16 halves the long product is bound by reading the rows of the factor below
+    // the block from HBM (64 flops per byte at 128 columns), so two block rows are brought up to
+    // date per product: every row read serves 256 columns (the second block's reading comes from
+    // L2).  The upper of the two then only lacks what the lower one adds once it is finished, a
+    // K = 128 product on the fp32 pipe.  (The pair's product also touches the block above the
+    // upper row's diagonal block; nothing reads the upper triangle.)
+    for (int a = nblk - 1; a >= 0;) {
+        const bool pair = halves && a >= 1;
+        if (int e = trailing_update(pair ? a - 1 : a, a)) return e;
+        if (int e = finish_block_row(a)) return e;
+        if (pair) {
+            forge::GemmArgs fix{};
+            fix.X = H; fix.At = H; fix.Bm = H; fix.ldx = fix.lda = fix.ldb = C;
+            fix.xs = fix.as = fix.bs = C * C;
+            fix.m0 = (a - 1) * NB; fix.m1 = a * NB; fix.n0 = 0; fix.n1 = a * NB;
+            fix.k0 = a * NB; fix.k1 = (a + 1) * NB;
+            fix.negate_a = true;
+            if (int e = forge::launch_chain_gemm(fix, batch, st)) return e;
+            if (int e = finish_block_row(a - 1)) return e;
+            a -= 2;
+        } else {
+            a -= 1;
+        }
     }
     if (factor_only) return FORGE_OK;
     forge::KernelTiming timing("chol_finish_rows", st,

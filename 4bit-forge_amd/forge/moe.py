@@ -87,10 +87,13 @@ class ExpertGroupGPTQ:
     # ------------------------------------------------------------------ solve
     @torch.no_grad()
     def quantize(self, chunk: int = 32, max_shrink: float = 0.2, n_grid: int = 100,
-                 norm: float = 2.4):
+                 norm: float = 2.4, overlap_scale_search: bool = True):
         """Returns one (qweight [E,R,C] u8, scales [E,R*G] f32, qzeros [E,R*G] f32) per stack;
         with algorithm="sparsegptq" a fourth element M [E, ceil(C/32), R] u32 (bit i of word w
-        <-> column 32 w + i of the SOLVER order, as the reference returns it)."""
+        <-> column 32 w + i of the SOLVER order, as the reference returns it).
+        overlap_scale_search=False keeps the scale search on the caller's stream instead of a
+        side stream (same results; for per-kernel timing, where no kernel's time should include
+        another stream's work)."""
         E, C, gs, dev = self.E, self.C, self.group_size, self.device
         G = (C + gs - 1) // gs
         mse = self.quantization_scale == "mse"
@@ -116,7 +119,7 @@ class ExpertGroupGPTQ:
             self.H[e].zero_()
             self.H[e].diagonal().fill_(1.0)
         failed = []
-        side = torch.cuda.Stream(device=dev)          # default priority
+        side = torch.cuda.Stream(device=dev) if overlap_scale_search else None   # default priority
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
@@ -176,8 +179,9 @@ class ExpertGroupGPTQ:
                 # the scale search only needs the weights: it runs on a side stream so that
                 # its VALU/transcendental work shares the CUs with the MFMA-bound factorisation
                 main = torch.cuda.current_stream()
-                side.wait_stream(main)
-                with torch.cuda.stream(side):
+                search = side if side is not None else main
+                search.wait_stream(main)
+                with torch.cuda.stream(search):
                     parts = []
                     for i in job:
                         # pruned columns are zero in the reference's W before the grid is built
@@ -185,7 +189,7 @@ class ExpertGroupGPTQ:
                         Wsrc = Wi.masked_fill(dead[:, None, :], 0) if has_dead else Wi
                         parts.append(kernels.quant_grid(Wsrc, gs, self.bits, self.symmetric, mse,
                                                         cand, norm))
-                        Wsrc.record_stream(side)
+                        Wsrc.record_stream(search)
                         del Wsrc
                     if len(parts) == 1:
                         scales, qzeros = parts[0]
@@ -224,7 +228,7 @@ class ExpertGroupGPTQ:
                 for i in job:
                     kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0)
                     r0 += sizes[i]
-                main.wait_stream(side)
+                main.wait_stream(search)
                 for t in (scales, qzeros, sT, zT):
                     t.record_stream(main)
                 M = None

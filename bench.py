@@ -144,7 +144,7 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
                 with torch.cuda.stream(stream):
                     grp = ExpertGroupGPTQ([w[a:b] for w in weights], **kw)
                     grp.update(rows[offs[a]:offs[b]], sub_offs)
-                    return grp.quantize(chunk=b - a)
+                    return grp.quantize(chunk=b - a, overlap_scale_search=overlap)
 
             for weights, rows, stream in (([wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]),
                                           ([wl["Wd"]], hs, STREAMS[2 * j + 1])):

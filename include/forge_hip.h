@@ -232,8 +232,8 @@ int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype);
  * blocks is left unwritten.  info[b] (int32) is 0 on
  * success or the 1-based index of the first non-positive pivot, in which case U[b] = I.
  * H[b] is destroyed (used as workspace).  ws: workspace of forge_chol_workspace_bytes
- * (128x128 inverse diagonal blocks, plus 768 bytes per column and matrix for the bf16
- * pieces of one panel), 256-byte aligned.
+ * (128x128 inverse diagonal blocks, plus 1540 bytes per column and matrix for the 16-bit
+ * pieces of two panels and the column scales), 256-byte aligned.
  * When C is a multiple of 128 the trailing updates are computed from three bf16 pieces per
  * fp32 operand on the bf16 matrix pipe (fp32-grade accuracy; not bit-identical to the fp32
  * update).  The option "fp32_blocked_sum" selects the fp32 update. */

@@ -37,9 +37,9 @@ def test_invalid_arguments_are_rejected_without_a_launch():
     rc = lib.forge_quant_grid(None, 7, 1, 0, 4, 128, 128, 128, 4, 1, 0, None, 0, 2.4, None, None, None)
     assert rc == 1 and b"w_dtype" in lib.forge_last_error()
     assert lib.forge_build_group_meta_packed(None, 0, 128, 4, 1, None, None, None) == 0   # empty: no-op
-    # inverse diagonal blocks (fp32) + the bf16 pieces of one 128-column panel (6 bytes per
-    # element) + one fp32 scale per column
-    assert lib.forge_chol_workspace_bytes(2, 256) == 2 * 2 * 128 * 128 * 4 + 2 * 256 * 128 * 6 + 2 * 256 * 4
+    # inverse diagonal blocks (fp32) + the 16-bit pieces of two 128-column panels (6 bytes per
+    # element each) + one fp32 scale per column
+    assert lib.forge_chol_workspace_bytes(2, 256) == 2 * 2 * 128 * 128 * 4 + 2 * 2 * 256 * 128 * 6 + 2 * 256 * 4
 
 
 def test_options_are_settings_of_the_library_not_of_the_environment(monkeypatch):
