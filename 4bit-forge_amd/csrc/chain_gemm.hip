@@ -509,8 +509,9 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 // of the multipliers' stage:
 //   multipliers, stage s:  MFMAs of k-step 0 | reads of k-step 1;  barrier s;
 //                          MFMAs of k-step 1 | reads of (stage s+1, k-step 0)
-//   producers, between barriers s-1 and s: stage s+1 into buffer (s+1)&1, then the global
-//                          loads of stage s+5 into the registers just consumed
+//   producers, between barriers s-1 and s: stage s+1 into buffer (s+1)&1, and between its
+//                          pieces the global loads of stage s+4 into the registers that the
+//                          previous iteration consumed
 // The A panel is the same for every workgroup of a matrix, so it is split once by
 // split_a_panel_kernel into the exact LDS image of each stage and the producers only copy it.
 // The multipliers never touch global memory: they start from zero, and at the end hand their
@@ -644,18 +645,26 @@ struct SplitPair {
 //   caller asks for it (the direct sweep's block updates, option "sweep_update_products").
 //   HALF (NP = 2, NPROD = 3): the pieces are fp16 halves of operands scaled by the powers of two
 //   g.scale[matrix][column] (split_pieces2h): fp32-grade from three products.
-template <int NP, int NPROD, bool HALF>
+//   MT = 2 (NP = 2 only; the problem has two m tiles): one workgroup computes both, 256 x 128
+//   outputs.  Every row of B is then loaded and split once for 256 output rows, a stage holds
+//   twice the matrix work behind the same number of B loads in flight (what the producers'
+//   four register sets can cover of the HBM latency doubles), and the LDS traffic per matrix
+//   instruction falls by a quarter.  The 128 accumulator registers leave no room for a second
+//   set of totals, so K is summed in one run, as an SGEMM does.
+template <int NP, int NPROD, bool HALF, int MT>
 __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
+    static_assert(MT == 1 || (MT == 2 && NP == 2), "two m tiles per workgroup: two-piece layouts only");
     const bool in_first = blockIdx.x < (unsigned)sp.pair.first_wgs;
     const GemmArgs& g = in_first ? sp.pair.first : sp.pair.second;
     const int wg = in_first ? (int)blockIdx.x : (int)blockIdx.x - sp.pair.first_wgs;
-    // [buffer][operand][piece][k group][position]
-    __shared__ __attribute__((aligned(16))) u32x4 L[2][2][NP][4][128];
+    // [buffer][operand: the A panel of each m tile, then B][piece][k group][position]
+    __shared__ __attribute__((aligned(16))) u32x4 L[2][MT + 1][NP][4][128];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // The m tiles of one (matrix, n tile) follow each other on the same XCD: they read the same
     // rows of B at about the same time, so the second reading is served by that XCD's L2.
-    const int per_matrix = g.n_tiles * g.m_tiles;
+    const int grid_m_tiles = MT == 2 ? 1 : g.m_tiles;
+    const int per_matrix = g.n_tiles * grid_m_tiles;
     int bz, rem;
     if (g.xcd_map) {
         const int xcd = wg & 7, slot = wg >> 3;
@@ -665,7 +674,7 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         bz = wg / per_matrix;
         rem = wg % per_matrix;
     }
-    const int tile = rem / g.m_tiles, mtile = rem % g.m_tiles;
+    const int tile = rem / grid_m_tiles, mtile = rem % grid_m_tiles;
     const int m0 = g.m0 + mtile * TM;
     const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile : tile;
     const int nt = g.n0 + tn * TN;
@@ -684,6 +693,9 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<u32x4*>(sp.Ap + (int64_t)mtile * sp.apt + (int64_t)bz * sp.aps), 0, 0x7FFFFFFF,
             0x00027000);
+        const __amdgpu_buffer_rsrc_t a_rsrc2 = __builtin_amdgcn_make_buffer_rsrc(   // second m tile
+            const_cast<u32x4*>(sp.Ap + (int64_t)(MT - 1) * sp.apt + (int64_t)bz * sp.aps), 0, 0x7FFFFFFF,
+            0x00027000);
         int ob[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) ob[j] = (int)(((int64_t)(4 * kh + j) * g.ldb + 4 * cq) * 4);
@@ -696,7 +708,7 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         int b_soff = 0, a_soff = 0, fetched = 0;
         int b_adv = (int)(SPLIT_TK * g.ldb * 4), a_adv = split_stage_words(NP) * 16;
         f32x4 xb[SPLIT_SETS][4];
-        u32x4 xa[SPLIT_SETS][2 * NP];
+        u32x4 xa[SPLIT_SETS][MT * 2 * NP];
 #define FORGE_SPLIT_FETCH(q)                                                                       \
     do {                                                                                           \
         ++fetched;                                                                                 \
@@ -705,13 +717,17 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             f32x4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ob[j], b_soff, 0));               \
         _Pragma("unroll") for (int j = 0; j < 2 * NP; ++j)                                         \
             xa[q][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, oa + j * 4096, a_soff, 0);    \
+        if (MT == 2) {                                                                             \
+            _Pragma("unroll") for (int j = 0; j < 2 * NP; ++j) xa[q][(MT - 1) * 2 * NP + j] =      \
+                __builtin_amdgcn_raw_buffer_load_b128(a_rsrc2, oa + j * 4096, a_soff, 0);          \
+        }                                                                                          \
         b_soff += b_adv;                                                                           \
         a_soff += a_adv;                                                                           \
     } while (0)
         // B word (piece, k group kh >> 1, position 32 e + cq), half kh & 1; A: plain copy
-        u32x2* const Lb = reinterpret_cast<u32x2*>(&L[0][1][0][kh >> 1][cq]) + (kh & 1);
+        u32x2* const Lb = reinterpret_cast<u32x2*>(&L[0][MT][0][kh >> 1][cq]) + (kh & 1);
         u32x4* const La = &L[0][0][0][0][0] + pt;
-        constexpr int BUF = 2 * split_stage_words(NP);   // words per buffer (both operands)
+        constexpr int BUF = (MT + 1) * split_stage_words(NP);   // words per buffer (all operands)
 #define FORGE_SPLIT_STAGE(buf, q)                                                                  \
     do {                                                                                           \
         _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
@@ -729,30 +745,65 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             Lb[((buf) * BUF + 32 * e) * 2] = p1;                                                   \
             Lb[((buf) * BUF + 512 + 32 * e) * 2] = p2;                                             \
         }                                                                                          \
-        _Pragma("unroll") for (int j = 0; j < 2 * NP; ++j) La[(buf) * BUF + j * 256] = xa[q][j];   \
+        _Pragma("unroll") for (int j = 0; j < MT * 2 * NP; ++j) La[(buf) * BUF + j * 256] = xa[q][j]; \
+    } while (0)
+        // One stage's split and LDS writes, with the loads of a later stage (into the register
+        // set qf, which the previous iteration consumed) spread between them: a wavefront does
+        // not go on until the texture unit has taken its load, and the unit takes 16 cycles per
+        // 1 KB instruction, so loads issued back to back by all four producers would hold them
+        // for as long as the unit needs for the whole stage.
+#define FORGE_SPLIT_STAGE_FETCH(buf, q, qf)                                                        \
+    do {                                                                                           \
+        ++fetched;                                                                                 \
+        if (fetched >= n_stage) { b_adv = 0; a_adv = 0; }                                          \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
+            xb[qf][e] = __builtin_bit_cast(                                                        \
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ob[e], b_soff, 0));           \
+            _Pragma("unroll") for (int j = e * NP / 2; j < (e + 1) * NP / 2; ++j) {                \
+                xa[qf][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, oa + j * 4096, a_soff, 0); \
+                if (MT == 2) xa[qf][2 * NP + j] =                                                  \
+                    __builtin_amdgcn_raw_buffer_load_b128(a_rsrc2, oa + j * 4096, a_soff, 0);      \
+            }                                                                                      \
+            float col[4];                                                                          \
+            u32x2 p1, p2, p3;                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) col[j] = xb[q][j][e];                    \
+            if (NP == 3) {                                                                         \
+                split_pieces<4>(col, p1, p2, p3);                                                  \
+                Lb[((buf) * BUF + (NP - 1) * 512 + 32 * e) * 2] = p3;                              \
+            } else if (HALF) {                                                                     \
+                split_pieces2h<4>(col, scb[e], p1, p2);                                            \
+            } else {                                                                               \
+                split_pieces2<4>(col, p1, p2);                                                     \
+            }                                                                                      \
+            Lb[((buf) * BUF + 32 * e) * 2] = p1;                                                   \
+            Lb[((buf) * BUF + 512 + 32 * e) * 2] = p2;                                             \
+            _Pragma("unroll") for (int j = e * MT * NP / 2; j < (e + 1) * MT * NP / 2; ++j)        \
+                La[(buf) * BUF + j * 256] = xa[q][j];                                              \
+            __builtin_amdgcn_sched_barrier(0);                                                     \
+        }                                                                                          \
+        b_soff += b_adv;                                                                           \
+        a_soff += a_adv;                                                                           \
     } while (0)
         FORGE_SPLIT_FETCH(0);
         FORGE_SPLIT_FETCH(1);
         FORGE_SPLIT_FETCH(2);
         FORGE_SPLIT_FETCH(3);
         FORGE_SPLIT_STAGE(0, 0);
-        FORGE_SPLIT_FETCH(0);
         __syncthreads();
         for (int s0 = 0; s0 < n_stage; s0 += 4) {
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                FORGE_SPLIT_STAGE((s + 1) & 1, (s + 1) & 3);
-                FORGE_SPLIT_FETCH((s + 1) & 3);
+                FORGE_SPLIT_STAGE_FETCH((s + 1) & 1, (s + 1) & 3, s & 3);
                 __syncthreads();
             }
         }
+#undef FORGE_SPLIT_STAGE_FETCH
 #undef FORGE_SPLIT_FETCH
 #undef FORGE_SPLIT_STAGE
         // Epilogue, on the producers so that it is coalesced: the multipliers leave their
-        // sums in LDS (over the stage buffers, free by then), row r of the tile at
-        // S[r][position]; thread = 16 rows x 4 consecutive columns, X is read and written in
-        // 16-byte pieces of whole 512-byte rows.
-        float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)m0 * g.ldx + nt + 4 * cq;
+        // sums in LDS (over the stage buffers, free by then), one m tile at a time, row r of
+        // the tile at S[r][position]; thread = 16 rows x 4 consecutive columns, X is read and
+        // written in 16-byte pieces of whole 512-byte rows.
         const float sgn = g.negate_a ? -1.0f : 1.0f;
         // fp16 halves: element (row, column) of the sums carries the factors of A's column
         // m0 + row and of B's column; powers of two, so dividing them out is exact
@@ -764,27 +815,33 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) ib[e] = sgn;
         }
-        const float* __restrict__ sca = HALF ? g.scale + (int64_t)bz * g.scale_stride + m0 : nullptr;
-        f32x4 xo[16];
-        if (!g.init_zero) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                xo[i] = *reinterpret_cast<const f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) xo[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-        __syncthreads();   // every multiplier has read its last operands
-        __syncthreads();   // the sums are in LDS
         const float* S = reinterpret_cast<const float*>(&L[0][0][0][0][0]);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float* Sr = S + (kh + 8 * i) * TN + cq;
-            const float ia = HALF ? 1.0f / sca[kh + 8 * i] : 1.0f;
-            f32x4 o;
+        for (int t = 0; t < MT; ++t) {
+            float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)(m0 + t * TM) * g.ldx + nt + 4 * cq;
+            const float* __restrict__ sca =
+                HALF ? g.scale + (int64_t)bz * g.scale_stride + m0 + t * TM : nullptr;
+            f32x4 xo[16];
+            if (!g.init_zero) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + (ib[e] * ia) * Sr[32 * e];
-            *reinterpret_cast<f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx) = o;
+                for (int i = 0; i < 16; ++i)
+                    xo[i] = *reinterpret_cast<const f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) xo[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            if (t == 0) __syncthreads();   // every multiplier has read its last operands
+            __syncthreads();               // the sums of m tile t are in LDS
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float* Sr = S + (kh + 8 * i) * TN + cq;
+                const float ia = HALF ? 1.0f / sca[kh + 8 * i] : 1.0f;
+                f32x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + (ib[e] * ia) * Sr[32 * e];
+                *reinterpret_cast<f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx) = o;
+            }
+            if (t + 1 < MT) __syncthreads();   // the staging area is free for the next m tile
         }
         return;
     }
@@ -796,21 +853,30 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     // element v of the accumulator is MFMA row (lane >> 5) * 4 + (v >> 2) * 8 + (v & 3),
     // column lane & 31.
     const int jrow = (lane >> 5) * 4, jcol = lane & 31;
-    f32x16 acc[2][2], tot[2][2];   // sums of the chunks; X itself is added in the epilogue
+    // One m tile: acc holds the sum of the current 128-row chunk, tot the sum of the chunks.
+    // Two m tiles: acc runs over all of K.  X itself is added in the epilogue.
+    constexpr bool CHUNKED = MT == 1;
+    f32x16 acc[MT][2][2], tot[2][2];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) tot[mi][ni][v] = 0.0f;
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    acc[t][mi][ni][v] = 0.0f;
+                    if (CHUNKED) tot[mi][ni][v] = 0.0f;
+                }
     const int rk = lane >> 5, ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    bf16x8 A0[NP][2], B0[NP][2], A1[NP][2], B1[NP][2];   // operands of k-step 0 / 1
+    bf16x8 A0[MT][NP][2], B0[NP][2], A1[MT][NP][2], B1[NP][2];   // operands of k-step 0 / 1
 #define FORGE_SPLIT_READ(buf, u, A, B)                                                             \
     do {                                                                                           \
         _Pragma("unroll") for (int p = 0; p < NP; ++p) _Pragma("unroll") for (int i = 0; i < 2; ++i) { \
-            A[p][i] = __builtin_bit_cast(bf16x8, L[buf][0][p][2 * (u) + rk][ra + 64 * i]);         \
-            B[p][i] = __builtin_bit_cast(bf16x8, L[buf][1][p][2 * (u) + rk][rb + 64 * i]);         \
+            _Pragma("unroll") for (int t = 0; t < MT; ++t)                                         \
+                A[t][p][i] = __builtin_bit_cast(bf16x8, L[buf][t][p][2 * (u) + rk][ra + 64 * i]);  \
+            B[p][i] = __builtin_bit_cast(bf16x8, L[buf][MT][p][2 * (u) + rk][rb + 64 * i]);        \
         }                                                                                          \
     } while (0)
     // piece products smallest first; the four tiles innermost so that consecutive MFMAs use
@@ -818,25 +884,26 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
 #define FORGE_SPLIT_MFMAS(A, B, fresh)                                                             \
     do {                                                                                           \
         constexpr int PA[6] = {NP - 1, 0, 1, 1, 0, 0}, PB[6] = {0, NP - 1, 1, 0, 1, 0};            \
-        _Pragma("unroll") for (int t = 6 - NPROD; t < 6; ++t) _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) \
-            _Pragma("unroll") for (int ni = 0; ni < 2; ++ni)                                       \
-                acc[mi][ni] = HALF ? __builtin_amdgcn_mfma_f32_32x32x16_f16(                       \
-                    __builtin_bit_cast(f16x8, A[PA[t]][mi]), __builtin_bit_cast(f16x8, B[PB[t]][ni]), \
-                    ((fresh) && t == 6 - NPROD) ? zero : acc[mi][ni], 0, 0, 0)                     \
+        _Pragma("unroll") for (int t = 6 - NPROD; t < 6; ++t) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) \
+            _Pragma("unroll") for (int mi = 0; mi < 2; ++mi) _Pragma("unroll") for (int ni = 0; ni < 2; ++ni) \
+                acc[mt][mi][ni] = HALF ? __builtin_amdgcn_mfma_f32_32x32x16_f16(                   \
+                    __builtin_bit_cast(f16x8, A[mt][PA[t]][mi]), __builtin_bit_cast(f16x8, B[PB[t]][ni]), \
+                    (CHUNKED && (fresh) && t == 6 - NPROD) ? zero : acc[mt][mi][ni], 0, 0, 0)      \
                     : __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                     \
-                    A[PA[t]][mi], B[PB[t]][ni], ((fresh) && t == 6 - NPROD) ? zero : acc[mi][ni], 0, 0, 0);\
+                    A[mt][PA[t]][mi], B[PB[t]][ni],                                                \
+                    (CHUNKED && (fresh) && t == 6 - NPROD) ? zero : acc[mt][mi][ni], 0, 0, 0);     \
     } while (0)
-    // 4 NPROD MFMAs and 4 NP LDS reads per k-step (24 and 12, or 12 and 8): the reads spread
-    // evenly between the MFMAs
+    // 4 NPROD MT MFMAs and 2 NP (MT + 1) LDS reads per k-step (24 and 12, or 12 and 8): the
+    // reads spread evenly between the MFMAs
 #define FORGE_SPLIT_SCHED()                                                                        \
     do {                                                                                           \
-        if (NPROD == 6) {                                                                          \
+        if (NPROD * MT == 6) {                                                                          \
             _Pragma("unroll") for (int i = 0; i < 12; ++i) {                                       \
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
             }                                                                                      \
-        } else if (NPROD == 3) {                                                                   \
+        } else if (NPROD * MT == 3) {                                                              \
             _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                        \
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
@@ -862,10 +929,12 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             FORGE_SPLIT_SCHED();
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (CHUNKED) {
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
+            for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) tot[mi][ni] += acc[mi][ni];
+                for (int ni = 0; ni < 2; ++ni) tot[mi][ni] += acc[0][mi][ni];
+        }
     }
 #undef FORGE_SPLIT_READ
 #undef FORGE_SPLIT_MFMAS
@@ -873,15 +942,19 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     __syncthreads();   // all operand reads done: the stage buffers become the output staging
     float* S = reinterpret_cast<float*>(&L[0][0][0][0][0]);
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int t = 0; t < MT; ++t) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = 4 * (jrow + (v >> 2) * 8 + (v & 3)) + wm + 2 * mi;
-                S[r * TN + 32 * (wn + 2 * ni) + jcol] = tot[mi][ni][v];
-            }
-    __syncthreads();
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = 4 * (jrow + (v >> 2) * 8 + (v & 3)) + wm + 2 * mi;
+                    S[r * TN + 32 * (wn + 2 * ni) + jcol] = CHUNKED ? tot[mi][ni][v] : acc[t][mi][ni][v];
+                }
+        __syncthreads();                     // the producers add them to X
+        if (t + 1 < MT) __syncthreads();     // and have read them all
+    }
 }
 
 }  // namespace
@@ -1030,15 +1103,21 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
     }
     KernelTiming timing(half ? "split_gemm_f16x2" : two ? "split_gemm_bf16x2" : "split_gemm_bf16x3", st,
                         a.flops + (b ? b->flops : 0.0), WORK_FLOPS);
-    const dim3 grid((unsigned)n_wg), block(512);
+    // two m tiles of a two-piece layout: one workgroup computes both
+    const bool wide = a.g.m_tiles == 2 && np == 2 && (half || products == 3);
+    const dim3 grid((unsigned)(wide ? n_wg / 2 : n_wg)), block(512);
     if (half) {
-        split_gemm_kernel<2, 3, true><<<grid, block, 0, st>>>(sp);
+        if (wide) split_gemm_kernel<2, 3, true, 2><<<grid, block, 0, st>>>(sp);
+        else split_gemm_kernel<2, 3, true, 1><<<grid, block, 0, st>>>(sp);
     } else {
         switch (products) {
-            case 1: split_gemm_kernel<2, 1, false><<<grid, block, 0, st>>>(sp); break;
-            case 3: split_gemm_kernel<2, 3, false><<<grid, block, 0, st>>>(sp); break;
-            case 4: split_gemm_kernel<2, 4, false><<<grid, block, 0, st>>>(sp); break;
-            default: split_gemm_kernel<3, 6, false><<<grid, block, 0, st>>>(sp); break;
+            case 1: split_gemm_kernel<2, 1, false, 1><<<grid, block, 0, st>>>(sp); break;
+            case 3:
+                if (wide) split_gemm_kernel<2, 3, false, 2><<<grid, block, 0, st>>>(sp);
+                else split_gemm_kernel<2, 3, false, 1><<<grid, block, 0, st>>>(sp);
+                break;
+            case 4: split_gemm_kernel<2, 4, false, 1><<<grid, block, 0, st>>>(sp); break;
+            default: split_gemm_kernel<3, 6, false, 1><<<grid, block, 0, st>>>(sp); break;
         }
     }
     FORGE_LAUNCH_CHECK();
