@@ -23,11 +23,15 @@ struct GemmArgs {
     bool b_lower_tri;  // Bm[k, n] == 0 for k < n: start each tile's K loop at its first column
     bool blocked_sum;  // sum K in blocks of 128 (more accurate; NOT the sweep's single chain)
     int products;      // bf16-piece path only: piece products per fp32 product (1, 3, 4; else 6)
-    // piece path only: not null = two fp16 pieces of every operand, column c of At and of Bm
-    // scaled by the power of two scale[matrix * scale_stride + c] (the caller's bound:
-    // |entry| * scale <= 2^14; At and Bm share their column indexing), three products, fp32-grade
-    const float* scale;
-    int64_t scale_stride;
+    // piece path only: both not null = two fp16 pieces of every operand, three products,
+    // fp32-grade.  bound_a[matrix * bound_a_stride + m] >= |At[k, m]| and
+    // bound_b[matrix * bound_b_stride + n] >= |Bm[k, n]| for every k of the product: column m of
+    // At and column n of Bm are scaled by the largest powers of two that keep them at or below
+    // 2^14 (fp16 overflows at 2^16), and the two factors are divided out of the sums, exactly.
+    const float* bound_a;
+    int64_t bound_a_stride;
+    const float* bound_b;
+    int64_t bound_b_stride;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;

@@ -580,6 +580,13 @@ __device__ __forceinline__ void split_pieces2(const float (&x)[N], W& p1, W& p2)
 // enters.
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+// The largest power of two sc with bound * sc <= 2^14 (bound = f * 2^e, f in [0.5, 1): 2^(14 - e)),
+// kept inside [2^-100, 2^114] so that it and its reciprocal are normal numbers.
+__device__ __forceinline__ float pow2_scale(float bound) {
+    int e = __builtin_amdgcn_frexp_expf(bound);
+    e = e < -100 ? -100 : (e > 114 ? 114 : e);
+    return __uint_as_float((unsigned)(127 + 14 - e) << 23);
+}
 template <int N, typename W>
 __device__ __forceinline__ void split_pieces2h(const float (&x)[N], float sc, W& p1, W& p2) {
 #pragma unroll
@@ -599,8 +606,8 @@ template <int NP, bool HALF>
 __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restrict__ At, int64_t lda,
                                                             int64_t as, int m0, int k0, int n_stage,
                                                             u32x4* __restrict__ Ap, int64_t aps,
-                                                            const float* __restrict__ scale,
-                                                            int64_t scale_stride) {
+                                                            const float* __restrict__ bound,
+                                                            int64_t bound_stride) {
     const int bz = blockIdx.x / n_stage, st = blockIdx.x % n_stage;
     const int t = threadIdx.x, kg = t >> 5, cq = t & 31;
     const float* src = At + (int64_t)bz * as + (int64_t)(k0 + SPLIT_TK * st + 8 * kg) * lda + m0 + 4 * cq;
@@ -609,7 +616,11 @@ __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restr
     for (int j = 0; j < 8; ++j) x[j] = *reinterpret_cast<const f32x4*>(src + (int64_t)j * lda);
     u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * split_stage_words(NP) + kg * 128 + cq;
     f32x4 sc4 = {1.f, 1.f, 1.f, 1.f};
-    if (HALF) sc4 = *reinterpret_cast<const f32x4*>(scale + (int64_t)bz * scale_stride + m0 + 4 * cq);
+    if (HALF) {
+        const f32x4 b4 = *reinterpret_cast<const f32x4*>(bound + (int64_t)bz * bound_stride + m0 + 4 * cq);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc4[e] = pow2_scale(b4[e]);
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float col[8];
@@ -701,7 +712,12 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         for (int j = 0; j < 4; ++j) ob[j] = (int)(((int64_t)(4 * kh + j) * g.ldb + 4 * cq) * 4);
         // fp16 halves: the power-of-two factors of this thread's four B columns
         f32x4 scb = {1.f, 1.f, 1.f, 1.f};
-        if (HALF) scb = *reinterpret_cast<const f32x4*>(g.scale + (int64_t)bz * g.scale_stride + nt + 4 * cq);
+        if (HALF) {
+            const f32x4 b4 =
+                *reinterpret_cast<const f32x4*>(g.bound_b + (int64_t)bz * g.bound_b_stride + nt + 4 * cq);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) scb[e] = pow2_scale(b4[e]);
+        }
         const int oa = pt * 16;
         // Every fetch stays inside [k0, k1): the offsets advance only while a further stage
         // exists; past the end the last stage is fetched again and never used.
@@ -820,7 +836,7 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
         for (int t = 0; t < MT; ++t) {
             float* __restrict__ Xt = g.X + (int64_t)bz * g.xs + (int64_t)(m0 + t * TM) * g.ldx + nt + 4 * cq;
             const float* __restrict__ sca =
-                HALF ? g.scale + (int64_t)bz * g.scale_stride + m0 + t * TM : nullptr;
+                HALF ? g.bound_a + (int64_t)bz * g.bound_a_stride + m0 + t * TM : nullptr;
             f32x4 xo[16];
             if (!g.init_zero) {
 #pragma unroll
@@ -835,7 +851,7 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const float* Sr = S + (kh + 8 * i) * TN + cq;
-                const float ia = HALF ? 1.0f / sca[kh + 8 * i] : 1.0f;
+                const float ia = HALF ? 1.0f / pow2_scale(sca[kh + 8 * i]) : 1.0f;
                 f32x4 o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = xo[i][e] + (ib[e] * ia) * Sr[32 * e];
@@ -1059,7 +1075,8 @@ bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t
     if (b) {
         const GemmArgs &x = a.g, &y = b->g;
         if (x.At != y.At || x.lda != y.lda || x.as != y.as || x.m0 != y.m0 || x.k0 != y.k0) return false;
-        if (x.scale != y.scale || x.scale_stride != y.scale_stride) return false;
+        if (x.bound_a != y.bound_a || x.bound_a_stride != y.bound_a_stride) return false;
+        if ((x.bound_b != nullptr) != (y.bound_b != nullptr)) return false;
         if (b->g.xcd_map && a.n_wg % 8 != 0) return false;
         if (y.k1 > k1) k1 = y.k1;
     }
@@ -1078,7 +1095,7 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
     sp.pair.second = b ? b->g : a.g;
     sp.pair.first_wgs = (int)a.n_wg;
     sp.Ap = static_cast<const u32x4*>(ws);
-    const bool half = a.g.scale != nullptr;                               // fp16 pieces, three products
+    const bool half = a.g.bound_a != nullptr && a.g.bound_b != nullptr;                               // fp16 pieces, three products
     const int products = half ? 3 : a.g.products;
     const bool two = products == 1 || products == 3 || products == 4;     // two-piece layout
     const int np = two ? 2 : 3;
@@ -1091,8 +1108,8 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
         u32x4* dst = static_cast<u32x4*>(ws) + (int64_t)mt * sp.apt;
         if (half)
             split_a_panel_kernel<2, true><<<pgrid, pblock, 0, st>>>(
-                a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, a.g.scale,
-                a.g.scale_stride);
+                a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, a.g.bound_a,
+                a.g.bound_a_stride);
         else if (two)
             split_a_panel_kernel<2, false><<<pgrid, pblock, 0, st>>>(
                 a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, nullptr, 0);

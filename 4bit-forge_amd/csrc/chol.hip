@@ -43,22 +43,17 @@ __global__ void add_damp_kernel(float* __restrict__ H, const float* __restrict__
     if (i < C) H[b * C * C + i * C + i] += damp[b];
 }
 
-// Power-of-two scales for the fp16-piece products of the factorisation, one per column: every
-// entry of the factor obeys |L2[k][j]| <= sqrt(A[j][j]) (column j of A = L2^T L2 sums its
-// squares), so scale[j] = 2^(14 - ceil(log2 sqrt(A[j][j]))) keeps scale[j] * |L2[.][j]| <= 2^14
-// (fp16 overflows at 2^16) whatever the spread of the diagonal (outlier channels).
-__global__ __launch_bounds__(256) void factor_scale_kernel(const float* __restrict__ H, int64_t C,
-                                                           float* __restrict__ scale) {
+// Bounds for the fp16-piece products of the factorisation, one per column: every entry of the
+// factor obeys |L2[k][j]| <= sqrt(A[j][j]) (column j of A = L2^T L2 sums its squares), whatever
+// the spread of the diagonal (outlier channels).  The products scale each column by the largest
+// power of two that keeps its bound at or below 2^14.
+__global__ __launch_bounds__(256) void factor_bound_kernel(const float* __restrict__ H, int64_t C,
+                                                           float* __restrict__ bound) {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= C) return;
     const float d = H[(int64_t)blockIdx.y * C * C + j * C + j];
-    float sc = 1.0f;
-    if (d > 0.0f && d < 3.0e38f) {                // (NaN fails both tests: such a matrix fails anyway)
-        int e;
-        (void)frexpf(sqrtf(d), &e);               // sqrt(d) = f * 2^e, f in [0.5, 1)
-        sc = ldexpf(1.0f, 14 - e);
-    }
-    scale[(int64_t)blockIdx.y * C + j] = sc;
+    // (NaN fails both tests: such a matrix fails anyway); 1.0001: sqrtf rounds to nearest
+    bound[(int64_t)blockIdx.y * C + j] = (d > 0.0f && d < 3.0e38f) ? 1.0001f * sqrtf(d) : 1.0f;
 }
 
 // 1b for one diagonal block of every matrix in the batch: P = D^T D (D lower triangular,
@@ -391,7 +386,7 @@ extern "C" int64_t forge_chol_workspace_bytes(int64_t batch, int64_t C) {
     // inverse diagonal blocks, then the split A panels of the trailing updates (two block rows
     // per product on the factor-only route)
     return batch * nblk * NB * NB * (int64_t)sizeof(float) + 2 * forge::split_gemm_workspace_bytes(batch, C) +
-           (batch * C * (int64_t)sizeof(float) + 255) / 256 * 256;   // + one scale per column
+           (batch * C * (int64_t)sizeof(float) + 255) / 256 * 256;   // + one bound per column
 }
 
 namespace {
@@ -405,7 +400,7 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
     const int64_t dinv_bytes = batch * nblk * NB * NB * (int64_t)sizeof(float);
     void* split_ws = (char*)ws + dinv_bytes;
     const int64_t split_ws_bytes = 2 * forge::split_gemm_workspace_bytes(batch, C);
-    float* scale = (float*)((char*)ws + dinv_bytes + split_ws_bytes);   // one per column and matrix
+    float* bound = (float*)((char*)ws + dinv_bytes + split_ws_bytes);   // one per column and matrix
     // Factor only (no triangular inverse follows): every operand of the trailing updates is a
     // finished row of the factor, whose entries are bounded by the diagonal of the matrix, so
     // the products can be formed from two fp16 halves (three products) instead of three bf16
@@ -426,8 +421,8 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
     }
 
     if (halves) {
-        factor_scale_kernel<<<dim3((unsigned)forge::ceil_div(C, 256), (unsigned)batch), dim3(256), 0, st>>>(
-            H, C, scale);
+        factor_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 256), (unsigned)batch), dim3(256), 0, st>>>(
+            H, C, bound);
         FORGE_LAUNCH_CHECK();
     }
     // 1a (+ 2a) for block rows [a_lo, a]: P[rows, 0..a] -= sum_{k > a} L2[k, rows]^T L2[k, 0..a].
@@ -442,7 +437,7 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
         g1a.xs = g1a.as = g1a.bs = C * C;
         g1a.m0 = m0; g1a.m1 = m1; g1a.n0 = 0; g1a.n1 = m1; g1a.k0 = m1; g1a.k1 = (int)C;
         g1a.negate_a = true; g1a.blocked_sum = true;
-        if (halves) { g1a.scale = scale; g1a.scale_stride = C; }
+        if (halves) { g1a.bound_a = g1a.bound_b = bound; g1a.bound_a_stride = g1a.bound_b_stride = C; }
         if (!factor_only) {
             g2a.X = U; g2a.At = H; g2a.Bm = U; g2a.ldx = g2a.lda = g2a.ldb = C;
             g2a.xs = g2a.as = g2a.bs = C * C;

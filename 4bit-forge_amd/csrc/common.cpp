@@ -125,7 +125,7 @@ std::atomic<int64_t> g_options[OPT_COUNT];
 
 bool valid_option(int o, int64_t v) {
     if (v < kOptions[o].lo || v > kOptions[o].hi) return false;
-    return o != OPT_SWEEP_PRODUCTS || v == 0 || v == 1 || v == 3 || v == 4 || v == 6;
+    return o != OPT_SWEEP_PRODUCTS || v == 0 || v == 1 || v == 2 || v == 3 || v == 4 || v == 6;
 }
 
 // Runs when the library is loaded: the environment is looked at here and nowhere else.

@@ -42,6 +42,7 @@ struct SweepArgs {
     uint32_t* M;           // [ceil(C/32),R] per matrix (sparse only)
     const float* uinv;     // [C] per matrix (sparse only)
     const float* W0;       // [C,R] per matrix: the untouched weights (displacement form only)
+    float* dbound;         // [R] per matrix or null: running max |d| of each row (displacement form)
     int64_t C, R, G;
     int64_t c0;            // first column of this block
     int bw;                // columns in this block (<= BW)
@@ -125,6 +126,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     const int bw = a.bw;
     const int nsub = (bw + SB - 1) / SB;
     const float maxq = (float)a.maxq;
+    float dmax = 0.0f;     // largest |d| this lane hands on in this block
 
     float x[BW];
 #pragma unroll
@@ -223,6 +225,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                 e = keep ? e : (DISP ? err[t] : x[t]);
             }
             err[t] = e;
+            if constexpr (DISP) dmax = fmaxf(dmax, fabsf(e));
             q[c * R] = (uint8_t)qf;
             if constexpr (ERR_IN_A) {
                 A[c * R] = e;
@@ -342,6 +345,41 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
 #pragma unroll
         for (int i = 0; i + SB < BW; ++i) x[i] = x[i + SB];
     }
+    if constexpr (DISP) {
+        // one lane per row: no other lane touches this entry (the first block starts it)
+        if (a.dbound) {
+            float* p = a.dbound + b * R + r;
+            *p = a.c0 == 0 ? dmax : fmaxf(*p, dmax);
+        }
+    }
+}
+
+// bound[m] = max_{t < m} |V[t, m]| for every column of the unit upper matrix V (the strict upper
+// triangle is all that the block updates read).  One workgroup per (128 columns, matrix).
+__global__ __launch_bounds__(256) void upper_column_bound_kernel(const float* __restrict__ V, int64_t C,
+                                                                 float* __restrict__ bound) {
+    __shared__ float red[8][128];
+    const int64_t b = blockIdx.y, m0 = (int64_t)blockIdx.x * 128;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const float* __restrict__ Vb = V + b * C * C;
+    float mx[4] = {0.f, 0.f, 0.f, 0.f};
+    const int64_t rows = (m0 + 128) < C ? (m0 + 128) : C;
+    for (int64_t t = ty; t < rows; t += 8) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int64_t m = m0 + 4 * tx + e;
+            if (m < C && t < m) mx[e] = fmaxf(mx[e], fabsf(Vb[t * C + m]));
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[ty][4 * tx + e] = mx[e];
+    __syncthreads();
+    if (threadIdx.x < 128) {
+        float v = red[0][threadIdx.x];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) v = fmaxf(v, red[i][threadIdx.x]);
+        if (m0 + threadIdx.x < C) bound[b * C + m0 + threadIdx.x] = v;
+    }
 }
 
 // U[i, :] *= 1/U[i,i]; uinv[i] = 1/U[i,i]   (solver_sparsegptq14.cu:153-155)
@@ -456,12 +494,30 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
     const int64_t forced = forge::option(forge::OPT_SWEEP_SCHEDULE);
     if (forced == 1) right_looking = false;
     if (forced == 2) right_looking = true;
-    // Piece products per fp32 product in the direct route's block updates.  By default three
-    // (two rounded pieces per operand) from 4096 columns on, where the codes' own sensitivity to
-    // fp32 rounding is an order of magnitude above what the shorter sum adds and where the
-    // updates are most of the sweep's time; six (fp32-grade) below.
+    // The direct route's block updates on the 16-bit matrix pipe, three products per fp32
+    // product.  Below 4096 columns two fp16 halves per operand, fp32-grade: the columns of V are
+    // scaled from their largest entry above the diagonal, the rows of displacements from a
+    // running maximum that the block kernel keeps.  From 4096 columns on two bf16 pieces, each
+    // rounded to nearest (~2^-17): there the codes' own sensitivity to fp32 rounding is an order
+    // of magnitude above what the shorter pieces add, the updates are most of the sweep's time,
+    // and under the power limit the bf16 instruction runs ~5 % faster than the fp16 one.  The
+    // option sweep_update_products overrides (2: fp16 halves; bf16 pieces: 6 three truncated
+    // pieces, fp32-grade; 3 / 4 two rounded pieces; 1 plain bf16).
     int products = (int)forge::option(forge::OPT_SWEEP_PRODUCTS);
-    if (products == 0) products = C >= 4096 ? 3 : 6;
+    if (products == 0) products = C >= 4096 ? 3 : 2;
+    const bool halves = ws && W0 && products == 2 && !right_looking && C > forge::kBW;
+    const int64_t split_bytes = C > forge::kBW ? 2 * forge::split_gemm_workspace_bytes(batch, C - forge::kBW) : 0;
+    float* vbound = nullptr;
+    float* dbound = nullptr;
+    if (halves) {
+        vbound = (float*)((char*)ws + split_bytes);
+        dbound = (float*)((char*)ws + split_bytes + (batch * C * 4 + 255) / 256 * 256);
+    }
+    if (halves) {
+        upper_column_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 128), (unsigned)batch), dim3(256), 0, st>>>(
+            U, C, vbound);
+        FORGE_LAUNCH_CHECK();
+    }
     for (int64_t start = 0; start < C; start += forge::kBW) {
         const int bw = (int)((C - start) < forge::kBW ? (C - start) : forge::kBW);
         forge::GemmArgs g{};
@@ -472,8 +528,8 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         if (right_looking) {
             // nothing to do here: the earlier blocks have already been pushed into this one
         } else if (ws) {
-            // sums of 128 products each from bf16 pieces of the operands on the bf16 matrix pipe
-            // where the block is a full tile (fp32 matrix pipe otherwise).  That product is
+            // sums from 16-bit pieces of the operands on the fp16 / bf16 matrix pipe where the
+            // block is a full tile (fp32 matrix pipe otherwise).  That product is
             // bound by reading the displacement rows of all earlier columns from HBM, so full
             // blocks are brought up to date two at a time: every row read then serves 256
             // columns (the second block's reading comes from L2), and the odd block only lacks
@@ -482,9 +538,13 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
             const bool odd = pairs && ((start / forge::kBW) & 1) != 0;
             if (!odd) {
                 g.blocked_sum = true;
-                g.products = products;
+                g.products = products == 2 ? 6 : products;
+                if (halves) {
+                    g.bound_a = vbound; g.bound_a_stride = C;
+                    g.bound_b = dbound; g.bound_b_stride = R;
+                }
                 if (pairs && start + 2 * forge::kBW <= C) g.m1 = (int)(start + 2 * forge::kBW);
-                if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, ws_bytes)) return e;
+                if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, split_bytes)) return e;
                 g.m1 = (int)(start + bw);
             } else {
                 g.k0 = (int)(start - forge::kBW);
@@ -497,6 +557,7 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
         a.W0 = W0;
+        a.dbound = halves ? dbound : nullptr;
         a.maxq = (1 << bits) - 1;
         int e = sparse14 ? (W0 ? launch_block<true, false, true>(a, batch, st)
                                : launch_block<true, false>(a, batch, st))
@@ -520,9 +581,12 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
                          bits, sparse14, nullptr, 0, stream);
 }
 
-extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C) {
-    if (batch <= 0 || C <= forge::kBW) return 0;
-    return 2 * forge::split_gemm_workspace_bytes(batch, C - forge::kBW);   // two column blocks per product
+extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R) {
+    if (batch <= 0 || C <= forge::kBW || R <= 0) return 0;
+    // the split A panels of two column blocks per product, one bound per column of V and one
+    // per row of displacements
+    return 2 * forge::split_gemm_workspace_bytes(batch, C - forge::kBW) +
+           (batch * C * 4 + 255) / 256 * 256 + (batch * R * 4 + 255) / 256 * 256;
 }
 
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
@@ -533,9 +597,9 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
                                                int bits, int sparse14, void* ws, int64_t ws_bytes,
                                                forge_stream_t stream) {
     FORGE_REQUIRE(W0 || batch == 0, "null pointer");
-    FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C),
+    FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C, R),
                   "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
-                  (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C));
+                  (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C, R));
     return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, M, mdiag, batch, C, R, G, bits,
                          sparse14, ws, ws_bytes, stream);
 }

@@ -51,7 +51,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
                                       vp], i32),
         "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                              i32, i32, vp, i64, vp], i32),
-        "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64], i64),
+        "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
@@ -305,7 +305,7 @@ class _HipKernels:
             M = torch.empty((B, (C + 31) // 32, R), dtype=torch.uint32, device=X.device)
             assert mdiag is not None and tuple(mdiag.shape) == (B, C) and mdiag.is_contiguous()
             assert mdiag.dtype == torch.float32
-        nbytes = 0 if exact_chain else int(self._lib.forge_gptq_sweep_direct_workspace_bytes(B, C))
+        nbytes = 0 if exact_chain else int(self._lib.forge_gptq_sweep_direct_workspace_bytes(B, C, R))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_gptq_sweep_direct_batched(

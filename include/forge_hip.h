@@ -55,14 +55,17 @@ int forge_kernel_timing_get(int index, char* name, int name_cap, int64_t* launch
  *                           1: left-looking, 2: right-looking -- see forge_gptq_sweep_batched
  *   "fp32_blocked_sum"      FORGE_FP32_BLOCKED_SUM=1          1: the factorisation's and the direct
  *                           sweep's blocked sums stay on the fp32 matrix instruction
- *   "sweep_update_products" FORGE_SWEEP_UPDATE_PRODUCTS=n     bf16 piece products per fp32 product in
- *                           the block updates of forge_gptq_sweep_direct_batched: 3 (two pieces
- *                           per operand, each rounded to nearest, products (2,1) (1,2) (1,1),
- *                           within ~2^-17 of the fp32 product), 4 (adds (2,2)), 6 (three
- *                           truncated pieces, every product of weight >= 2^-16: fp32-grade), 1
- *                           (operands rounded to bf16; for measurements: it moves 2-16 % of
- *                           the codes) or 0 (default): 3 from C = 4096 on, 6 below; the
- *                           factorisation always uses 6
+ *   "sweep_update_products" FORGE_SWEEP_UPDATE_PRODUCTS=n     how the block updates of
+ *                           forge_gptq_sweep_direct_batched form an fp32 product on the 16-bit
+ *                           matrix pipe.  2: two fp16 halves per operand, three products,
+ *                           fp32-grade (columns of V scaled by powers of two from their largest
+ *                           entry, rows of displacements from a running maximum).  bf16 piece
+ *                           products: 6 (three truncated pieces, every product of weight
+ *                           >= 2^-16: fp32-grade), 3 (two pieces per operand, each rounded to
+ *                           nearest, products (2,1) (1,2) (1,1), within ~2^-17 of the fp32
+ *                           product), 4 (adds (2,2)), 1 (operands rounded to bf16; for
+ *                           measurements: it moves 2-16 % of the codes).  0 (default): 3 from
+ *                           C = 4096 on, 2 below
  *   "factor_pieces"         FORGE_FACTOR_PIECES=1             0 (default): where only the factor of H is
  *                           computed (forge_chol_reverse_lower_batched, C a multiple of 128) the
  *                           trailing updates take two fp16 halves of every operand, each column
@@ -154,17 +157,17 @@ int forge_gptq_sweep_batched(float* X, const float* U, const float* scalesT,
  * ws == NULL: the update of a column block by all earlier columns is one fp32 fused
  * multiply-add per earlier column, in ascending order (the chain of solver.cu:91-94 carried
  * across blocks), reproducible bit for bit on a CPU.  With a workspace of
- * forge_gptq_sweep_direct_workspace_bytes(batch, C) bytes that update is summed in blocks of
- * 128 columns from bf16 pieces of the fp32 operands on the bf16 matrix pipe wherever a block
- * is a full 128 x 128 tile and the left-looking schedule applies (see "sweep_update_products"
- * under forge_set_option: different rounding than the chain, faster). */
+ * forge_gptq_sweep_direct_workspace_bytes(batch, C, R) bytes that update is summed from
+ * 16-bit pieces of the fp32 operands on the fp16 / bf16 matrix pipe wherever a block is a full
+ * 128 x 128 tile and the left-looking schedule applies (see "sweep_update_products" under
+ * forge_set_option: different rounding than the chain, faster). */
 int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                     const float* scalesT, const float* qzerosT,
                                     const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
                                     const float* mdiag, int64_t batch, int64_t C, int64_t R,
                                     int64_t G, int bits, int sparse14, void* ws,
                                     int64_t ws_bytes, forge_stream_t stream);
-int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C);
+int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R);
 
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private

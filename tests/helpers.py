@@ -50,8 +50,8 @@ class Float64StagesGPTQ(oracle.GPTQ):
     arithmetic as the oracle's own; everything else (activation order from the fp32 diagonal,
     damping, grid search, the in-block kernel) is the oracle's code unchanged.
 
-    flips(oracle, this) is the FLOOR the end-to-end tests use: how far the reference's codes
-    move when only the rounding inside its library calls changes."""
+    One of the realisations that reference_floor compares: how far the reference's codes move
+    when only the rounding inside its library calls changes."""
 
     def __init__(self, *a, **kw):
         super().__init__(*a, **kw)
@@ -82,9 +82,11 @@ def reference_floor(W, batches, qo, **kw):
     """(floor, out64).  Two other valid realisations of the reference on the same inputs:
     (a) Float64StagesGPTQ (out64 = what it returns), (b) the oracle itself with every
     calibration batch fed in three pieces, i.e. the running-mean Hessian of gptq.py:73-79
-    summed in another order by the same fp32 SGEMM.  floor = the larger of the two shares of
-    the oracle's codes `qo` that differ: the codes' own sensitivity is heavy-tailed (one early
-    flip cascades along its row), and a single alternative underestimates it as often as not."""
+    summed in another order by the same fp32 SGEMM.  floor = the largest share of codes that
+    differ between any two of the three (the oracle's codes `qo`, a, b): the codes' own
+    sensitivity is heavy-tailed (one early flip cascades along its row), a single pair
+    underestimates it as often as not, and two realisations that each sit f away from the
+    exact-arithmetic result sit up to 2 f away from each other."""
     t = Float64StagesGPTQ(linear(W), trail_mode=oracle.TRAIL_GEMM, **kw)
     for b in batches:
         t.update(b)
@@ -95,5 +97,6 @@ def reference_floor(W, batches, qo, **kw):
         for b in batches:
             for part in torch.chunk(b, 3):
                 c.update(part)
-        floor = max(floor, flip_rate(qo, c.quantize()[0]))
+        qc = c.quantize()[0]
+        floor = max(floor, flip_rate(qo, qc), flip_rate(out[0], qc))
     return floor, out

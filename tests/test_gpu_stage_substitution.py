@@ -106,11 +106,12 @@ def test_direct_route_sweep_on_the_oracles_hessian(hip, name):
     the GPU (factor of H itself), the matrix V is copied back, and the displacement-form
     sweep runs on both sides with that V: the fp32-chain form equals its CPU checker bit for
     bit.  The block updates the library ships for batches of experts (left-looking schedule,
-    sums of 128 products from bf16 pieces) are a different fp32-grade summation, not a chain:
-    their codes are compared with the chain's for 6, 3 (the default) and 1 piece products per
-    fp32 product.  6 and 3 must stay within max(0.1 %, a quarter of the floor) -- the floor
-    being what the reference's own codes move by between two fp32 realisations of its
-    library stages; plain bf16 operands (1 product) are reported: they move 2-16 %."""
+    sums on the 16-bit matrix pipe) are a different fp32-grade summation, not a chain: their
+    codes are compared with the chain's for two fp16 halves per operand (2) and
+    for 6, 3 and 1 bf16 piece products per fp32 product.  All but the last must stay within
+    max(0.1 %, a quarter of the floor) -- the floor being what the reference's own codes move
+    by between two fp32 realisations of its library stages; plain bf16 operands (1 product)
+    are reported: they move 2-16 %."""
     W, X, kw = _case(name)
     R, C = W.shape
     sparse = kw.get("algorithm") == "sparsegptq"
@@ -144,16 +145,17 @@ def test_direct_route_sweep_on_the_oracles_hessian(hip, name):
     bound = max(1e-3, 0.25 * floor)
     hip.set_option("sweep_schedule", 1)               # what a batch of experts takes
     try:
-        for products in (6, 3, 1):
+        for products in (2, 6, 3, 1):
             old = hip.set_option("sweep_update_products", products)
             try:
                 q_s, M_s = gpu()
             finally:
                 hip.set_option("sweep_update_products", old)
             flips = (q_x != q_s).float().mean().item()
-            print(f"{name}: block updates from {products} piece product(s) vs fp32 chain: flips "
+            what = "fp16 halves" if products == 2 else f"{products} bf16 piece product(s)"
+            print(f"{name}: block updates from {what} vs fp32 chain: flips "
                   f"{flips:.2e} (floor {floor:.2e})")
-            if products > 1:
+            if products != 1:
                 assert flips <= bound, (products, flips, floor)
                 if sparse:
                     assert (M_x.view(torch.int32) != M_s.view(torch.int32)).float().mean().item() <= bound
