@@ -248,6 +248,25 @@ def hessian_buckets(C=7168, E=64):
                      "the kernels compute; bytes 2nC + 4C^2 per expert")
 
 
+def mfma_ceiling():
+    """What the matrix pipe itself sustains on this device (forge_mfma_rate_probe: back-to-back
+    32x32x16 matrix instructions from registers, nothing else): with operands of ones, and with
+    pseudo-random operands, whose toggling bits make the device's power management slow the
+    pipe.  The random-operand rate is the ceiling of any GEMM on real data."""
+    from forge.backend.hip import kernels
+    out = {}
+    for name, f16, rnd in (("bf16_ones", False, False), ("bf16_random", False, True),
+                           ("f16_ones", True, False), ("f16_random", True, True)):
+        kernels.mfma_rate_probe(f16, rnd)                                          # warm-up
+        stats = timing_pass(lambda: [kernels.mfma_rate_probe(f16, rnd) for _ in range(3)])
+        s = stats["mfma_rate_" + name]
+        out[name] = dict(tflops=round(s["work"] / s["ms"] / 1e9, 1),
+                         frac_of_published_peak=round(s["work"] / s["ms"] / 1e9 / PEAK["mfma_bf16"], 4))
+    out["note"] = ("executed TFLOP/s of v_mfma_f32_32x32x16 issued back to back from registers on "
+                   "every CU, ~7 ms per launch; published peak 2500")
+    return out
+
+
 def hbm_kernels(wl):
     """min/max grid, int4 pack and fp8 block dequant on the chunk's gate_proj stack (64 x 2048 x
     7168): achieved GB/s of the algorithmic bytes against 8 TB/s."""
@@ -488,6 +507,7 @@ def main():
             value=round(a.steps * chunk / dt, 3), unit="experts/s")
         out["hessian_buckets"] = hessian_buckets(cfg["hidden"], min(chunk, 64))
         out["hbm_kernels"] = hbm_kernels(wl)
+        out["mfma_ceiling"] = mfma_ceiling()
         out["other_configs"] = other_configs()
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, cfg)

@@ -79,24 +79,32 @@ class Float64StagesGPTQ(oracle.GPTQ):
 
 
 def reference_floor(W, batches, qo, **kw):
-    """(floor, out64).  Two other valid realisations of the reference on the same inputs:
-    (a) Float64StagesGPTQ (out64 = what it returns), (b) the oracle itself with every
+    """(floor, out64).  Other valid realisations of the reference on the same inputs:
+    (a) Float64StagesGPTQ (out64 = what it returns); (b) the oracle itself with every
     calibration batch fed in three pieces, i.e. the running-mean Hessian of gptq.py:73-79
-    summed in another order by the same fp32 SGEMM.  floor = the largest share of codes that
-    differ between any two of the three (the oracle's codes `qo`, a, b): the codes' own
-    sensitivity is heavy-tailed (one early flip cascades along its row), a single pair
-    underestimates it as often as not, and two realisations that each sit f away from the
-    exact-arithmetic result sit up to 2 f away from each other."""
+    summed in another order by the same fp32 SGEMM; and, for matrices of up to 2048 x 2048
+    (where a run takes seconds), (c) two pieces with the trailing update as one BLAS SGEMM per
+    block (dense solve; summed from zero otherwise) and (d) five pieces with the trailing update summed from zero.  floor = the largest
+    share of codes that differ between any two of them and the oracle's codes `qo`: the codes'
+    own sensitivity is heavy-tailed (one early flip cascades along its row), a single pair
+    underestimates it as often as not (the same pair measured on two hosts, whose BLAS sums in
+    different orders, gave 8.1e-4 and 1.1e-3), and two realisations that each sit f away from
+    the exact-arithmetic result sit up to 2 f away from each other."""
     t = Float64StagesGPTQ(linear(W), trail_mode=oracle.TRAIL_GEMM, **kw)
     for b in batches:
         t.update(b)
     out = t.quantize()
-    floor = flip_rate(qo, out[0])
+    codes = [qo, out[0]]
     if sum(int(b.shape[0]) for b in batches) >= 3:
-        c = oracle.GPTQ(linear(W), **kw)
-        for b in batches:
-            for part in torch.chunk(b, 3):
-                c.update(part)
-        qc = c.quantize()[0]
-        floor = max(floor, flip_rate(qo, qc), flip_rate(out[0], qc))
+        variants = [(3, None)]
+        if W.numel() <= 2048 * 2048:
+            blas = oracle.TRAIL_BLAS if kw.get("algorithm", "gptq") == "gptq" else oracle.TRAIL_GEMM
+            variants += [(2, blas), (5, oracle.TRAIL_GEMM)]
+        for pieces, mode in variants:
+            c = oracle.GPTQ(linear(W), **(dict(kw, trail_mode=mode) if mode is not None else kw))
+            for b in batches:
+                for part in torch.chunk(b, pieces):
+                    c.update(part)
+            codes.append(c.quantize()[0])
+    floor = max(flip_rate(a, b) for i, a in enumerate(codes) for b in codes[i + 1:])
     return floor, out

@@ -6,17 +6,14 @@ bit-exact at the benchmark shapes (test_gpu_stage_substitution).  End to end the
 and the factorisation are fp32 library calls in the reference (an SGEMM and LAPACK's
 potrf/potri/potrf, gptq.py:79,160-164) whose summation order it does not fix, and GPTQ's
 rounding decisions amplify their last bits: a flipped code changes the error fed to every
-later column of its row.  FLOOR = the largest share of codes that differ between any two of
-three valid realisations of the reference: the oracle, the same with those two library stages
-computed in float64 and rounded to fp32 once and the trailing update's SGEMM
-(solver.cu:146-150) summing in another valid order (helpers.Float64StagesGPTQ), and the oracle
-with its Hessian accumulated in three calls instead of one (helpers.reference_floor).
-The GPU result must stay within max(1e-3, 2 * FLOOR) of the oracle (two results that each sit
-f away from the exact-arithmetic codes sit up to 2 f apart, and FLOOR is itself such a pair
-distance: every variant of the GPU path -- fp32 sums everywhere, either factor route, any
-piece count -- lands between 1.0 and 1.6 FLOOR on the matrices tried), at benchmark sizes also
-within 1.5 * FLOOR of the float64-stage result, and its layer output error ||WX - QX||^2
-within 1 % of the oracle's.
+later column of its row.  FLOOR = the largest share of codes that differ between any two
+valid realisations of the reference out of three to five (helpers.reference_floor): the oracle,
+the same with those two library stages computed in float64 and rounded to fp32 once
+(helpers.Float64StagesGPTQ), and the oracle with its Hessian accumulated in two, three or five
+calls instead of one and the trailing update's SGEMM (solver.cu:146-150) summing in another
+valid order.  The GPU result must stay within max(1e-3, 1.5 * FLOOR) of the oracle, at benchmark
+sizes also of the float64-stage result, and its layer output error ||WX - QX||^2 within 1 % of
+the oracle's.
 """
 import numpy as np
 import pytest
@@ -29,8 +26,7 @@ from helpers import linear, flip_rate, expand_meta, reference_floor
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-FLOORS = 2.0        # GPU vs oracle
-FLOORS64 = 1.5      # GPU vs the float64-stage realisation (benchmark sizes)
+FLOORS = 1.5
 
 
 def _isolated_ties(qo, qg, order):
@@ -68,7 +64,7 @@ def _codes_at_floor(tag, qo, qg, W, batches, kw, both=False, order=None):
         return flips, floor, out64
     assert flips <= bound, (tag, flips, floor)
     if both:
-        assert to64 <= max(1e-3, FLOORS64 * floor), (tag, to64, floor)
+        assert to64 <= bound, (tag, to64, floor)
     return flips, floor, out64
 
 
