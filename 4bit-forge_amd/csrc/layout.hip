@@ -13,13 +13,20 @@ __device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
     return __uint_as_float(static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(p)) << 16);
 }
 
+__device__ __forceinline__ void st_from_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st_from_f32(__hip_bfloat16* p, float v) {   // v is a bf16 value
+    *reinterpret_cast<uint16_t*>(p) = (uint16_t)(__float_as_uint(v) >> 16);
+}
+
 // Xout[b][perm_inv[c]][r] = W[b][r][c]  (64x64 tiles through LDS; the W.T[perm] of
 // forge/gptq.py:133 written as a scatter of whole output rows so that both sides coalesce).
+// W0out (may be null): the same matrix once more in the weights' own type, the untouched copy
+// that the displacement-form sweep reads beside the values it updates.
 template <typename T>
 __global__ __launch_bounds__(256) void to_solver_order_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const int64_t* __restrict__ perm_inv,
-    const uint8_t* __restrict__ dead, float* __restrict__ Xout, int64_t R, int64_t C,
-    int64_t ldo, int64_t o_stride) {
+    const uint8_t* __restrict__ dead, float* __restrict__ Xout, T* __restrict__ W0out, int64_t R,
+    int64_t C, int64_t ldo, int64_t o_stride) {
     __shared__ float tile[64][65];
     const int64_t b = blockIdx.z;
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
@@ -34,7 +41,11 @@ __global__ __launch_bounds__(256) void to_solver_order_kernel(
     __syncthreads();
     for (int j = ty; j < 64; j += 4) {
         const int64_t c = c0 + j, r = r0 + tx;
-        if (c < C && r < R) Xout[b * o_stride + perm_inv[b * C + c] * ldo + r] = tile[tx][j];
+        if (c < C && r < R) {
+            const int64_t at = b * o_stride + perm_inv[b * C + c] * ldo + r;
+            Xout[at] = tile[tx][j];
+            if (W0out) st_from_f32(W0out + at, tile[tx][j]);
+        }
     }
 }
 
@@ -65,7 +76,8 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
 __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw,
     const int64_t* __restrict__ perm_inv, const uint8_t* __restrict__ dead,
-    float* __restrict__ Xout, int64_t R, int64_t C, int64_t ldo, int64_t o_stride) {
+    float* __restrict__ Xout, uint16_t* __restrict__ W0out, int64_t R, int64_t C, int64_t ldo,
+    int64_t o_stride) {
     constexpr int TC = 64, TR = 256, PITCH = TR + 4;     // rows stay 8-byte aligned
     __shared__ __attribute__((aligned(8))) uint16_t tile[TC][PITCH];
     const int64_t b = blockIdx.z;
@@ -98,7 +110,9 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
             const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
             const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
                                          __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
-            *reinterpret_cast<float4*>(Xout + b * o_stride + perm_inv[b * C + c0 + c] * ldo + r0 + r4) = o;
+            const int64_t at = b * o_stride + perm_inv[b * C + c0 + c] * ldo + r0 + r4;
+            *reinterpret_cast<float4*>(Xout + at) = o;
+            if (W0out) *reinterpret_cast<uint2*>(W0out + at) = v;
         }
     }
 }
@@ -307,11 +321,11 @@ __global__ __launch_bounds__(256) void pack_int4_fast_kernel(const uint8_t* __re
 
 }  // namespace
 
-extern "C" int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_stride,
-                                                    int64_t ldw, const int64_t* perm_inv,
-                                                    const uint8_t* dead, float* Xout, int64_t ldo,
-                                                    int64_t o_stride, int64_t batch, int64_t R,
-                                                    int64_t C, forge_stream_t stream) {
+extern "C" int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stride,
+                                                 int64_t ldw, const int64_t* perm_inv,
+                                                 const uint8_t* dead, float* Xout, void* W0out,
+                                                 int64_t ldo, int64_t o_stride, int64_t batch,
+                                                 int64_t R, int64_t C, forge_stream_t stream) {
     FORGE_REQUIRE(w_dtype == FORGE_F32 || w_dtype == FORGE_BF16, "w_dtype=%d", w_dtype);
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0 && ldw >= C, "bad shape");
     FORGE_REQUIRE(ldo >= R && o_stride >= (C > 0 ? (C - 1) * ldo + R : 0), "output pitch too small");
@@ -320,25 +334,36 @@ extern "C" int forge_weight_to_solver_order_strided(const void* W, int w_dtype, 
     dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
     FORGE_REQUIRE(grid.y < 65536, "R too large");
     forge::KernelTiming timing("weight_to_solver_order", (hipStream_t)stream,
-                               (double)batch * R * C * (4.0 + (w_dtype == FORGE_F32 ? 4.0 : 2.0)),
+                               (double)batch * R * C * (4.0 + (w_dtype == FORGE_F32 ? 4.0 : 2.0) * (W0out ? 2.0 : 1.0)),
                                forge::WORK_BYTES);
     const bool fast = w_dtype == FORGE_BF16 && (R % 256) == 0 && (C % 64) == 0 && (ldw % 4) == 0 &&
                       (w_stride % 4) == 0 && (reinterpret_cast<uintptr_t>(W) % 8) == 0 &&
                       (reinterpret_cast<uintptr_t>(Xout) % 16) == 0 && (ldo % 4) == 0 &&
-                      (o_stride % 4) == 0 && R / 256 < 65536;
+                      (o_stride % 4) == 0 && R / 256 < 65536 &&
+                      (reinterpret_cast<uintptr_t>(W0out) % 8) == 0;
     if (fast) {
         const dim3 tiles((unsigned)(C / 64), (unsigned)(R / 256), (unsigned)batch);
         to_solver_order_bf16_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(
-            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
+            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, (uint16_t*)W0out, R, C, ldo, o_stride);
     } else if (w_dtype == FORGE_F32) {
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
-            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
+            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, (float*)W0out, R, C, ldo, o_stride);
     } else {
         to_solver_order_kernel<__hip_bfloat16><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
-            (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, R, C, ldo, o_stride);
+            (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, (__hip_bfloat16*)W0out, R, C,
+            ldo, o_stride);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
+}
+
+extern "C" int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_stride,
+                                                    int64_t ldw, const int64_t* perm_inv,
+                                                    const uint8_t* dead, float* Xout, int64_t ldo,
+                                                    int64_t o_stride, int64_t batch, int64_t R,
+                                                    int64_t C, forge_stream_t stream) {
+    return forge_weight_to_solver_order_pair(W, w_dtype, w_stride, ldw, perm_inv, dead, Xout, nullptr,
+                                             ldo, o_stride, batch, R, C, stream);
 }
 
 extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride,

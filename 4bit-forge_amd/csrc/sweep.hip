@@ -41,7 +41,8 @@ struct SweepArgs {
     uint8_t* q;            // [C,R] per matrix
     uint32_t* M;           // [ceil(C/32),R] per matrix (sparse only)
     const float* uinv;     // [C] per matrix (sparse only)
-    const float* W0;       // [C,R] per matrix: the untouched weights (displacement form only)
+    const void* W0;        // [C,R] per matrix: the untouched weights (displacement form only),
+    bool w0_bf16;          // as f32 or, when set, as bf16 (exact for weights that are bf16)
     float* dbound;         // [R] per matrix or null: running max |d| of each row (displacement form)
     int64_t C, R, G;
     int64_t c0;            // first column of this block
@@ -101,7 +102,11 @@ __device__ __forceinline__ float dpp_source(float u) {
 // Values of columns that are NOT yet reached differ between the forms; the 1:4 mask score,
 // which looks three columns ahead, rebuilds the error form's values from the 4x4 diagonal
 // block of V (see select_and_quantize).
-template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false>
+__device__ __forceinline__ float w0_as_f32(const float* p) { return *p; }
+__device__ __forceinline__ float w0_as_f32(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
+
+template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false,
+          typename W0T = float>
 __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
     constexpr int RING = FORGE_SWEEP_RING;   // LDS read-ahead: RING-1 steps of 16 columns
@@ -122,7 +127,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     const float* __restrict__ uinv = SPARSE ? a.uinv + b * C : nullptr;
     uint32_t* __restrict__ Mw = SPARSE ? a.M + b * ((C + 31) / 32) * R + r : nullptr;
     uint8_t* __restrict__ q = a.q + b * C * R + r;
-    const float* __restrict__ W0 = DISP ? a.W0 + b * C * R + r : nullptr;
+    const W0T* __restrict__ W0 = DISP ? static_cast<const W0T*>(a.W0) + b * C * R + r : nullptr;
     const int bw = a.bw;
     const int nsub = (bw + SB - 1) / SB;
     const float maxq = (float)a.maxq;
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
         if constexpr (!TAIL) {
             if constexpr (DISP) {
 #pragma unroll
-                for (int t = 0; t < SB; ++t) err[t] = W0[(cs + t) * R];
+                for (int t = 0; t < SB; ++t) err[t] = w0_as_f32(W0 + (cs + t) * R);
             }
             // fetch the next sub-block's panel (rows cs+32.., columns cs+32..) into registers
             const bool more = sb + 1 < nsub;
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
         } else {
             if constexpr (DISP) {
 #pragma unroll 1
-                for (int t = 0; t < SB; ++t) err[t] = (t < rem) ? W0[(cs + t) * R] : 0.0f;
+                for (int t = 0; t < SB; ++t) err[t] = (t < rem) ? w0_as_f32(W0 + (cs + t) * R) : 0.0f;
             }
 #pragma unroll 1
             for (int t = 0; t < SB; ++t) {
@@ -390,7 +395,7 @@ __global__ void row_normalise_kernel(float* __restrict__ U, float* __restrict__ 
     if (threadIdx.x == 0) uinv[i] = inv;
 }
 
-template <bool SPARSE, bool PER_ELEM, bool DISP = false>
+template <bool SPARSE, bool PER_ELEM, bool DISP = false, typename W0T = float>
 int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
     constexpr bool ERR_IN_A = !PER_ELEM;  // batched form keeps the errors in place
     forge::KernelTiming timing(SPARSE ? "sweep_block_sparse14" : "sweep_block", st,
@@ -401,15 +406,15 @@ int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
                       (reinterpret_cast<uintptr_t>(a.U) % 16) == 0;
     if (fast && a.R % 256 == 0) {
         dim3 grid((unsigned)(a.R / 256), (unsigned)batch);
-        sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false, DISP>
+        sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false, DISP, W0T>
             <<<grid, dim3(256), 0, st>>>(a);
     } else {
         dim3 grid((unsigned)forge::ceil_div(a.R, 64), (unsigned)batch);
         if (fast)
-            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, false, DISP>
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, false, DISP, W0T>
                 <<<grid, dim3(64), 0, st>>>(a);
         else
-            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, true, DISP>
+            sweep_block_kernel<forge_kBW, 64, SPARSE, PER_ELEM, ERR_IN_A, true, DISP, W0T>
                 <<<grid, dim3(64), 0, st>>>(a);
     }
     FORGE_LAUNCH_CHECK();
@@ -473,7 +478,7 @@ extern "C" int forge_sparsegptq14_solver(float* W, float* U, const float* scales
 
 // Left-looking schedule for a batch of equally shaped matrices, errors (or, with W0, the
 // displacements) kept in X.
-static int sweep_batched(float* X, const float* W0, const float* U, const float* scalesT,
+static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U, const float* scalesT,
                          const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                          uint32_t* M, const float* uinv, int64_t batch, int64_t C, int64_t R,
                          int64_t G, int bits, int sparse14, void* ws, int64_t ws_bytes,
@@ -557,12 +562,17 @@ static int sweep_batched(float* X, const float* W0, const float* U, const float*
         a.A = X; a.B = nullptr; a.U = U; a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx;
         a.q = qweight; a.M = M; a.uinv = uinv; a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = bw;
         a.W0 = W0;
+        a.w0_bf16 = w0_bf16;
         a.dbound = halves ? dbound : nullptr;
         a.maxq = (1 << bits) - 1;
-        int e = sparse14 ? (W0 ? launch_block<true, false, true>(a, batch, st)
-                               : launch_block<true, false>(a, batch, st))
-                : W0     ? launch_block<false, false, true>(a, batch, st)
-                         : launch_block<false, false>(a, batch, st);
+        int e;
+        if (!W0) e = sparse14 ? launch_block<true, false>(a, batch, st) : launch_block<false, false>(a, batch, st);
+        else if (w0_bf16)
+            e = sparse14 ? launch_block<true, false, true, uint16_t>(a, batch, st)
+                         : launch_block<false, false, true, uint16_t>(a, batch, st);
+        else
+            e = sparse14 ? launch_block<true, false, true>(a, batch, st)
+                         : launch_block<false, false, true>(a, batch, st);
         if (e) return e;
         if (right_looking && start + bw < C) {
             g.m0 = (int)(start + bw); g.m1 = (int)C; g.k0 = (int)start; g.k1 = (int)(start + bw);
@@ -577,7 +587,7 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
                                         uint8_t* qweight, uint32_t* M, const float* uinv,
                                         int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
                                         int sparse14, forge_stream_t stream) {
-    return sweep_batched(X, nullptr, U, scalesT, qzerosT, g_idx, qweight, M, uinv, batch, C, R, G,
+    return sweep_batched(X, nullptr, false, U, scalesT, qzerosT, g_idx, qweight, M, uinv, batch, C, R, G,
                          bits, sparse14, nullptr, 0, stream);
 }
 
@@ -589,6 +599,22 @@ extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_
            (batch * C * 4 + 255) / 256 * 256 + (batch * R * 4 + 255) / 256 * 256;
 }
 
+extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
+                                                  const float* scalesT, const float* qzerosT,
+                                                  const int32_t* g_idx, uint8_t* qweight,
+                                                  uint32_t* M, const float* mdiag,
+                                                  int64_t batch, int64_t C, int64_t R, int64_t G,
+                                                  int bits, int sparse14, void* ws, int64_t ws_bytes,
+                                                  forge_stream_t stream) {
+    FORGE_REQUIRE(W0 || batch == 0, "null pointer");
+    FORGE_REQUIRE(w0_dtype == FORGE_F32 || w0_dtype == FORGE_BF16, "w0_dtype=%d", w0_dtype);
+    FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C, R),
+                  "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
+                  (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C, R));
+    return sweep_batched(X, W0, w0_dtype == FORGE_BF16, V, scalesT, qzerosT, g_idx, qweight, M, mdiag,
+                         batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
+}
+
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                                const float* scalesT, const float* qzerosT,
                                                const int32_t* g_idx, uint8_t* qweight,
@@ -596,12 +622,8 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
                                                int64_t batch, int64_t C, int64_t R, int64_t G,
                                                int bits, int sparse14, void* ws, int64_t ws_bytes,
                                                forge_stream_t stream) {
-    FORGE_REQUIRE(W0 || batch == 0, "null pointer");
-    FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C, R),
-                  "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
-                  (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C, R));
-    return sweep_batched(X, W0, V, scalesT, qzerosT, g_idx, qweight, M, mdiag, batch, C, R, G, bits,
-                         sparse14, ws, ws_bytes, stream);
+    return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, V, scalesT, qzerosT, g_idx, qweight, M,
+                                              mdiag, batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

@@ -53,6 +53,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
                                       vp], i32),
         "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                              i32, i32, vp, i64, vp], i32),
+        "forge_gptq_sweep_direct_batched_w0": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64,
+                                                i64, i32, i32, vp, i64, vp], i32),
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
@@ -69,6 +71,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_weight_to_solver_order_strided": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, i64, i64,
                                                   vp], i32),
+        "forge_weight_to_solver_order_pair": ([vp, i32, i64, i64, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                               vp], i32),
         "forge_codes_to_layer_order_strided": ([vp, i64, i64, vp, vp, i64, i64, i64, vp], i32),
         "forge_pack_int4": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_fp8_e4m3_block_dequant": ([vp, vp, vp, i32, i64, i64, i64, i64, i64, vp], i32),
@@ -96,6 +100,7 @@ EXPORTED_SYMBOLS = (
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_weight_to_solver_order_strided", "forge_codes_to_layer_order_strided",
+    "forge_weight_to_solver_order_pair", "forge_gptq_sweep_direct_batched_w0",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
     "forge_dequantize_groups", "forge_gather_scaled_rows",
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
@@ -314,7 +319,7 @@ class _HipKernels:
         assert tuple(qzerosT.shape) == (B, G, R) and tuple(g_idx.shape) == (B, C)
         if W0 is None:
             W0 = X.clone()
-        assert W0.is_contiguous() and W0.shape == X.shape and W0.dtype == torch.float32
+        assert W0.is_contiguous() and W0.shape == X.shape and W0.dtype in (torch.float32, torch.bfloat16)
         assert W0.data_ptr() != X.data_ptr() or X.numel() == 0
         q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
         M = None
@@ -325,8 +330,8 @@ class _HipKernels:
         nbytes = 0 if exact_chain else int(self._lib.forge_gptq_sweep_direct_workspace_bytes(B, C, R))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
-            self._check(self._lib.forge_gptq_sweep_direct_batched(
-                _ptr(X), _ptr(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
+            self._check(self._lib.forge_gptq_sweep_direct_batched_w0(
+                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
                 _ptr(M), _ptr(mdiag), B, C, R, G, int(bits), int(bool(sparse14)), _ptr(ws), nbytes,
                 _stream()))
         return (q, M) if sparse14 else q
@@ -450,10 +455,12 @@ class _HipKernels:
                 _stream()))
         return Hp, damp
 
-    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0):
+    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None):
         """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c].
         With ``out`` [B,C,Rtot] (f32, contiguous) the rows land at out[:, :, row0:row0+R]: stacks
-        that share a factor fill one tall matrix without being concatenated first."""
+        that share a factor fill one tall matrix without being concatenated first.  ``out0``
+        (shape of ``out``, dtype of W) receives the same values in W's own type: the untouched
+        copy for gptq_sweep_direct_batched(W0=...)."""
         _need_cuda(W, perm_inv, dead, out)
         B, R, C = W.shape
         assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
@@ -465,10 +472,15 @@ class _HipKernels:
         assert out.is_contiguous() and out.dtype == torch.float32 and out.dim() == 3
         Rtot = out.shape[2]
         assert tuple(out.shape[:2]) == (B, C) and 0 <= row0 and row0 + R <= Rtot
+        p0 = None
+        if out0 is not None:
+            _need_cuda(out0)
+            assert out0.is_contiguous() and out0.dtype == W.dtype and out0.shape == out.shape
+            p0 = ctypes.c_void_p(out0.data_ptr() + out0.element_size() * row0)
         with torch.cuda.device(W.device):
-            self._check(self._lib.forge_weight_to_solver_order_strided(
+            self._check(self._lib.forge_weight_to_solver_order_pair(
                 _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
-                out.data_ptr() + 4 * row0, Rtot, C * Rtot, B, R, C, _stream()))
+                ctypes.c_void_p(out.data_ptr() + 4 * row0), p0, Rtot, C * Rtot, B, R, C, _stream()))
         return out
 
     def codes_to_layer_order(self, q, perm_inv, out=None, row0=0, rows=None):

@@ -233,7 +233,10 @@ class GPTQ(object):
             zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
             q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
             return kernels.codes_to_layer_order(q, perm_r_inv.view(1, C))[0], scales, qzeros
-        X = kernels.weight_to_solver_order(W.view(1, R, C), self.perm_inv.view(1, C))
+        W0 = None
+        if self.factor_route == "direct":
+            W0 = torch.empty((1, C, R), dtype=W.dtype, device=W.device)
+        X = kernels.weight_to_solver_order(W.view(1, R, C), self.perm_inv.view(1, C), out0=W0)
         g_idx = (self.perm // gs).to(torch.int32).view(1, C)
         sT = scales.view(R, G).t().contiguous().view(1, G, R)
         zT = qzeros.view(R, G).t().contiguous().view(1, G, R)
@@ -242,14 +245,14 @@ class GPTQ(object):
         if self.algorithm == "sparsegptq":
             if self.factor_route == "direct":
                 q, M = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits,
-                                                         sparse14=True, mdiag=self._score_weight)
+                                                         W0=W0, sparse14=True, mdiag=self._score_weight)
             else:
                 q, M = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits,
                                                   sparse14=True, uinv=self._score_weight)
             qw = kernels.codes_to_layer_order(q, self.perm_inv.view(1, C))[0]
             return qw, scales, qzeros, M[0]
         if self.factor_route == "direct":
-            q = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
+            q = kernels.gptq_sweep_direct_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits, W0=W0)
         else:
             q = kernels.gptq_sweep_batched(X, U.view(1, C, C), sT, zT, g_idx, self.bits)
         qw = kernels.codes_to_layer_order(q, self.perm_inv.view(1, C))[0]

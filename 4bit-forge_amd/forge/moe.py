@@ -224,25 +224,31 @@ class ExpertGroupGPTQ:
                 del Hp
                 failed.append((e0, info))
                 X = torch.empty((B, C, R), dtype=torch.float32, device=dev)
+                # the displacement form also reads the untouched weights: the layout pass writes
+                # them a second time in their own type instead of X being copied afterwards
+                W0 = None
+                if direct and len({self.W[i].dtype for i in job}) == 1:
+                    W0 = torch.empty((B, C, R), dtype=self.W[job[0]].dtype, device=dev)
                 r0 = 0
                 for i in job:
-                    kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0)
+                    kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0,
+                                                   out0=W0)
                     r0 += sizes[i]
                 main.wait_stream(search)
                 for t in (scales, qzeros, sT, zT):
                     t.record_stream(main)
                 M = None
                 if direct and sparse:
-                    q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits,
+                    q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0,
                                                              sparse14=True, mdiag=uinv)
                 elif sparse:
                     q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
                                                       uinv=uinv)
                 elif direct:
-                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits)
+                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0)
                 else:
                     q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
-                del X, U
+                del X, U, W0
                 r0 = 0
                 for i in job:
                     Ri = sizes[i]

@@ -180,6 +180,15 @@ int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
                                     int64_t G, int bits, int sparse14, void* ws,
                                     int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R);
+/* The same with the untouched weights W0 in f32 (w0_dtype = FORGE_F32) or in bf16 (FORGE_BF16:
+ * exact when the layer's weights are bf16, and half the bytes to read);
+ * forge_weight_to_solver_order_pair writes X and W0 in one pass. */
+int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
+                                       const float* scalesT, const float* qzerosT,
+                                       const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
+                                       const float* mdiag, int64_t batch, int64_t C, int64_t R,
+                                       int64_t G, int bits, int sparse14, void* ws,
+                                       int64_t ws_bytes, forge_stream_t stream);
 
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private
@@ -309,6 +318,14 @@ int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_s
                                          const int64_t* perm_inv, const uint8_t* dead, float* Xout,
                                          int64_t ldo, int64_t o_stride, int64_t batch, int64_t R,
                                          int64_t C, forge_stream_t stream);
+/* _pair: additionally writes W0out (may be NULL), the same matrix in the weights' own type
+ * (w_dtype) with the same pitches in elements: the untouched copy that
+ * forge_gptq_sweep_direct_batched_w0 reads beside the values it updates, produced in the pass
+ * that lays X out instead of by a copy of X afterwards. */
+int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                                      const int64_t* perm_inv, const uint8_t* dead, float* Xout,
+                                      void* W0out, int64_t ldo, int64_t o_stride, int64_t batch,
+                                      int64_t R, int64_t C, forge_stream_t stream);
 int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
                                        const int64_t* perm_inv, uint8_t* qout, int64_t batch,
                                        int64_t R, int64_t C, forge_stream_t stream);

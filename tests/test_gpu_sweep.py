@@ -115,6 +115,48 @@ def test_direct_sweep_bit_exact(hip, C, R):
     assert (X2 - X).abs().max().item() <= 0.05 * X.abs().max().item()
 
 
+@pytest.mark.parametrize("C,R,dtype", [(512, 256, torch.bfloat16), (384, 192, torch.bfloat16),
+                                       (200, 70, torch.bfloat16), (256, 128, torch.float32)])
+def test_direct_sweep_untouched_weights_from_the_layout_pass(hip, C, R, dtype):
+    """The layout pass writes the solver-order weights twice, as f32 (the values the sweep
+    updates) and in the weights' own type (the untouched copy the displacement form reads):
+    both equal the plain pass's output, also for a band of a taller matrix, and the sweep
+    returns the same codes and displacements whether that copy is bf16, f32 or made inside the
+    wrapper.  Fast (whole 256-row tiles) and general layout kernels."""
+    B, gs = 2, 128
+    G = (C + gs - 1) // gs
+    g0 = torch.Generator().manual_seed(C + R)
+    W = (0.02 * torch.randn(B, R, C, generator=g0)).to(dtype)
+    perm = torch.stack([torch.randperm(C, generator=g0) for _ in range(B)])
+    perm_inv = torch.argsort(perm, dim=1)
+    Vs, sT, zT = [], [], []
+    for b in range(B):
+        pr = random_problem(C=C, R=R, seed=300 + b)
+        Vs.append(torch.from_numpy(mathref.direct_factor(pr["H"].double().numpy(), 0.01)).float().contiguous())
+        s_, z_ = oracle.build_group_meta_packed(
+            torch.nn.functional.pad(W[b].float(), (0, G * gs - C)).reshape(R * G, gs), 4, True)
+        sT.append(s_.view(R, G).t().contiguous()); zT.append(z_.view(R, G).t().contiguous())
+    Wd, pd = W.to(DEV), perm_inv.to(DEV)
+    X = hip.weight_to_solver_order(Wd, pd)
+    W0 = torch.empty((B, C, R), dtype=dtype, device=DEV)
+    X2 = hip.weight_to_solver_order(Wd, pd, out=torch.empty_like(X), out0=W0)
+    assert torch.equal(X, X2) and torch.equal(W0.float(), X)
+    assert torch.equal(X[0].cpu(), W[0].float().t()[perm[0]])
+    # a band of a taller pair
+    tall, tall0 = torch.zeros((B, C, 2 * R), device=DEV), torch.zeros((B, C, 2 * R), dtype=dtype, device=DEV)
+    hip.weight_to_solver_order(Wd, pd, out=tall, row0=R, out0=tall0)
+    assert torch.equal(tall[:, :, R:], X) and torch.equal(tall0[:, :, R:].float(), X)
+    assert not tall[:, :, :R].any() and not tall0[:, :, :R].any()
+    args = (torch.stack(Vs).to(DEV), torch.stack(sT).to(DEV), torch.stack(zT).to(DEV),
+            (perm // gs).int().to(DEV), 4)
+    Xa, Xb, Xc = X.clone(), X.clone(), X.clone()
+    qa = hip.gptq_sweep_direct_batched(Xa, *args)
+    qb = hip.gptq_sweep_direct_batched(Xb, *args, W0=W0)
+    qc = hip.gptq_sweep_direct_batched(Xc, *args, W0=W0.float())
+    assert torch.equal(qa, qb) and torch.equal(qa, qc)
+    assert torch.equal(Xa, Xb) and torch.equal(Xa, Xc)
+
+
 @pytest.mark.parametrize("C,R,n", [(256, 64, 500), (512, 256, 300), (200, 33, 150)])
 def test_direct_sparse14_sweep_bit_exact(hip, C, R, n):
     """1:4 joint solve in the displacement form against its CPU checker: codes and masks bit
