@@ -32,6 +32,14 @@ struct GemmArgs {
     int64_t bound_a_stride;
     const float* bound_b;
     int64_t bound_b_stride;
+    // piece path only: not null = At is not read; its panel is formed from a lower triangular
+    // matrix instead, At[k, m] = -(Al[m, k] * (1 / Al[m, m])) for k < m (the matrix V of the
+    // displacement-form sweep straight from the factor of H; zero where a_info[matrix] != 0).
+    // Al has pitch a_lower_ld and batch stride a_lower_stride.  Problems that do not take the
+    // piece path need At.
+    const float* a_lower;
+    int64_t a_lower_ld, a_lower_stride;
+    const int32_t* a_info;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;
@@ -56,5 +64,8 @@ int launch_chain_gemm(const GemmArgs& g, int64_t batch, hipStream_t st);
 int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,
                            hipStream_t st, void* split_ws = nullptr, int64_t split_ws_bytes = 0);
 int64_t split_gemm_workspace_bytes(int64_t batch, int64_t k_rows);
+// True when launch_chain_gemm_pair(g, {}, batch, st, ws, ws_bytes) with a workspace of that
+// size would run `g` on the piece path (and so would not read g.At when g.a_lower is set).
+bool split_path_applies(const GemmArgs& g, int64_t batch, int64_t ws_bytes);
 
 }  // namespace forge

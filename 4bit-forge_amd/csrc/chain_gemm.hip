@@ -640,6 +640,49 @@ __global__ __launch_bounds__(128) void split_a_panel_kernel(const float* __restr
     }
 }
 
+// The same panel taken from a lower triangular matrix: element (k, m) = -(Al[m, k] * (1 / Al[m, m]))
+// for k < m, zero elsewhere and for matrices whose info is not 0.  A thread reads the 8
+// consecutive k of a word from ONE row of Al (32 contiguous bytes; four neighbouring lanes cover
+// the 128 bytes that a row contributes to the stage), so nothing is transposed.
+template <int NP, bool HALF>
+__global__ __launch_bounds__(128) void split_a_panel_lower_kernel(
+    const float* __restrict__ Al, int64_t ldl, int64_t ls, const int32_t* __restrict__ info, int m0,
+    int k0, int n_stage, u32x4* __restrict__ Ap, int64_t aps, const float* __restrict__ bound,
+    int64_t bound_stride) {
+    const int bz = blockIdx.x / n_stage, st = blockIdx.x % n_stage;
+    const int t = threadIdx.x, kg = t & 3, mr = t >> 2;     // k group of 8, row within a pass of 32
+    const int kb = k0 + SPLIT_TK * st + 8 * kg;             // first of this thread's 8 k
+    const float* __restrict__ Ab = Al + (int64_t)bz * ls;
+    const bool failed = info != nullptr && info[bz] != 0;
+    u32x4* dst = Ap + (int64_t)bz * aps + (int64_t)st * split_stage_words(NP) + kg * 128;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int c = 32 * e + mr, m = m0 + c;              // column of the tile, row of Al
+        const float* row = Ab + (int64_t)m * ldl;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(row + kb);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(row + kb + 4);
+        const float rcp = 1.0f / row[m];
+        float col[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float a = j < 4 ? lo[j] : hi[j - 4];
+            col[j] = (failed || kb + j >= m) ? 0.0f : -(a * rcp);
+        }
+        const int pos = (c & 3) * 32 + (c >> 2);            // the stage image's place of column c
+        u32x4 p1, p2, p3;
+        if (NP == 3) {
+            split_pieces<8>(col, p1, p2, p3);
+            dst[1024 + pos] = p3;
+        } else if (HALF) {
+            split_pieces2h<8>(col, pow2_scale(bound[(int64_t)bz * bound_stride + m]), p1, p2);
+        } else {
+            split_pieces2<8>(col, p1, p2);
+        }
+        dst[pos] = p1;
+        dst[512 + pos] = p2;
+    }
+}
+
 struct SplitPair {
     GemmPair pair;
     const u32x4* Ap;   // split A panel of both problems (same At, m0, k0)
@@ -1075,6 +1118,9 @@ bool split_eligible(const Prepared& a, const Prepared* b, int64_t batch, int64_t
     if (b) {
         const GemmArgs &x = a.g, &y = b->g;
         if (x.At != y.At || x.lda != y.lda || x.as != y.as || x.m0 != y.m0 || x.k0 != y.k0) return false;
+        if (x.a_lower != y.a_lower || x.a_lower_ld != y.a_lower_ld || x.a_lower_stride != y.a_lower_stride ||
+            x.a_info != y.a_info)
+            return false;
         if (x.bound_a != y.bound_a || x.bound_a_stride != y.bound_a_stride) return false;
         if ((x.bound_b != nullptr) != (y.bound_b != nullptr)) return false;
         if (b->g.xcd_map && a.n_wg % 8 != 0) return false;
@@ -1106,7 +1152,21 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
                             WORK_BYTES);
         const dim3 pgrid((unsigned)(batch * n_stage)), pblock(128);
         u32x4* dst = static_cast<u32x4*>(ws) + (int64_t)mt * sp.apt;
-        if (half)
+        if (a.g.a_lower) {
+            const int m0 = a.g.m0 + mt * TM;
+            if (half)
+                split_a_panel_lower_kernel<2, true><<<pgrid, pblock, 0, st>>>(
+                    a.g.a_lower, a.g.a_lower_ld, a.g.a_lower_stride, a.g.a_info, m0, a.g.k0, n_stage, dst,
+                    sp.aps, a.g.bound_a, a.g.bound_a_stride);
+            else if (two)
+                split_a_panel_lower_kernel<2, false><<<pgrid, pblock, 0, st>>>(
+                    a.g.a_lower, a.g.a_lower_ld, a.g.a_lower_stride, a.g.a_info, m0, a.g.k0, n_stage, dst,
+                    sp.aps, nullptr, 0);
+            else
+                split_a_panel_lower_kernel<3, false><<<pgrid, pblock, 0, st>>>(
+                    a.g.a_lower, a.g.a_lower_ld, a.g.a_lower_stride, a.g.a_info, m0, a.g.k0, n_stage, dst,
+                    sp.aps, nullptr, 0);
+        } else if (half)
             split_a_panel_kernel<2, true><<<pgrid, pblock, 0, st>>>(
                 a.g.At, a.g.lda, a.g.as, a.g.m0 + mt * TM, a.g.k0, n_stage, dst, sp.aps, a.g.bound_a,
                 a.g.bound_a_stride);
@@ -1146,6 +1206,12 @@ int launch_split(const Prepared& a, const Prepared* b, int64_t batch, int n_stag
 int64_t split_gemm_workspace_bytes(int64_t batch, int64_t k_rows) {
     if (batch <= 0 || k_rows <= 0) return 0;
     return batch * ceil_div(k_rows, (int64_t)SPLIT_TK) * SPLIT_STAGE_WORDS * 16;
+}
+
+bool split_path_applies(const GemmArgs& g, int64_t batch, int64_t ws_bytes) {
+    const Prepared p = prepare(g, batch);
+    int n_stage = 0;
+    return !p.empty && split_eligible(p, nullptr, batch, ws_bytes, &n_stage);
 }
 
 int launch_chain_gemm_pair(const GemmArgs& first, const GemmArgs& second, int64_t batch,

@@ -519,13 +519,17 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
 template <bool FLIP>
 __global__ __launch_bounds__(256) void unit_upper_from_lower_kernel(
     const float* __restrict__ L, const int32_t* __restrict__ info, float* __restrict__ U, int64_t C,
-    float sign, bool upper_tiles_only) {
+    float sign, bool upper_tiles_only, bool band) {
     __shared__ float tile[32][33];
-    if (upper_tiles_only && blockIdx.y > blockIdx.x) return;   // whole tile below the diagonal
+    // band: the grid's x covers the eight tile columns of the row's own 128-column block and
+    // the next one only
+    const unsigned tile_col = band ? 4u * (blockIdx.y / 4u) + blockIdx.x : blockIdx.x;
+    if (band && (int64_t)tile_col * 32 >= C) return;
+    if (upper_tiles_only && blockIdx.y > tile_col) return;   // whole tile below the diagonal
     const int64_t b = blockIdx.z;
     const float* __restrict__ Lb = L + b * C * C;
     float* __restrict__ Ub = U + b * C * C;
-    const int64_t t0 = (int64_t)blockIdx.y * 32, k0 = (int64_t)blockIdx.x * 32;   // U tile rows t, columns k
+    const int64_t t0 = (int64_t)blockIdx.y * 32, k0 = (int64_t)tile_col * 32;   // U tile rows t, columns k
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;                      // 32 x 8
     const bool failed = info != nullptr && info[b] != 0;
     if (!failed && k0 + 31 >= t0) {
@@ -586,13 +590,17 @@ extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, 
     FORGE_REQUIRE(L && U && L != U, "null or aliased pointer");
     hipStream_t st = (hipStream_t)stream;
     const unsigned nt = (unsigned)forge::ceil_div(C, 32);
-    forge::KernelTiming timing("unit_upper_from_lower", st, 6.0 * C * C * (double)batch, forge::WORK_BYTES);
+    forge::KernelTiming timing("unit_upper_from_lower", st,
+                               ((flipped_upper & 8) ? 8.0 * 256.0 * C : 6.0 * C * C) * (double)batch,
+                               forge::WORK_BYTES);
     const float sign = (flipped_upper & 2) ? -1.0f : 1.0f;
     const bool skip = (flipped_upper & 4) != 0;
+    const bool band = (flipped_upper & 8) != 0;
+    const dim3 grid(band ? 8u : nt, nt, (unsigned)batch);
     if (flipped_upper & 1)
-        unit_upper_from_lower_kernel<true><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign, skip);
+        unit_upper_from_lower_kernel<true><<<grid, dim3(256), 0, st>>>(L, info, U, C, sign, skip, band);
     else
-        unit_upper_from_lower_kernel<false><<<dim3(nt, nt, (unsigned)batch), dim3(256), 0, st>>>(L, info, U, C, sign, skip);
+        unit_upper_from_lower_kernel<false><<<grid, dim3(256), 0, st>>>(L, info, U, C, sign, skip, band);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

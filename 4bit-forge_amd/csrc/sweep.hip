@@ -359,6 +359,26 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     }
 }
 
+// The same bounds from the lower factor that V is made of, V[t, m] = -(Al[m, t] * (1 / Al[m, m])):
+// the largest |Al[m, t]|, t < m, times |1 / Al[m, m]| (rounding is monotone, so this is the
+// largest |V[t, m]| exactly).  One wavefront per row; 0 for matrices whose info is not 0.
+__global__ __launch_bounds__(256) void lower_row_bound_kernel(const float* __restrict__ Al, int64_t C,
+                                                              const int32_t* __restrict__ info,
+                                                              float* __restrict__ bound) {
+    const int64_t b = blockIdx.y, m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (m >= C) return;
+    const int lane = threadIdx.x & 63;
+    const float* __restrict__ row = Al + b * C * C + m * C;
+    float mx = 0.0f;
+    for (int64_t t = lane; t < m; t += 64) mx = fmaxf(mx, fabsf(row[t]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if (lane == 0) {
+        const bool failed = info != nullptr && info[b] != 0;
+        bound[b * C + m] = failed ? 0.0f : fabsf(mx * (1.0f / row[m]));
+    }
+}
+
 // bound[m] = max_{t < m} |V[t, m]| for every column of the unit upper matrix V (the strict upper
 // triangle is all that the block updates read).  One workgroup per (128 columns, matrix).
 __global__ __launch_bounds__(256) void upper_column_bound_kernel(const float* __restrict__ V, int64_t C,
@@ -476,9 +496,48 @@ extern "C" int forge_sparsegptq14_solver(float* W, float* U, const float* scales
     return solve_single<true>(W, U, scales, qzeros, bits, C, R, qweight, M, E, uinv, st);
 }
 
+// Few matrices: a left-looking step has only batch * R/128 tiles, far fewer than the GPU
+// has CUs.  Then every finished block is pushed into ALL later columns at once instead
+// (K = 128, (C - start)/128 times as many tiles); the weights are re-read per step, which
+// a batch could not afford.  Same fma chain per element, hence the same bits.
+static bool right_looking_schedule(int64_t batch, int64_t R) {
+    bool right_looking = batch * forge::ceil_div(R, 128) < 128;
+    const int64_t forced = forge::option(forge::OPT_SWEEP_SCHEDULE);
+    if (forced == 1) right_looking = false;
+    if (forced == 2) right_looking = true;
+    return right_looking;
+}
+
+// The even blocks' long product, as sweep_batched launches it for block `start`.
+static forge::GemmArgs even_block_update(float* X, const float* U, int64_t C, int64_t R, int64_t start) {
+    forge::GemmArgs g{};
+    g.X = X; g.At = U; g.Bm = X; g.ldx = R; g.lda = C; g.ldb = R;
+    g.xs = C * R; g.as = C * C; g.bs = C * R;
+    g.m0 = (int)start; g.n1 = (int)R; g.k0 = 0; g.k1 = (int)start;
+    g.m1 = (int)(start + 2 * forge::kBW <= C ? start + 2 * forge::kBW : start + forge::kBW);
+    g.negate_a = true;
+    g.blocked_sum = true;
+    g.products = 3;
+    return g;
+}
+
+// True when, given the lower factor, the displacement-form sweep reads V only within one
+// 128-column block of its diagonal: left-looking schedule and every even block's product on the
+// piece path (whole 128 x 128 tiles, aligned rows), whose A panels then come from the factor.
+static bool sweep_reads_band_only(float* X, const float* U, int64_t batch, int64_t C, int64_t R,
+                                  int64_t split_bytes) {
+    if (right_looking_schedule(batch, R) || C % forge::kBW != 0 || C <= forge::kBW) return false;
+    // the last even block has the longest K (and the largest offsets); alignment is the same for all
+    const int64_t nblk = C / forge::kBW, last_even = ((nblk - 1) / 2) * 2;
+    if (last_even == 0) return false;
+    return forge::split_path_applies(even_block_update(X, U, C, R, last_even * forge::kBW), batch, split_bytes) &&
+           forge::split_path_applies(even_block_update(X, U, C, R, 2 * forge::kBW), batch, split_bytes);
+}
+
 // Left-looking schedule for a batch of equally shaped matrices, errors (or, with W0, the
 // displacements) kept in X.
-static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U, const float* scalesT,
+static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U, const float* Lf,
+                         const int32_t* Linfo, const float* scalesT,
                          const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                          uint32_t* M, const float* uinv, int64_t batch, int64_t C, int64_t R,
                          int64_t G, int bits, int sparse14, void* ws, int64_t ws_bytes,
@@ -491,14 +550,7 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U,
     FORGE_REQUIRE(!sparse14 || (M && uinv), "sparse14 needs M and uinv");
     FORGE_REQUIRE(W0 != X, "W0 must be a copy of X, not X itself");
     hipStream_t st = (hipStream_t)stream;
-    // Few matrices: a left-looking step has only batch * R/128 tiles, far fewer than the GPU
-    // has CUs.  Then every finished block is pushed into ALL later columns at once instead
-    // (K = 128, (C - start)/128 times as many tiles); the weights are re-read per step, which
-    // a batch could not afford.  Same fma chain per element, hence the same bits.
-    bool right_looking = batch * forge::ceil_div(R, 128) < 128;
-    const int64_t forced = forge::option(forge::OPT_SWEEP_SCHEDULE);
-    if (forced == 1) right_looking = false;
-    if (forced == 2) right_looking = true;
+    const bool right_looking = right_looking_schedule(batch, R);
     // The direct route's block updates on the 16-bit matrix pipe, three products per fp32
     // product.  Below 4096 columns two fp16 halves per operand, fp32-grade: the columns of V are
     // scaled from their largest entry above the diagonal, the rows of displacements from a
@@ -518,9 +570,18 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U,
         vbound = (float*)((char*)ws + split_bytes);
         dbound = (float*)((char*)ws + split_bytes + (batch * C * 4 + 255) / 256 * 256);
     }
+    // With the lower factor at hand the even blocks' A panels are formed from its rows: V is
+    // then read only within one block of its diagonal (in-block chains, odd blocks' K = 128
+    // products), provided every even block takes the piece path.
+    const bool from_lower = Lf != nullptr && ws && W0 &&
+                            sweep_reads_band_only(X, U, batch, C, R, split_bytes);
     if (halves) {
-        upper_column_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 128), (unsigned)batch), dim3(256), 0, st>>>(
-            U, C, vbound);
+        if (from_lower)
+            lower_row_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 4), (unsigned)batch), dim3(256), 0, st>>>(
+                Lf, C, Linfo, vbound);
+        else
+            upper_column_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 128), (unsigned)batch), dim3(256), 0, st>>>(
+                U, C, vbound);
         FORGE_LAUNCH_CHECK();
     }
     for (int64_t start = 0; start < C; start += forge::kBW) {
@@ -548,9 +609,13 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U,
                     g.bound_a = vbound; g.bound_a_stride = C;
                     g.bound_b = dbound; g.bound_b_stride = R;
                 }
+                if (from_lower) {
+                    g.a_lower = Lf; g.a_lower_ld = C; g.a_lower_stride = C * C; g.a_info = Linfo;
+                }
                 if (pairs && start + 2 * forge::kBW <= C) g.m1 = (int)(start + 2 * forge::kBW);
                 if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, split_bytes)) return e;
                 g.m1 = (int)(start + bw);
+                g.a_lower = nullptr;
             } else {
                 g.k0 = (int)(start - forge::kBW);
                 if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
@@ -587,8 +652,8 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
                                         uint8_t* qweight, uint32_t* M, const float* uinv,
                                         int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
                                         int sparse14, forge_stream_t stream) {
-    return sweep_batched(X, nullptr, false, U, scalesT, qzerosT, g_idx, qweight, M, uinv, batch, C, R, G,
-                         bits, sparse14, nullptr, 0, stream);
+    return sweep_batched(X, nullptr, false, U, nullptr, nullptr, scalesT, qzerosT, g_idx, qweight, M, uinv,
+                         batch, C, R, G, bits, sparse14, nullptr, 0, stream);
 }
 
 extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R) {
@@ -599,7 +664,16 @@ extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_
            (batch * C * 4 + 255) / 256 * 256 + (batch * R * 4 + 255) / 256 * 256;
 }
 
+extern "C" int forge_gptq_sweep_direct_reads_band_only(int64_t batch, int64_t C, int64_t R) {
+    if (batch <= 0 || C <= 0 || R <= 0) return 0;
+    // stand-in pointers: only their alignment is looked at (device allocations are aligned)
+    float* aligned = reinterpret_cast<float*>(uintptr_t(256));
+    const int64_t split_bytes = C > forge::kBW ? 2 * forge::split_gemm_workspace_bytes(batch, C - forge::kBW) : 0;
+    return sweep_reads_band_only(aligned, aligned, batch, C, R, split_bytes) ? 1 : 0;
+}
+
 extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
+                                                  const float* L, const int32_t* info,
                                                   const float* scalesT, const float* qzerosT,
                                                   const int32_t* g_idx, uint8_t* qweight,
                                                   uint32_t* M, const float* mdiag,
@@ -611,8 +685,8 @@ extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int 
     FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C, R),
                   "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
                   (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C, R));
-    return sweep_batched(X, W0, w0_dtype == FORGE_BF16, V, scalesT, qzerosT, g_idx, qweight, M, mdiag,
-                         batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
+    return sweep_batched(X, W0, w0_dtype == FORGE_BF16, V, L, info, scalesT, qzerosT, g_idx, qweight, M,
+                         mdiag, batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
 }
 
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
@@ -622,8 +696,9 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
                                                int64_t batch, int64_t C, int64_t R, int64_t G,
                                                int bits, int sparse14, void* ws, int64_t ws_bytes,
                                                forge_stream_t stream) {
-    return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, V, scalesT, qzerosT, g_idx, qweight, M,
-                                              mdiag, batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
+    return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, V, nullptr, nullptr, scalesT, qzerosT, g_idx,
+                                              qweight, M, mdiag, batch, C, R, G, bits, sparse14, ws,
+                                              ws_bytes, stream);
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

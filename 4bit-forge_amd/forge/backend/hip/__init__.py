@@ -53,8 +53,9 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
                                       vp], i32),
         "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                              i32, i32, vp, i64, vp], i32),
-        "forge_gptq_sweep_direct_batched_w0": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64,
-                                                i64, i32, i32, vp, i64, vp], i32),
+        "forge_gptq_sweep_direct_batched_w0": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64,
+                                                i64, i64, i32, i32, vp, i64, vp], i32),
+        "forge_gptq_sweep_direct_reads_band_only": ([i64, i64, i64], i32),
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
@@ -101,6 +102,7 @@ EXPORTED_SYMBOLS = (
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_weight_to_solver_order_strided", "forge_codes_to_layer_order_strided",
     "forge_weight_to_solver_order_pair", "forge_gptq_sweep_direct_batched_w0",
+    "forge_gptq_sweep_direct_reads_band_only",
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
     "forge_dequantize_groups", "forge_gather_scaled_rows",
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
@@ -301,17 +303,28 @@ class _HipKernels:
                 _ptr(uinv), B, C, R, G, int(bits), int(bool(sparse14)), _stream()))
         return (q, M) if sparse14 else q
 
+    def sweep_direct_reads_band_only(self, B, C, R) -> bool:
+        """True when gptq_sweep_direct_batched(..., L=...) reads V only within one 128-column
+        block of its diagonal for this shape (unit_upper_from_lower(band=True) then suffices)."""
+        return bool(self._lib.forge_gptq_sweep_direct_reads_band_only(int(B), int(C), int(R)))
+
     def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None,
-                                  exact_chain=False, sparse14=False, mdiag=None):
+                                  exact_chain=False, sparse14=False, mdiag=None, L=None, info=None):
         """The sweep fed by the factor of H itself: V [B,C,C] = -M[t,k]/M[k,k] above the
         diagonal (``unit_upper_from_lower(L, info, negate=True)``).  X [B,C,R] f32 in/out
         (displacements w0 - deq on exit); W0: untouched copy of X (made here when None).
         exact_chain: keep the block updates as one fp32 fma chain per element (reproducible
         on a CPU) instead of blocked sums on the bf16 matrix pipe.  sparse14: the 1:4 joint
-        solve, with mdiag [B,C] = diag(L) (1 where the factorisation failed).
+        solve, with mdiag [B,C] = diag(L) (1 where the factorisation failed).  L [B,C,C], info
+        [B] int32: the lower factor V was made from and its failure flags; the long block
+        updates then take their V operand from L's rows (same numbers).
         Returns qweight [B,C,R] u8 (and M [B, ceil(C/32), R] u32)."""
-        _need_cuda(X, V, scalesT, qzerosT, g_idx, W0)
+        _need_cuda(X, V, scalesT, qzerosT, g_idx, W0, L, info)
         B, C, R = X.shape
+        assert L is None or (L.is_contiguous() and L.dtype == torch.float32 and L.shape == V.shape)
+        assert info is None or (info.dtype == torch.int32 and info.is_contiguous() and info.numel() == B)
+        if exact_chain:
+            L = None
         G = scalesT.shape[1]
         assert X.is_contiguous() and V.is_contiguous() and scalesT.is_contiguous()
         assert qzerosT.is_contiguous() and g_idx.is_contiguous() and g_idx.dtype == torch.int32
@@ -331,7 +344,8 @@ class _HipKernels:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_gptq_sweep_direct_batched_w0(
-                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(V), _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
+                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(V), _ptr(L), _ptr(info if L is not None else None),
+                _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
                 _ptr(M), _ptr(mdiag), B, C, R, G, int(bits), int(bool(sparse14)), _ptr(ws), nbytes,
                 _stream()))
         return (q, M) if sparse14 else q
@@ -403,18 +417,20 @@ class _HipKernels:
         return H, info
 
     def unit_upper_from_lower(self, L, info=None, flipped_upper=False, negate=False,
-                              upper_only=False):
+                              upper_only=False, band=False):
         """U [B,C,C]: U[t,k] = L[k,t] / L[k,k] (k > t), unit diagonal, zero below; identity
         where info != 0.  flipped_upper: L is the upper factor A with both orders reversed.
         negate: entries above the diagonal with the opposite sign.  upper_only: 32x32 tiles
-        wholly below the diagonal are left unwritten (uninitialised memory)."""
+        wholly below the diagonal are left unwritten (uninitialised memory).  band: only the
+        columns of each row's own 128-column block and of the next one are written."""
         _need_cuda(L, info)
         B, C, _ = L.shape
         assert L.is_contiguous() and L.dtype == torch.float32
         U = torch.empty_like(L)
         with torch.cuda.device(L.device):
             self._check(self._lib.forge_unit_upper_from_lower(
-                _ptr(L), _ptr(info), _ptr(U), B, C, int(bool(flipped_upper)) | (2 if negate else 0) | (4 if upper_only else 0),
+                _ptr(L), _ptr(info), _ptr(U), B, C,
+                int(bool(flipped_upper)) | (2 if negate else 0) | (4 if upper_only else 0) | (8 if band else 0),
                 _stream()))
         return U
 

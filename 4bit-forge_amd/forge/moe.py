@@ -205,12 +205,16 @@ class ExpertGroupGPTQ:
                     del L
                 elif direct:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True)
+                    # the sweep's long products read V straight from L's rows; where that covers
+                    # everything beyond one block of the diagonal, only that band of V is written
+                    band = kernels.sweep_direct_reads_band_only(B, C, R)
+                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True, band=band)
                     if sparse:
                         # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the
                         # diagonal of the factor of H itself; U = I where it failed
                         uinv = torch.where((info != 0)[:, None], torch.ones((), device=dev),
                                            L.diagonal(dim1=1, dim2=2)).contiguous()
+                    Lf = L
                     del L
                 elif sparse:
                     # un-normalised factor, rows then scaled by the rounded reciprocal of the
@@ -240,15 +244,17 @@ class ExpertGroupGPTQ:
                 M = None
                 if direct and sparse:
                     q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0,
-                                                             sparse14=True, mdiag=uinv)
+                                                             sparse14=True, mdiag=uinv, L=Lf, info=info)
                 elif sparse:
                     q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
                                                       uinv=uinv)
                 elif direct:
-                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0)
+                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0, L=Lf,
+                                                          info=info)
                 else:
                     q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
                 del X, U, W0
+                Lf = None
                 r0 = 0
                 for i in job:
                     Ri = sizes[i]

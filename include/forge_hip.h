@@ -182,8 +182,16 @@ int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
 int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R);
 /* The same with the untouched weights W0 in f32 (w0_dtype = FORGE_F32) or in bf16 (FORGE_BF16:
  * exact when the layer's weights are bf16, and half the bytes to read);
- * forge_weight_to_solver_order_pair writes X and W0 in one pass. */
+ * forge_weight_to_solver_order_pair writes X and W0 in one pass.
+ * L, info (may be NULL): the lower factor that V was made from
+ * (forge_chol_reverse_lower_batched) and its failure flags.  With them the long block updates
+ * take their V operand straight from the rows of L, the same numbers, and when
+ * forge_gptq_sweep_direct_reads_band_only(batch, C, R) returns 1 (left-looking schedule, whole
+ * 128 x 128 tiles, workspace given) V is read only within one 128-column block of its diagonal:
+ * forge_unit_upper_from_lower with bit 3 then suffices. */
+int forge_gptq_sweep_direct_reads_band_only(int64_t batch, int64_t C, int64_t R);
 int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
+                                       const float* L, const int32_t* info,
                                        const float* scalesT, const float* qzerosT,
                                        const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
                                        const float* mdiag, int64_t batch, int64_t C, int64_t R,
@@ -282,7 +290,10 @@ int forge_chol_reverse_lower_batched(float* H, const float* damp, int32_t* info,
  * flipped_upper bit 0: L is given as the reference's upper factor A instead,
  * L[k][t] = A[C-1-k][C-1-t].  Bit 1: the entries above the diagonal are negated (the matrix V
  * of forge_gptq_sweep_direct_batched).  Bit 2: 32 x 32 tiles that lie wholly below the
- * diagonal are left unwritten (no sweep reads them).  L and U must not overlap. */
+ * diagonal are left unwritten (no sweep reads them).  Bit 3: only the columns of each row's own
+ * 128-column block and of the next block are written (all that
+ * forge_gptq_sweep_direct_batched_w0 reads when it is given L and
+ * forge_gptq_sweep_direct_reads_band_only says so).  L and U must not overlap. */
 int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U, int64_t batch,
                                 int64_t C, int flipped_upper, forge_stream_t stream);
 

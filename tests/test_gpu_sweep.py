@@ -157,6 +157,54 @@ def test_direct_sweep_untouched_weights_from_the_layout_pass(hip, C, R, dtype):
     assert torch.equal(Xa, Xb) and torch.equal(Xa, Xc)
 
 
+@pytest.mark.parametrize("C,products", [(512, 0), (640, 3), (384, 6)])
+def test_direct_sweep_reads_its_v_operand_from_the_lower_factor(hip, C, products):
+    """Given the lower factor, the long block updates form their V operand from its rows
+    instead of reading V: same numbers, so codes and displacements are bit-identical, also
+    when everything of V beyond one block of its diagonal was never written (NaN here) and
+    for a matrix whose factorisation failed (V = I).  Left-looking schedule, both piece kinds."""
+    B, R, gs = 3, 256, 128
+    G = C // gs
+    g0 = torch.Generator().manual_seed(C)
+    H = torch.stack([random_problem(C=C, R=8, seed=400 + b)["H"] for b in range(B)])
+    H[2] = -H[2]                                                  # not positive definite
+    W = 0.02 * torch.randn(B, R, C, generator=g0)
+    perm = torch.stack([torch.randperm(C, generator=g0) for _ in range(B)])
+    sT, zT = [], []
+    for b in range(B):
+        s_, z_ = oracle.build_group_meta_packed(W[b].reshape(R * G, gs), 4, True)
+        sT.append(s_.view(R, G).t().contiguous()); zT.append(z_.view(R, G).t().contiguous())
+    damp = torch.full((B,), 0.01) * H.diagonal(dim1=1, dim2=2).mean(dim=1).abs()
+    L, info = hip.chol_reverse_lower_batched(H.to(DEV).clone(), damp.to(DEV))
+    assert info.cpu().tolist()[:2] == [0, 0] and info.cpu().tolist()[2] != 0
+    X = hip.weight_to_solver_order(W.to(DEV), torch.argsort(perm, dim=1).to(DEV))
+    args = (torch.stack(sT).to(DEV), torch.stack(zT).to(DEV), (perm // gs).int().to(DEV), 4)
+    hip.set_option("sweep_schedule", 1)
+    old = hip.set_option("sweep_update_products", products)
+    try:
+        assert hip.sweep_direct_reads_band_only(B, C, R)
+        assert not hip.sweep_direct_reads_band_only(B, C + 4, R)       # ragged last block
+        V = hip.unit_upper_from_lower(L, info, negate=True, upper_only=True)
+        Xa = X.clone()
+        qa = hip.gptq_sweep_direct_batched(Xa, V, *args)
+        Vb = torch.full_like(V, float("nan"))
+        with torch.cuda.device(DEV):
+            hip._check(hip._lib.forge_unit_upper_from_lower(
+                L.data_ptr(), info.data_ptr(), Vb.data_ptr(), B, C, 2 | 4 | 8, None))
+        idx = torch.arange(C, device=DEV)
+        blk = idx // 128
+        upper = idx[None, :] >= idx[:, None]                          # row t, column k >= t
+        in_band = upper & (blk[None, :] <= blk[:, None] + 1)
+        assert torch.equal(Vb[:, in_band], V[:, in_band])
+        assert torch.isnan(Vb[:, upper & ~in_band]).all()
+        Xb = X.clone()
+        qb = hip.gptq_sweep_direct_batched(Xb, Vb, *args, L=L, info=info)
+        assert torch.equal(qa, qb) and torch.equal(Xa, Xb)
+    finally:
+        hip.set_option("sweep_update_products", old)
+        hip.set_option("sweep_schedule", 0)
+
+
 @pytest.mark.parametrize("C,R,n", [(256, 64, 500), (512, 256, 300), (200, 33, 150)])
 def test_direct_sparse14_sweep_bit_exact(hip, C, R, n):
     """1:4 joint solve in the displacement form against its CPU checker: codes and masks bit
