@@ -24,6 +24,7 @@
 // bf16 and f32 values are exact there) and the update beta*old + alpha*sum is rounded to
 // fp32 once; the rank-k kernels write that value where row == column.
 #include "common.h"
+#include <type_traits>
 #include <hip/hip_bf16.h>
 #include <algorithm>
 #include <cstring>
@@ -100,27 +101,36 @@ __global__ __launch_bounds__(256) void diag_float64_kernel(const T* __restrict__
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t c0 = (int64_t)blockIdx.x * 128 + 2 * lane;
     const bool in0 = c0 < C, in1 = c0 + 1 < C;
+    // columns past the end read column 0 instead and count as zero: unconditional loads, so that
+    // the sixteen rows really are in flight together (a load inside a branch is waited for at once)
     const T* __restrict__ col = X + g.row0 * ldx + (in0 ? c0 : 0);
+    const int off1 = in1 ? 1 : 0;
+    const double m0 = in0 ? 1.0 : 0.0, m1 = in1 ? 1.0 : 0.0;
     double s0 = 0.0, s1 = 0.0;
     int t = wave;
-    for (; t + 12 < g.n; t += 16) {             // four rows in flight per wavefront
-        T a[4], b[4];
+    // sixteen rows in flight per wavefront: a heavy group's columns are walked by ONE workgroup,
+    // whose time is the rows' load latency divided by what is in flight
+    // (16-bit values are held one per 32-bit register: packed pairs would chain the loads)
+    using Held = typename std::conditional<sizeof(T) == 2, uint32_t, T>::type;
+    for (; t + 60 < g.n; t += 64) {
+        Held a[16], b[16];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 16; ++u) {
             const T* r = col + (int64_t)(t + 4 * u) * ldx;
-            a[u] = in0 ? r[0] : T(0);
-            b[u] = in1 ? r[1] : T(0);
+            a[u] = r[0];
+            b[u] = r[off1];
         }
+        __builtin_amdgcn_sched_barrier(0);      // all 32 loads are issued before the first is used
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const double x = as_double<T>(a[u]), y = as_double<T>(b[u]);
+        for (int u = 0; u < 16; ++u) {
+            const double x = m0 * as_double<T>((T)a[u]), y = m1 * as_double<T>((T)b[u]);
             s0 = __builtin_fma(x, x, s0);
             s1 = __builtin_fma(y, y, s1);
         }
     }
     for (; t < g.n; t += 4) {
         const T* r = col + (int64_t)t * ldx;
-        const double x = as_double<T>(in0 ? r[0] : T(0)), y = as_double<T>(in1 ? r[1] : T(0));
+        const double x = m0 * as_double<T>(r[0]), y = m1 * as_double<T>(r[off1]);
         s0 = __builtin_fma(x, x, s0);
         s1 = __builtin_fma(y, y, s1);
     }
