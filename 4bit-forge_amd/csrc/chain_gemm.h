@@ -40,6 +40,11 @@ struct GemmArgs {
     const float* a_lower;
     int64_t a_lower_ld, a_lower_stride;
     const int32_t* a_info;
+    // piece path only: not null = the sums start from x_init (same pitch and batch stride as X,
+    // in elements; f32 or, with x_init_bf16, bf16) instead of from X, which is then only written.
+    // Problems that do not take the piece path ignore it and start from X.
+    const void* x_init;
+    bool x_init_bf16;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;

@@ -881,7 +881,20 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
             const float* __restrict__ sca =
                 HALF ? g.bound_a + (int64_t)bz * g.bound_a_stride + m0 + t * TM : nullptr;
             f32x4 xo[16];
-            if (!g.init_zero) {
+            if (g.x_init && g.x_init_bf16) {
+                const uint16_t* __restrict__ X0 = static_cast<const uint16_t*>(g.x_init) + (Xt - g.X);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const u32x2 w = *reinterpret_cast<const u32x2*>(X0 + (int64_t)(kh + 8 * i) * g.ldx);
+                    xo[i] = f32x4{__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xFFFF0000u),
+                                  __uint_as_float(w[1] << 16), __uint_as_float(w[1] & 0xFFFF0000u)};
+                }
+            } else if (g.x_init) {
+                const float* __restrict__ X0 = static_cast<const float*>(g.x_init) + (Xt - g.X);
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    xo[i] = *reinterpret_cast<const f32x4*>(X0 + (int64_t)(kh + 8 * i) * g.ldx);
+            } else if (!g.init_zero) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
                     xo[i] = *reinterpret_cast<const f32x4*>(Xt + (int64_t)(kh + 8 * i) * g.ldx);

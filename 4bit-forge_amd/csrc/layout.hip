@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void to_solver_order_kernel(
         const int64_t c = c0 + j, r = r0 + tx;
         if (c < C && r < R) {
             const int64_t at = b * o_stride + perm_inv[b * C + c] * ldo + r;
-            Xout[at] = tile[tx][j];
+            if (Xout) Xout[at] = tile[tx][j];
             if (W0out) st_from_f32(W0out + at, tile[tx][j]);
         }
     }
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
             const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
                                          __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
             const int64_t at = b * o_stride + perm_inv[b * C + c0 + c] * ldo + r0 + r4;
-            *reinterpret_cast<float4*>(Xout + at) = o;
+            if (Xout) *reinterpret_cast<float4*>(Xout + at) = o;
             if (W0out) *reinterpret_cast<uint2*>(W0out + at) = v;
         }
     }
@@ -330,11 +330,11 @@ extern "C" int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0 && ldw >= C, "bad shape");
     FORGE_REQUIRE(ldo >= R && o_stride >= (C > 0 ? (C - 1) * ldo + R : 0), "output pitch too small");
     if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
-    FORGE_REQUIRE(W && perm_inv && Xout, "null pointer");
+    FORGE_REQUIRE(W && perm_inv && (Xout || W0out), "null pointer");
     dim3 grid((unsigned)forge::ceil_div(C, 64), (unsigned)forge::ceil_div(R, 64), (unsigned)batch);
     FORGE_REQUIRE(grid.y < 65536, "R too large");
     forge::KernelTiming timing("weight_to_solver_order", (hipStream_t)stream,
-                               (double)batch * R * C * (4.0 + (w_dtype == FORGE_F32 ? 4.0 : 2.0) * (W0out ? 2.0 : 1.0)),
+                               (double)batch * R * C * ((Xout ? 4.0 : 0.0) + (w_dtype == FORGE_F32 ? 4.0 : 2.0) * (W0out ? 2.0 : 1.0)),
                                forge::WORK_BYTES);
     const bool fast = w_dtype == FORGE_BF16 && (R % 256) == 0 && (C % 64) == 0 && (ldw % 4) == 0 &&
                       (w_stride % 4) == 0 && (reinterpret_cast<uintptr_t>(W) % 8) == 0 &&

@@ -379,6 +379,16 @@ __global__ __launch_bounds__(256) void lower_row_bound_kernel(const float* __res
     }
 }
 
+// X[b][c][r] = W0[b][c][r] for the first `rows` solver columns c of every matrix (the blocks that
+// no long product writes before they are swept).
+template <typename W0T>
+__global__ __launch_bounds__(256) void rows_from_w0_kernel(float* __restrict__ X, const W0T* __restrict__ W0,
+                                                           int64_t C, int64_t R, int64_t rows) {
+    const int64_t b = blockIdx.y, n = rows * R;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        X[b * C * R + i] = w0_as_f32(W0 + b * C * R + i);
+}
+
 // bound[m] = max_{t < m} |V[t, m]| for every column of the unit upper matrix V (the strict upper
 // triangle is all that the block updates read).  One workgroup per (128 columns, matrix).
 __global__ __launch_bounds__(256) void upper_column_bound_kernel(const float* __restrict__ V, int64_t C,
@@ -536,8 +546,8 @@ static bool sweep_reads_band_only(float* X, const float* U, int64_t batch, int64
 
 // Left-looking schedule for a batch of equally shaped matrices, errors (or, with W0, the
 // displacements) kept in X.
-static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U, const float* Lf,
-                         const int32_t* Linfo, const float* scalesT,
+static int sweep_batched(float* X, const void* W0, bool w0_bf16, bool x_from_w0, const float* U,
+                         const float* Lf, const int32_t* Linfo, const float* scalesT,
                          const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
                          uint32_t* M, const float* uinv, int64_t batch, int64_t C, int64_t R,
                          int64_t G, int bits, int sparse14, void* ws, int64_t ws_bytes,
@@ -573,8 +583,21 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U,
     // With the lower factor at hand the even blocks' A panels are formed from its rows: V is
     // then read only within one block of its diagonal (in-block chains, odd blocks' K = 128
     // products), provided every even block takes the piece path.
-    const bool from_lower = Lf != nullptr && ws && W0 &&
-                            sweep_reads_band_only(X, U, batch, C, R, split_bytes);
+    const bool all_pieces = ws && W0 && sweep_reads_band_only(X, U, batch, C, R, split_bytes);
+    const bool from_lower = Lf != nullptr && all_pieces;
+    // X not laid out by the caller: every block from the third on is first written by its long
+    // product, which then starts from W0; the first two are copied here
+    FORGE_REQUIRE(!x_from_w0 || all_pieces,
+                  "x_from_w0 needs the shape for which forge_gptq_sweep_direct_reads_band_only returns 1");
+    if (x_from_w0) {
+        const int64_t rows = C < 2 * forge::kBW ? C : 2 * forge::kBW;
+        const dim3 grid((unsigned)forge::ceil_div(rows * R, 256 * 8), (unsigned)batch);
+        if (w0_bf16)
+            rows_from_w0_kernel<uint16_t><<<grid, dim3(256), 0, st>>>(X, (const uint16_t*)W0, C, R, rows);
+        else
+            rows_from_w0_kernel<float><<<grid, dim3(256), 0, st>>>(X, (const float*)W0, C, R, rows);
+        FORGE_LAUNCH_CHECK();
+    }
     if (halves) {
         if (from_lower)
             lower_row_bound_kernel<<<dim3((unsigned)forge::ceil_div(C, 4), (unsigned)batch), dim3(256), 0, st>>>(
@@ -612,10 +635,12 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, const float* U,
                 if (from_lower) {
                     g.a_lower = Lf; g.a_lower_ld = C; g.a_lower_stride = C * C; g.a_info = Linfo;
                 }
+                if (x_from_w0) { g.x_init = W0; g.x_init_bf16 = w0_bf16; }
                 if (pairs && start + 2 * forge::kBW <= C) g.m1 = (int)(start + 2 * forge::kBW);
                 if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, ws, split_bytes)) return e;
                 g.m1 = (int)(start + bw);
                 g.a_lower = nullptr;
+                g.x_init = nullptr;
             } else {
                 g.k0 = (int)(start - forge::kBW);
                 if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
@@ -652,8 +677,8 @@ extern "C" int forge_gptq_sweep_batched(float* X, const float* U, const float* s
                                         uint8_t* qweight, uint32_t* M, const float* uinv,
                                         int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
                                         int sparse14, forge_stream_t stream) {
-    return sweep_batched(X, nullptr, false, U, nullptr, nullptr, scalesT, qzerosT, g_idx, qweight, M, uinv,
-                         batch, C, R, G, bits, sparse14, nullptr, 0, stream);
+    return sweep_batched(X, nullptr, false, false, U, nullptr, nullptr, scalesT, qzerosT, g_idx, qweight, M,
+                         uinv, batch, C, R, G, bits, sparse14, nullptr, 0, stream);
 }
 
 extern "C" int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_t R) {
@@ -672,8 +697,8 @@ extern "C" int forge_gptq_sweep_direct_reads_band_only(int64_t batch, int64_t C,
     return sweep_reads_band_only(aligned, aligned, batch, C, R, split_bytes) ? 1 : 0;
 }
 
-extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
-                                                  const float* L, const int32_t* info,
+extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, int x_from_w0,
+                                                  const float* V, const float* L, const int32_t* info,
                                                   const float* scalesT, const float* qzerosT,
                                                   const int32_t* g_idx, uint8_t* qweight,
                                                   uint32_t* M, const float* mdiag,
@@ -685,8 +710,8 @@ extern "C" int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int 
     FORGE_REQUIRE(!ws || ws_bytes >= forge_gptq_sweep_direct_workspace_bytes(batch, C, R),
                   "workspace of %lld bytes, %lld needed", (long long)ws_bytes,
                   (long long)forge_gptq_sweep_direct_workspace_bytes(batch, C, R));
-    return sweep_batched(X, W0, w0_dtype == FORGE_BF16, V, L, info, scalesT, qzerosT, g_idx, qweight, M,
-                         mdiag, batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
+    return sweep_batched(X, W0, w0_dtype == FORGE_BF16, x_from_w0 != 0, V, L, info, scalesT, qzerosT, g_idx,
+                         qweight, M, mdiag, batch, C, R, G, bits, sparse14, ws, ws_bytes, stream);
 }
 
 extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const float* V,
@@ -696,7 +721,7 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
                                                int64_t batch, int64_t C, int64_t R, int64_t G,
                                                int bits, int sparse14, void* ws, int64_t ws_bytes,
                                                forge_stream_t stream) {
-    return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, V, nullptr, nullptr, scalesT, qzerosT, g_idx,
+    return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, 0, V, nullptr, nullptr, scalesT, qzerosT, g_idx,
                                               qweight, M, mdiag, batch, C, R, G, bits, sparse14, ws,
                                               ws_bytes, stream);
 }

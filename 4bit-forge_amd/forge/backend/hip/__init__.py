@@ -53,8 +53,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
                                       vp], i32),
         "forge_gptq_sweep_direct_batched": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                              i32, i32, vp, i64, vp], i32),
-        "forge_gptq_sweep_direct_batched_w0": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64,
-                                                i64, i64, i32, i32, vp, i64, vp], i32),
+        "forge_gptq_sweep_direct_batched_w0": ([vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64,
+                                                i64, i64, i64, i32, i32, vp, i64, vp], i32),
         "forge_gptq_sweep_direct_reads_band_only": ([i64, i64, i64], i32),
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
@@ -309,7 +309,8 @@ class _HipKernels:
         return bool(self._lib.forge_gptq_sweep_direct_reads_band_only(int(B), int(C), int(R)))
 
     def gptq_sweep_direct_batched(self, X, V, scalesT, qzerosT, g_idx, bits, W0=None,
-                                  exact_chain=False, sparse14=False, mdiag=None, L=None, info=None):
+                                  exact_chain=False, sparse14=False, mdiag=None, L=None, info=None,
+                                  x_from_w0=False):
         """The sweep fed by the factor of H itself: V [B,C,C] = -M[t,k]/M[k,k] above the
         diagonal (``unit_upper_from_lower(L, info, negate=True)``).  X [B,C,R] f32 in/out
         (displacements w0 - deq on exit); W0: untouched copy of X (made here when None).
@@ -317,7 +318,8 @@ class _HipKernels:
         on a CPU) instead of blocked sums on the bf16 matrix pipe.  sparse14: the 1:4 joint
         solve, with mdiag [B,C] = diag(L) (1 where the factorisation failed).  L [B,C,C], info
         [B] int32: the lower factor V was made from and its failure flags; the long block
-        updates then take their V operand from L's rows (same numbers).
+        updates then take their V operand from L's rows (same numbers).  x_from_w0: X is
+        uninitialised on entry (shapes with sweep_direct_reads_band_only only).
         Returns qweight [B,C,R] u8 (and M [B, ceil(C/32), R] u32)."""
         _need_cuda(X, V, scalesT, qzerosT, g_idx, W0, L, info)
         B, C, R = X.shape
@@ -344,7 +346,8 @@ class _HipKernels:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
         with torch.cuda.device(X.device):
             self._check(self._lib.forge_gptq_sweep_direct_batched_w0(
-                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(V), _ptr(L), _ptr(info if L is not None else None),
+                _ptr(X), _ptr(W0), _dtype_code(W0), int(bool(x_from_w0)), _ptr(V), _ptr(L),
+                _ptr(info if L is not None else None),
                 _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q),
                 _ptr(M), _ptr(mdiag), B, C, R, G, int(bits), int(bool(sparse14)), _ptr(ws), nbytes,
                 _stream()))
@@ -471,12 +474,13 @@ class _HipKernels:
                 _stream()))
         return Hp, damp
 
-    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None):
+    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None, skip_out=False):
         """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c].
         With ``out`` [B,C,Rtot] (f32, contiguous) the rows land at out[:, :, row0:row0+R]: stacks
         that share a factor fill one tall matrix without being concatenated first.  ``out0``
         (shape of ``out``, dtype of W) receives the same values in W's own type: the untouched
-        copy for gptq_sweep_direct_batched(W0=...)."""
+        copy for gptq_sweep_direct_batched(W0=...).  skip_out: only ``out0`` is written
+        (``out`` then only gives the shape; for gptq_sweep_direct_batched(x_from_w0=True))."""
         _need_cuda(W, perm_inv, dead, out)
         B, R, C = W.shape
         assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
@@ -496,7 +500,8 @@ class _HipKernels:
         with torch.cuda.device(W.device):
             self._check(self._lib.forge_weight_to_solver_order_pair(
                 _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
-                ctypes.c_void_p(out.data_ptr() + 4 * row0), p0, Rtot, C * Rtot, B, R, C, _stream()))
+                None if skip_out else ctypes.c_void_p(out.data_ptr() + 4 * row0), p0, Rtot, C * Rtot, B,
+                R, C, _stream()))
         return out
 
     def codes_to_layer_order(self, q, perm_inv, out=None, row0=0, rows=None):

@@ -233,10 +233,13 @@ class ExpertGroupGPTQ:
                 W0 = None
                 if direct and len({self.W[i].dtype for i in job}) == 1:
                     W0 = torch.empty((B, C, R), dtype=self.W[job[0]].dtype, device=dev)
+                # where every column block is first written by its long product, that product
+                # starts from W0 and X is not laid out at all
+                lazy_x = W0 is not None and band
                 r0 = 0
                 for i in job:
                     kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0,
-                                                   out0=W0)
+                                                   out0=W0, skip_out=lazy_x)
                     r0 += sizes[i]
                 main.wait_stream(search)
                 for t in (scales, qzeros, sT, zT):
@@ -244,13 +247,14 @@ class ExpertGroupGPTQ:
                 M = None
                 if direct and sparse:
                     q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0,
-                                                             sparse14=True, mdiag=uinv, L=Lf, info=info)
+                                                             sparse14=True, mdiag=uinv, L=Lf, info=info,
+                                                             x_from_w0=lazy_x)
                 elif sparse:
                     q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
                                                       uinv=uinv)
                 elif direct:
                     q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0, L=Lf,
-                                                          info=info)
+                                                          info=info, x_from_w0=lazy_x)
                 else:
                     q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
                 del X, U, W0

@@ -188,10 +188,13 @@ int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_
  * take their V operand straight from the rows of L, the same numbers, and when
  * forge_gptq_sweep_direct_reads_band_only(batch, C, R) returns 1 (left-looking schedule, whole
  * 128 x 128 tiles, workspace given) V is read only within one 128-column block of its diagonal:
- * forge_unit_upper_from_lower with bit 3 then suffices. */
+ * forge_unit_upper_from_lower with bit 3 then suffices.
+ * x_from_w0 != 0 (only where that function returns 1; an error otherwise): X need not hold the
+ * weights on entry -- forge_weight_to_solver_order_pair may be called with Xout = NULL -- since
+ * every column block is then first written by its long product, which starts from W0. */
 int forge_gptq_sweep_direct_reads_band_only(int64_t batch, int64_t C, int64_t R);
-int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, const float* V,
-                                       const float* L, const int32_t* info,
+int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, int x_from_w0,
+                                       const float* V, const float* L, const int32_t* info,
                                        const float* scalesT, const float* qzerosT,
                                        const int32_t* g_idx, uint8_t* qweight, uint32_t* M,
                                        const float* mdiag, int64_t batch, int64_t C, int64_t R,
@@ -332,7 +335,8 @@ int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_s
 /* _pair: additionally writes W0out (may be NULL), the same matrix in the weights' own type
  * (w_dtype) with the same pitches in elements: the untouched copy that
  * forge_gptq_sweep_direct_batched_w0 reads beside the values it updates, produced in the pass
- * that lays X out instead of by a copy of X afterwards. */
+ * that lays X out instead of by a copy of X afterwards.  Xout may be NULL when only W0out is
+ * wanted. */
 int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
                                       const int64_t* perm_inv, const uint8_t* dead, float* Xout,
                                       void* W0out, int64_t ldo, int64_t o_stride, int64_t batch,

@@ -161,8 +161,9 @@ def test_direct_sweep_untouched_weights_from_the_layout_pass(hip, C, R, dtype):
 def test_direct_sweep_reads_its_v_operand_from_the_lower_factor(hip, C, products):
     """Given the lower factor, the long block updates form their V operand from its rows
     instead of reading V: same numbers, so codes and displacements are bit-identical, also
-    when everything of V beyond one block of its diagonal was never written (NaN here) and
-    for a matrix whose factorisation failed (V = I).  Left-looking schedule, both piece kinds."""
+    when everything of V beyond one block of its diagonal was never written (NaN here), when X
+    itself was never laid out (NaN; the products start from the untouched copy) and for a
+    matrix whose factorisation failed (V = I).  Left-looking schedule, both piece kinds."""
     B, R, gs = 3, 256, 128
     G = C // gs
     g0 = torch.Generator().manual_seed(C)
@@ -200,6 +201,21 @@ def test_direct_sweep_reads_its_v_operand_from_the_lower_factor(hip, C, products
         Xb = X.clone()
         qb = hip.gptq_sweep_direct_batched(Xb, Vb, *args, L=L, info=info)
         assert torch.equal(qa, qb) and torch.equal(Xa, Xb)
+        # X not laid out at all: every block is first written by its long product, which then
+        # starts from the untouched copy (f32 here; bf16 in the layout-pass test's shapes)
+        Xc = torch.full_like(X, float("nan"))
+        qc = hip.gptq_sweep_direct_batched(Xc, Vb, *args, W0=X.clone(), L=L, info=info, x_from_w0=True)
+        assert torch.equal(qa, qc) and torch.equal(Xa, Xc)
+        Wb = W.bfloat16()
+        X0 = torch.empty((B, C, R), dtype=torch.bfloat16, device=DEV)
+        pinv = torch.argsort(perm, dim=1).to(DEV)
+        Xd = hip.weight_to_solver_order(Wb.to(DEV), pinv, out=torch.full_like(X, float("nan")), out0=X0,
+                                        skip_out=True)
+        assert torch.isnan(Xd).all()
+        qd = hip.gptq_sweep_direct_batched(Xd, Vb, *args, W0=X0, L=L, info=info, x_from_w0=True)
+        Xe = hip.weight_to_solver_order(Wb.to(DEV), pinv)
+        qe = hip.gptq_sweep_direct_batched(Xe, V, *args)
+        assert torch.equal(qd, qe) and torch.equal(Xd, Xe)
     finally:
         hip.set_option("sweep_update_products", old)
         hip.set_option("sweep_schedule", 0)
