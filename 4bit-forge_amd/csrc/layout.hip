@@ -184,10 +184,12 @@ __global__ __launch_bounds__(256) void hessian_permute_kernel(
 // once per workgroup instead of once per row; rows move as float4 on both sides and the
 // two LDS row buffers alternate, which leaves one barrier per row.
 constexpr int kPermuteRows = 16;
+// lower_blocks: columns beyond the row's own 128-column block are not written (a factorisation
+// that works on the lower triangle in 128 x 128 blocks never reads them).
 template <int NCH>
 __global__ __launch_bounds__(256) void hessian_permute_rows_kernel(
     const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
-    float* __restrict__ Hp, int C) {
+    float* __restrict__ Hp, int C, bool lower_blocks) {
     extern __shared__ float srow[];                 // 2 * C floats
     const int64_t b = blockIdx.y;
     const int i0 = blockIdx.x * kPermuteRows;
@@ -238,8 +240,10 @@ __global__ __launch_bounds__(256) void hessian_permute_rows_kernel(
         const int i = i0 + r;
         const bool dead_i = db && db[i];
         float* __restrict__ dst = Hpb + (int64_t)i * C;
+        const int jmax = lower_blocks ? (i / 128 + 1) * 128 : C;
 #pragma unroll
         for (int u = 0; u < NCH; ++u) {
+            if (4 * (tid + 256 * u) >= jmax) continue;
             float4 v;
             v.x = buf[src_col[u][0]];
             v.y = buf[src_col[u][1]];
@@ -406,26 +410,27 @@ extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* per
     return forge_codes_to_layer_order_strided(qin, R, C * R, perm_inv, qout, batch, R, C, stream);
 }
 
-extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead,
-                                     float* Hp, float* damp, float rel_damp, int64_t batch,
-                                     int64_t C, forge_stream_t stream) {
+static int hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
+                           float* damp, float rel_damp, int64_t batch, int64_t C, bool lower_blocks,
+                           forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1, "bad shape");
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(H && perm && Hp && damp, "null pointer");
     FORGE_REQUIRE(H != Hp, "hessian_permute cannot run in place");
     hipStream_t st = (hipStream_t)stream;
-    forge::KernelTiming timing("hessian_permute", st, 8.0 * C * C * (double)batch, forge::WORK_BYTES);
+    forge::KernelTiming timing("hessian_permute", st, (lower_blocks ? 6.0 : 8.0) * C * C * (double)batch,
+                               forge::WORK_BYTES);
     const bool vec_ok = (C % 4) == 0 && C <= 8192 && (reinterpret_cast<uintptr_t>(H) % 16) == 0 &&
                         (reinterpret_cast<uintptr_t>(Hp) % 16) == 0;
     if (vec_ok) {
         const dim3 grid((unsigned)forge::ceil_div(C, kPermuteRows), (unsigned)batch);
         const size_t lds = 2 * (size_t)C * sizeof(float);   // <= 64 KB
         if (C <= 2048)
-            hessian_permute_rows_kernel<2><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+            hessian_permute_rows_kernel<2><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
         else if (C <= 4096)
-            hessian_permute_rows_kernel<4><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+            hessian_permute_rows_kernel<4><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
         else
-            hessian_permute_rows_kernel<8><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C);
+            hessian_permute_rows_kernel<8><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
     } else {
         const size_t lds = C <= kPermuteLdsFloats ? (size_t)C * sizeof(float) : 0;
         hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), lds, st>>>(
@@ -435,6 +440,18 @@ extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const 
     damp_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(Hp, damp, rel_damp, C);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
+}
+
+extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead,
+                                     float* Hp, float* damp, float rel_damp, int64_t batch,
+                                     int64_t C, forge_stream_t stream) {
+    return hessian_permute(H, perm, dead, Hp, damp, rel_damp, batch, C, false, stream);
+}
+
+extern "C" int forge_hessian_permute_lower(const float* H, const int64_t* perm, const uint8_t* dead,
+                                           float* Hp, float* damp, float rel_damp, int64_t batch,
+                                           int64_t C, forge_stream_t stream) {
+    return hessian_permute(H, perm, dead, Hp, damp, rel_damp, batch, C, true, stream);
 }
 
 extern "C" int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_t* packed,

@@ -68,6 +68,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_babai_solver": ([vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp, vp, i64, vp], i32),
         "forge_babai_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_permute": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
+        "forge_hessian_permute_lower": ([vp, vp, vp, vp, vp, f32, i64, i64, vp], i32),
         "forge_weight_to_solver_order": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_codes_to_layer_order": ([vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_weight_to_solver_order_strided": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, i64, i64,
@@ -99,6 +100,7 @@ EXPORTED_SYMBOLS = (
     "forge_hessian_workspace_bytes",
     "forge_hessian_update_static", "forge_hessian_update_static_max_rows",
     "forge_chol_inv_upper_batched", "forge_chol_workspace_bytes", "forge_hessian_permute",
+    "forge_hessian_permute_lower",
     "forge_weight_to_solver_order", "forge_codes_to_layer_order", "forge_pack_int4",
     "forge_weight_to_solver_order_strided", "forge_codes_to_layer_order_strided",
     "forge_weight_to_solver_order_pair", "forge_gptq_sweep_direct_batched_w0",
@@ -461,7 +463,10 @@ class _HipKernels:
                 int(G), _ptr(q), _ptr(ws), nbytes, _stream()))
         return q
 
-    def hessian_permute(self, H, perm, dead, rel_damp):
+    def hessian_permute(self, H, perm, dead, rel_damp, lower_blocks=False):
+        """Hp[b] = H[b][perm][:, perm] with dead rows/columns cleared (unit diagonal), damp[b] =
+        rel_damp * mean(diag).  lower_blocks: in row i only the columns up to the end of its own
+        128-column block are written (what the factorisations read)."""
         _need_cuda(H, perm, dead)
         B, C, _ = H.shape
         assert H.is_contiguous() and perm.dtype == torch.int64 and perm.is_contiguous()
@@ -469,9 +474,9 @@ class _HipKernels:
         Hp = torch.empty_like(H)
         damp = torch.empty(B, dtype=torch.float32, device=H.device)
         with torch.cuda.device(H.device):
-            self._check(self._lib.forge_hessian_permute(
-                _ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
-                _stream()))
+            fn = self._lib.forge_hessian_permute_lower if lower_blocks else self._lib.forge_hessian_permute
+            self._check(fn(_ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
+                           _stream()))
         return Hp, damp
 
     def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None, skip_out=False):

@@ -198,7 +198,9 @@ class ExpertGroupGPTQ:
                         qzeros = torch.cat([p[1].view(B, sizes[i], G) for p, i in zip(parts, job)], dim=1)
                     sT = scales.view(B, R, G).transpose(1, 2).contiguous()
                     zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
-                Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp))
+                # the factorisations read their input's lower triangle in 128 x 128 blocks only
+                Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp),
+                                                   lower_blocks=True)
                 if babai:
                     L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                     U = kernels.unit_upper_from_lower(L, info, upper_only=True)

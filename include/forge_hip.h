@@ -306,6 +306,12 @@ int forge_unit_upper_from_lower(const float* L, const int32_t* info, float* U, i
 int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
                           float* damp, float rel_damp, int64_t batch, int64_t C,
                           forge_stream_t stream);
+/* The same, but in row i only the columns up to the end of the row's own 128-column block are
+ * written (three quarters of the bytes): all that forge_chol_reverse_lower_batched and
+ * forge_chol_inv_upper_batched read of their input. */
+int forge_hessian_permute_lower(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
+                                float* damp, float rel_damp, int64_t batch, int64_t C,
+                                forge_stream_t stream);
 
 /* ------------------------------------------------------------------ layout helpers */
 

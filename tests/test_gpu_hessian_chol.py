@@ -255,6 +255,12 @@ def test_hessian_permute_sizes(hip, C):
     ref[d, :] = 0; ref[:, d] = 0; ref[d, d] = 1
     assert torch.equal(Hp[0].cpu(), ref)
     assert dmp[0].item() == pytest.approx(0.01 * ref.diag().mean().item(), rel=1e-5)
+    # the form that writes, in each row, only up to the end of the row's own 128-column block
+    # (the scalar form writes everything): equal there, and the same damping
+    Hl, dl = hip.hessian_permute(Hh.to(DEV), perm.to(DEV), dead.to(DEV), 0.01, lower_blocks=True)
+    idx = torch.arange(C)
+    keep = (idx[None, :] // 128) <= (idx[:, None] // 128)
+    assert torch.equal(Hl[0].cpu()[keep], ref[keep]) and torch.equal(dl, dmp)
 
 
 
