@@ -315,14 +315,18 @@ def test_expert_group_dead_and_zero_columns(zero_weight_column):
                 assert torch.equal(qo[:, [37, 200]], q[e].cpu()[:, [37, 200]])
 
 
-@pytest.mark.parametrize("factor_route", ["direct", "inverse"])
-def test_expert_group_sparse14_matches_per_expert_oracle(factor_route):
+@pytest.mark.parametrize("factor_route,R,C", [("direct", 64, 256), ("inverse", 64, 256),
+                                              ("direct", 128, 384)])
+def test_expert_group_sparse14_matches_per_expert_oracle(factor_route, R, C, hip):
     """algorithm="sparsegptq" through the batched front end: codes, keep-masks (solver order)
     and scales against oracle.GPTQ expert by expert; one kept weight in every group of four.
-    Both routes to the sweep's matrix."""
+    Both routes to the sweep's matrix; the last case with the left-looking schedule a large
+    batch takes (whole 128 x 128 tiles: long products from 16-bit pieces, their V operand from
+    the factor's rows, X never laid out)."""
     from forge.moe import ExpertGroupGPTQ
     g = torch.Generator().manual_seed(31)
-    E, R, C = 3, 64, 256
+    E = 3
+    left = R % 128 == 0
     Wg = (0.02 * torch.randn(E, R, C, generator=g)).bfloat16()
     Wu = (0.02 * torch.randn(E, R, C, generator=g)).bfloat16()
     xs = [torch.randn(n, C, generator=g).bfloat16() for n in (500, 320, 640)]
@@ -331,7 +335,13 @@ def test_expert_group_sparse14_matches_per_expert_oracle(factor_route):
               quantization_order="default", algorithm="sparsegptq")
     grp = ExpertGroupGPTQ([Wg.to(DEV), Wu.to(DEV)], device=DEV, factor_route=factor_route, **kw)
     grp.update(torch.cat(xs).to(DEV), offs)
-    (qg, sg, zg, Mg), (qu, su, zu, Mu) = grp.quantize(chunk=4)
+    if left:
+        hip.set_option("sweep_schedule", 1)
+    try:
+        assert hip.sweep_direct_reads_band_only(E, C, 2 * R) == left
+        (qg, sg, zg, Mg), (qu, su, zu, Mu) = grp.quantize(chunk=4)
+    finally:
+        hip.set_option("sweep_schedule", 0)
     for e in range(E):
         for W, (q, s, z, M) in ((Wg[e], (qg, sg, zg, Mg)), (Wu[e], (qu, su, zu, Mu))):
             o = oracle.GPTQ(linear(W), **kw)
@@ -557,9 +567,11 @@ def test_expert_group_few_tokens_routes_agree():
             assert err(q, s, z) < 0.5 * rtn
 
 
-def test_config2_qwen3_experts_at_full_shape():
+def test_config2_qwen3_experts_at_full_shape(hip):
     """Eight Qwen3-30B-A3B-shaped experts (768x2048 / 2048x768 bf16, asymmetric, MSE) with the
-    layer's ragged routing, batched, against per-expert oracle handles."""
+    layer's ragged routing, batched, against per-expert oracle handles.  With the left-looking
+    schedule that the layer's 128 experts take (eight alone would be swept right-looking): long
+    products from fp16 halves, their V operand from the factor's rows, X never laid out."""
     from forge.moe import ExpertGroupGPTQ
     moe = synth.qwen3_moe(experts=8, seed=6)
     E = 8
@@ -571,8 +583,13 @@ def test_config2_qwen3_experts_at_full_shape():
     dn = ExpertGroupGPTQ([moe.Wd.to(DEV)], device=DEV, **kw)
     gu.update(torch.cat(xs).to(DEV), offs)
     dn.update(torch.cat(hs).to(DEV), offs)
-    (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=8)
-    (qd, sd, zd), = dn.quantize(chunk=8)
+    hip.set_option("sweep_schedule", 1)
+    try:
+        assert hip.sweep_direct_reads_band_only(8, 2048, 1536) and hip.sweep_direct_reads_band_only(8, 768, 2048)
+        (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=8)
+        (qd, sd, zd), = dn.quantize(chunk=8)
+    finally:
+        hip.set_option("sweep_schedule", 0)
     # ||WX - QX||^2 summed over the tokens each expert saw: the layer's output error.  Per
     # expert the ratio is only meaningful with enough tokens (an expert that saw 3 tokens has
     # a rank-3 Hessian and its error moves by several % between equally good solutions).
