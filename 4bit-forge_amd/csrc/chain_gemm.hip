@@ -500,6 +500,13 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 // are folded into running totals every 128 k like the fp32 blocked sum, so the error is that
 // of an fp32 dot product.  Six bf16 MFMAs do the work of sixteen fp32 ones.
 //
+// Two-piece forms of the same kernel (template parameters NP, NPROD, HALF, MT below): two bf16
+// pieces each rounded to nearest with three products (~2^-17), and two fp16 halves of operands
+// scaled by powers of two with three products (fp32-grade); with two pieces one workgroup can
+// compute both m tiles of a 256-row problem (MT = 2).  What the matrix pipe sustains is set by
+// the device's power management (about two thirds of the nominal rate on operands with random
+// bits), so the kernel's job is to keep the pipe issuing and everything else out of its way.
+//
 // The fp32 matrix instruction shares the vector ALU, the bf16 one does not, so here the
 // split arithmetic has somewhere to run; but a wavefront that holds 128 accumulators and the
 // operands of the next step has no registers left for it.  Hence 8 wavefronts with two roles:
@@ -513,7 +520,8 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
 //                          pieces the global loads of stage s+4 into the registers that the
 //                          previous iteration consumed
 // The A panel is the same for every workgroup of a matrix, so it is split once by
-// split_a_panel_kernel into the exact LDS image of each stage and the producers only copy it.
+// split_a_panel_kernel (or split_a_panel_lower_kernel, from the rows of a lower triangular
+// factor) into the exact LDS image of each stage and the producers only copy it.
 // The multipliers never touch global memory: they start from zero, and at the end hand their
 // sums to the producers through LDS, who add the old X (X + s * sum, s = -1 for a negated A)
 // with coalesced 16-byte accesses.
