@@ -188,7 +188,8 @@ int64_t forge_gptq_sweep_direct_workspace_bytes(int64_t batch, int64_t C, int64_
  * take their V operand straight from the rows of L, the same numbers, and when
  * forge_gptq_sweep_direct_reads_band_only(batch, C, R) returns 1 (left-looking schedule, whole
  * 128 x 128 tiles, workspace given) V is read only within one 128-column block of its diagonal:
- * forge_unit_upper_from_lower with bit 3 then suffices.
+ * forge_unit_upper_from_lower with bit 3 then suffices (the answer depends on the library's
+ * options: do not change them between the query and the sweep).
  * x_from_w0 != 0 (only where that function returns 1; an error otherwise): X need not hold the
  * weights on entry -- forge_weight_to_solver_order_pair may be called with Xout = NULL -- since
  * every column block is then first written by its long product, which starts from W0. */
