@@ -480,8 +480,8 @@ int chol_run(float* H, const float* damp, float* U, float* udiag, int32_t* info,
     };
     // With the fp16 halves the long product is bound by reading the rows of the factor below
     // the block from HBM (64 flops per byte at 128 columns), so two block rows are brought up to
-    // date per product: every row read serves 256 columns (the second block's reading comes from
-    // L2).  The upper of the two then only lacks what the lower one adds once it is finished, a
+    // date per product: every row read serves 256 columns (one workgroup computes both blocks'
+    // tiles).  The upper of the two then only lacks what the lower one adds once it is finished, a
     // K = 128 product on the fp32 pipe.  (The pair's product also touches the block above the
     // upper row's diagonal block; nothing reads the upper triangle.)
     for (int a = nblk - 1; a >= 0;) {

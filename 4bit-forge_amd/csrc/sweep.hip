@@ -621,8 +621,9 @@ static int sweep_batched(float* X, const void* W0, bool w0_bf16, bool x_from_w0,
             // block is a full tile (fp32 matrix pipe otherwise).  That product is
             // bound by reading the displacement rows of all earlier columns from HBM, so full
             // blocks are brought up to date two at a time: every row read then serves 256
-            // columns (the second block's reading comes from L2), and the odd block only lacks
-            // what its even neighbour adds, a K = 128 product on the fp32 pipe.
+            // columns (one workgroup computes both blocks' tiles where the pieces allow it), and
+            // the odd block only lacks what its even neighbour adds, a K = 128 product on the
+            // fp32 pipe.
             const bool pairs = C % forge::kBW == 0;
             const bool odd = pairs && ((start / forge::kBW) & 1) != 0;
             if (!odd) {
