@@ -150,8 +150,12 @@ __device__ __forceinline__ float pow_abs(float e, float norm) {
 template <bool FLOOR>
 __device__ __forceinline__ float element_loss(float x, float s, float rcp, float q0, float maxq,
                                               float norm) {
-    const float q = clampf(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq);
-    const float diff = __builtin_fmaf(q - q0, s, -x);
+    // q - q0 directly: round(x*rcp) clamped to [-q0, maxq - q0].  q0 is a small integer, so
+    // this is the reference's clamp(round(fma(x, rcp, q0)), 0, maxq) - q0 except where the
+    // fma's own rounding lands x*rcp + q0 on a half-integer that x*rcp is not; there the two
+    // neighbouring levels are equally far from x to within one ulp of the sum.
+    const float qc = __builtin_amdgcn_fmed3f(__builtin_rintf(x * rcp), -q0, maxq - q0);
+    const float diff = __builtin_fmaf(qc, s, -x);
     return pow_abs(FLOOR ? fmaxf(fabsf(diff), 1e-20f) : fabsf(diff), norm);
 }
 
