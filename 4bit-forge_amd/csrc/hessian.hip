@@ -720,6 +720,46 @@ extern "C" int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_g
     return bytes;
 }
 
+// Shared body of the two grouped entry points: group e = rows row0[e] .. row0[e] + n[e] - 1.
+static int update_ranges(const void* X, int x_dtype, int64_t ldx, int64_t C, const int64_t* row0_host,
+                         const int64_t* n_host, int64_t n_groups, const float* alpha_host,
+                         const float* beta_host, float* H, void* ws, int64_t ws_bytes,
+                         hipStream_t st) {
+    std::vector<GroupDesc> gd((size_t)n_groups);
+    int64_t off = 0, total = 0;
+    int max_chunks = 0, min_tokens = 1 << 30;
+    bool any = false, any_blend = false;
+    for (int64_t e = 0; e < n_groups; ++e) {
+        const int64_t n = n_host[e];
+        FORGE_REQUIRE(n >= 0 && n < (1LL << 31) && row0_host[e] >= 0, "bad row range of group %lld",
+                      (long long)e);
+        gd[e].row0 = row0_host[e];
+        gd[e].n = (int32_t)n;
+        gd[e].nchunk = (int32_t)forge::ceil_div(n, 16);
+        gd[e].pack_off = off;
+        gd[e].alpha = alpha_host[e];
+        gd[e].beta = beta_host[e];
+        off += pack_units(n, C);
+        total += n;
+        if (gd[e].nchunk > max_chunks) max_chunks = gd[e].nchunk;
+        if (n > 0 && n < min_tokens) min_tokens = (int)n;
+        any |= n > 0;
+        any_blend |= n > 0 && beta_host[e] != 0.0f;
+    }
+    if (!any) return FORGE_OK;
+    FORGE_REQUIRE(X, "X is null");
+    FORGE_REQUIRE(ws_bytes >= forge_hessian_workspace_bytes(total, n_groups, C, x_dtype),
+                  "workspace too small");
+    GroupDesc* gd_dev = (GroupDesc*)ws;
+    const int64_t desc_bytes = round256(n_groups * (int64_t)sizeof(GroupDesc));
+    float* dnew = (float*)((char*)ws + desc_bytes);
+    uint4* pack = (uint4*)((char*)ws + desc_bytes + round256(n_groups * C * 4));
+    // through a pinned block of the library's own: the host does not wait for the copy
+    if (int rc = upload_async(gd.data(), n_groups * (int64_t)sizeof(GroupDesc), gd_dev, st)) return rc;
+    return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, min_tokens, any_blend,
+                         H, dnew, pack, st);
+}
+
 extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_t C,
                                             const int64_t* offsets_host, int64_t n_groups,
                                             const float* alpha_host, const float* beta_host,
@@ -731,41 +771,28 @@ extern "C" int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t 
                   (long long)ldx);
     if (n_groups == 0) return FORGE_OK;
     FORGE_REQUIRE(offsets_host && alpha_host && beta_host && H && ws, "null pointer");
-    const int64_t total = offsets_host[n_groups] - offsets_host[0];
-    FORGE_REQUIRE(total >= 0, "offsets must be non-decreasing");
-    FORGE_REQUIRE(total == 0 || X, "X is null");
-    FORGE_REQUIRE(ws_bytes >= forge_hessian_workspace_bytes(total, n_groups, C, x_dtype),
-                  "workspace too small");
-    hipStream_t st = (hipStream_t)stream;
-
-    std::vector<GroupDesc> gd((size_t)n_groups);
-    int64_t off = 0;
-    int max_chunks = 0, min_tokens = 1 << 30;
-    bool any = false, any_blend = false;
+    std::vector<int64_t> n((size_t)n_groups);
     for (int64_t e = 0; e < n_groups; ++e) {
-        const int64_t n = offsets_host[e + 1] - offsets_host[e];
-        FORGE_REQUIRE(n >= 0 && n < (1LL << 31), "offsets must be non-decreasing");
-        gd[e].row0 = offsets_host[e];
-        gd[e].n = (int32_t)n;
-        gd[e].nchunk = (int32_t)forge::ceil_div(n, 16);
-        gd[e].pack_off = off;
-        gd[e].alpha = alpha_host[e];
-        gd[e].beta = beta_host[e];
-        off += pack_units(n, C);
-        if (gd[e].nchunk > max_chunks) max_chunks = gd[e].nchunk;
-        if (n > 0 && n < min_tokens) min_tokens = (int)n;
-        any |= n > 0;
-        any_blend |= n > 0 && beta_host[e] != 0.0f;
+        n[e] = offsets_host[e + 1] - offsets_host[e];
+        FORGE_REQUIRE(n[e] >= 0, "offsets must be non-decreasing");
     }
-    if (!any) return FORGE_OK;
-    GroupDesc* gd_dev = (GroupDesc*)ws;
-    const int64_t desc_bytes = round256(n_groups * (int64_t)sizeof(GroupDesc));
-    float* dnew = (float*)((char*)ws + desc_bytes);
-    uint4* pack = (uint4*)((char*)ws + desc_bytes + round256(n_groups * C * 4));
-    // through a pinned block of the library's own: the host does not wait for the copy
-    if (int rc = upload_async(gd.data(), n_groups * (int64_t)sizeof(GroupDesc), gd_dev, st)) return rc;
-    return launch_update(X, x_dtype, ldx, C, gd_dev, n_groups, total, max_chunks, min_tokens, any_blend,
-                         H, dnew, pack, st);
+    return update_ranges(X, x_dtype, ldx, C, offsets_host, n.data(), n_groups, alpha_host, beta_host, H,
+                         ws, ws_bytes, (hipStream_t)stream);
+}
+
+extern "C" int forge_hessian_update_ranges(const void* X, int x_dtype, int64_t ldx, int64_t C,
+                                           const int64_t* row0_host, const int64_t* n_host,
+                                           int64_t n_groups, const float* alpha_host,
+                                           const float* beta_host, float* H, void* ws,
+                                           int64_t ws_bytes, forge_stream_t stream) {
+    FORGE_REQUIRE(x_dtype == FORGE_F32 || x_dtype == FORGE_BF16, "x_dtype=%d", x_dtype);
+    FORGE_REQUIRE(n_groups >= 0 && n_groups < 65536 && C >= 1 && C < (1 << 24) && ldx >= C,
+                  "bad shape n_groups=%lld C=%lld ldx=%lld", (long long)n_groups, (long long)C,
+                  (long long)ldx);
+    if (n_groups == 0) return FORGE_OK;
+    FORGE_REQUIRE(row0_host && n_host && alpha_host && beta_host && H && ws, "null pointer");
+    return update_ranges(X, x_dtype, ldx, C, row0_host, n_host, n_groups, alpha_host, beta_host, H, ws,
+                         ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int64_t forge_hessian_update_static_max_rows(int64_t C, int x_dtype) {

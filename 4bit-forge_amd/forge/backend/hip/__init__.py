@@ -59,6 +59,10 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_gptq_sweep_direct_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
+        "forge_hessian_update_ranges": ([vp, i32, i64, i64, vp, vp, i64, vp, vp, vp, vp, i64, vp], i32),
+        "forge_lowrank_factor": ([vp, vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_gptq_sweep_lowrank": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i64,
+                                      vp], i32),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
         "forge_hessian_update_static_max_rows": ([i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
@@ -108,7 +112,8 @@ EXPORTED_SYMBOLS = (
     "forge_fp8_e4m3_block_dequant", "forge_pack_sparsegptq14_to_u64x2",
     "forge_dequantize_groups", "forge_gather_scaled_rows",
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
-    "forge_babai_workspace_bytes",
+    "forge_babai_workspace_bytes", "forge_hessian_update_ranges", "forge_lowrank_factor",
+    "forge_gptq_sweep_lowrank",
 )
 
 
@@ -374,6 +379,60 @@ class _HipKernels:
                 nbytes, _stream()))
         return H
 
+    def hessian_update_ranges(self, X, row0, counts, H, alpha, beta):
+        """hessian_update_grouped with every group's rows given as (row0[e], counts[e]): groups
+        with counts[e] == 0 leave H[e] untouched wherever their rows lie in X."""
+        _need_cuda(X, H)
+        E = H.shape[0]
+        C = H.shape[-1]
+        assert len(row0) == E and len(counts) == E
+        r0 = (ctypes.c_int64 * E)(*[int(o) for o in row0])
+        cn = (ctypes.c_int64 * E)(*[int(o) for o in counts])
+        al = (ctypes.c_float * E)(*[float(a) for a in alpha])
+        be = (ctypes.c_float * E)(*[float(b) for b in beta])
+        assert X.stride(1) == 1 and H.is_contiguous() and H.dtype == torch.float32
+        total = sum(int(c) for c in counts)
+        nbytes = int(self._lib.forge_hessian_workspace_bytes(total, E, C, _dtype_code(X)))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=X.device)
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_hessian_update_ranges(
+                _ptr(X), _dtype_code(X), X.stride(0), C, r0, cn, E, al, be, _ptr(H), _ptr(ws), nbytes,
+                _stream()))
+        return H
+
+    def lowrank_factor(self, Bp, D):
+        """Bp [B,C,16] f32, D [B,C] f32 -> (Hm [B,C,16] f32, info [B] i32): the factor of
+        D + Bp^T Bp as the 16-vectors the low-rank sweep reads (see forge_hip.h)."""
+        _need_cuda(Bp, D)
+        B, C, n = Bp.shape
+        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and n == 16
+        assert D.is_contiguous() and D.dtype == torch.float32 and tuple(D.shape) == (B, C)
+        Hm = torch.empty_like(Bp)
+        info = torch.empty(B, dtype=torch.int32, device=Bp.device)
+        with torch.cuda.device(Bp.device):
+            self._check(self._lib.forge_lowrank_factor(_ptr(Bp), _ptr(D), _ptr(Hm), _ptr(info), B, C, n,
+                                                       _stream()))
+        return Hm, info
+
+    def gptq_sweep_lowrank(self, W0, Bp, Hm, info, scalesT, qzerosT, g_idx, bits):
+        """W0 [B,C,R] (f32/bf16, solver order), Bp/Hm [B,C,16], scalesT/qzerosT [B,G,R], g_idx
+        [B,C] i32 -> codes [B,C,R] u8."""
+        _need_cuda(W0, Bp, Hm, info, scalesT, qzerosT, g_idx)
+        B, C, R = W0.shape
+        G = scalesT.shape[1]
+        assert W0.is_contiguous() and Bp.is_contiguous() and Hm.is_contiguous()
+        assert tuple(Bp.shape) == (B, C, 16) and tuple(Hm.shape) == (B, C, 16)
+        assert scalesT.is_contiguous() and qzerosT.is_contiguous() and tuple(scalesT.shape) == (B, G, R)
+        assert tuple(qzerosT.shape) == (B, G, R) and scalesT.dtype == torch.float32
+        assert g_idx.dtype == torch.int32 and g_idx.is_contiguous() and tuple(g_idx.shape) == (B, C)
+        assert info.dtype == torch.int32 and info.numel() == B
+        q = torch.empty((B, C, R), dtype=torch.uint8, device=W0.device)
+        with torch.cuda.device(W0.device):
+            self._check(self._lib.forge_gptq_sweep_lowrank(
+                _ptr(W0), _dtype_code(W0), _ptr(Bp), _ptr(Hm), _ptr(info), _ptr(scalesT), _ptr(qzerosT),
+                _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), 16, _stream()))
+        return q
+
     def hessian_update_static(self, X, H, alpha, beta):
         """H [C,C] f32 <- beta*H + alpha * X^T X for X [n,C] (bf16/f32) through the entry point
         that allocates nothing (its workspace is a device array of the library's own; see
@@ -463,16 +522,24 @@ class _HipKernels:
                 int(G), _ptr(q), _ptr(ws), nbytes, _stream()))
         return q
 
-    def hessian_permute(self, H, perm, dead, rel_damp, lower_blocks=False):
+    def hessian_permute(self, H, perm, dead, rel_damp, lower_blocks=False, out=None):
         """Hp[b] = H[b][perm][:, perm] with dead rows/columns cleared (unit diagonal), damp[b] =
         rel_damp * mean(diag).  lower_blocks: in row i only the columns up to the end of its own
-        128-column block are written (what the factorisations read)."""
+        128-column block are written (what the factorisations read).  out = (Hp, damp): write
+        into these (contiguous slices of a larger batch, say) instead of new tensors."""
         _need_cuda(H, perm, dead)
         B, C, _ = H.shape
         assert H.is_contiguous() and perm.dtype == torch.int64 and perm.is_contiguous()
         assert dead.dtype == torch.uint8 and dead.is_contiguous()
-        Hp = torch.empty_like(H)
-        damp = torch.empty(B, dtype=torch.float32, device=H.device)
+        assert tuple(perm.shape) == (B, C) and tuple(dead.shape) == (B, C)
+        if out is not None:
+            Hp, damp = out
+            _need_cuda(Hp, damp)
+            assert Hp.is_contiguous() and Hp.dtype == torch.float32 and Hp.shape == H.shape
+            assert damp.is_contiguous() and damp.dtype == torch.float32 and damp.numel() == B
+        else:
+            Hp = torch.empty_like(H)
+            damp = torch.empty(B, dtype=torch.float32, device=H.device)
         with torch.cuda.device(H.device):
             fn = self._lib.forge_hessian_permute_lower if lower_blocks else self._lib.forge_hessian_permute
             self._check(fn(_ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
@@ -491,16 +558,21 @@ class _HipKernels:
         assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
         assert tuple(perm_inv.shape) == (B, C)
         assert dead is None or (dead.dtype == torch.uint8 and dead.is_contiguous())
-        if out is None:
-            out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
-            row0 = 0
-        assert out.is_contiguous() and out.dtype == torch.float32 and out.dim() == 3
-        Rtot = out.shape[2]
-        assert tuple(out.shape[:2]) == (B, C) and 0 <= row0 and row0 + R <= Rtot
+        if out is None and skip_out and out0 is not None:
+            shape = tuple(out0.shape)                 # only out0 is written: it also gives the shape
+        else:
+            if out is None:
+                out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
+                row0 = 0
+            assert out.is_contiguous() and out.dtype == torch.float32
+            shape = tuple(out.shape)
+        assert len(shape) == 3
+        Rtot = shape[2]
+        assert shape[:2] == (B, C) and 0 <= row0 and row0 + R <= Rtot
         p0 = None
         if out0 is not None:
             _need_cuda(out0)
-            assert out0.is_contiguous() and out0.dtype == W.dtype and out0.shape == out.shape
+            assert out0.is_contiguous() and out0.dtype == W.dtype and tuple(out0.shape) == shape
             p0 = ctypes.c_void_p(out0.data_ptr() + out0.element_size() * row0)
         with torch.cuda.device(W.device):
             self._check(self._lib.forge_weight_to_solver_order_pair(

@@ -8,6 +8,12 @@ takes the routed tokens of ALL experts at once (rows grouped by expert + offsets
 issues one ragged MFMA launch; ``quantize`` runs the scale search, the factorisation
 and the sweep for a chunk of experts per launch so that every kernel fills the GPU.
 Arithmetic per expert is the one of ``forge.gptq.GPTQ``.
+
+Experts that saw at most ``low_rank_tokens`` rows (most experts of a large routed layer see a
+handful of the calibration tokens, many none) never get a C x C Hessian: their rows are kept,
+and the solve runs on the closed form that H = D + B^T B has in those few rows
+(``kernels.lowrank_factor`` / ``kernels.gptq_sweep_lowrank``): the same result in exact
+arithmetic.
 """
 from __future__ import annotations
 
@@ -22,7 +28,8 @@ class ExpertGroupGPTQ:
     def __init__(self, weights: Sequence[torch.Tensor], bits: int = 4, group_size: int = 128,
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
-                 algorithm: str = "gptq", device=None, factor_route: str = "direct"):
+                 algorithm: str = "gptq", device=None, factor_route: str = "direct",
+                 low_rank_tokens: int = 16):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
@@ -31,7 +38,11 @@ class ExpertGroupGPTQ:
         errors; "direct" stops at the factor of H itself and sweeps with the displacements
         w0 - deq (``kernels.gptq_sweep_direct_batched``): the same solve in exact arithmetic
         at half the factorisation work, codes differing only where fp32 rounding decides a
-        near-tie."""
+        near-tie.
+        low_rank_tokens (0..16; algorithm "gptq" on the direct route, C a multiple of 16):
+        experts with at most this many calibration rows are solved from the rows themselves,
+        see the module text; 0 = every expert through its Hessian.  ``self.H[e]`` of such an
+        expert is never written."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         if factor_route not in ("direct", "inverse"):
@@ -56,6 +67,15 @@ class ExpertGroupGPTQ:
         self.rel_damp = rel_damp
         self.H: Optional[torch.Tensor] = None           # [E, C, C] f32
         self.num_samples = [0] * self.E                 # host-side counts
+        if not 0 <= int(low_rank_tokens) <= 16:
+            raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..16")
+        ok = algorithm == "gptq" and factor_route == "direct" and self.C % 16 == 0 \
+            and len({w.dtype for w in self.W}) == 1
+        self.low_rank_tokens = int(low_rank_tokens) if ok else 0
+        # rows of the experts that are still on the low-rank route, [E, 16, C] f32 (zero rows
+        # beyond num_samples[e]); low_rank[e] turns False for good once an expert has seen more
+        self.low_rank = [self.low_rank_tokens > 0] * self.E
+        self._kept: Optional[torch.Tensor] = None
         self.issue_non_invertible = torch.zeros(self.E, dtype=torch.bool)
 
     # ------------------------------------------------------------------ Hessians
@@ -72,15 +92,43 @@ class ExpertGroupGPTQ:
             X = X.contiguous()
         if self.H is None:
             self.H = torch.empty((self.E, self.C, self.C), dtype=torch.float32, device=self.device)
-        alpha, beta = [], []
+        if self._kept is None and self.low_rank_tokens:
+            self._kept = torch.zeros((self.E, 16, self.C), dtype=torch.float32, device=self.device)
+        row0, counts, alpha, beta = [], [], [], []
+        src, dst, late = [], [], []
         for e in range(self.E):
-            new = int(offsets[e + 1]) - int(offsets[e])
+            o, new = int(offsets[e]), int(offsets[e + 1]) - int(offsets[e])
             n = self.num_samples[e]
-            total = max(n + new, 1)
-            alpha.append(2.0 / total)
-            beta.append(n / total)
-            self.num_samples[e] = n + new
-        kernels.hessian_update_grouped(X, [int(o) for o in offsets], self.H, alpha, beta)
+            total = n + new
+            self.num_samples[e] = total
+            if self.low_rank[e] and total <= self.low_rank_tokens:
+                src.extend(range(o, o + new))                     # keep the rows, no Hessian
+                dst.extend(range(e * 16 + n, e * 16 + total))
+                new = 0
+            elif self.low_rank[e]:
+                self.low_rank[e] = False
+                if n > 0:
+                    late.append((e, n, o, new))                   # H[e] was never written
+                    new = 0
+            row0.append(o)
+            counts.append(new)
+            alpha.append(2.0 / max(total, 1))
+            beta.append(n / max(total, 1))
+        if src:
+            self._kept.view(self.E * 16, self.C)[torch.tensor(dst, device=self.device)] = \
+                X[torch.tensor(src, device=self.device)].float()
+        kernels.hessian_update_ranges(X, row0, counts, self.H, alpha, beta)
+        if late:
+            # experts that leave the low-rank route: their Hessian from the kept rows and the
+            # new ones together, (2/total) X^T X, what the running mean equals
+            parts, row0, counts, alpha = [], [0] * self.E, [0] * self.E, [0.0] * self.E
+            at = 0
+            for e, n, o, new in late:
+                parts += [self._kept[e, :n].to(X.dtype), X[o:o + new]]
+                row0[e], counts[e], alpha[e] = at, n + new, 2.0 / (n + new)
+                at += n + new
+                self._kept[e].zero_()
+            kernels.hessian_update_ranges(torch.cat(parts), row0, counts, self.H, alpha, [0.0] * self.E)
 
     add_batch = update
 
@@ -103,7 +151,21 @@ class ExpertGroupGPTQ:
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
         seen = torch.tensor([n > 0 for n in self.num_samples], device=dev)
         diag_all = self.H.diagonal(dim1=1, dim2=2)                        # [E, C] view
+        lr_host = list(self.low_rank)
+        any_lr = any(lr_host)
+        if any_lr:
+            # low-rank experts: diag(H) = (2/n) sum of squares of their kept rows (float64, rounded
+            # once, as the Hessian kernel does for the others); H[e] itself holds nothing
+            if self._kept is None:
+                self._kept = torch.zeros((E, 16, C), dtype=torch.float32, device=dev)
+            lr_dev = torch.tensor(lr_host, device=dev)
+            alpha32 = torch.tensor([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32,
+                                   device=dev)
+            d_lr = ((self._kept.double() ** 2).sum(dim=1) * alpha32.double()[:, None]).float()
+            diag_all = torch.where(lr_dev[:, None], d_lr, diag_all)
         bad = (~seen) | torch.isnan(diag_all).any(dim=1)
+        if any_lr:
+            diag_all = torch.where((bad & lr_dev)[:, None], torch.ones((), device=dev), diag_all)
         # Weights with pruned columns zeroed decide the (unpermuted-index) zero-column mask
         # that the reference applies to the permuted Hessian (forge/gptq.py:145-149).  A column
         # can only be all zero if its first rows are: one look at 8 rows of every expert (fp8-
@@ -116,26 +178,40 @@ class ExpertGroupGPTQ:
         # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
         # fraction of the fill rate)
         for e in host_flags[0].nonzero().flatten().tolist():
+            if lr_host[e]:
+                continue                       # no matrix: its rows count as none (below)
             self.H[e].zero_()
             self.H[e].diagonal().fill_(1.0)
+            diag_all = self.H.diagonal(dim1=1, dim2=2) if not any_lr else diag_all.index_fill(
+                0, torch.tensor([e], device=dev), 1.0)
         failed = []
         side = torch.cuda.Stream(device=dev) if overlap_scale_search else None   # default priority
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
         direct = self.algorithm in ("gptq", "sparsegptq") and self.factor_route == "direct"
+        babai = self.algorithm == "babai"
         outs = [[torch.empty((E, R, C), dtype=torch.uint8, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev),
                  torch.empty((E, R * G), dtype=torch.float32, device=dev)]
                 + ([torch.empty((E, (C + 31) // 32, R), dtype=torch.uint32, device=dev)] if sparse else [])
                 for R in sizes]
+
+        def runs_of(ids):
+            """[(first expert, count, position in ids)] of the consecutive runs of a sorted list."""
+            out = []
+            for pos, e in enumerate(ids):
+                if out and out[-1][0] + out[-1][1] == e:
+                    out[-1][1] += 1
+                else:
+                    out.append([e, 1, pos])
+            return [tuple(r) for r in out]
+
         for e0 in range(0, E, chunk):
             e1 = min(E, e0 + chunk)
             B = e1 - e0
-            H = self.H[e0:e1]
-            diag = H.diagonal(dim1=1, dim2=2)
+            diag = diag_all[e0:e1]
             dead = diag == 0                                             # [B, C]
-            babai = self.algorithm == "babai"
             if self.quantization_order == "activation":
                 # Babai walks back to front: ascending order (forge/gptq.py:107-108)
                 perm = torch.argsort(torch.where(dead, torch.ones_like(diag), diag), dim=1,
@@ -169,6 +245,9 @@ class ExpertGroupGPTQ:
                     if len(masks) > 1 else True
                 if babai:   # positions of the reference's order -> positions of the reversed one
                     masks = [m.flip(1).contiguous() for m in masks]
+            # the experts of the chunk by route (positions in the chunk, ascending)
+            lr_ids = [e - e0 for e in range(e0, e1) if lr_host[e]]
+            dn_ids = [e - e0 for e in range(e0, e1) if not lr_host[e]]
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
             for job in jobs:
@@ -198,78 +277,145 @@ class ExpertGroupGPTQ:
                         qzeros = torch.cat([p[1].view(B, sizes[i], G) for p, i in zip(parts, job)], dim=1)
                     sT = scales.view(B, R, G).transpose(1, 2).contiguous()
                     zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
-                # the factorisations read their input's lower triangle in 128 x 128 blocks only
-                Hp, damp = kernels.hessian_permute(H, perm, masks[job[0]], float(self.rel_damp),
-                                                   lower_blocks=True)
-                if babai:
-                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    U = kernels.unit_upper_from_lower(L, info, upper_only=True)
-                    del L
-                elif direct:
-                    L, info = kernels.chol_reverse_lower_batched(Hp, damp)
-                    # the sweep's long products read V straight from L's rows; where that covers
-                    # everything beyond one block of the diagonal, only that band of V is written
-                    band = kernels.sweep_direct_reads_band_only(B, C, R)
-                    U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True, band=band)
-                    if sparse:
-                        # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the
-                        # diagonal of the factor of H itself; U = I where it failed
-                        uinv = torch.where((info != 0)[:, None], torch.ones((), device=dev),
-                                           L.diagonal(dim1=1, dim2=2)).contiguous()
-                    Lf = L
-                    del L
-                elif sparse:
-                    # un-normalised factor, rows then scaled by the rounded reciprocal of the
-                    # diagonal as solver_sparsegptq14.cu:153-155 does
-                    U, udiag, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=False,
-                                                                   upper_only=True)
-                    uinv = (1.0 / udiag).contiguous()
-                    U.mul_(uinv.unsqueeze(-1))
-                else:
-                    U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
-                del Hp
-                failed.append((e0, info))
-                X = torch.empty((B, C, R), dtype=torch.float32, device=dev)
-                # the displacement form also reads the untouched weights: the layout pass writes
-                # them a second time in their own type instead of X being copied afterwards
-                W0 = None
-                if direct and len({self.W[i].dtype for i in job}) == 1:
-                    W0 = torch.empty((B, C, R), dtype=self.W[job[0]].dtype, device=dev)
-                # where every column block is first written by its long product, that product
-                # starts from W0 and X is not laid out at all
-                lazy_x = W0 is not None and band
-                r0 = 0
-                for i in job:
-                    kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0,
-                                                   out0=W0, skip_out=lazy_x)
-                    r0 += sizes[i]
-                main.wait_stream(search)
-                for t in (scales, qzeros, sT, zT):
-                    t.record_stream(main)
-                M = None
-                if direct and sparse:
-                    q, M = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0,
-                                                             sparse14=True, mdiag=uinv, L=Lf, info=info,
-                                                             x_from_w0=lazy_x)
-                elif sparse:
-                    q, M = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits, sparse14=True,
-                                                      uinv=uinv)
-                elif direct:
-                    q = kernels.gptq_sweep_direct_batched(X, U, sT, zT, g_idx, self.bits, W0=W0, L=Lf,
-                                                          info=info, x_from_w0=lazy_x)
-                else:
-                    q = kernels.gptq_sweep_batched(X, U, sT, zT, g_idx, self.bits)
-                del X, U, W0
-                Lf = None
+                mask = masks[job[0]]
+                waited = False
+
+                def layout_in(ids, W0, X=None, skip_out=False):
+                    """weights of the chunk's experts `ids` -> solver order, run by run"""
+                    for first, count, pos in runs_of(ids):
+                        sl = slice(pos, pos + count)
+                        ex = slice(e0 + first, e0 + first + count)
+                        ch = slice(first, first + count)
+                        r0 = 0
+                        for i in job:
+                            kernels.weight_to_solver_order(
+                                self.W[i][ex], perm_inv[ch], dead_u8[ch], out=None if X is None else X[sl],
+                                row0=r0, out0=None if W0 is None else W0[sl], skip_out=skip_out)
+                            r0 += sizes[i]
+
+                def layout_out(ids, q, M=None):
+                    for first, count, pos in runs_of(ids):
+                        sl = slice(pos, pos + count)
+                        ex = slice(e0 + first, e0 + first + count)
+                        ch = slice(first, first + count)
+                        r0 = 0
+                        for i in job:
+                            Ri = sizes[i]
+                            kernels.codes_to_layer_order(q[sl], perm_inv[ch], out=outs[i][0][ex], row0=r0,
+                                                         rows=Ri)
+                            if M is not None:
+                                outs[i][3][ex] = M[sl, :, r0:r0 + Ri]
+                            r0 += Ri
+
+                # ---------------------------------------------------------- low-rank experts
+                if lr_ids:
+                    li = torch.tensor(lr_ids, device=dev)
+                    Bl = len(lr_ids)
+                    msk = mask[li].bool()                                   # [Bl, C], solver order
+                    rows = self._kept[e0:e1][li]                            # [Bl, 16, C]
+                    rows = torch.where(bad[e0:e1][li][:, None, None], torch.zeros((), device=dev), rows)
+                    root = alpha32[e0:e1][li].double().sqrt()[:, None, None]
+                    Bp = torch.gather((rows.double() * root).float(), 2,
+                                      perm[li][:, None, :].expand(-1, 16, -1))
+                    Bp = Bp.masked_fill(msk[:, None, :], 0).transpose(1, 2).contiguous()   # [Bl, C, 16]
+                    dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[li], 1, perm[li]))
+                    D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
+                    Hm, info = kernels.lowrank_factor(Bp, D.contiguous())
+                    failed.append((torch.tensor([e0 + i for i in lr_ids]), info))
+                    W0 = torch.empty((Bl, C, R), dtype=self.W[job[0]].dtype, device=dev)
+                    layout_in(lr_ids, W0, skip_out=True)
+                    main.wait_stream(search)
+                    waited = True
+                    for t in (scales, qzeros, sT, zT):
+                        t.record_stream(main)
+                    q = kernels.gptq_sweep_lowrank(W0, Bp, Hm, info, sT[li], zT[li], g_idx[li].contiguous(),
+                                                   self.bits)
+                    layout_out(lr_ids, q)
+                    del W0, q, Bp, Hm
+
+                # ---------------------------------------------------------- through the Hessian
+                if dn_ids:
+                    whole = len(dn_ids) == B
+                    di = None if whole else torch.tensor(dn_ids, device=dev)
+                    pick = (lambda t: t) if whole else (lambda t: t[di].contiguous())
+                    Bd = len(dn_ids)
+                    # the factorisations read their input's lower triangle in 128 x 128 blocks only
+                    if whole:
+                        Hp, damp = kernels.hessian_permute(self.H[e0:e1], perm, mask, float(self.rel_damp),
+                                                           lower_blocks=True)
+                    else:
+                        Hp = torch.empty((Bd, C, C), dtype=torch.float32, device=dev)
+                        damp = torch.empty(Bd, dtype=torch.float32, device=dev)
+                        for first, count, pos in runs_of(dn_ids):
+                            ch = slice(first, first + count)
+                            kernels.hessian_permute(self.H[e0 + first:e0 + first + count], perm[ch], mask[ch],
+                                                    float(self.rel_damp), lower_blocks=True,
+                                                    out=(Hp[pos:pos + count], damp[pos:pos + count]))
+                    if babai:
+                        L, info = kernels.chol_reverse_lower_batched(Hp, damp)
+                        U = kernels.unit_upper_from_lower(L, info, upper_only=True)
+                        del L
+                    elif direct:
+                        L, info = kernels.chol_reverse_lower_batched(Hp, damp)
+                        # the sweep's long products read V straight from L's rows; where that covers
+                        # everything beyond one block of the diagonal, only that band of V is written
+                        band = kernels.sweep_direct_reads_band_only(Bd, C, R)
+                        U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True, band=band)
+                        if sparse:
+                            # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the
+                            # diagonal of the factor of H itself; U = I where it failed
+                            uinv = torch.where((info != 0)[:, None], torch.ones((), device=dev),
+                                               L.diagonal(dim1=1, dim2=2)).contiguous()
+                        Lf = L
+                        del L
+                    elif sparse:
+                        # un-normalised factor, rows then scaled by the rounded reciprocal of the
+                        # diagonal as solver_sparsegptq14.cu:153-155 does
+                        U, udiag, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=False,
+                                                                       upper_only=True)
+                        uinv = (1.0 / udiag).contiguous()
+                        U.mul_(uinv.unsqueeze(-1))
+                    else:
+                        U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
+                    del Hp
+                    failed.append((torch.tensor([e0 + i for i in dn_ids]), info))
+                    X = torch.empty((Bd, C, R), dtype=torch.float32, device=dev)
+                    # the displacement form also reads the untouched weights: the layout pass writes
+                    # them a second time in their own type instead of X being copied afterwards
+                    W0 = None
+                    if direct and len({self.W[i].dtype for i in job}) == 1:
+                        W0 = torch.empty((Bd, C, R), dtype=self.W[job[0]].dtype, device=dev)
+                    # where every column block is first written by its long product, that product
+                    # starts from W0 and X is not laid out at all
+                    lazy_x = W0 is not None and band
+                    layout_in(dn_ids, W0, X, skip_out=lazy_x)
+                    if not waited:
+                        main.wait_stream(search)
+                        for t in (scales, qzeros, sT, zT):
+                            t.record_stream(main)
+                    sTd, zTd, gd = pick(sT), pick(zT), pick(g_idx)
+                    M = None
+                    if direct and sparse:
+                        q, M = kernels.gptq_sweep_direct_batched(X, U, sTd, zTd, gd, self.bits, W0=W0,
+                                                                 sparse14=True, mdiag=uinv, L=Lf, info=info,
+                                                                 x_from_w0=lazy_x)
+                    elif sparse:
+                        q, M = kernels.gptq_sweep_batched(X, U, sTd, zTd, gd, self.bits, sparse14=True,
+                                                          uinv=uinv)
+                    elif direct:
+                        q = kernels.gptq_sweep_direct_batched(X, U, sTd, zTd, gd, self.bits, W0=W0, L=Lf,
+                                                              info=info, x_from_w0=lazy_x)
+                    else:
+                        q = kernels.gptq_sweep_batched(X, U, sTd, zTd, gd, self.bits)
+                    del X, U, W0
+                    Lf = None
+                    layout_out(dn_ids, q, M)
                 r0 = 0
                 for i in job:
                     Ri = sizes[i]
-                    kernels.codes_to_layer_order(q, perm_inv, out=outs[i][0][e0:e1], row0=r0, rows=Ri)
                     outs[i][1][e0:e1] = scales.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     outs[i][2][e0:e1] = qzeros.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
-                    if sparse:
-                        outs[i][3][e0:e1] = M[:, :, r0:r0 + Ri]
                     r0 += Ri
-        for e0, info in failed:
-            self.issue_non_invertible[e0:e0 + info.numel()] |= (info > 0).cpu()
+        for ids, info in failed:
+            self.issue_non_invertible[ids] |= (info > 0).cpu()
         return [tuple(o) for o in outs]

@@ -202,6 +202,29 @@ int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, i
                                        int64_t G, int bits, int sparse14, void* ws,
                                        int64_t ws_bytes, forge_stream_t stream);
 
+/* GPTQ.quantize for a layer that saw n <= 16 calibration rows (gptq.py:128-166 with
+ * solver.cu:9-154), without the C x C Hessian.  Such a layer's damped, pruned, permuted Hessian
+ * (gptq.py:97-119,145-153) is  D + Bp^T Bp  with  Bp[k][j] = sqrt(2/n) x_j[perm[k]]  (0 in pruned
+ * and all-zero-weight columns) and D[k] = damp (+ 1 in those columns), and every number the sweep
+ * takes from the factor of that matrix is an n-term dot product:
+ *   forge_lowrank_factor: Bp [batch][C][16] f32 (rows beyond n zero), D [batch][C] f32 ->
+ *     Hm [batch][C][16] f32 with  Hm[k] . Bp[t] = M[k][t] / M[k][k]  (t < k) for the lower factor
+ *     M of forge_chol_reverse_lower_batched; info[b] = 1 where a pivot is not positive (or NaN).
+ *     One wavefront per matrix, recurrence in float64.
+ *   forge_gptq_sweep_lowrank: W0 [batch][C][R] (w0_dtype f32 or bf16, solver order, pruned columns
+ *     zero: forge_weight_to_solver_order_pair's W0out), scalesT/qzerosT [batch][G][R], g_idx
+ *     [batch][C] -> qweight [batch][C][R] u8.  Column k of a row is quantised at
+ *     w0_k + Hm[k] . a  and then adds (w0_k - deq_k) Bp[k] to the row's 16-vector a: the values
+ *     forge_gptq_sweep_direct_batched reaches in exact arithmetic, the reference's quantiser
+ *     (solver.cu:9-23).  Matrices with info != 0 are swept uncoupled (gptq.py:172-175).
+ * n must be 16 (pad with zero rows; a layer that saw no rows at all is Bp = 0), C % 16 == 0. */
+int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, int32_t* info, int64_t batch,
+                         int64_t C, int64_t n, forge_stream_t stream);
+int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, const float* Hm,
+                             const int32_t* info, const float* scalesT, const float* qzerosT,
+                             const int32_t* g_idx, uint8_t* qweight, int64_t batch, int64_t C,
+                             int64_t R, int64_t G, int bits, int64_t n, forge_stream_t stream);
+
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private
  * copy with the dequantised values), A [C, C] f32 upper Cholesky factor of H (H = A^T A),
@@ -237,6 +260,14 @@ int forge_hessian_update_grouped(const void* X, int x_dtype, int64_t ldx, int64_
                                  void* ws, int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_hessian_workspace_bytes(int64_t total_rows, int64_t n_groups, int64_t C,
                                       int x_dtype);
+/* The same update with each group's rows given as a range of its own, rows row0_host[e] ..
+ * row0_host[e] + n_host[e] - 1 of X: groups need not follow one another, so that a caller can
+ * leave out the experts it handles by forge_lowrank_factor (n_host[e] = 0 leaves H[e] untouched)
+ * while their rows stay where they are in X.  total_rows of the workspace query = sum of n_host. */
+int forge_hessian_update_ranges(const void* X, int x_dtype, int64_t ldx, int64_t C,
+                                const int64_t* row0_host, const int64_t* n_host, int64_t n_groups,
+                                const float* alpha_host, const float* beta_host, float* H, void* ws,
+                                int64_t ws_bytes, forge_stream_t stream);
 
 /* GPTQ.update for ONE matrix without any allocation: H <- beta*H + alpha * X^T X for the
  * n_rows rows of X ([n_rows, C], pitch ldx, dtype x_dtype), the same kernels and the same
