@@ -60,7 +60,11 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_hessian_update_grouped": ([vp, i32, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp], i32),
         "forge_hessian_workspace_bytes": ([i64, i64, i64, i32], i64),
         "forge_hessian_update_ranges": ([vp, i32, i64, i64, vp, vp, i64, vp, vp, vp, vp, i64, vp], i32),
-        "forge_lowrank_factor": ([vp, vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_lowrank_factor": ([vp, vp, vp, vp, i64, i64, i64, vp, i64, vp], i32),
+        "forge_lowrank_workspace_bytes": ([i64, i64, i64], i64),
+        "forge_gptq_sweep_lowrank_mixed": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
+                                            vp], i32),
+        "forge_round_to_nearest": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, i64, i32, vp], i32),
         "forge_gptq_sweep_lowrank": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i64,
                                       vp], i32),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
@@ -113,7 +117,8 @@ EXPORTED_SYMBOLS = (
     "forge_dequantize_groups", "forge_gather_scaled_rows",
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
     "forge_babai_workspace_bytes", "forge_hessian_update_ranges", "forge_lowrank_factor",
-    "forge_gptq_sweep_lowrank",
+    "forge_gptq_sweep_lowrank", "forge_round_to_nearest", "forge_lowrank_workspace_bytes",
+    "forge_gptq_sweep_lowrank_mixed",
 )
 
 
@@ -400,28 +405,77 @@ class _HipKernels:
                 _stream()))
         return H
 
-    def lowrank_factor(self, Bp, D):
-        """Bp [B,C,16] f32, D [B,C] f32 -> (Hm [B,C,16] f32, info [B] i32): the factor of
-        D + Bp^T Bp as the 16-vectors the low-rank sweep reads (see forge_hip.h)."""
+    def round_to_nearest(self, W, scales, qzeros, gs, bits, out=None):
+        """W [B,R,C] (bf16/f32, layer layout), scales/qzeros [B,R*G] -> codes [B,R,C] u8 of the
+        reference's quantiser applied weight by weight (a layer with H = I)."""
+        _need_cuda(W, scales, qzeros, out)
+        B, R, C = W.shape
+        G = (C + gs - 1) // gs
+        assert W.stride(2) == 1 and scales.is_contiguous() and qzeros.is_contiguous()
+        assert tuple(scales.shape) == (B, R * G) and tuple(qzeros.shape) == (B, R * G)
+        assert scales.dtype == torch.float32 and qzeros.dtype == torch.float32
+        if out is None:
+            out = torch.empty((B, R, C), dtype=torch.uint8, device=W.device)
+        assert out.is_contiguous() and out.dtype == torch.uint8 and tuple(out.shape) == (B, R, C)
+        with torch.cuda.device(W.device):
+            self._check(self._lib.forge_round_to_nearest(
+                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(scales), _ptr(qzeros), _ptr(out),
+                B, R, C, int(gs), int(bits), _stream()))
+        return out
+
+    def lowrank_factor(self, Bp, D, out=None):
+        """Bp [B,C,n] f32 (n = 16, 32 or 64), D [B,C] f32 -> (Hm [B,C,n] f32, info [B] i32): the
+        factor of D + Bp^T Bp as the n-vectors the low-rank sweep reads (see forge_hip.h)."""
         _need_cuda(Bp, D)
         B, C, n = Bp.shape
-        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and n == 16
+        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and n in (16, 32, 64)
         assert D.is_contiguous() and D.dtype == torch.float32 and tuple(D.shape) == (B, C)
-        Hm = torch.empty_like(Bp)
-        info = torch.empty(B, dtype=torch.int32, device=Bp.device)
+        if out is not None:
+            Hm, info = out
+            _need_cuda(Hm, info)
+            assert Hm.is_contiguous() and Hm.dtype == torch.float32 and Hm.shape == Bp.shape
+            assert info.is_contiguous() and info.dtype == torch.int32 and info.numel() == B
+        else:
+            Hm = torch.empty_like(Bp)
+            info = torch.empty(B, dtype=torch.int32, device=Bp.device)
+        nbytes = int(self._lib.forge_lowrank_workspace_bytes(B, C, n))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=Bp.device)
         with torch.cuda.device(Bp.device):
             self._check(self._lib.forge_lowrank_factor(_ptr(Bp), _ptr(D), _ptr(Hm), _ptr(info), B, C, n,
-                                                       _stream()))
+                                                       _ptr(ws), nbytes, _stream()))
         return Hm, info
 
-    def gptq_sweep_lowrank(self, W0, Bp, Hm, info, scalesT, qzerosT, g_idx, bits):
-        """W0 [B,C,R] (f32/bf16, solver order), Bp/Hm [B,C,16], scalesT/qzerosT [B,G,R], g_idx
-        [B,C] i32 -> codes [B,C,R] u8."""
+    def gptq_sweep_lowrank_mixed(self, W0, Bp, Hm, ns, info, scalesT, qzerosT, g_idx, bits):
+        """gptq_sweep_lowrank for matrices of different n in one launch: ns[b] in (16, 32, 64);
+        Bp/Hm flat f32 buffers holding matrix b's [C, ns[b]] vectors one after the other."""
         _need_cuda(W0, Bp, Hm, info, scalesT, qzerosT, g_idx)
         B, C, R = W0.shape
         G = scalesT.shape[1]
+        assert len(ns) == B and all(int(n) in (16, 32, 64) for n in ns)
+        total = C * sum(int(n) for n in ns)
         assert W0.is_contiguous() and Bp.is_contiguous() and Hm.is_contiguous()
-        assert tuple(Bp.shape) == (B, C, 16) and tuple(Hm.shape) == (B, C, 16)
+        assert Bp.numel() == total and Hm.numel() == total and Bp.dtype == Hm.dtype == torch.float32
+        assert scalesT.is_contiguous() and qzerosT.is_contiguous() and tuple(scalesT.shape) == (B, G, R)
+        assert tuple(qzerosT.shape) == (B, G, R) and scalesT.dtype == torch.float32
+        assert g_idx.dtype == torch.int32 and g_idx.is_contiguous() and tuple(g_idx.shape) == (B, C)
+        assert info.dtype == torch.int32 and info.is_contiguous() and info.numel() == B
+        q = torch.empty((B, C, R), dtype=torch.uint8, device=W0.device)
+        nh = (ctypes.c_int64 * max(B, 1))(*[int(n) for n in ns])
+        with torch.cuda.device(W0.device):
+            self._check(self._lib.forge_gptq_sweep_lowrank_mixed(
+                _ptr(W0), _dtype_code(W0), _ptr(Bp), _ptr(Hm), nh, _ptr(info), _ptr(scalesT),
+                _ptr(qzerosT), _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), _stream()))
+        return q
+
+    def gptq_sweep_lowrank(self, W0, Bp, Hm, info, scalesT, qzerosT, g_idx, bits):
+        """W0 [B,C,R] (f32/bf16, solver order), Bp/Hm [B,C,n] (n = 16, 32 or 64), scalesT/qzerosT
+        [B,G,R], g_idx [B,C] i32 -> codes [B,C,R] u8."""
+        _need_cuda(W0, Bp, Hm, info, scalesT, qzerosT, g_idx)
+        B, C, R = W0.shape
+        G = scalesT.shape[1]
+        n = Bp.shape[2]
+        assert W0.is_contiguous() and Bp.is_contiguous() and Hm.is_contiguous()
+        assert n in (16, 32, 64) and tuple(Bp.shape) == (B, C, n) and tuple(Hm.shape) == (B, C, n)
         assert scalesT.is_contiguous() and qzerosT.is_contiguous() and tuple(scalesT.shape) == (B, G, R)
         assert tuple(qzerosT.shape) == (B, G, R) and scalesT.dtype == torch.float32
         assert g_idx.dtype == torch.int32 and g_idx.is_contiguous() and tuple(g_idx.shape) == (B, C)
@@ -430,7 +484,7 @@ class _HipKernels:
         with torch.cuda.device(W0.device):
             self._check(self._lib.forge_gptq_sweep_lowrank(
                 _ptr(W0), _dtype_code(W0), _ptr(Bp), _ptr(Hm), _ptr(info), _ptr(scalesT), _ptr(qzerosT),
-                _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), 16, _stream()))
+                _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), n, _stream()))
         return q
 
     def hessian_update_static(self, X, H, alpha, beta):

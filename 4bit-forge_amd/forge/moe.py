@@ -29,7 +29,7 @@ class ExpertGroupGPTQ:
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
                  algorithm: str = "gptq", device=None, factor_route: str = "direct",
-                 low_rank_tokens: int = 16):
+                 low_rank_tokens: int = 64):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
@@ -39,7 +39,7 @@ class ExpertGroupGPTQ:
         w0 - deq (``kernels.gptq_sweep_direct_batched``): the same solve in exact arithmetic
         at half the factorisation work, codes differing only where fp32 rounding decides a
         near-tie.
-        low_rank_tokens (0..16; algorithm "gptq" on the direct route, C a multiple of 16):
+        low_rank_tokens (0..64; algorithm "gptq" on the direct route, C a multiple of 16):
         experts with at most this many calibration rows are solved from the rows themselves,
         see the module text; 0 = every expert through its Hessian.  ``self.H[e]`` of such an
         expert is never written."""
@@ -67,13 +67,14 @@ class ExpertGroupGPTQ:
         self.rel_damp = rel_damp
         self.H: Optional[torch.Tensor] = None           # [E, C, C] f32
         self.num_samples = [0] * self.E                 # host-side counts
-        if not 0 <= int(low_rank_tokens) <= 16:
-            raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..16")
+        if not 0 <= int(low_rank_tokens) <= 64:
+            raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..64")
         ok = algorithm == "gptq" and factor_route == "direct" and self.C % 16 == 0 \
             and len({w.dtype for w in self.W}) == 1
         self.low_rank_tokens = int(low_rank_tokens) if ok else 0
-        # rows of the experts that are still on the low-rank route, [E, 16, C] f32 (zero rows
+        # rows of the experts that are still on the low-rank route, [E, _cap, C] f32 (zero rows
         # beyond num_samples[e]); low_rank[e] turns False for good once an expert has seen more
+        self._cap = next(n for n in (16, 32, 64) if n >= max(self.low_rank_tokens, 1))
         self.low_rank = [self.low_rank_tokens > 0] * self.E
         self._kept: Optional[torch.Tensor] = None
         self.issue_non_invertible = torch.zeros(self.E, dtype=torch.bool)
@@ -93,7 +94,7 @@ class ExpertGroupGPTQ:
         if self.H is None:
             self.H = torch.empty((self.E, self.C, self.C), dtype=torch.float32, device=self.device)
         if self._kept is None and self.low_rank_tokens:
-            self._kept = torch.zeros((self.E, 16, self.C), dtype=torch.float32, device=self.device)
+            self._kept = torch.zeros((self.E, self._cap, self.C), dtype=torch.float32, device=self.device)
         row0, counts, alpha, beta = [], [], [], []
         src, dst, late = [], [], []
         for e in range(self.E):
@@ -103,7 +104,7 @@ class ExpertGroupGPTQ:
             self.num_samples[e] = total
             if self.low_rank[e] and total <= self.low_rank_tokens:
                 src.extend(range(o, o + new))                     # keep the rows, no Hessian
-                dst.extend(range(e * 16 + n, e * 16 + total))
+                dst.extend(range(e * self._cap + n, e * self._cap + total))
                 new = 0
             elif self.low_rank[e]:
                 self.low_rank[e] = False
@@ -115,7 +116,7 @@ class ExpertGroupGPTQ:
             alpha.append(2.0 / max(total, 1))
             beta.append(n / max(total, 1))
         if src:
-            self._kept.view(self.E * 16, self.C)[torch.tensor(dst, device=self.device)] = \
+            self._kept.view(self.E * self._cap, self.C)[torch.tensor(dst, device=self.device)] = \
                 X[torch.tensor(src, device=self.device)].float()
         kernels.hessian_update_ranges(X, row0, counts, self.H, alpha, beta)
         if late:
@@ -157,7 +158,7 @@ class ExpertGroupGPTQ:
             # low-rank experts: diag(H) = (2/n) sum of squares of their kept rows (float64, rounded
             # once, as the Hessian kernel does for the others); H[e] itself holds nothing
             if self._kept is None:
-                self._kept = torch.zeros((E, 16, C), dtype=torch.float32, device=dev)
+                self._kept = torch.zeros((E, self._cap, C), dtype=torch.float32, device=dev)
             lr_dev = torch.tensor(lr_host, device=dev)
             alpha32 = torch.tensor([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32,
                                    device=dev)
@@ -186,6 +187,9 @@ class ExpertGroupGPTQ:
                 0, torch.tensor([e], device=dev), 1.0)
         failed = []
         side = torch.cuda.Stream(device=dev) if overlap_scale_search else None   # default priority
+        # the low-rank experts' kernels are chains of dependent steps on a few wavefronts: on a
+        # stream of their own they run beside the other experts' matrix products
+        lr_side = torch.cuda.Stream(device=dev) if overlap_scale_search and any_lr else None
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
@@ -246,7 +250,8 @@ class ExpertGroupGPTQ:
                 if babai:   # positions of the reference's order -> positions of the reversed one
                     masks = [m.flip(1).contiguous() for m in masks]
             # the experts of the chunk by route (positions in the chunk, ascending)
-            lr_ids = [e - e0 for e in range(e0, e1) if lr_host[e]]
+            none_ids = [e - e0 for e in range(e0, e1) if lr_host[e] and bool(host_flags[0, e])]
+            lr_ids = [e - e0 for e in range(e0, e1) if lr_host[e] and not bool(host_flags[0, e])]
             dn_ids = [e - e0 for e in range(e0, e1) if not lr_host[e]]
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
@@ -278,7 +283,6 @@ class ExpertGroupGPTQ:
                     sT = scales.view(B, R, G).transpose(1, 2).contiguous()
                     zT = qzeros.view(B, R, G).transpose(1, 2).contiguous()
                 mask = masks[job[0]]
-                waited = False
 
                 def layout_in(ids, W0, X=None, skip_out=False):
                     """weights of the chunk's experts `ids` -> solver order, run by run"""
@@ -308,30 +312,64 @@ class ExpertGroupGPTQ:
                             r0 += Ri
 
                 # ---------------------------------------------------------- low-rank experts
-                if lr_ids:
-                    li = torch.tensor(lr_ids, device=dev)
-                    Bl = len(lr_ids)
-                    msk = mask[li].bool()                                   # [Bl, C], solver order
-                    rows = self._kept[e0:e1][li]                            # [Bl, 16, C]
-                    rows = torch.where(bad[e0:e1][li][:, None, None], torch.zeros((), device=dev), rows)
-                    root = alpha32[e0:e1][li].double().sqrt()[:, None, None]
-                    Bp = torch.gather((rows.double() * root).float(), 2,
-                                      perm[li][:, None, :].expand(-1, 16, -1))
-                    Bp = Bp.masked_fill(msk[:, None, :], 0).transpose(1, 2).contiguous()   # [Bl, C, 16]
-                    dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[li], 1, perm[li]))
-                    D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
-                    Hm, info = kernels.lowrank_factor(Bp, D.contiguous())
-                    failed.append((torch.tensor([e0 + i for i in lr_ids]), info))
-                    W0 = torch.empty((Bl, C, R), dtype=self.W[job[0]].dtype, device=dev)
-                    layout_in(lr_ids, W0, skip_out=True)
-                    main.wait_stream(search)
-                    waited = True
-                    for t in (scales, qzeros, sT, zT):
-                        t.record_stream(main)
-                    q = kernels.gptq_sweep_lowrank(W0, Bp, Hm, info, sT[li], zT[li], g_idx[li].contiguous(),
-                                                   self.bits)
-                    layout_out(lr_ids, q)
-                    del W0, q, Bp, Hm
+                lr_stream = main
+                if lr_ids or none_ids:
+                    lr_stream = lr_side if lr_side is not None and dn_ids else main
+                    lr_stream.wait_stream(main)
+                with torch.cuda.stream(lr_stream):
+                    # by the number of rows the kernels are compiled for: 16, 32 or 64
+                    buckets = []
+                    for lo, nr in ((0, 16), (16, 32), (32, 64)):
+                        ids = [i for i in lr_ids if lo < self.num_samples[e0 + i] <= nr]
+                        if ids:
+                            buckets.append((nr, ids))
+                    # one sweep launch for all of them: their vectors laid end to end
+                    ids_all = [i for _, ids in buckets for i in ids]
+                    ns = [nr for nr, ids in buckets for _ in ids]
+                    if ids_all:
+                        Bp_all = torch.empty(C * sum(ns), dtype=torch.float32, device=dev)
+                        Hm_all = torch.empty_like(Bp_all)
+                        info = torch.empty(len(ids_all), dtype=torch.int32, device=dev)
+                        W0 = torch.empty((len(ids_all), C, R), dtype=self.W[job[0]].dtype, device=dev)
+                    pos = at = 0
+                    for nr, ids in buckets:
+                        li = torch.tensor(ids, device=dev)
+                        msk = mask[li].bool()                               # [Bl, C], solver order
+                        root = alpha32[e0:e1][li].double().sqrt()[:, None, None]
+                        Bp = torch.gather((self._kept[e0:e1][li][:, :nr].double() * root).float(), 2,
+                                          perm[li][:, None, :].expand(-1, nr, -1))
+                        Bp = Bp.masked_fill(msk[:, None, :], 0).transpose(1, 2)            # [Bl, C, nr]
+                        span = slice(at, at + len(ids) * C * nr)
+                        Bpv = Bp_all[span].view(len(ids), C, nr)
+                        Bpv.copy_(Bp)
+                        dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[li], 1, perm[li]))
+                        D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
+                        kernels.lowrank_factor(Bpv, D.contiguous(),
+                                               out=(Hm_all[span].view(len(ids), C, nr), info[pos:pos + len(ids)]))
+                        layout_in(ids, W0[pos:pos + len(ids)], skip_out=True)
+                        pos += len(ids)
+                        at += len(ids) * C * nr
+                    if lr_ids or none_ids:
+                        lr_stream.wait_stream(search)
+                        for t in (scales, qzeros, sT, zT) + tuple(x for p in parts for x in p):
+                            t.record_stream(lr_stream)
+                    if ids_all:
+                        failed.append((torch.tensor([e0 + i for i in ids_all]), info))
+                        la = torch.tensor(ids_all, device=dev)
+                        q = kernels.gptq_sweep_lowrank_mixed(W0, Bp_all, Hm_all, ns, info, sT[la], zT[la],
+                                                             g_idx[la].contiguous(), self.bits)
+                        pos = 0
+                        for nr, ids in buckets:
+                            layout_out(ids, q[pos:pos + len(ids)])
+                            pos += len(ids)
+                        del W0, q, Bp_all, Hm_all
+                    # experts without a single row (or with NaN rows): H = I, plain rounding
+                    for first, count, _ in runs_of(none_ids):
+                        ex = slice(e0 + first, e0 + first + count)
+                        ch = slice(first, first + count)
+                        for (sc_i, qz_i), i in zip(parts, job):
+                            kernels.round_to_nearest(self.W[i][ex], sc_i[ch], qz_i[ch], gs, self.bits,
+                                                     out=outs[i][0][ex])
 
                 # ---------------------------------------------------------- through the Hessian
                 if dn_ids:
@@ -389,10 +427,9 @@ class ExpertGroupGPTQ:
                     # starts from W0 and X is not laid out at all
                     lazy_x = W0 is not None and band
                     layout_in(dn_ids, W0, X, skip_out=lazy_x)
-                    if not waited:
-                        main.wait_stream(search)
-                        for t in (scales, qzeros, sT, zT):
-                            t.record_stream(main)
+                    main.wait_stream(search)
+                    for t in (scales, qzeros, sT, zT):
+                        t.record_stream(main)
                     sTd, zTd, gd = pick(sT), pick(zT), pick(g_idx)
                     M = None
                     if direct and sparse:
@@ -410,6 +447,10 @@ class ExpertGroupGPTQ:
                     del X, U, W0
                     Lf = None
                     layout_out(dn_ids, q, M)
+                main.wait_stream(search)
+                main.wait_stream(lr_stream)
+                for t in (scales, qzeros):
+                    t.record_stream(main)
                 r0 = 0
                 for i in job:
                     Ri = sizes[i]

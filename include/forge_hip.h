@@ -202,24 +202,43 @@ int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, i
                                        int64_t G, int bits, int sparse14, void* ws,
                                        int64_t ws_bytes, forge_stream_t stream);
 
-/* GPTQ.quantize for a layer that saw n <= 16 calibration rows (gptq.py:128-166 with
+/* GPTQ.quantize for a layer that saw n <= 64 calibration rows (gptq.py:128-166 with
  * solver.cu:9-154), without the C x C Hessian.  Such a layer's damped, pruned, permuted Hessian
  * (gptq.py:97-119,145-153) is  D + Bp^T Bp  with  Bp[k][j] = sqrt(2/n) x_j[perm[k]]  (0 in pruned
  * and all-zero-weight columns) and D[k] = damp (+ 1 in those columns), and every number the sweep
  * takes from the factor of that matrix is an n-term dot product:
- *   forge_lowrank_factor: Bp [batch][C][16] f32 (rows beyond n zero), D [batch][C] f32 ->
- *     Hm [batch][C][16] f32 with  Hm[k] . Bp[t] = M[k][t] / M[k][k]  (t < k) for the lower factor
+ *   forge_lowrank_factor: Bp [batch][C][n] f32 (rows beyond the layer's own count zero), D
+ *     [batch][C] f32 -> Hm [batch][C][n] f32 with  Hm[k] . Bp[t] = M[k][t] / M[k][k]  (t < k) for the lower factor
  *     M of forge_chol_reverse_lower_batched; info[b] = 1 where a pivot is not positive (or NaN).
- *     One wavefront per matrix, recurrence in float64.
+ *     Recurrence in float64, 128-column blocks side by side; ws: device workspace of
+ *     forge_lowrank_workspace_bytes(batch, C, n), 16-byte aligned.
  *   forge_gptq_sweep_lowrank: W0 [batch][C][R] (w0_dtype f32 or bf16, solver order, pruned columns
  *     zero: forge_weight_to_solver_order_pair's W0out), scalesT/qzerosT [batch][G][R], g_idx
  *     [batch][C] -> qweight [batch][C][R] u8.  Column k of a row is quantised at
- *     w0_k + Hm[k] . a  and then adds (w0_k - deq_k) Bp[k] to the row's 16-vector a: the values
+ *     w0_k + Hm[k] . a  and then adds (w0_k - deq_k) Bp[k] to the row's n-vector a: the values
  *     forge_gptq_sweep_direct_batched reaches in exact arithmetic, the reference's quantiser
  *     (solver.cu:9-23).  Matrices with info != 0 are swept uncoupled (gptq.py:172-175).
- * n must be 16 (pad with zero rows; a layer that saw no rows at all is Bp = 0), C % 16 == 0. */
+ * n is 16, 32 or 64 (pad with zero rows), C % 16 == 0. */
+/* GPTQ.quantize for a layer that saw NO calibration rows: H = I (gptq.py:97-99), its factor is
+ * the identity, nothing couples the columns and the sweep of solver.cu:9-154 is its quantiser
+ * (solver.cu:9-23) applied to every weight.  W [batch][R][C] (w_dtype f32 or bf16, row pitch ldw,
+ * batch stride w_stride, layer layout), scales/qzeros [batch][R*G] (index r*G + c/gs) ->
+ * qweight [batch][R][C] u8, layer layout: no permutation, no layout pass. */
+int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                           const float* scales, const float* qzeros, uint8_t* qweight, int64_t batch,
+                           int64_t R, int64_t C, int64_t gs, int bits, forge_stream_t stream);
 int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, int32_t* info, int64_t batch,
-                         int64_t C, int64_t n, forge_stream_t stream);
+                         int64_t C, int64_t n, void* ws, int64_t ws_bytes, forge_stream_t stream);
+int64_t forge_lowrank_workspace_bytes(int64_t batch, int64_t C, int64_t n);
+/* forge_gptq_sweep_lowrank for matrices of different n in ONE launch (each of the three sizes
+ * alone leaves most of the GPU idle): n_host[b] in {16, 32, 64} (host array), and matrix b's
+ * vectors start C * (n_host[0] + ... + n_host[b-1]) floats into Bp and into Hm, i.e. the per-size
+ * [batch_n][C][n] arrays laid end to end in batch order.  Everything else as above. */
+int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, const float* Bp, const float* Hm,
+                                   const int64_t* n_host, const int32_t* info, const float* scalesT,
+                                   const float* qzerosT, const int32_t* g_idx, uint8_t* qweight,
+                                   int64_t batch, int64_t C, int64_t R, int64_t G, int bits,
+                                   forge_stream_t stream);
 int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, const float* Hm,
                              const int32_t* info, const float* scalesT, const float* qzerosT,
                              const int32_t* g_idx, uint8_t* qweight, int64_t batch, int64_t C,

@@ -1,4 +1,4 @@
-"""The low-rank route (layers that saw at most 16 calibration rows) against dense float64
+"""The low-rank route (layers that saw at most 64 calibration rows) against dense float64
 algebra and against the route through the Hessian.
 
 The closed forms are pinned by the dense computation they replace: the lower factor M of
@@ -26,7 +26,7 @@ def _lower_factor(H):
 
 def _problem(C, n, seed, dead=()):
     g = torch.Generator().manual_seed(seed)
-    Bp = torch.zeros(C, 16)
+    Bp = torch.zeros(C, 16 if n <= 16 else 32 if n <= 32 else 64)
     Bp[:, :n] = torch.randn(C, n, generator=g) * (2.0 / max(n, 1)) ** 0.5
     Bp[:, 0] *= torch.linspace(3.0, 0.3, C)                 # an "activation-ordered" spread
     D = torch.full((C,), 0.02)
@@ -36,7 +36,7 @@ def _problem(C, n, seed, dead=()):
     return Bp, D
 
 
-@pytest.mark.parametrize("n", [0, 1, 5, 16])
+@pytest.mark.parametrize("n", [0, 1, 5, 16, 23, 64])
 def test_factor_matches_the_dense_float64_factor(hip, n):
     C = 384
     probs = [_problem(C, n, s, dead=(7, 200) if s == 1 else ()) for s in range(3)]
@@ -78,7 +78,8 @@ def _float64_gptq(W, H, s, z, maxq=15.0):
 
 
 @pytest.mark.parametrize("n,dtype", [(1, torch.float32), (4, torch.bfloat16), (16, torch.bfloat16),
-                                     (0, torch.float32)])
+                                     (0, torch.float32), (30, torch.bfloat16), (64, torch.float32),
+                                     (50, torch.bfloat16)])
 def test_sweep_matches_float64_gptq_on_the_dense_factor(hip, n, dtype):
     C, R, gs = 256, 300, 128
     G = C // gs
@@ -120,7 +121,7 @@ def test_failed_factor_sweeps_uncoupled(hip):
     s, z = oracle.build_group_meta_packed(W0.t().contiguous().reshape(R, gs), 4, True)
     g_idx = torch.zeros(C, dtype=torch.int32)
     args = (s.view(1, 1, R).to(DEV), z.view(1, 1, R).to(DEV), g_idx[None].to(DEV), 4)
-    Hm = torch.full((1, C, 16), float("nan"), device=DEV)
+    Hm = torch.full((1, C, 16), float("nan"), device=DEV)          # never read
     bad = torch.ones(1, dtype=torch.int32, device=DEV)
     q = hip.gptq_sweep_lowrank(W0[None].to(DEV), Bp[None].to(DEV), Hm, bad, *args)[0].cpu()
     # the quantiser's fma(x, 1/(s+eps), z): the product of two floats is exact in float64
@@ -129,6 +130,24 @@ def test_failed_factor_sweeps_uncoupled(hip):
     v = (W0.double() * inv.double() + z[None, :].double()).float()
     want = torch.clamp(torch.round(v), 0, 15).to(torch.uint8)
     assert torch.equal(q, want)
+
+
+@pytest.mark.parametrize("dtype,C,gs", [(torch.bfloat16, 512, 128), (torch.float32, 200, 64),
+                                         (torch.bfloat16, 77, 32)])
+def test_round_to_nearest_is_the_quantiser_weight_by_weight(hip, dtype, C, gs):
+    g = torch.Generator().manual_seed(4)
+    B, R = 3, 37
+    G = (C + gs - 1) // gs
+    W = (0.02 * torch.randn(B, R, C + 8, generator=g)).to(dtype)[:, :, :C]     # pitched rows
+    Wp = torch.nn.functional.pad(W.float(), (0, G * gs - C))
+    s, z = oracle.build_group_meta_packed(Wp.reshape(B * R * G, gs), 4, False)
+    s, z = s.view(B, R * G), z.view(B, R * G)
+    q = hip.round_to_nearest(W.to(DEV), s.to(DEV), z.to(DEV), gs, 4).cpu()
+    se = s.view(B, R, G).repeat_interleave(gs, dim=2)[:, :, :C]
+    ze = z.view(B, R, G).repeat_interleave(gs, dim=2)[:, :, :C]
+    inv = 1.0 / (se + 1e-12)
+    v = (W.double() * inv.double() + ze.double()).float()    # fma: the product is exact in float64
+    assert torch.equal(q, torch.clamp(torch.round(v), 0, 15).to(torch.uint8))
 
 
 def test_hessian_ranges_skip_groups_in_place(hip):
