@@ -226,7 +226,9 @@ class ExpertGroupGPTQ:
             if babai:
                 # the solve runs as a forward sweep over the reversed order (see forge/gptq.py)
                 perm = perm.flip(1).contiguous()
-            perm_inv = torch.argsort(perm, dim=1)
+            # the inverse permutation by a scatter (argsort(perm), forge/gptq.py:113, sorts again)
+            perm_inv = torch.empty_like(perm).scatter_(
+                1, perm, torch.arange(C, device=dev).expand(B, C))
             g_idx = (perm // gs).to(torch.int32).contiguous()
             dead_u8 = dead.to(torch.uint8).contiguous()
             has_dead = bool(host_flags[1, e0:e1].any())

@@ -10,7 +10,10 @@ forge.synth.deepseek_v3_moe (seed 0) on the GPU.  One STEP = one pass of the hot
 one chunk of experts, everything already resident in HBM: ragged Hessian accumulation for
 gate/up and for down, then per expert two factorisations (gate and up share theirs), three
 scale searches and three sweeps.  Successive steps walk through the layer's experts chunk
-by chunk (their routed-token lists differ).
+by chunk (128 experts a step; their routed-token lists differ).  Experts with at most 64
+routed rows (most of them: 8192 tokens over 256 experts with Zipf popularity) take the
+library's low-rank route, which reaches the same result from the rows themselves without a
+C x C Hessian; `config.experts_by_route` counts them.
 value = experts quantised per second = steps * chunk / elapsed.
 
 After the timed steps:
@@ -22,6 +25,7 @@ After the timed steps:
   and with random operands;
 * `reference_route`: the same steps on the reference's route (factor of inv(H), fp32-chain
   sweep: every integer stage bit-exact against the CPU oracle);
+* `every_expert_through_its_hessian`: the same steps with the low-rank route switched off;
 * `hessian_buckets`: the rank-k kernel alone at 16 / 256 / 1024 / 4096 tokens per expert;
 * `hbm_kernels`: min/max grid, int4 pack, fp8 block dequant at benchmark shapes;
 * `other_configs`: configs 1, 2, 4, 5 of the benchmark definition, end to end;
@@ -69,11 +73,15 @@ KERNEL_BOUND = {
     "sweep_block": ("valu", "valu_f32", 1.0),
     "sweep_block_sparse14": ("valu", "valu_f32", 1.0),
     "chol_diag_block": ("latency", "valu_f32", 1.0),
+    # the low-rank route: a serial chain per output row (sweep) and per 128-column block (factor)
+    "lowrank_sweep": ("valu", "valu_f32", 1.0),
+    "lowrank_factor": ("latency", "valu_f32", 1.0),
+    "round_to_nearest": ("hbm", "hbm", 1.0),
 }
 
 CONFIGS = {
     "deepseek_v3": dict(n_experts=256, hidden=7168, inter=2048, tokens=8192, fp8=True,
-                        symmetric=True, order="activation", chunk=64),
+                        symmetric=True, order="activation", chunk=128),
     "qwen3": dict(n_experts=128, hidden=2048, inter=768, tokens=4096, fp8=False,
                   symmetric=False, order="default", chunk=128),
 }
@@ -106,7 +114,7 @@ def make_workload(name, cfg, chunk, seed=0):
 STREAMS = []
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"):
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=64):
     """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
     jobs one after the other (per-kernel event times are then exclusive)."""
     import torch
@@ -128,7 +136,7 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
         offs.append(offs[-1] + wl["counts"][e])
     kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"],
               quantization_scale="mse" if mse else "absmax", quantization_order=cfg["order"],
-              rel_damp=0.01, device="cuda", factor_route=factor_route)
+              rel_damp=0.01, device="cuda", factor_route=factor_route, low_rank_tokens=low_rank_tokens)
     # gate/up (shared Hessian) and down are independent: one host thread and one HIP stream
     # each, so that the MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale
     # search and the latency-bound diagonal blocks of the other
@@ -162,6 +170,14 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
     for s in STREAMS:
         cur.wait_stream(s)
     return results[0::2], results[1::2]
+
+
+def route_counts(wl, chunk, low_rank_tokens):
+    """How many of the layer's experts take which route (whole layer, by routed rows)."""
+    c = wl["counts"]
+    none = sum(1 for n in c if n == 0) if low_rank_tokens else 0
+    low = sum(1 for n in c if 0 < n <= low_rank_tokens)
+    return dict(no_rows=none, low_rank=low, through_hessian=len(c) - none - low)
 
 
 def timed_steps(wl, cfg, chunk, steps, warmup, first_step=0, **kw):
@@ -273,8 +289,8 @@ def mfma_ceiling():
 
 
 def hbm_kernels(wl):
-    """min/max grid, int4 pack and fp8 block dequant on the chunk's gate_proj stack (64 x 2048 x
-    7168): achieved GB/s of the algorithmic bytes against 8 TB/s."""
+    """min/max grid, int4 pack and fp8 block dequant on the chunk's gate_proj stack (chunk x 2048
+    x 7168): achieved GB/s of the algorithmic bytes against 8 TB/s."""
     import torch
     from forge.backend.hip import kernels
     Wg = wl["Wg"]
@@ -431,6 +447,9 @@ def main():
     ap.add_argument("--factor-route", default="direct", choices=["direct", "inverse"],
                     help="direct (default): sweep fed by the factor of H itself; inverse: the "
                          "reference's factor of inv(H) and fp32-chain sweep")
+    ap.add_argument("--low-rank-tokens", type=int, default=64,
+                    help="experts with at most this many routed rows are solved from the rows themselves "
+                         "(0: every expert through its Hessian)")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run of "
@@ -456,12 +475,12 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    elapsed = timed_steps(wl, cfg, chunk, a.steps, a.warmup, mse=mse, factor_route=a.factor_route)
+    route = dict(factor_route=a.factor_route, low_rank_tokens=a.low_rank_tokens)
+    elapsed = timed_steps(wl, cfg, chunk, a.steps, a.warmup, mse=mse, **route)
 
     # one more step with per-kernel HIP-event timing (on the stream the kernels run on); its
     # jobs run one after the other so that no kernel's time includes another stream's work
-    stats = timing_pass(lambda: run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False,
-                                         factor_route=a.factor_route))
+    stats = timing_pass(lambda: run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False, **route))
     breakdown = kernel_table(stats)
     # `roofline` describes the longest-running kernel among those that an HBM or a matrix-pipe
     # roofline bounds; a kernel bound by the vector ALU (the shrink search, the in-block chains)
@@ -473,7 +492,7 @@ def main():
     roofline = dict(kernel=dom, bound="mfma" if bound == "mfma" else "hbm", achieved=d["rate"],
                     peak=PEAK[peak_key], unit=d["rate_unit"], frac=d["frac"],
                     traffic=measured_traffic(a.config, chunk, dom)
-                    if a.split == 1 and a.factor_route == "direct" and mse else None,
+                    if a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 64 else None,
                     avg_launch_us=d["avg_us"], launches=d["launches"],
                     note="achieved = algorithmic work (2*M*N*K counted once per fp32 product) / event time")
     if by_time != dom:
@@ -500,7 +519,9 @@ def main():
                                f" 4-bit {'sym' if cfg['symmetric'] else 'asym'} g128"
                                f" {'act-order' if cfg['order'] == 'activation' else 'no act-order'}"
                                f" {'mse' if mse else 'absmax'} grid",
-                   "experts_per_step": chunk, "factor_route": a.factor_route},
+                   "experts_per_step": chunk, "factor_route": a.factor_route,
+                   "low_rank_tokens": a.low_rank_tokens if a.factor_route == "direct" else 0,
+                   "experts_by_route": route_counts(wl, chunk, a.low_rank_tokens if a.factor_route == "direct" else 0)},
         "roofline": roofline,
         "kernels": breakdown,
     }
@@ -520,6 +541,11 @@ def main():
         out["reference_route" if other == "inverse" else "direct_route"] = dict(
             factor_route=other, ms_per_step=round(1e3 * dt / a.steps, 2),
             value=round(a.steps * chunk / dt, 3), unit="experts/s")
+        if a.factor_route == "direct" and a.low_rank_tokens:
+            dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route="direct", low_rank_tokens=0)
+            out["every_expert_through_its_hessian"] = dict(
+                low_rank_tokens=0, ms_per_step=round(1e3 * dt / a.steps, 2),
+                value=round(a.steps * chunk / dt, 3), unit="experts/s")
         out["hessian_buckets"] = hessian_buckets(cfg["hidden"], min(chunk, 64))
         out["hbm_kernels"] = hbm_kernels(wl)
         out["mfma_ceiling"] = mfma_ceiling()
