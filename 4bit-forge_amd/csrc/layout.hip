@@ -26,23 +26,23 @@ template <typename T>
 __global__ __launch_bounds__(256) void to_solver_order_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const int64_t* __restrict__ perm_inv,
     const uint8_t* __restrict__ dead, float* __restrict__ Xout, T* __restrict__ W0out, int64_t R,
-    int64_t C, int64_t ldo, int64_t o_stride) {
+    int64_t C, int64_t ldo, int64_t o_stride, const int64_t* __restrict__ index) {
     __shared__ float tile[64][65];
-    const int64_t b = blockIdx.z;
+    const int64_t b = blockIdx.z, sb = index ? index[b] : b;    // output slot, source slot
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const T* __restrict__ Wb = W + b * w_stride;
+    const T* __restrict__ Wb = W + sb * w_stride;
     for (int i = ty; i < 64; i += 4) {
         const int64_t r = r0 + i, c = c0 + tx;
         float v = 0.0f;
-        if (r < R && c < C && !(dead && dead[b * C + c])) v = ld_as_f32(Wb + r * ldw + c);
+        if (r < R && c < C && !(dead && dead[sb * C + c])) v = ld_as_f32(Wb + r * ldw + c);
         tile[i][tx] = v;
     }
     __syncthreads();
     for (int j = ty; j < 64; j += 4) {
         const int64_t c = c0 + j, r = r0 + tx;
         if (c < C && r < R) {
-            const int64_t at = b * o_stride + perm_inv[b * C + c] * ldo + r;
+            const int64_t at = b * o_stride + perm_inv[sb * C + c] * ldo + r;
             if (Xout) Xout[at] = tile[tx][j];
             if (W0out) st_from_f32(W0out + at, tile[tx][j]);
         }
@@ -52,19 +52,20 @@ __global__ __launch_bounds__(256) void to_solver_order_kernel(
 // qout[b][r][c] = qin[b][perm_inv[c]][r]   (qweight[perm_inv].T of forge/gptq.py:139)
 __global__ __launch_bounds__(256) void to_layer_order_kernel(
     const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
-    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride) {
+    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride,
+    const int64_t* __restrict__ index) {
     __shared__ uint8_t tile[64][65];
-    const int64_t b = blockIdx.z;
+    const int64_t b = blockIdx.z, sb = index ? index[b] : b;    // input slot, destination slot
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int j = ty; j < 64; j += 4) {
         const int64_t c = c0 + j, r = r0 + tx;
-        tile[j][tx] = (c < C && r < R) ? qin[b * i_stride + perm_inv[b * C + c] * ldi + r] : 0;
+        tile[j][tx] = (c < C && r < R) ? qin[b * i_stride + perm_inv[sb * C + c] * ldi + r] : 0;
     }
     __syncthreads();
     for (int i = ty; i < 64; i += 4) {
         const int64_t r = r0 + i, c = c0 + tx;
-        if (r < R && c < C) qout[b * R * C + r * C + c] = tile[tx][i];
+        if (r < R && c < C) qout[sb * R * C + r * C + c] = tile[tx][i];
     }
 }
 
@@ -77,18 +78,18 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw,
     const int64_t* __restrict__ perm_inv, const uint8_t* __restrict__ dead,
     float* __restrict__ Xout, uint16_t* __restrict__ W0out, int64_t R, int64_t C, int64_t ldo,
-    int64_t o_stride) {
+    int64_t o_stride, const int64_t* __restrict__ index) {
     constexpr int TC = 64, TR = 256, PITCH = TR + 4;     // rows stay 8-byte aligned
     __shared__ __attribute__((aligned(8))) uint16_t tile[TC][PITCH];
-    const int64_t b = blockIdx.z;
+    const int64_t b = blockIdx.z, sb = index ? index[b] : b;
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
-    const uint16_t* __restrict__ Wb = W + b * w_stride;
+    const uint16_t* __restrict__ Wb = W + sb * w_stride;
     {   // 16 lanes x 8 bytes cover one 128-byte row piece; 16 rows per pass
         const int rr = tid >> 4, c4 = (tid & 15) * 4;
         uint32_t keep = 0xF;
         if (dead) {
-            const uint8_t* d = dead + b * C + c0 + c4;
+            const uint8_t* d = dead + sb * C + c0 + c4;
             keep = (d[0] ? 0u : 1u) | (d[1] ? 0u : 2u) | (d[2] ? 0u : 4u) | (d[3] ? 0u : 8u);
         }
 #pragma unroll 4
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
             const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
             const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
                                          __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
-            const int64_t at = b * o_stride + perm_inv[b * C + c0 + c] * ldo + r0 + r4;
+            const int64_t at = b * o_stride + perm_inv[sb * C + c0 + c] * ldo + r0 + r4;
             if (Xout) *reinterpret_cast<float4*>(Xout + at) = o;
             if (W0out) *reinterpret_cast<uint2*>(W0out + at) = v;
         }
@@ -121,10 +122,11 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
 // back four bytes (four values of c) per lane.
 __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
     const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
-    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride) {
+    uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride,
+    const int64_t* __restrict__ index) {
     constexpr int TC = 128, TR = 256, PITCH = TR + 4;    // 65 words per row: odd
     __shared__ __attribute__((aligned(4))) uint8_t tile[TC][PITCH];
-    const int64_t b = blockIdx.z;
+    const int64_t b = blockIdx.z, sb = index ? index[b] : b;
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
     {   // a wavefront reads the 256 bytes of one source row per instruction
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
         for (int cc = 0; cc < TC; cc += 4) {
             const int c = cc + cw;
             const uint32_t v = *reinterpret_cast<const uint32_t*>(
-                qin + b * i_stride + perm_inv[b * C + c0 + c] * ldi + r0 + r4);
+                qin + b * i_stride + perm_inv[sb * C + c0 + c] * ldi + r0 + r4);
             *reinterpret_cast<uint32_t*>(&tile[c][r4]) = v;
         }
     }
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
             const int r = 8 * p + rr;
             const uint32_t v = (uint32_t)tile[c4][r] | ((uint32_t)tile[c4 + 1][r] << 8) |
                                ((uint32_t)tile[c4 + 2][r] << 16) | ((uint32_t)tile[c4 + 3][r] << 24);
-            *reinterpret_cast<uint32_t*>(qout + b * R * C + (r0 + r) * C + c0 + c4) = v;
+            *reinterpret_cast<uint32_t*>(qout + sb * R * C + (r0 + r) * C + c0 + c4) = v;
         }
     }
 }
@@ -158,12 +160,12 @@ __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
 // General form: one workgroup per output row, scalar accesses, LDS staging when C fits.
 __global__ __launch_bounds__(256) void hessian_permute_kernel(
     const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
-    float* __restrict__ Hp, int64_t C) {
+    float* __restrict__ Hp, int64_t C, const int64_t* __restrict__ index) {
     extern __shared__ float srow[];                 // C floats, or nothing when C is too large
-    const int64_t b = blockIdx.y, i = blockIdx.x;
-    const int64_t* __restrict__ pb = perm + b * C;
-    const uint8_t* __restrict__ db = dead ? dead + b * C : nullptr;
-    const float* __restrict__ src = H + b * C * C + pb[i] * C;
+    const int64_t b = blockIdx.y, i = blockIdx.x, sb = index ? index[b] : b;
+    const int64_t* __restrict__ pb = perm + sb * C;
+    const uint8_t* __restrict__ db = dead ? dead + sb * C : nullptr;
+    const float* __restrict__ src = H + sb * C * C + pb[i] * C;
     float* __restrict__ dst = Hp + b * C * C + i * C;
     const bool dead_i = db && db[i];
     const bool staged = C <= kPermuteLdsFloats;
@@ -189,14 +191,14 @@ constexpr int kPermuteRows = 16;
 template <int NCH>
 __global__ __launch_bounds__(256) void hessian_permute_rows_kernel(
     const float* __restrict__ H, const int64_t* __restrict__ perm, const uint8_t* __restrict__ dead,
-    float* __restrict__ Hp, int C, bool lower_blocks) {
+    float* __restrict__ Hp, int C, bool lower_blocks, const int64_t* __restrict__ index) {
     extern __shared__ float srow[];                 // 2 * C floats
-    const int64_t b = blockIdx.y;
+    const int64_t b = blockIdx.y, sb = index ? index[b] : b;
     const int i0 = blockIdx.x * kPermuteRows;
     const int tid = threadIdx.x;
-    const int64_t* __restrict__ pb = perm + b * C;
-    const uint8_t* __restrict__ db = dead ? dead + b * C : nullptr;
-    const float* __restrict__ Hb = H + b * (int64_t)C * C;
+    const int64_t* __restrict__ pb = perm + sb * C;
+    const uint8_t* __restrict__ db = dead ? dead + sb * C : nullptr;
+    const float* __restrict__ Hb = H + sb * (int64_t)C * C;
     float* __restrict__ Hpb = Hp + b * (int64_t)C * C;
 
     // Column chunks past the end are clamped onto the last one: they move the same data a
@@ -325,11 +327,10 @@ __global__ __launch_bounds__(256) void pack_int4_fast_kernel(const uint8_t* __re
 
 }  // namespace
 
-extern "C" int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stride,
-                                                 int64_t ldw, const int64_t* perm_inv,
-                                                 const uint8_t* dead, float* Xout, void* W0out,
-                                                 int64_t ldo, int64_t o_stride, int64_t batch,
-                                                 int64_t R, int64_t C, forge_stream_t stream) {
+static int weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                                  const int64_t* index, const int64_t* perm_inv, const uint8_t* dead,
+                                  float* Xout, void* W0out, int64_t ldo, int64_t o_stride,
+                                  int64_t batch, int64_t R, int64_t C, forge_stream_t stream) {
     FORGE_REQUIRE(w_dtype == FORGE_F32 || w_dtype == FORGE_BF16, "w_dtype=%d", w_dtype);
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0 && ldw >= C, "bad shape");
     FORGE_REQUIRE(ldo >= R && o_stride >= (C > 0 ? (C - 1) * ldo + R : 0), "output pitch too small");
@@ -348,17 +349,38 @@ extern "C" int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int
     if (fast) {
         const dim3 tiles((unsigned)(C / 64), (unsigned)(R / 256), (unsigned)batch);
         to_solver_order_bf16_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(
-            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, (uint16_t*)W0out, R, C, ldo, o_stride);
+            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, (uint16_t*)W0out, R, C, ldo, o_stride,
+            index);
     } else if (w_dtype == FORGE_F32) {
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
-            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, (float*)W0out, R, C, ldo, o_stride);
+            (const float*)W, w_stride, ldw, perm_inv, dead, Xout, (float*)W0out, R, C, ldo, o_stride, index);
     } else {
         to_solver_order_kernel<__hip_bfloat16><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
             (const __hip_bfloat16*)W, w_stride, ldw, perm_inv, dead, Xout, (__hip_bfloat16*)W0out, R, C,
-            ldo, o_stride);
+            ldo, o_stride, index);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
+}
+
+extern "C" int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stride,
+                                                 int64_t ldw, const int64_t* perm_inv,
+                                                 const uint8_t* dead, float* Xout, void* W0out,
+                                                 int64_t ldo, int64_t o_stride, int64_t batch,
+                                                 int64_t R, int64_t C, forge_stream_t stream) {
+    return weight_to_solver_order(W, w_dtype, w_stride, ldw, nullptr, perm_inv, dead, Xout, W0out, ldo,
+                                  o_stride, batch, R, C, stream);
+}
+
+extern "C" int forge_weight_to_solver_order_gather(const void* W, int w_dtype, int64_t w_stride,
+                                                   int64_t ldw, const int64_t* index,
+                                                   const int64_t* perm_inv, const uint8_t* dead,
+                                                   float* Xout, void* W0out, int64_t ldo,
+                                                   int64_t o_stride, int64_t batch, int64_t R,
+                                                   int64_t C, forge_stream_t stream) {
+    FORGE_REQUIRE(index || batch == 0, "null index");
+    return weight_to_solver_order(W, w_dtype, w_stride, ldw, index, perm_inv, dead, Xout, W0out, ldo,
+                                  o_stride, batch, R, C, stream);
 }
 
 extern "C" int forge_weight_to_solver_order_strided(const void* W, int w_dtype, int64_t w_stride,
@@ -378,10 +400,9 @@ extern "C" int forge_weight_to_solver_order(const void* W, int w_dtype, int64_t 
                                                 C * R, batch, R, C, stream);
 }
 
-extern "C" int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
-                                                  const int64_t* perm_inv, uint8_t* qout,
-                                                  int64_t batch, int64_t R, int64_t C,
-                                                  forge_stream_t stream) {
+static int codes_to_layer_order(const uint8_t* qin, int64_t ldi, int64_t i_stride, const int64_t* index,
+                                const int64_t* perm_inv, uint8_t* qout, int64_t batch, int64_t R,
+                                int64_t C, forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0, "bad shape");
     FORGE_REQUIRE(ldi >= R && i_stride >= (C > 0 ? (C - 1) * ldi + R : 0), "input pitch too small");
     if (batch == 0 || R == 0 || C == 0) return FORGE_OK;
@@ -395,13 +416,28 @@ extern "C" int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ld
     if (fast) {
         const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
         to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C,
-                                                                                 ldi, i_stride);
+                                                                                 ldi, i_stride, index);
     } else {
         to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C, ldi,
-                                                                           i_stride);
+                                                                           i_stride, index);
     }
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
+}
+
+extern "C" int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
+                                                  const int64_t* perm_inv, uint8_t* qout,
+                                                  int64_t batch, int64_t R, int64_t C,
+                                                  forge_stream_t stream) {
+    return codes_to_layer_order(qin, ldi, i_stride, nullptr, perm_inv, qout, batch, R, C, stream);
+}
+
+extern "C" int forge_codes_to_layer_order_scatter(const uint8_t* qin, int64_t ldi, int64_t i_stride,
+                                                  const int64_t* index, const int64_t* perm_inv,
+                                                  uint8_t* qout, int64_t batch, int64_t R, int64_t C,
+                                                  forge_stream_t stream) {
+    FORGE_REQUIRE(index || batch == 0, "null index");
+    return codes_to_layer_order(qin, ldi, i_stride, index, perm_inv, qout, batch, R, C, stream);
 }
 
 extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* perm_inv,
@@ -410,9 +446,9 @@ extern "C" int forge_codes_to_layer_order(const uint8_t* qin, const int64_t* per
     return forge_codes_to_layer_order_strided(qin, R, C * R, perm_inv, qout, batch, R, C, stream);
 }
 
-static int hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
-                           float* damp, float rel_damp, int64_t batch, int64_t C, bool lower_blocks,
-                           forge_stream_t stream) {
+static int hessian_permute(const float* H, const int64_t* index, const int64_t* perm,
+                           const uint8_t* dead, float* Hp, float* damp, float rel_damp, int64_t batch,
+                           int64_t C, bool lower_blocks, forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1, "bad shape");
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(H && perm && Hp && damp, "null pointer");
@@ -426,15 +462,15 @@ static int hessian_permute(const float* H, const int64_t* perm, const uint8_t* d
         const dim3 grid((unsigned)forge::ceil_div(C, kPermuteRows), (unsigned)batch);
         const size_t lds = 2 * (size_t)C * sizeof(float);   // <= 64 KB
         if (C <= 2048)
-            hessian_permute_rows_kernel<2><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
+            hessian_permute_rows_kernel<2><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks, index);
         else if (C <= 4096)
-            hessian_permute_rows_kernel<4><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
+            hessian_permute_rows_kernel<4><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks, index);
         else
-            hessian_permute_rows_kernel<8><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks);
+            hessian_permute_rows_kernel<8><<<grid, dim3(256), lds, st>>>(H, perm, dead, Hp, (int)C, lower_blocks, index);
     } else {
         const size_t lds = C <= kPermuteLdsFloats ? (size_t)C * sizeof(float) : 0;
         hessian_permute_kernel<<<dim3((unsigned)C, (unsigned)batch), dim3(256), lds, st>>>(
-            H, perm, dead, Hp, C);
+            H, perm, dead, Hp, C, index);
     }
     FORGE_LAUNCH_CHECK();
     damp_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(Hp, damp, rel_damp, C);
@@ -445,13 +481,21 @@ static int hessian_permute(const float* H, const int64_t* perm, const uint8_t* d
 extern "C" int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* dead,
                                      float* Hp, float* damp, float rel_damp, int64_t batch,
                                      int64_t C, forge_stream_t stream) {
-    return hessian_permute(H, perm, dead, Hp, damp, rel_damp, batch, C, false, stream);
+    return hessian_permute(H, nullptr, perm, dead, Hp, damp, rel_damp, batch, C, false, stream);
 }
 
 extern "C" int forge_hessian_permute_lower(const float* H, const int64_t* perm, const uint8_t* dead,
                                            float* Hp, float* damp, float rel_damp, int64_t batch,
                                            int64_t C, forge_stream_t stream) {
-    return hessian_permute(H, perm, dead, Hp, damp, rel_damp, batch, C, true, stream);
+    return hessian_permute(H, nullptr, perm, dead, Hp, damp, rel_damp, batch, C, true, stream);
+}
+
+extern "C" int forge_hessian_permute_gather(const float* H, const int64_t* index, const int64_t* perm,
+                                            const uint8_t* dead, float* Hp, float* damp,
+                                            float rel_damp, int64_t batch, int64_t C, int lower_blocks,
+                                            forge_stream_t stream) {
+    FORGE_REQUIRE(index || batch == 0, "null index");
+    return hessian_permute(H, index, perm, dead, Hp, damp, rel_damp, batch, C, lower_blocks != 0, stream);
 }
 
 extern "C" int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_t* packed,

@@ -401,11 +401,11 @@ template <typename T>
 __global__ __launch_bounds__(256) void round_to_nearest_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const float* __restrict__ scales,
     const float* __restrict__ qzeros, uint8_t* __restrict__ q, int64_t R, int64_t C, int64_t gs,
-    int64_t G, float maxq) {
+    int64_t G, float maxq, const int64_t* __restrict__ index) {
     const int64_t per_row = (C + 7) / 8;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= R * per_row) return;
-    const int64_t b = blockIdx.y, r = idx / per_row, c0 = (idx - r * per_row) * 8;
+    const int64_t b = index ? index[blockIdx.y] : blockIdx.y, r = idx / per_row, c0 = (idx - r * per_row) * 8;
     const T* __restrict__ src = W + b * w_stride + r * ldw + c0;
     const float* __restrict__ sc = scales + (b * R + r) * G;
     const float* __restrict__ qz = qzeros + (b * R + r) * G;
@@ -450,9 +450,9 @@ __global__ __launch_bounds__(256) void round_to_nearest_kernel(
 }  // namespace
 
 extern "C" int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
-                                      const float* scales, const float* qzeros, uint8_t* qweight,
-                                      int64_t batch, int64_t R, int64_t C, int64_t gs, int bits,
-                                      forge_stream_t stream) {
+                                      const int64_t* index, const float* scales, const float* qzeros,
+                                      uint8_t* qweight, int64_t batch, int64_t R, int64_t C, int64_t gs,
+                                      int bits, forge_stream_t stream) {
     FORGE_REQUIRE(w_dtype == FORGE_F32 || w_dtype == FORGE_BF16, "w_dtype=%d", w_dtype);
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && R >= 0 && C >= 0 && gs >= 1 && ldw >= C &&
                       R < (1LL << 30) && C < (1LL << 30),
@@ -471,10 +471,10 @@ extern "C" int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stri
                                forge::WORK_BYTES);
     if (w_dtype == FORGE_BF16)
         round_to_nearest_kernel<uint16_t><<<grid, block, 0, st>>>((const uint16_t*)W, w_stride, ldw, scales,
-                                                                  qzeros, qweight, R, C, gs, G, maxq);
+                                                                  qzeros, qweight, R, C, gs, G, maxq, index);
     else
         round_to_nearest_kernel<float><<<grid, block, 0, st>>>((const float*)W, w_stride, ldw, scales,
-                                                               qzeros, qweight, R, C, gs, G, maxq);
+                                                               qzeros, qweight, R, C, gs, G, maxq, index);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

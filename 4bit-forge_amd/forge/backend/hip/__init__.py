@@ -64,7 +64,11 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_lowrank_workspace_bytes": ([i64, i64, i64], i64),
         "forge_gptq_sweep_lowrank_mixed": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
                                             vp], i32),
-        "forge_round_to_nearest": ([vp, i32, i64, i64, vp, vp, vp, i64, i64, i64, i64, i32, vp], i32),
+        "forge_round_to_nearest": ([vp, i32, i64, i64, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp], i32),
+        "forge_hessian_permute_gather": ([vp, vp, vp, vp, vp, vp, f32, i64, i64, i32, vp], i32),
+        "forge_weight_to_solver_order_gather": ([vp, i32, i64, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64,
+                                                 i64, vp], i32),
+        "forge_codes_to_layer_order_scatter": ([vp, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_gptq_sweep_lowrank": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i64,
                                       vp], i32),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
@@ -118,7 +122,8 @@ EXPORTED_SYMBOLS = (
     "forge_chol_reverse_lower_batched", "forge_unit_upper_from_lower", "forge_babai_solver",
     "forge_babai_workspace_bytes", "forge_hessian_update_ranges", "forge_lowrank_factor",
     "forge_gptq_sweep_lowrank", "forge_round_to_nearest", "forge_lowrank_workspace_bytes",
-    "forge_gptq_sweep_lowrank_mixed",
+    "forge_gptq_sweep_lowrank_mixed", "forge_hessian_permute_gather",
+    "forge_weight_to_solver_order_gather", "forge_codes_to_layer_order_scatter",
 )
 
 
@@ -405,22 +410,28 @@ class _HipKernels:
                 _stream()))
         return H
 
-    def round_to_nearest(self, W, scales, qzeros, gs, bits, out=None):
+    def round_to_nearest(self, W, scales, qzeros, gs, bits, out=None, index=None):
         """W [B,R,C] (bf16/f32, layer layout), scales/qzeros [B,R*G] -> codes [B,R,C] u8 of the
-        reference's quantiser applied weight by weight (a layer with H = I)."""
-        _need_cuda(W, scales, qzeros, out)
+        reference's quantiser applied weight by weight (a layer with H = I).  index (int64,
+        device): only these matrices of the stacks are worked on (``out`` required then)."""
+        _need_cuda(W, scales, qzeros, out, index)
         B, R, C = W.shape
         G = (C + gs - 1) // gs
         assert W.stride(2) == 1 and scales.is_contiguous() and qzeros.is_contiguous()
         assert tuple(scales.shape) == (B, R * G) and tuple(qzeros.shape) == (B, R * G)
         assert scales.dtype == torch.float32 and qzeros.dtype == torch.float32
         if out is None:
+            assert index is None
             out = torch.empty((B, R, C), dtype=torch.uint8, device=W.device)
         assert out.is_contiguous() and out.dtype == torch.uint8 and tuple(out.shape) == (B, R, C)
+        n = B
+        if index is not None:
+            assert index.dtype == torch.int64 and index.is_contiguous() and index.dim() == 1
+            n = index.numel()
         with torch.cuda.device(W.device):
             self._check(self._lib.forge_round_to_nearest(
-                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(scales), _ptr(qzeros), _ptr(out),
-                B, R, C, int(gs), int(bits), _stream()))
+                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(index), _ptr(scales), _ptr(qzeros),
+                _ptr(out), n, R, C, int(gs), int(bits), _stream()))
         return out
 
     def lowrank_factor(self, Bp, D, out=None):
@@ -576,81 +587,116 @@ class _HipKernels:
                 int(G), _ptr(q), _ptr(ws), nbytes, _stream()))
         return q
 
-    def hessian_permute(self, H, perm, dead, rel_damp, lower_blocks=False, out=None):
+    def hessian_permute(self, H, perm, dead, rel_damp, lower_blocks=False, out=None, index=None):
         """Hp[b] = H[b][perm][:, perm] with dead rows/columns cleared (unit diagonal), damp[b] =
         rel_damp * mean(diag).  lower_blocks: in row i only the columns up to the end of its own
         128-column block are written (what the factorisations read).  out = (Hp, damp): write
-        into these (contiguous slices of a larger batch, say) instead of new tensors."""
-        _need_cuda(H, perm, dead)
+        into these instead of new tensors.  index (int64 [n], device): output b is made from
+        matrix index[b] of H and rows index[b] of perm and dead."""
+        _need_cuda(H, perm, dead, index)
         B, C, _ = H.shape
         assert H.is_contiguous() and perm.dtype == torch.int64 and perm.is_contiguous()
         assert dead.dtype == torch.uint8 and dead.is_contiguous()
         assert tuple(perm.shape) == (B, C) and tuple(dead.shape) == (B, C)
+        n = B
+        if index is not None:
+            assert index.dtype == torch.int64 and index.is_contiguous() and index.dim() == 1
+            n = index.numel()
         if out is not None:
             Hp, damp = out
             _need_cuda(Hp, damp)
-            assert Hp.is_contiguous() and Hp.dtype == torch.float32 and Hp.shape == H.shape
-            assert damp.is_contiguous() and damp.dtype == torch.float32 and damp.numel() == B
+            assert Hp.is_contiguous() and Hp.dtype == torch.float32 and tuple(Hp.shape) == (n, C, C)
+            assert damp.is_contiguous() and damp.dtype == torch.float32 and damp.numel() == n
         else:
-            Hp = torch.empty_like(H)
-            damp = torch.empty(B, dtype=torch.float32, device=H.device)
+            Hp = torch.empty((n, C, C), dtype=torch.float32, device=H.device)
+            damp = torch.empty(n, dtype=torch.float32, device=H.device)
         with torch.cuda.device(H.device):
-            fn = self._lib.forge_hessian_permute_lower if lower_blocks else self._lib.forge_hessian_permute
-            self._check(fn(_ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
-                           _stream()))
+            if index is not None:
+                self._check(self._lib.forge_hessian_permute_gather(
+                    _ptr(H), _ptr(index), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), n,
+                    C, int(bool(lower_blocks)), _stream()))
+            else:
+                fn = self._lib.forge_hessian_permute_lower if lower_blocks else self._lib.forge_hessian_permute
+                self._check(fn(_ptr(H), _ptr(perm), _ptr(dead), _ptr(Hp), _ptr(damp), float(rel_damp), B, C,
+                               _stream()))
         return Hp, damp
 
-    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None, skip_out=False):
+    def weight_to_solver_order(self, W, perm_inv, dead=None, out=None, row0=0, out0=None, skip_out=False,
+                               index=None):
         """W [B,R,C] (bf16/f32) -> X [B,C,R] f32, X[b, perm_inv[b,c], r] = W[b, r, c].
         With ``out`` [B,C,Rtot] (f32, contiguous) the rows land at out[:, :, row0:row0+R]: stacks
         that share a factor fill one tall matrix without being concatenated first.  ``out0``
         (shape of ``out``, dtype of W) receives the same values in W's own type: the untouched
         copy for gptq_sweep_direct_batched(W0=...).  skip_out: only ``out0`` is written
-        (``out`` then only gives the shape; for gptq_sweep_direct_batched(x_from_w0=True))."""
-        _need_cuda(W, perm_inv, dead, out)
+        (``out`` then only gives the shape; for gptq_sweep_direct_batched(x_from_w0=True)).
+        index (int64 [n], device): output b is made from W[index[b]], perm_inv[index[b]] and
+        dead[index[b]]; ``out`` / ``out0`` are then [n,C,Rtot]."""
+        _need_cuda(W, perm_inv, dead, out, index)
         B, R, C = W.shape
         assert W.stride(2) == 1 and perm_inv.dtype == torch.int64 and perm_inv.is_contiguous()
         assert tuple(perm_inv.shape) == (B, C)
         assert dead is None or (dead.dtype == torch.uint8 and dead.is_contiguous())
+        n = B
+        if index is not None:
+            assert index.dtype == torch.int64 and index.is_contiguous() and index.dim() == 1
+            n = index.numel()
         if out is None and skip_out and out0 is not None:
             shape = tuple(out0.shape)                 # only out0 is written: it also gives the shape
         else:
             if out is None:
-                out = torch.empty((B, C, R), dtype=torch.float32, device=W.device)
+                out = torch.empty((n, C, R), dtype=torch.float32, device=W.device)
                 row0 = 0
             assert out.is_contiguous() and out.dtype == torch.float32
             shape = tuple(out.shape)
         assert len(shape) == 3
         Rtot = shape[2]
-        assert shape[:2] == (B, C) and 0 <= row0 and row0 + R <= Rtot
+        assert shape[:2] == (n, C) and 0 <= row0 and row0 + R <= Rtot
         p0 = None
         if out0 is not None:
             _need_cuda(out0)
             assert out0.is_contiguous() and out0.dtype == W.dtype and tuple(out0.shape) == shape
             p0 = ctypes.c_void_p(out0.data_ptr() + out0.element_size() * row0)
+        px = None if skip_out else ctypes.c_void_p(out.data_ptr() + 4 * row0)
         with torch.cuda.device(W.device):
-            self._check(self._lib.forge_weight_to_solver_order_pair(
-                _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
-                None if skip_out else ctypes.c_void_p(out.data_ptr() + 4 * row0), p0, Rtot, C * Rtot, B,
-                R, C, _stream()))
+            if index is not None:
+                self._check(self._lib.forge_weight_to_solver_order_gather(
+                    _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(index), _ptr(perm_inv),
+                    _ptr(dead), px, p0, Rtot, C * Rtot, n, R, C, _stream()))
+            else:
+                self._check(self._lib.forge_weight_to_solver_order_pair(
+                    _ptr(W), _dtype_code(W), W.stride(0), W.stride(1), _ptr(perm_inv), _ptr(dead),
+                    px, p0, Rtot, C * Rtot, B, R, C, _stream()))
         return out
 
-    def codes_to_layer_order(self, q, perm_inv, out=None, row0=0, rows=None):
+    def codes_to_layer_order(self, q, perm_inv, out=None, row0=0, rows=None, index=None):
         """q [B,C,R] u8 (solver order) -> [B,R,C] u8, out[b, r, c] = q[b, perm_inv[b,c], r].
         ``row0``/``rows`` select a band of q's rows (a stack of a tall shared-factor matrix);
-        ``out`` [B,rows,C] (contiguous) receives it."""
-        _need_cuda(q, perm_inv, out)
+        ``out`` [B,rows,C] (contiguous) receives it.  index (int64 [B], device): q[b] goes to
+        out[index[b]] through perm_inv[index[b]] (``out`` and ``perm_inv`` are then the larger
+        stack's)."""
+        _need_cuda(q, perm_inv, out, index)
         B, C, Rtot = q.shape
         R = Rtot - row0 if rows is None else int(rows)
         assert q.is_contiguous() and q.dtype == torch.uint8 and perm_inv.is_contiguous()
-        assert perm_inv.dtype == torch.int64 and tuple(perm_inv.shape) == (B, C)
+        assert perm_inv.dtype == torch.int64 and perm_inv.shape[1] == C
         assert 0 <= row0 and R >= 0 and row0 + R <= Rtot
-        if out is None:
-            out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
-        assert out.is_contiguous() and out.dtype == torch.uint8 and tuple(out.shape) == (B, R, C)
+        if index is None:
+            assert perm_inv.shape[0] == B
+            if out is None:
+                out = torch.empty((B, R, C), dtype=torch.uint8, device=q.device)
+            assert tuple(out.shape) == (B, R, C)
+        else:
+            assert index.dtype == torch.int64 and index.is_contiguous() and index.numel() == B
+            assert out is not None and tuple(out.shape) == (perm_inv.shape[0], R, C)
+        assert out.is_contiguous() and out.dtype == torch.uint8
         with torch.cuda.device(q.device):
-            self._check(self._lib.forge_codes_to_layer_order_strided(
-                q.data_ptr() + row0, Rtot, C * Rtot, _ptr(perm_inv), _ptr(out), B, R, C, _stream()))
+            if index is not None:
+                self._check(self._lib.forge_codes_to_layer_order_scatter(
+                    q.data_ptr() + row0, Rtot, C * Rtot, _ptr(index), _ptr(perm_inv), _ptr(out), B, R, C,
+                    _stream()))
+            else:
+                self._check(self._lib.forge_codes_to_layer_order_strided(
+                    q.data_ptr() + row0, Rtot, C * Rtot, _ptr(perm_inv), _ptr(out), B, R, C, _stream()))
         return out
 
     def pack_int4(self, codes, qzeros, group_size):

@@ -201,16 +201,6 @@ class ExpertGroupGPTQ:
                 + ([torch.empty((E, (C + 31) // 32, R), dtype=torch.uint32, device=dev)] if sparse else [])
                 for R in sizes]
 
-        def runs_of(ids):
-            """[(first expert, count, position in ids)] of the consecutive runs of a sorted list."""
-            out = []
-            for pos, e in enumerate(ids):
-                if out and out[-1][0] + out[-1][1] == e:
-                    out[-1][1] += 1
-                else:
-                    out.append([e, 1, pos])
-            return [tuple(r) for r in out]
-
         for e0 in range(0, E, chunk):
             e1 = min(E, e0 + chunk)
             B = e1 - e0
@@ -287,31 +277,29 @@ class ExpertGroupGPTQ:
                 mask = masks[job[0]]
 
                 def layout_in(ids, W0, X=None, skip_out=False):
-                    """weights of the chunk's experts `ids` -> solver order, run by run"""
-                    for first, count, pos in runs_of(ids):
-                        sl = slice(pos, pos + count)
-                        ex = slice(e0 + first, e0 + first + count)
-                        ch = slice(first, first + count)
-                        r0 = 0
-                        for i in job:
-                            kernels.weight_to_solver_order(
-                                self.W[i][ex], perm_inv[ch], dead_u8[ch], out=None if X is None else X[sl],
-                                row0=r0, out0=None if W0 is None else W0[sl], skip_out=skip_out)
-                            r0 += sizes[i]
+                    """weights of the chunk's experts `ids` -> solver order: one launch per stack"""
+                    whole = len(ids) == B
+                    idx = None if whole else torch.tensor(ids, device=dev)
+                    r0 = 0
+                    for i in job:
+                        kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0,
+                                                       out0=W0, skip_out=skip_out, index=idx)
+                        r0 += sizes[i]
 
                 def layout_out(ids, q, M=None):
-                    for first, count, pos in runs_of(ids):
-                        sl = slice(pos, pos + count)
-                        ex = slice(e0 + first, e0 + first + count)
-                        ch = slice(first, first + count)
-                        r0 = 0
-                        for i in job:
-                            Ri = sizes[i]
-                            kernels.codes_to_layer_order(q[sl], perm_inv[ch], out=outs[i][0][ex], row0=r0,
-                                                         rows=Ri)
-                            if M is not None:
-                                outs[i][3][ex] = M[sl, :, r0:r0 + Ri]
-                            r0 += Ri
+                    whole = len(ids) == B
+                    idx = None if whole else torch.tensor(ids, device=dev)
+                    r0 = 0
+                    for i in job:
+                        Ri = sizes[i]
+                        kernels.codes_to_layer_order(q, perm_inv, out=outs[i][0][e0:e1], row0=r0, rows=Ri,
+                                                     index=idx)
+                        if M is not None:
+                            if whole:
+                                outs[i][3][e0:e1] = M[:, :, r0:r0 + Ri]
+                            else:
+                                outs[i][3][e0:e1][idx] = M[:, :, r0:r0 + Ri]
+                        r0 += Ri
 
                 # ---------------------------------------------------------- low-rank experts
                 lr_stream = main
@@ -366,12 +354,11 @@ class ExpertGroupGPTQ:
                             pos += len(ids)
                         del W0, q, Bp_all, Hm_all
                     # experts without a single row (or with NaN rows): H = I, plain rounding
-                    for first, count, _ in runs_of(none_ids):
-                        ex = slice(e0 + first, e0 + first + count)
-                        ch = slice(first, first + count)
+                    if none_ids:
+                        ni = torch.tensor(none_ids, device=dev)
                         for (sc_i, qz_i), i in zip(parts, job):
-                            kernels.round_to_nearest(self.W[i][ex], sc_i[ch], qz_i[ch], gs, self.bits,
-                                                     out=outs[i][0][ex])
+                            kernels.round_to_nearest(self.W[i][e0:e1], sc_i, qz_i, gs, self.bits,
+                                                     out=outs[i][0][e0:e1], index=ni)
 
                 # ---------------------------------------------------------- through the Hessian
                 if dn_ids:
@@ -380,17 +367,8 @@ class ExpertGroupGPTQ:
                     pick = (lambda t: t) if whole else (lambda t: t[di].contiguous())
                     Bd = len(dn_ids)
                     # the factorisations read their input's lower triangle in 128 x 128 blocks only
-                    if whole:
-                        Hp, damp = kernels.hessian_permute(self.H[e0:e1], perm, mask, float(self.rel_damp),
-                                                           lower_blocks=True)
-                    else:
-                        Hp = torch.empty((Bd, C, C), dtype=torch.float32, device=dev)
-                        damp = torch.empty(Bd, dtype=torch.float32, device=dev)
-                        for first, count, pos in runs_of(dn_ids):
-                            ch = slice(first, first + count)
-                            kernels.hessian_permute(self.H[e0 + first:e0 + first + count], perm[ch], mask[ch],
-                                                    float(self.rel_damp), lower_blocks=True,
-                                                    out=(Hp[pos:pos + count], damp[pos:pos + count]))
+                    Hp, damp = kernels.hessian_permute(self.H[e0:e1], perm, mask, float(self.rel_damp),
+                                                       lower_blocks=True, index=di)
                     if babai:
                         L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                         U = kernels.unit_upper_from_lower(L, info, upper_only=True)

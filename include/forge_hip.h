@@ -223,10 +223,13 @@ int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, i
  * the identity, nothing couples the columns and the sweep of solver.cu:9-154 is its quantiser
  * (solver.cu:9-23) applied to every weight.  W [batch][R][C] (w_dtype f32 or bf16, row pitch ldw,
  * batch stride w_stride, layer layout), scales/qzeros [batch][R*G] (index r*G + c/gs) ->
- * qweight [batch][R][C] u8, layer layout: no permutation, no layout pass. */
+ * qweight [batch][R][C] u8, layer layout: no permutation, no layout pass.  index (device, int64
+ * [batch], may be NULL): launch entry b works on matrix index[b] of all three arrays, so that a
+ * scattered subset of a stack is handled in place by one launch. */
 int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
-                           const float* scales, const float* qzeros, uint8_t* qweight, int64_t batch,
-                           int64_t R, int64_t C, int64_t gs, int bits, forge_stream_t stream);
+                           const int64_t* index, const float* scales, const float* qzeros,
+                           uint8_t* qweight, int64_t batch, int64_t R, int64_t C, int64_t gs, int bits,
+                           forge_stream_t stream);
 int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, int32_t* info, int64_t batch,
                          int64_t C, int64_t n, void* ws, int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_lowrank_workspace_bytes(int64_t batch, int64_t C, int64_t n);
@@ -363,6 +366,12 @@ int forge_hessian_permute(const float* H, const int64_t* perm, const uint8_t* de
 int forge_hessian_permute_lower(const float* H, const int64_t* perm, const uint8_t* dead, float* Hp,
                                 float* damp, float rel_damp, int64_t batch, int64_t C,
                                 forge_stream_t stream);
+/* The same for a scattered subset of a larger stack in one launch: output b (Hp[b], damp[b]) is
+ * made from matrix index[b] of H and rows index[b] of perm and dead (index: device, int64
+ * [batch]); lower_blocks != 0 as forge_hessian_permute_lower. */
+int forge_hessian_permute_gather(const float* H, const int64_t* index, const int64_t* perm,
+                                 const uint8_t* dead, float* Hp, float* damp, float rel_damp,
+                                 int64_t batch, int64_t C, int lower_blocks, forge_stream_t stream);
 
 /* ------------------------------------------------------------------ layout helpers */
 
@@ -401,6 +410,18 @@ int forge_weight_to_solver_order_pair(const void* W, int w_dtype, int64_t w_stri
 int forge_codes_to_layer_order_strided(const uint8_t* qin, int64_t ldi, int64_t i_stride,
                                        const int64_t* perm_inv, uint8_t* qout, int64_t batch,
                                        int64_t R, int64_t C, forge_stream_t stream);
+/* The two strided layout passes for a scattered subset of a larger stack in one launch (index:
+ * device, int64 [batch]).  _gather: output b (Xout / W0out + b * o_stride) is made from matrix
+ * index[b] of W and rows index[b] of perm_inv and dead.  _scatter: input b (qin + b * i_stride)
+ * goes to matrix index[b] of qout, through row index[b] of perm_inv. */
+int forge_weight_to_solver_order_gather(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
+                                        const int64_t* index, const int64_t* perm_inv,
+                                        const uint8_t* dead, float* Xout, void* W0out, int64_t ldo,
+                                        int64_t o_stride, int64_t batch, int64_t R, int64_t C,
+                                        forge_stream_t stream);
+int forge_codes_to_layer_order_scatter(const uint8_t* qin, int64_t ldi, int64_t i_stride,
+                                       const int64_t* index, const int64_t* perm_inv, uint8_t* qout,
+                                       int64_t batch, int64_t R, int64_t C, forge_stream_t stream);
 
 /* Nibble packing of [R, C] u8 codes into the compressed-tensors "pack-quantized" int32
  * layout consumed by pack_quantized.py:279-313: value = code - zero + 8 (offset binary of

@@ -167,6 +167,45 @@ def test_hessian_ranges_skip_groups_in_place(hip):
     assert torch.equal(got[2], H0[2]) and torch.equal(got[0], want[0]) and torch.equal(got[3], want[3])
 
 
+def test_layout_passes_on_a_scattered_subset(hip):
+    """The gather / scatter forms (one launch for a subset of a stack) against the plain forms on
+    the same matrices one by one."""
+    g = torch.Generator().manual_seed(6)
+    B, R, C = 5, 256, 256
+    W = (0.02 * torch.randn(B, R, C, generator=g)).bfloat16().to(DEV)
+    perm_inv = torch.stack([torch.randperm(C, generator=g) for _ in range(B)]).to(DEV)
+    dead = (torch.rand(B, C, generator=g) < 0.02).to(torch.uint8).to(DEV)
+    H = torch.randn(B, C, C, generator=g).to(DEV)
+    idx = torch.tensor([3, 0, 4], device=DEV)
+    X = torch.empty((3, C, R), dtype=torch.float32, device=DEV)
+    W0 = torch.empty((3, C, R), dtype=torch.bfloat16, device=DEV)
+    hip.weight_to_solver_order(W, perm_inv, dead, out=X, out0=W0, index=idx)
+    Hp, damp = hip.hessian_permute(H, perm_inv, dead, 0.01, lower_blocks=True, index=idx)
+    codes = torch.randint(0, 16, (3, C, R), generator=g, dtype=torch.uint8).to(DEV)
+    out = torch.zeros((B, R, C), dtype=torch.uint8, device=DEV)
+    hip.codes_to_layer_order(codes, perm_inv, out=out, index=idx)
+    for pos, e in enumerate(idx.tolist()):
+        sl = slice(e, e + 1)
+        X1 = hip.weight_to_solver_order(W[sl], perm_inv[sl].contiguous(), dead[sl].contiguous())
+        assert torch.equal(X[pos], X1[0]) and torch.equal(W0[pos].float(), X1[0])
+        H1, d1 = hip.hessian_permute(H[sl], perm_inv[sl].contiguous(), dead[sl].contiguous(), 0.01,
+                                     lower_blocks=True)
+        keep = torch.ones(C, C, dtype=torch.bool, device=DEV).tril()
+        for blk in range(0, C, 128):                             # what lower_blocks writes
+            keep[blk:blk + 128, :blk + 128] = True
+        assert torch.equal(Hp[pos][keep], H1[0][keep]) and torch.equal(damp[pos], d1[0])
+        q1 = hip.codes_to_layer_order(codes[pos:pos + 1], perm_inv[sl].contiguous())
+        assert torch.equal(out[e], q1[0])
+    assert not out[1].any() and not out[2].any()                 # untouched slots
+    G = C // 128
+    s, z = oracle.build_group_meta_packed(W.float().cpu().reshape(B * R * G, 128), 4, False)
+    s, z = s.view(B, R * G).to(DEV), z.view(B, R * G).to(DEV)
+    full = hip.round_to_nearest(W, s, z, 128, 4)
+    part = torch.zeros_like(full)
+    hip.round_to_nearest(W, s, z, 128, 4, out=part, index=idx)
+    assert torch.equal(part[idx], full[idx]) and not part[1].any() and not part[2].any()
+
+
 def test_expert_group_low_rank_route_against_the_dense_route_and_the_oracle():
     """Experts with 0 .. 16 rows through the low-rank route, the same experts with
     low_rank_tokens=0 through their Hessians, and the reference-form oracle: scales identical,
