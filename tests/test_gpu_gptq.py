@@ -444,11 +444,13 @@ def test_config5_sparse14_full_size():
     assert torch.equal(words, want)
 
 
-@pytest.mark.parametrize("n_tokens", [1536, 200])
+@pytest.mark.parametrize("n_tokens", [1536, 200, 40])
 def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 512 of
     its 2048 rows, rows being independent, to keep the CPU oracle's sweeps short) with a heavy
-    expert's tokens and with 200 (Hessian of rank 200 before damping).  At this size the
+    expert's tokens, with 200 (Hessian of rank 200 before damping) and with 40 (the batched
+    front end's default route then solves from the 40 rows themselves, without a Hessian).  At
+    this size the
     problem is ill conditioned: the oracle's own codes move by 1-2 % between two valid fp32
     realisations of its library stages (the floor).  Three GPU routes are held to that floor
     against the reference-form oracle: the drop-in class (reference's factor of inv(H), fp32
