@@ -18,7 +18,8 @@
 // dense route in exact arithmetic; in floating point this route is the more accurate one (the
 // recurrence runs in float64, where S shrinks from 1 to damp / |b|^2 without losing its digits).
 //
-// Compiled for n = 16, 32 and 64 rows of B (rows beyond a layer's own count are zero rows):
+// Compiled for n = 16, 32, 64 and 128 rows of B (rows beyond a layer's own count are zero rows;
+// 128 with four threads per row of S in the factor):
 //   lowrank_gram/suffix/block_kernel   the recurrence, cut into blocks of 128 columns that
 //                                      start from their own S and run side by side; writes h_k.
 //   lowrank_sweep_kernel               n/16 lanes per output row walk k = 0 .. C-1: dot,
@@ -229,6 +230,166 @@ __global__ __launch_bounds__(64) void lowrank_block_kernel(const float* __restri
     if (threadIdx.x == 0 && bad) atomicOr(info + b, 1);
 }
 
+// ---- n = 128: a row of S no longer fits one lane's registers.  NS = 4 threads share a row, 32
+// columns each (512 threads, thread = (row, quarter)); what crosses threads goes through LDS
+// with a workgroup barrier.  Same arithmetic as the one-wavefront kernels above except that the
+// dot products are summed quarter by quarter.
+constexpr int WN = 128, WS = 4, WQ = WN / WS;      // rows, threads per row, columns per thread
+
+__global__ __launch_bounds__(WN * WS) void lowrank_gram_wide_kernel(const float* __restrict__ Bp,
+                                                                    const float* __restrict__ D,
+                                                                    double* __restrict__ gram,
+                                                                    int64_t C, int nblk) {
+    __shared__ __attribute__((aligned(16))) float bsh[2][WN];
+    const int row = threadIdx.x & (WN - 1), qt = threadIdx.x / WN;
+    const int blk = blockIdx.x;
+    const int64_t b = blockIdx.y;
+    const int64_t k_lo = (int64_t)blk * FB, k_hi = (k_lo + FB < C ? k_lo + FB : C) - 1;
+    const float* __restrict__ Bb = Bp + b * C * WN + row;
+    const float* __restrict__ Db = D + b * C;
+    double acc[WQ];
+#pragma unroll
+    for (int j = 0; j < WQ; ++j) acc[j] = 0.0;
+    if (qt == 0) bsh[k_hi & 1][row] = Bb[k_hi * WN];
+    float nd = Db[k_hi];
+    for (int64_t k = k_hi; k >= k_lo; --k) {
+        const double dk = (double)nd;
+        float nxt = 0.0f;
+        if (k > k_lo) {
+            if (qt == 0) nxt = Bb[(k - 1) * WN];
+            nd = Db[k - 1];
+        }
+        __syncthreads();
+        const double mine = (double)bsh[k & 1][row] / dk;
+#pragma unroll
+        for (int j = 0; j < WQ; j += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(&bsh[k & 1][qt * WQ + j]);
+            acc[j + 0] = __builtin_fma(mine, (double)v.x, acc[j + 0]);
+            acc[j + 1] = __builtin_fma(mine, (double)v.y, acc[j + 1]);
+            acc[j + 2] = __builtin_fma(mine, (double)v.z, acc[j + 2]);
+            acc[j + 3] = __builtin_fma(mine, (double)v.w, acc[j + 3]);
+        }
+        if (k > k_lo && qt == 0) bsh[(k - 1) & 1][row] = nxt;
+    }
+    double* __restrict__ out = gram + ((b * nblk + blk) * WN + row) * WN + qt * WQ;
+#pragma unroll
+    for (int j = 0; j < WQ; ++j) out[j] = acc[j];
+}
+
+__global__ __launch_bounds__(WN * WS) void lowrank_block_wide_kernel(const float* __restrict__ Bp,
+                                                                     const float* __restrict__ D,
+                                                                     const double* __restrict__ later,
+                                                                     float* __restrict__ Hm,
+                                                                     int32_t* __restrict__ info,
+                                                                     int64_t C, int nblk) {
+    __shared__ __attribute__((aligned(16))) float bsh[2][WN];
+    __shared__ __attribute__((aligned(16))) double rowsh[WN];      // pivot row / s
+    __shared__ __attribute__((aligned(16))) double colsh[WN];      // pivot column
+    __shared__ __attribute__((aligned(16))) double part[WS][WN];   // partial dots
+    __shared__ double psum[WS];
+    const int row = threadIdx.x & (WN - 1), qt = threadIdx.x / WN;
+    const int blk = blockIdx.x;
+    const int64_t b = blockIdx.y;
+    const int64_t k_lo = (int64_t)blk * FB, k_hi = (k_lo + FB < C ? k_lo + FB : C) - 1;
+    const float* __restrict__ Bb = Bp + b * C * WN + row;
+    const float* __restrict__ Db = D + b * C;
+    float* __restrict__ Hb = Hm + b * C * WN + row;
+    if (qt == 0) bsh[k_hi & 1][row] = Bb[k_hi * WN];
+    float nd = Db[k_hi];
+    bool bad = false;
+
+    double S[WQ];                                   // S[row][qt * WQ + j]
+#pragma unroll
+    for (int j = 0; j < WQ; ++j) S[j] = (qt * WQ + j == row) ? 1.0 : 0.0;
+    if (blk + 1 < nblk) {
+        const double* __restrict__ src = later + ((b * nblk + blk) * WN + row) * WN + qt * WQ;
+#pragma unroll
+        for (int j = 0; j < WQ; ++j) S[j] += src[j];
+#pragma unroll
+        for (int m = 0; m < WN; ++m) {
+            __syncthreads();                       // the previous pivot row and column have been read
+            if (row == m) {
+#pragma unroll
+                for (int j = 0; j < WQ; ++j) rowsh[qt * WQ + j] = S[j];
+            }
+            if (qt == m / WQ) colsh[row] = S[m % WQ];
+            __syncthreads();
+            double piv[WQ];
+#pragma unroll
+            for (int j = 0; j < WQ; j += 2) {
+                const double2 v = *reinterpret_cast<const double2*>(&rowsh[qt * WQ + j]);
+                piv[j] = v.x;
+                piv[j + 1] = v.y;
+            }
+            const double p = rowsh[m];
+            bad |= !(p > 0.0);
+            const double rp = 1.0 / p;
+            const bool is_m = row == m;
+            const double keep = is_m ? 0.0 : 1.0;
+            const double g = is_m ? rp : -(colsh[row] * rp);
+#pragma unroll
+            for (int j = 0; j < WQ; ++j) S[j] = __builtin_fma(g, piv[j], keep * S[j]);
+            if (qt == m / WQ) S[m % WQ] = g;
+        }
+    }
+
+    for (int64_t k = k_hi; k >= k_lo; --k) {
+        const double dk = (double)nd;
+        float nxt = 0.0f;
+        if (k > k_lo) {
+            if (qt == 0) nxt = Bb[(k - 1) * WN];
+            nd = Db[k - 1];
+        }
+        __syncthreads();                           // b_k is in place; last column's LDS reads are done
+        double bd[WQ];
+#pragma unroll
+        for (int j = 0; j < WQ; j += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(&bsh[k & 1][qt * WQ + j]);
+            bd[j + 0] = (double)v.x; bd[j + 1] = (double)v.y;
+            bd[j + 2] = (double)v.z; bd[j + 3] = (double)v.w;
+        }
+        double c0 = 0.0, c1 = 0.0, c2 = 0.0, c3 = 0.0;
+#pragma unroll
+        for (int j = 0; j < WQ; j += 4) {
+            c0 = __builtin_fma(S[j + 0], bd[j + 0], c0);
+            c1 = __builtin_fma(S[j + 1], bd[j + 1], c1);
+            c2 = __builtin_fma(S[j + 2], bd[j + 2], c2);
+            c3 = __builtin_fma(S[j + 3], bd[j + 3], c3);
+        }
+        part[qt][row] = (c0 + c1) + (c2 + c3);
+        __syncthreads();
+        const double s = (part[0][row] + part[1][row]) + (part[2][row] + part[3][row]);
+        if (qt == 0) rowsh[row] = s;
+        __syncthreads();
+        double sj[WQ];
+#pragma unroll
+        for (int j = 0; j < WQ; j += 2) {
+            const double2 v = *reinterpret_cast<const double2*>(&rowsh[qt * WQ + j]);
+            sj[j] = v.x;
+            sj[j + 1] = v.y;
+        }
+        // b . s: every thread of a quarter forms the same partial sum; one of them posts it
+        double p0 = 0.0, p1 = 0.0, p2 = 0.0, p3 = 0.0;
+#pragma unroll
+        for (int j = 0; j < WQ; j += 4) {
+            p0 = __builtin_fma(bd[j + 0], sj[j + 0], p0);
+            p1 = __builtin_fma(bd[j + 1], sj[j + 1], p1);
+            p2 = __builtin_fma(bd[j + 2], sj[j + 2], p2);
+            p3 = __builtin_fma(bd[j + 3], sj[j + 3], p3);
+        }
+        if (row == 0) psum[qt] = (p0 + p1) + (p2 + p3);
+        __syncthreads();
+        const double p = dk + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
+        bad |= !(p > 0.0);
+        const double h = s / p;
+        if (qt == 0) Hb[k * WN] = (float)h;
+#pragma unroll
+        for (int j = 0; j < WQ; ++j) S[j] = __builtin_fma(-h, sj[j], S[j]);
+        if (k > k_lo && qt == 0) bsh[(k - 1) & 1][row] = nxt;
+    }
+    if (threadIdx.x == 0 && bad) atomicOr(info + b, 1);
+}
+
 __device__ __forceinline__ float w0_as_f32(const float* p) { return *p; }
 __device__ __forceinline__ float w0_as_f32(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
 
@@ -346,6 +507,7 @@ __device__ __forceinline__ void lowrank_sweep_body(
             float dot = (c0 + c1) + (c2 + c3);
             if constexpr (L >= 2) dot += quad_swap<0xB1>(dot);      // lanes 0<->1, 2<->3
             if constexpr (L >= 4) dot += quad_swap<0x4E>(dot);      // lanes 0<->2, 1<->3
+            if constexpr (L >= 8) dot += quad_swap<0x141>(dot);     // lane i <-> 7 - i of every eight
             const float x = wv[t] + dot;
             const float qf = __builtin_amdgcn_fmed3f(
                 __builtin_rintf(__builtin_fmaf(x, rv[t], zv[t])), 0.0f, maxq);
@@ -390,8 +552,10 @@ __global__ __launch_bounds__(256) void lowrank_sweep_kernel(
         lowrank_sweep_body<16, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
     else if (nr == 32)
         lowrank_sweep_body<32, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
-    else
+    else if (nr == 64)
         lowrank_sweep_body<64, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
+    else
+        lowrank_sweep_body<128, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
 }
 
 // A layer that saw no rows at all has H = I (gptq.py:97-99): nothing couples its columns and the
@@ -504,8 +668,8 @@ extern "C" int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, 
                                     forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1LL << 22), "bad shape batch=%lld C=%lld",
                   (long long)batch, (long long)C);
-    FORGE_REQUIRE(n == 16 || n == 32 || n == 64, "n=%lld: 16, 32 or 64 rows (pad with zero rows)",
-                  (long long)n);
+    FORGE_REQUIRE(n == 16 || n == 32 || n == 64 || n == 128,
+                  "n=%lld: 16, 32, 64 or 128 rows (pad with zero rows)", (long long)n);
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(Bp && D && Hm && info && ws, "null pointer");
     FORGE_REQUIRE(ws_bytes >= forge_lowrank_workspace_bytes(batch, C, n), "workspace too small");
@@ -519,7 +683,18 @@ extern "C" int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, 
                                forge::WORK_FLOPS);
     if (n == 16) return launch_lowrank_factor<16>(Bp, D, Hm, info, batch, C, (double*)ws, st);
     if (n == 32) return launch_lowrank_factor<32>(Bp, D, Hm, info, batch, C, (double*)ws, st);
-    return launch_lowrank_factor<64>(Bp, D, Hm, info, batch, C, (double*)ws, st);
+    if (n == 64) return launch_lowrank_factor<64>(Bp, D, Hm, info, batch, C, (double*)ws, st);
+    double* gram = (double*)ws;
+    const int nblk = (int)forge::ceil_div(C, FB);
+    const dim3 grid((unsigned)nblk, (unsigned)batch), block(WN * WS);
+    lowrank_gram_wide_kernel<<<grid, block, 0, st>>>(Bp, D, gram, C, nblk);
+    FORGE_LAUNCH_CHECK();
+    lowrank_suffix_kernel<<<dim3((unsigned)forge::ceil_div(WN * WN, 256), (unsigned)batch), dim3(256), 0,
+                            st>>>(gram, info, nblk, WN * WN);
+    FORGE_LAUNCH_CHECK();
+    lowrank_block_wide_kernel<<<grid, block, 0, st>>>(Bp, D, gram, Hm, info, C, nblk);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
 }
 
 extern "C" int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, const float* Bp,
@@ -542,8 +717,8 @@ extern "C" int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, cons
                   "Bp and Hm must be 16-byte aligned");
     double rows = 0.0;
     for (int64_t b = 0; b < batch; ++b) {
-        FORGE_REQUIRE(n_host[b] == 16 || n_host[b] == 32 || n_host[b] == 64,
-                      "n[%lld]=%lld: 16, 32 or 64 rows (pad with zero rows)", (long long)b,
+        FORGE_REQUIRE(n_host[b] == 16 || n_host[b] == 32 || n_host[b] == 64 || n_host[b] == 128,
+                      "n[%lld]=%lld: 16, 32, 64 or 128 rows (pad with zero rows)", (long long)b,
                       (long long)n_host[b]);
         rows += (double)n_host[b];
     }

@@ -39,9 +39,11 @@ class ExpertGroupGPTQ:
         w0 - deq (``kernels.gptq_sweep_direct_batched``): the same solve in exact arithmetic
         at half the factorisation work, codes differing only where fp32 rounding decides a
         near-tie.
-        low_rank_tokens (0..64; algorithm "gptq" on the direct route, C a multiple of 16):
+        low_rank_tokens (0..128; algorithm "gptq" on the direct route, C a multiple of 16):
         experts with at most this many calibration rows are solved from the rows themselves,
-        see the module text; 0 = every expert through its Hessian.  ``self.H[e]`` of such an
+        see the module text; 0 = every expert through its Hessian.  Beyond 64 rows the per-row
+        vector sweep costs about what the route through the Hessian costs (measured), hence
+        the default.  ``self.H[e]`` of such an
         expert is never written."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
@@ -67,14 +69,14 @@ class ExpertGroupGPTQ:
         self.rel_damp = rel_damp
         self.H: Optional[torch.Tensor] = None           # [E, C, C] f32
         self.num_samples = [0] * self.E                 # host-side counts
-        if not 0 <= int(low_rank_tokens) <= 64:
-            raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..64")
+        if not 0 <= int(low_rank_tokens) <= 128:
+            raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..128")
         ok = algorithm == "gptq" and factor_route == "direct" and self.C % 16 == 0 \
             and len({w.dtype for w in self.W}) == 1
         self.low_rank_tokens = int(low_rank_tokens) if ok else 0
         # rows of the experts that are still on the low-rank route, [E, _cap, C] f32 (zero rows
         # beyond num_samples[e]); low_rank[e] turns False for good once an expert has seen more
-        self._cap = next(n for n in (16, 32, 64) if n >= max(self.low_rank_tokens, 1))
+        self._cap = next(n for n in (16, 32, 64, 128) if n >= max(self.low_rank_tokens, 1))
         self.low_rank = [self.low_rank_tokens > 0] * self.E
         self._kept: Optional[torch.Tensor] = None
         self.issue_non_invertible = torch.zeros(self.E, dtype=torch.bool)
@@ -307,9 +309,9 @@ class ExpertGroupGPTQ:
                     lr_stream = lr_side if lr_side is not None and dn_ids else main
                     lr_stream.wait_stream(main)
                 with torch.cuda.stream(lr_stream):
-                    # by the number of rows the kernels are compiled for: 16, 32 or 64
+                    # by the number of rows the kernels are compiled for: 16, 32, 64 or 128
                     buckets = []
-                    for lo, nr in ((0, 16), (16, 32), (32, 64)):
+                    for lo, nr in ((0, 16), (16, 32), (32, 64), (64, 128)):
                         ids = [i for i in lr_ids if lo < self.num_samples[e0 + i] <= nr]
                         if ids:
                             buckets.append((nr, ids))
