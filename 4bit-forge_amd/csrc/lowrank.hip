@@ -18,7 +18,7 @@
 // dense route in exact arithmetic; in floating point this route is the more accurate one (the
 // recurrence runs in float64, where S shrinks from 1 to damp / |b|^2 without losing its digits).
 //
-// Compiled for n = 16, 32, 64 and 128 rows of B (rows beyond a layer's own count are zero rows;
+// Compiled for n = 4, 16, 32, 64 and 128 rows of B (rows beyond a layer's own count are zero rows;
 // 128 with four threads per row of S in the factor):
 //   lowrank_gram/suffix/block_kernel   the recurrence, cut into blocks of 128 columns that
 //                                      start from their own S and run side by side; writes h_k.
@@ -394,7 +394,8 @@ __device__ __forceinline__ float w0_as_f32(const float* p) { return *p; }
 __device__ __forceinline__ float w0_as_f32(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
 
 // ---------------------------------------------------------------- sweep
-// A row's n-vector a is spread over L = NR / 16 neighbouring lanes, sixteen entries each: the
+// A row's n-vector a is spread over L = NR / 16 neighbouring lanes, sixteen entries each (one
+// lane with four entries for NR = 4, the experts with a handful of rows): the
 // dot product is sixteen multiply-adds per lane and a butterfly over the L lanes (both
 // partners add the same two numbers, so all of them hold the same value and quantise alike),
 // the update sixteen more.  256 / L rows per workgroup.  h_k and b_k are the same for every row:
@@ -415,7 +416,8 @@ __device__ __forceinline__ void lowrank_sweep_body(
     const int32_t* __restrict__ info, uint8_t* __restrict__ q, int64_t C, int64_t R, int64_t G,
     float maxq) {
     constexpr int TK = 16;                        // columns per staged tile
-    constexpr int L = NR / 16;                    // lanes per row
+    constexpr int NA = NR < 16 ? NR : 16;         // entries of a per lane
+    constexpr int L = NR / NA;                    // lanes per row
     constexpr int Q = NR / 4;                     // float4 per column
     __shared__ float4 Ts[2][2][TK][Q];            // [buffer][0 = h, 1 = b][column][quarter]
     const int64_t b = blockIdx.y;
@@ -455,9 +457,9 @@ __device__ __forceinline__ void lowrank_sweep_body(
         }
     };
 
-    float a[16];
+    float a[NA];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) a[j] = 0.0f;
+    for (int j = 0; j < NA; ++j) a[j] = 0.0f;
 
     float wv[TK], sv[TK], rv[TK], zv[TK];
     auto load_meta = [&](int64_t k0, float (&w)[TK], float (&s)[TK], float (&z)[TK]) {
@@ -490,15 +492,15 @@ __device__ __forceinline__ void lowrank_sweep_body(
         for (int t = 0; t < TK; ++t) rv[t] = 1.0f / (sv[t] + kEps);
 #pragma unroll
         for (int t = 0; t < TK; ++t) {
-            float h[16], bb[16];
+            float h[NA], bb[NA];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4 v = Ts[buf][0][t][4 * part + j];
+            for (int j = 0; j < NA / 4; ++j) {
+                const float4 v = Ts[buf][0][t][(NA / 4) * part + j];
                 h[4 * j + 0] = v.x; h[4 * j + 1] = v.y; h[4 * j + 2] = v.z; h[4 * j + 3] = v.w;
             }
             float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, c3 = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 16; j += 4) {
+            for (int j = 0; j < NA; j += 4) {
                 c0 = __builtin_fmaf(a[j + 0], h[j + 0], c0);
                 c1 = __builtin_fmaf(a[j + 1], h[j + 1], c1);
                 c2 = __builtin_fmaf(a[j + 2], h[j + 2], c2);
@@ -515,12 +517,12 @@ __device__ __forceinline__ void lowrank_sweep_body(
             const float d = wv[t] - deq;
             if (live) qo[(k0 + t) * R] = (uint8_t)qf;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4 v = Ts[buf][1][t][4 * part + j];
+            for (int j = 0; j < NA / 4; ++j) {
+                const float4 v = Ts[buf][1][t][(NA / 4) * part + j];
                 bb[4 * j + 0] = v.x; bb[4 * j + 1] = v.y; bb[4 * j + 2] = v.z; bb[4 * j + 3] = v.w;
             }
 #pragma unroll
-            for (int j = 0; j < 16; ++j) a[j] = __builtin_fmaf(d, bb[j], a[j]);
+            for (int j = 0; j < NA; ++j) a[j] = __builtin_fmaf(d, bb[j], a[j]);
         }
         if (more) {
             stash(buf ^ 1, stage);
@@ -548,7 +550,9 @@ __global__ __launch_bounds__(256) void lowrank_sweep_kernel(
     float maxq, MixedTable tab) {
     const int nr = tab.nr[blockIdx.y];
     const int64_t off = tab.off[blockIdx.y];
-    if (nr == 16)
+    if (nr == 4)
+        lowrank_sweep_body<4, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
+    else if (nr == 16)
         lowrank_sweep_body<16, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
     else if (nr == 32)
         lowrank_sweep_body<32, W0T>(W0, Bp + off, Hm + off, scT, qzT, g_idx, info, q, C, R, G, maxq);
@@ -668,8 +672,8 @@ extern "C" int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, 
                                     forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= 1 && C < (1LL << 22), "bad shape batch=%lld C=%lld",
                   (long long)batch, (long long)C);
-    FORGE_REQUIRE(n == 16 || n == 32 || n == 64 || n == 128,
-                  "n=%lld: 16, 32, 64 or 128 rows (pad with zero rows)", (long long)n);
+    FORGE_REQUIRE(n == 4 || n == 16 || n == 32 || n == 64 || n == 128,
+                  "n=%lld: 4, 16, 32, 64 or 128 rows (pad with zero rows)", (long long)n);
     if (batch == 0) return FORGE_OK;
     FORGE_REQUIRE(Bp && D && Hm && info && ws, "null pointer");
     FORGE_REQUIRE(ws_bytes >= forge_lowrank_workspace_bytes(batch, C, n), "workspace too small");
@@ -681,6 +685,7 @@ extern "C" int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, 
     forge::KernelTiming timing("lowrank_factor", st,
                                ((6.0 * n * n + 2.0 * n) * C + 2.0 * n * n * n * nb) * (double)batch,
                                forge::WORK_FLOPS);
+    if (n == 4) return launch_lowrank_factor<4>(Bp, D, Hm, info, batch, C, (double*)ws, st);
     if (n == 16) return launch_lowrank_factor<16>(Bp, D, Hm, info, batch, C, (double*)ws, st);
     if (n == 32) return launch_lowrank_factor<32>(Bp, D, Hm, info, batch, C, (double*)ws, st);
     if (n == 64) return launch_lowrank_factor<64>(Bp, D, Hm, info, batch, C, (double*)ws, st);
@@ -717,8 +722,9 @@ extern "C" int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, cons
                   "Bp and Hm must be 16-byte aligned");
     double rows = 0.0;
     for (int64_t b = 0; b < batch; ++b) {
-        FORGE_REQUIRE(n_host[b] == 16 || n_host[b] == 32 || n_host[b] == 64 || n_host[b] == 128,
-                      "n[%lld]=%lld: 16, 32, 64 or 128 rows (pad with zero rows)", (long long)b,
+        FORGE_REQUIRE(n_host[b] == 4 || n_host[b] == 16 || n_host[b] == 32 || n_host[b] == 64 ||
+                          n_host[b] == 128,
+                      "n[%lld]=%lld: 4, 16, 32, 64 or 128 rows (pad with zero rows)", (long long)b,
                       (long long)n_host[b]);
         rows += (double)n_host[b];
     }
@@ -737,7 +743,7 @@ extern "C" int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, cons
             off += C * n_host[b0 + i];
             if (n_host[b0 + i] > most) most = (int)n_host[b0 + i];
         }
-        const dim3 grid((unsigned)forge::ceil_div(R, 256 / (most / 16)), (unsigned)nb), block(256);
+        const dim3 grid((unsigned)forge::ceil_div(R, 256 / (most <= 16 ? 1 : most / 16)), (unsigned)nb), block(256);
         const char* w0 = (const char*)W0 + (size_t)(b0 * C * R) * w0_size;
         if (w0_dtype == FORGE_BF16)
             lowrank_sweep_kernel<uint16_t><<<grid, block, 0, st>>>(

@@ -435,11 +435,11 @@ class _HipKernels:
         return out
 
     def lowrank_factor(self, Bp, D, out=None):
-        """Bp [B,C,n] f32 (n = 16, 32, 64 or 128), D [B,C] f32 -> (Hm [B,C,n] f32, info [B] i32): the
+        """Bp [B,C,n] f32 (n = 4, 16, 32, 64 or 128), D [B,C] f32 -> (Hm [B,C,n] f32, info [B] i32): the
         factor of D + Bp^T Bp as the n-vectors the low-rank sweep reads (see forge_hip.h)."""
         _need_cuda(Bp, D)
         B, C, n = Bp.shape
-        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and n in (16, 32, 64, 128)
+        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and n in (4, 16, 32, 64, 128)
         assert D.is_contiguous() and D.dtype == torch.float32 and tuple(D.shape) == (B, C)
         if out is not None:
             Hm, info = out
@@ -457,12 +457,12 @@ class _HipKernels:
         return Hm, info
 
     def gptq_sweep_lowrank_mixed(self, W0, Bp, Hm, ns, info, scalesT, qzerosT, g_idx, bits):
-        """gptq_sweep_lowrank for matrices of different n in one launch: ns[b] in (16, 32, 64, 128);
+        """gptq_sweep_lowrank for matrices of different n in one launch: ns[b] in (4, 16, 32, 64, 128);
         Bp/Hm flat f32 buffers holding matrix b's [C, ns[b]] vectors one after the other."""
         _need_cuda(W0, Bp, Hm, info, scalesT, qzerosT, g_idx)
         B, C, R = W0.shape
         G = scalesT.shape[1]
-        assert len(ns) == B and all(int(n) in (16, 32, 64, 128) for n in ns)
+        assert len(ns) == B and all(int(n) in (4, 16, 32, 64, 128) for n in ns)
         total = C * sum(int(n) for n in ns)
         assert W0.is_contiguous() and Bp.is_contiguous() and Hm.is_contiguous()
         assert Bp.numel() == total and Hm.numel() == total and Bp.dtype == Hm.dtype == torch.float32
@@ -479,14 +479,14 @@ class _HipKernels:
         return q
 
     def gptq_sweep_lowrank(self, W0, Bp, Hm, info, scalesT, qzerosT, g_idx, bits):
-        """W0 [B,C,R] (f32/bf16, solver order), Bp/Hm [B,C,n] (n = 16, 32, 64 or 128), scalesT/qzerosT
+        """W0 [B,C,R] (f32/bf16, solver order), Bp/Hm [B,C,n] (n = 4, 16, 32, 64 or 128), scalesT/qzerosT
         [B,G,R], g_idx [B,C] i32 -> codes [B,C,R] u8."""
         _need_cuda(W0, Bp, Hm, info, scalesT, qzerosT, g_idx)
         B, C, R = W0.shape
         G = scalesT.shape[1]
         n = Bp.shape[2]
         assert W0.is_contiguous() and Bp.is_contiguous() and Hm.is_contiguous()
-        assert n in (16, 32, 64, 128) and tuple(Bp.shape) == (B, C, n) and tuple(Hm.shape) == (B, C, n)
+        assert n in (4, 16, 32, 64, 128) and tuple(Bp.shape) == (B, C, n) and tuple(Hm.shape) == (B, C, n)
         assert scalesT.is_contiguous() and qzerosT.is_contiguous() and tuple(scalesT.shape) == (B, G, R)
         assert tuple(qzerosT.shape) == (B, G, R) and scalesT.dtype == torch.float32
         assert g_idx.dtype == torch.int32 and g_idx.is_contiguous() and tuple(g_idx.shape) == (B, C)

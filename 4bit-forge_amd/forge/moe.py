@@ -309,9 +309,9 @@ class ExpertGroupGPTQ:
                     lr_stream = lr_side if lr_side is not None and dn_ids else main
                     lr_stream.wait_stream(main)
                 with torch.cuda.stream(lr_stream):
-                    # by the number of rows the kernels are compiled for: 16, 32, 64 or 128
+                    # by the number of rows the kernels are compiled for: 4, 16, 32, 64 or 128
                     buckets = []
-                    for lo, nr in ((0, 16), (16, 32), (32, 64), (64, 128)):
+                    for lo, nr in ((0, 4), (4, 16), (16, 32), (32, 64), (64, 128)):
                         ids = [i for i in lr_ids if lo < self.num_samples[e0 + i] <= nr]
                         if ids:
                             buckets.append((nr, ids))

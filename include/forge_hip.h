@@ -218,7 +218,7 @@ int forge_gptq_sweep_direct_batched_w0(float* X, const void* W0, int w0_dtype, i
  *     w0_k + Hm[k] . a  and then adds (w0_k - deq_k) Bp[k] to the row's n-vector a: the values
  *     forge_gptq_sweep_direct_batched reaches in exact arithmetic, the reference's quantiser
  *     (solver.cu:9-23).  Matrices with info != 0 are swept uncoupled (gptq.py:172-175).
- * n is 16, 32, 64 or 128 (pad with zero rows), C % 16 == 0. */
+ * n is 4, 16, 32, 64 or 128 (pad with zero rows), C % 16 == 0. */
 /* GPTQ.quantize for a layer that saw NO calibration rows: H = I (gptq.py:97-99), its factor is
  * the identity, nothing couples the columns and the sweep of solver.cu:9-154 is its quantiser
  * (solver.cu:9-23) applied to every weight.  W [batch][R][C] (w_dtype f32 or bf16, row pitch ldw,
@@ -234,7 +234,7 @@ int forge_lowrank_factor(const float* Bp, const float* D, float* Hm, int32_t* in
                          int64_t C, int64_t n, void* ws, int64_t ws_bytes, forge_stream_t stream);
 int64_t forge_lowrank_workspace_bytes(int64_t batch, int64_t C, int64_t n);
 /* forge_gptq_sweep_lowrank for matrices of different n in ONE launch (each of the three sizes
- * alone leaves most of the GPU idle): n_host[b] in {16, 32, 64, 128} (host array), and matrix b's
+ * alone leaves most of the GPU idle): n_host[b] in {4, 16, 32, 64, 128} (host array), and matrix b's
  * vectors start C * (n_host[0] + ... + n_host[b-1]) floats into Bp and into Hm, i.e. the per-size
  * [batch_n][C][n] arrays laid end to end in batch order.  Everything else as above. */
 int forge_gptq_sweep_lowrank_mixed(const void* W0, int w0_dtype, const float* Bp, const float* Hm,

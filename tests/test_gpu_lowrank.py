@@ -26,7 +26,7 @@ def _lower_factor(H):
 
 def _problem(C, n, seed, dead=()):
     g = torch.Generator().manual_seed(seed)
-    Bp = torch.zeros(C, 16 if n <= 16 else 32 if n <= 32 else 64 if n <= 64 else 128)
+    Bp = torch.zeros(C, 4 if 0 < n <= 4 else 16 if n <= 16 else 32 if n <= 32 else 64 if n <= 64 else 128)
     Bp[:, :n] = torch.randn(C, n, generator=g) * (2.0 / max(n, 1)) ** 0.5
     Bp[:, 0] *= torch.linspace(3.0, 0.3, C)                 # an "activation-ordered" spread
     D = torch.full((C,), 0.02)
@@ -36,7 +36,7 @@ def _problem(C, n, seed, dead=()):
     return Bp, D
 
 
-@pytest.mark.parametrize("n", [0, 1, 5, 16, 23, 64, 100, 128])
+@pytest.mark.parametrize("n", [0, 1, 3, 5, 16, 23, 64, 100, 128])
 def test_factor_matches_the_dense_float64_factor(hip, n):
     C = 384
     probs = [_problem(C, n, s, dead=(7, 200) if s == 1 else ()) for s in range(3)]
@@ -79,7 +79,7 @@ def _float64_gptq(W, H, s, z, maxq=15.0):
 
 @pytest.mark.parametrize("n,dtype", [(1, torch.float32), (4, torch.bfloat16), (16, torch.bfloat16),
                                      (0, torch.float32), (30, torch.bfloat16), (64, torch.float32),
-                                     (50, torch.bfloat16), (128, torch.bfloat16), (90, torch.float32)])
+                                     (50, torch.bfloat16), (128, torch.bfloat16), (90, torch.float32), (3, torch.bfloat16)])
 def test_sweep_matches_float64_gptq_on_the_dense_factor(hip, n, dtype):
     C, R, gs = 256, 300, 128
     G = C // gs
@@ -121,7 +121,7 @@ def test_failed_factor_sweeps_uncoupled(hip):
     s, z = oracle.build_group_meta_packed(W0.t().contiguous().reshape(R, gs), 4, True)
     g_idx = torch.zeros(C, dtype=torch.int32)
     args = (s.view(1, 1, R).to(DEV), z.view(1, 1, R).to(DEV), g_idx[None].to(DEV), 4)
-    Hm = torch.full((1, C, 16), float("nan"), device=DEV)          # never read
+    Hm = torch.full((1, C, Bp.shape[1]), float("nan"), device=DEV)  # never read
     bad = torch.ones(1, dtype=torch.int32, device=DEV)
     q = hip.gptq_sweep_lowrank(W0[None].to(DEV), Bp[None].to(DEV), Hm, bad, *args)[0].cpu()
     # the quantiser's fma(x, 1/(s+eps), z): the product of two floats is exact in float64
