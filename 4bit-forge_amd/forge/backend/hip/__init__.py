@@ -396,6 +396,8 @@ class _HipKernels:
         E = H.shape[0]
         C = H.shape[-1]
         assert len(row0) == E and len(counts) == E
+        assert all(int(c) >= 0 and int(o) >= 0 and (int(c) == 0 or int(o) + int(c) <= X.shape[0])
+                   for o, c in zip(row0, counts)), "row range outside X"
         r0 = (ctypes.c_int64 * E)(*[int(o) for o in row0])
         cn = (ctypes.c_int64 * E)(*[int(o) for o in counts])
         al = (ctypes.c_float * E)(*[float(a) for a in alpha])
