@@ -415,7 +415,9 @@ __device__ __forceinline__ void lowrank_sweep_body(
     const float* __restrict__ scT, const float* __restrict__ qzT, const int32_t* __restrict__ g_idx,
     const int32_t* __restrict__ info, uint8_t* __restrict__ q, int64_t C, int64_t R, int64_t G,
     float maxq) {
-    constexpr int TK = 16;                        // columns per staged tile
+    constexpr int TK = 8;                         // columns per staged tile (16: twice the registers for the
+                                                  // prefetched weights, scales and zeros, half the wavefronts per
+                                                  // SIMD, 28 % slower; 4: no faster)
     constexpr int NA = NR < 16 ? NR : 16;         // entries of a per lane
     constexpr int L = NR / NA;                    // lanes per row
     constexpr int Q = NR / 4;                     // float4 per column
