@@ -572,48 +572,53 @@ __global__ __launch_bounds__(256) void round_to_nearest_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const float* __restrict__ scales,
     const float* __restrict__ qzeros, uint8_t* __restrict__ q, int64_t R, int64_t C, int64_t gs,
     int64_t G, float maxq, const int64_t* __restrict__ index) {
-    const int64_t per_row = (C + 7) / 8;
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= R * per_row) return;
-    const int64_t b = index ? index[blockIdx.y] : blockIdx.y, r = idx / per_row, c0 = (idx - r * per_row) * 8;
-    const T* __restrict__ src = W + b * w_stride + r * ldw + c0;
-    const float* __restrict__ sc = scales + (b * R + r) * G;
-    const float* __restrict__ qz = qzeros + (b * R + r) * G;
-    uint8_t* __restrict__ dst = q + (b * R + r) * C + c0;
-    float v[8];
-    const bool whole = c0 + 8 <= C;
-    if (whole && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && sizeof(T) == 2) {
-        const uint4 w = *reinterpret_cast<const uint4*>(src);
-        v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
-        v[2] = __uint_as_float(w.y << 16); v[3] = __uint_as_float(w.y & 0xffff0000u);
-        v[4] = __uint_as_float(w.z << 16); v[5] = __uint_as_float(w.z & 0xffff0000u);
-        v[6] = __uint_as_float(w.w << 16); v[7] = __uint_as_float(w.w & 0xffff0000u);
-    } else {
+    // grid: (eight-column pieces of a row / 256, rows, matrices): no division to find the row,
+    // one 32-bit division to find the first group, boundaries counted from there
+    const uint32_t c0 = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    if ((int64_t)c0 >= C) return;
+    const int64_t b = index ? index[blockIdx.z] : blockIdx.z;
+    const uint32_t gs32 = (uint32_t)gs, C32 = (uint32_t)C;
+    const bool whole = c0 + 8 <= C32;
+    for (int64_t r = blockIdx.y; r < R; r += gridDim.y) {
+        const T* __restrict__ src = W + b * w_stride + r * ldw + c0;
+        const float* __restrict__ sc = scales + (b * R + r) * G;
+        const float* __restrict__ qz = qzeros + (b * R + r) * G;
+        uint8_t* __restrict__ dst = q + (b * R + r) * C + c0;
+        float v[8];
+        if (whole && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && sizeof(T) == 2) {
+            const uint4 w = *reinterpret_cast<const uint4*>(src);
+            v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
+            v[2] = __uint_as_float(w.y << 16); v[3] = __uint_as_float(w.y & 0xffff0000u);
+            v[4] = __uint_as_float(w.z << 16); v[5] = __uint_as_float(w.z & 0xffff0000u);
+            v[6] = __uint_as_float(w.w << 16); v[7] = __uint_as_float(w.w & 0xffff0000u);
+        } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (c0 + i < C) ? w0_as_f32(src + i) : 0.0f;
-    }
-    uint32_t lo = 0, hi = 0;
-    int64_t g_have = -1;
-    float s = 0.0f, z = 0.0f, rcp = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int64_t g = (c0 + i < C ? c0 + i : C - 1) / gs;
-        if (g != g_have) {
-            g_have = g;
-            s = sc[g];
-            z = qz[g];
-            rcp = 1.0f / (s + kEps);
+            for (int i = 0; i < 8; ++i) v[i] = (c0 + i < C32) ? w0_as_f32(src + i) : 0.0f;
         }
-        const uint32_t code = (uint32_t)__builtin_amdgcn_fmed3f(
-            __builtin_rintf(__builtin_fmaf(v[i], rcp, z)), 0.0f, maxq);
-        if (i < 4) lo |= code << (8 * i); else hi |= code << (8 * (i - 4));
-    }
-    if (whole && (reinterpret_cast<uintptr_t>(dst) & 7u) == 0) {
-        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
-    } else {
+        uint32_t lo = 0, hi = 0;
+        uint32_t g = c0 / gs32, next = (g + 1) * gs32;      // first column of the next group
+        float s = sc[g], z = qz[g];
+        float rcp = 1.0f / (s + kEps);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (c0 + i < C) dst[i] = (uint8_t)(((i < 4 ? lo : hi) >> (8 * (i & 3))) & 0xffu);
+        for (int i = 0; i < 8; ++i) {
+            if (c0 + i >= next && c0 + i < C32) {
+                ++g;
+                next += gs32;
+                s = sc[g];
+                z = qz[g];
+                rcp = 1.0f / (s + kEps);
+            }
+            const uint32_t code = (uint32_t)__builtin_amdgcn_fmed3f(
+                __builtin_rintf(__builtin_fmaf(v[i], rcp, z)), 0.0f, maxq);
+            if (i < 4) lo |= code << (8 * i); else hi |= code << (8 * (i - 4));
+        }
+        if (whole && (reinterpret_cast<uintptr_t>(dst) & 7u) == 0) {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (c0 + i < C32) dst[i] = (uint8_t)(((i < 4 ? lo : hi) >> (8 * (i & 3))) & 0xffu);
+        }
     }
 }
 
@@ -633,8 +638,9 @@ extern "C" int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stri
     FORGE_REQUIRE(W && scales && qzeros && qweight, "null pointer");
     hipStream_t st = (hipStream_t)stream;
     const int64_t G = forge::ceil_div(C, gs);
-    const int64_t threads = R * ((C + 7) / 8);
-    const dim3 grid((unsigned)forge::ceil_div(threads, 256), (unsigned)batch), block(256);
+    const dim3 grid((unsigned)forge::ceil_div((C + 7) / 8, 256), (unsigned)(R < 65535 ? R : 65535),
+                    (unsigned)batch),
+        block(256);
     const float maxq = (float)((1 << bits) - 1);
     forge::KernelTiming timing("round_to_nearest", st,
                                (double)batch * R * C * ((w_dtype == FORGE_BF16 ? 2.0 : 4.0) + 1.0),
