@@ -29,7 +29,7 @@ class ExpertGroupGPTQ:
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
                  algorithm: str = "gptq", device=None, factor_route: str = "direct",
-                 low_rank_tokens: int = 64):
+                 low_rank_tokens: int = 128):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
@@ -41,9 +41,9 @@ class ExpertGroupGPTQ:
         near-tie.
         low_rank_tokens (0..128; algorithm "gptq" on the direct route, C a multiple of 16):
         experts with at most this many calibration rows are solved from the rows themselves,
-        see the module text; 0 = every expert through its Hessian.  Beyond 64 rows the per-row
-        vector sweep costs about what the route through the Hessian costs (measured), hence
-        the default.  ``self.H[e]`` of such an
+        see the module text; 0 = every expert through its Hessian.  At 65-128 rows the per-row
+        vector sweep costs nearly what the route through the Hessian costs (measured: 1 % of a
+        benchmark step in its favour).  ``self.H[e]`` of such an
         expert is never written."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")

@@ -10,7 +10,7 @@ forge.synth.deepseek_v3_moe (seed 0) on the GPU.  One STEP = one pass of the hot
 one chunk of experts, everything already resident in HBM: ragged Hessian accumulation for
 gate/up and for down, then per expert two factorisations (gate and up share theirs), three
 scale searches and three sweeps.  Successive steps walk through the layer's experts chunk
-by chunk (128 experts a step; their routed-token lists differ).  Experts with at most 64
+by chunk (128 experts a step; their routed-token lists differ).  Experts with at most 128
 routed rows (most of them: 8192 tokens over 256 experts with Zipf popularity) take the
 library's low-rank route, which reaches the same result from the rows themselves without a
 C x C Hessian; `config.experts_by_route` counts them.
@@ -114,7 +114,7 @@ def make_workload(name, cfg, chunk, seed=0):
 STREAMS = []
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=64):
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128):
     """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
     jobs one after the other (per-kernel event times are then exclusive)."""
     import torch
@@ -447,7 +447,7 @@ def main():
     ap.add_argument("--factor-route", default="direct", choices=["direct", "inverse"],
                     help="direct (default): sweep fed by the factor of H itself; inverse: the "
                          "reference's factor of inv(H) and fp32-chain sweep")
-    ap.add_argument("--low-rank-tokens", type=int, default=64,
+    ap.add_argument("--low-rank-tokens", type=int, default=128,
                     help="experts with at most this many routed rows are solved from the rows themselves "
                          "(0: every expert through its Hessian)")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
@@ -492,7 +492,7 @@ def main():
     roofline = dict(kernel=dom, bound="mfma" if bound == "mfma" else "hbm", achieved=d["rate"],
                     peak=PEAK[peak_key], unit=d["rate_unit"], frac=d["frac"],
                     traffic=measured_traffic(a.config, chunk, dom)
-                    if a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 64 else None,
+                    if a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 128 else None,
                     avg_launch_us=d["avg_us"], launches=d["launches"],
                     note="achieved = algorithmic work (2*M*N*K counted once per fp32 product) / event time")
     if by_time != dom:
