@@ -1,4 +1,4 @@
-"""The low-rank route (layers that saw at most 64 calibration rows) against dense float64
+"""The low-rank route (layers that saw at most 128 calibration rows) against dense float64
 algebra and against the route through the Hessian.
 
 The closed forms are pinned by the dense computation they replace: the lower factor M of
