@@ -17,6 +17,8 @@ arithmetic.
 """
 from __future__ import annotations
 
+import collections
+import threading
 from typing import List, Optional, Sequence
 
 import torch
@@ -25,6 +27,14 @@ from forge.backend.hip import kernels
 
 
 class ExpertGroupGPTQ:
+    # quantize() queues its work and returns without waiting for the GPU.  A caller that builds
+    # group after group (a layer's chunks, a model's layers) would otherwise run arbitrarily far
+    # ahead of the device, each call holding tens of GB of workspace that cannot be reused before
+    # its kernels have run: every call waits for the call before the last MAX_IN_FLIGHT to finish.
+    MAX_IN_FLIGHT = 2
+    _in_flight = collections.deque()
+    _in_flight_lock = threading.Lock()
+
     def __init__(self, weights: Sequence[torch.Tensor], bits: int = 4, group_size: int = 128,
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
@@ -79,7 +89,24 @@ class ExpertGroupGPTQ:
         self._cap = next(n for n in (16, 32, 64, 128) if n >= max(self.low_rank_tokens, 1))
         self.low_rank = [self.low_rank_tokens > 0] * self.E
         self._kept: Optional[torch.Tensor] = None
-        self.issue_non_invertible = torch.zeros(self.E, dtype=torch.bool)
+        self._non_invertible = torch.zeros(self.E, dtype=torch.bool)
+        self._pending_info = []                          # (expert ids, device flags) not yet fetched
+
+    @property
+    def issue_non_invertible(self) -> torch.Tensor:
+        """[E] bool: experts whose factorisation failed in a quantize() so far (they were solved
+        with the identity instead, forge/gptq.py:168-175).  Reading it waits for the GPU."""
+        for ids, info in self._pending_info:
+            self._non_invertible[ids] |= (info > 0).cpu()
+        self._pending_info = []
+        return self._non_invertible
+
+    def _dev(self, values, dtype=None):
+        """A small host list as a device tensor without stopping the host: through pinned memory
+        and an asynchronous copy (torch.tensor(..., device=...) copies from pageable memory and
+        returns only when the stream has reached the copy, i.e. when all the work queued before
+        it is done)."""
+        return torch.tensor(values, dtype=dtype).pin_memory().to(self.device, non_blocking=True)
 
     # ------------------------------------------------------------------ Hessians
     @torch.no_grad()
@@ -118,8 +145,7 @@ class ExpertGroupGPTQ:
             alpha.append(2.0 / max(total, 1))
             beta.append(n / max(total, 1))
         if src:
-            self._kept.view(self.E * self._cap, self.C)[torch.tensor(dst, device=self.device)] = \
-                X[torch.tensor(src, device=self.device)].float()
+            self._kept.view(self.E * self._cap, self.C)[self._dev(dst)] = X[self._dev(src)].float()
         kernels.hessian_update_ranges(X, row0, counts, self.H, alpha, beta)
         if late:
             # experts that leave the low-rank route: their Hessian from the kept rows and the
@@ -152,7 +178,7 @@ class ExpertGroupGPTQ:
         if self.H is None:
             self.H = torch.empty((E, C, C), dtype=torch.float32, device=dev)
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
-        seen = torch.tensor([n > 0 for n in self.num_samples], device=dev)
+        seen = self._dev([n > 0 for n in self.num_samples])
         diag_all = self.H.diagonal(dim1=1, dim2=2)                        # [E, C] view
         lr_host = list(self.low_rank)
         any_lr = any(lr_host)
@@ -161,9 +187,8 @@ class ExpertGroupGPTQ:
             # once, as the Hessian kernel does for the others); H[e] itself holds nothing
             if self._kept is None:
                 self._kept = torch.zeros((E, self._cap, C), dtype=torch.float32, device=dev)
-            lr_dev = torch.tensor(lr_host, device=dev)
-            alpha32 = torch.tensor([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32,
-                                   device=dev)
+            lr_dev = self._dev(lr_host)
+            alpha32 = self._dev([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32)
             d_lr = ((self._kept.double() ** 2).sum(dim=1) * alpha32.double()[:, None]).float()
             diag_all = torch.where(lr_dev[:, None], d_lr, diag_all)
         bad = (~seen) | torch.isnan(diag_all).any(dim=1)
@@ -186,7 +211,7 @@ class ExpertGroupGPTQ:
             self.H[e].zero_()
             self.H[e].diagonal().fill_(1.0)
             diag_all = self.H.diagonal(dim1=1, dim2=2) if not any_lr else diag_all.index_fill(
-                0, torch.tensor([e], device=dev), 1.0)
+                0, self._dev([e]), 1.0)
         failed = []
         side = torch.cuda.Stream(device=dev) if overlap_scale_search else None   # default priority
         # the low-rank experts' kernels are chains of dependent steps on a few wavefronts: on a
@@ -281,7 +306,7 @@ class ExpertGroupGPTQ:
                 def layout_in(ids, W0, X=None, skip_out=False):
                     """weights of the chunk's experts `ids` -> solver order: one launch per stack"""
                     whole = len(ids) == B
-                    idx = None if whole else torch.tensor(ids, device=dev)
+                    idx = None if whole else self._dev(ids)
                     r0 = 0
                     for i in job:
                         kernels.weight_to_solver_order(self.W[i][e0:e1], perm_inv, dead_u8, out=X, row0=r0,
@@ -290,7 +315,7 @@ class ExpertGroupGPTQ:
 
                 def layout_out(ids, q, M=None):
                     whole = len(ids) == B
-                    idx = None if whole else torch.tensor(ids, device=dev)
+                    idx = None if whole else self._dev(ids)
                     r0 = 0
                     for i in job:
                         Ri = sizes[i]
@@ -325,7 +350,7 @@ class ExpertGroupGPTQ:
                         W0 = torch.empty((len(ids_all), C, R), dtype=self.W[job[0]].dtype, device=dev)
                     pos = at = 0
                     for nr, ids in buckets:
-                        li = torch.tensor(ids, device=dev)
+                        li = self._dev(ids)
                         msk = mask[li].bool()                               # [Bl, C], solver order
                         root = alpha32[e0:e1][li].double().sqrt()[:, None, None]
                         Bp = torch.gather((self._kept[e0:e1][li][:, :nr].double() * root).float(), 2,
@@ -347,7 +372,7 @@ class ExpertGroupGPTQ:
                             t.record_stream(lr_stream)
                     if ids_all:
                         failed.append((torch.tensor([e0 + i for i in ids_all]), info))
-                        la = torch.tensor(ids_all, device=dev)
+                        la = self._dev(ids_all)
                         q = kernels.gptq_sweep_lowrank_mixed(W0, Bp_all, Hm_all, ns, info, sT[la], zT[la],
                                                              g_idx[la].contiguous(), self.bits)
                         pos = 0
@@ -357,7 +382,7 @@ class ExpertGroupGPTQ:
                         del W0, q, Bp_all, Hm_all
                     # experts without a single row (or with NaN rows): H = I, plain rounding
                     if none_ids:
-                        ni = torch.tensor(none_ids, device=dev)
+                        ni = self._dev(none_ids)
                         for (sc_i, qz_i), i in zip(parts, job):
                             kernels.round_to_nearest(self.W[i][e0:e1], sc_i, qz_i, gs, self.bits,
                                                      out=outs[i][0][e0:e1], index=ni)
@@ -365,7 +390,7 @@ class ExpertGroupGPTQ:
                 # ---------------------------------------------------------- through the Hessian
                 if dn_ids:
                     whole = len(dn_ids) == B
-                    di = None if whole else torch.tensor(dn_ids, device=dev)
+                    di = None if whole else self._dev(dn_ids)
                     pick = (lambda t: t) if whole else (lambda t: t[di].contiguous())
                     Bd = len(dn_ids)
                     # the factorisations read their input's lower triangle in 128 x 128 blocks only
@@ -439,6 +464,16 @@ class ExpertGroupGPTQ:
                     outs[i][1][e0:e1] = scales.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     outs[i][2][e0:e1] = qzeros.view(B, R, G)[:, r0:r0 + Ri].reshape(B, Ri * G)
                     r0 += Ri
-        for ids, info in failed:
-            self.issue_non_invertible[ids] |= (info > 0).cpu()
+        # the failure flags stay on the device until someone looks (issue_non_invertible): quantize()
+        # itself never waits for the GPU after its one look at the Hessian diagonals
+        self._pending_info.extend(failed)
+        done = torch.cuda.Event()
+        done.record()
+        oldest = None
+        with ExpertGroupGPTQ._in_flight_lock:
+            ExpertGroupGPTQ._in_flight.append(done)
+            if len(ExpertGroupGPTQ._in_flight) > ExpertGroupGPTQ.MAX_IN_FLIGHT:
+                oldest = ExpertGroupGPTQ._in_flight.popleft()
+        if oldest is not None:
+            oldest.synchronize()
         return [tuple(o) for o in outs]

@@ -477,6 +477,7 @@ def main():
         del src, dst
     route = dict(factor_route=a.factor_route, low_rank_tokens=a.low_rank_tokens)
     elapsed = timed_steps(wl, cfg, chunk, a.steps, a.warmup, mse=mse, **route)
+    peak_gb = torch.cuda.max_memory_reserved() / 1e9      # workload and the steps in flight
 
     # one more step with per-kernel HIP-event timing (on the stream the kernels run on); its
     # jobs run one after the other so that no kernel's time includes another stream's work
@@ -524,6 +525,7 @@ def main():
                    "experts_by_route": route_counts(wl, chunk, a.low_rank_tokens if a.factor_route == "direct" else 0)},
         "roofline": roofline,
         "kernels": breakdown,
+        "peak_device_memory_gb": round(peak_gb, 1),
     }
     if "mse_grid" in breakdown and mse:
         # nominal candidate evaluations: P = 100 shrink factors for every weight of the step
