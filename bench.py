@@ -434,8 +434,8 @@ def cpu_baseline(wl, cfg, reps=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="deepseek_v3", choices=sorted(CONFIGS))
     ap.add_argument("--chunk", type=int, default=0, help="experts per step (0 = config default)")
     ap.add_argument("--split", type=int, default=1,
