@@ -170,9 +170,10 @@ __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, flo
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int l = Q + 4 * j;
-        float loss = 0.0f;
+        // (the reference starts from 0 and adds: the same value, every term being >= +0)
+        float loss = element_loss<FLOOR>(v[l], s, rcp, q0, maxq, norm);
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) loss += element_loss<FLOOR>(v[l + 32 * i], s, rcp, q0, maxq, norm);
+        for (int i = 1; i < VPL; ++i) loss += element_loss<FLOOR>(v[l + 32 * i], s, rcp, q0, maxq, norm);
         p[j] = loss;
     }
     return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
