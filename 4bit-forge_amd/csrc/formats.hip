@@ -80,6 +80,52 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(
     }
 }
 
+// I and the scale tile width multiples of 16, input and output 16-byte aligned: one workgroup
+// per row (row, scale row and batch come from the block index once, in scalar registers), one
+// 16-byte piece per thread and turn, and the conversions the matrix cores' input formats
+// brought along: two fp8 -> two f32 and two f32 -> two bf16 (round to nearest even) in one
+// instruction each.  Both are exact restatements of the bit arithmetic above for every input
+// that is no NaN; a NaN stays a NaN.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(1024) void fp8_block_dequant_rows_kernel(
+    const uint4* __restrict__ w, const float* __restrict__ sinv, void* __restrict__ out, uint32_t O,
+    uint32_t per_row, uint32_t so, uint32_t si16, uint32_t nO, uint32_t nI) {
+    const uint32_t row = blockIdx.x;                  // batch * O + r
+    const uint32_t b = row / O, r = row - b * O;
+    const float* srow = sinv + ((size_t)b * nO + r / so) * nI;
+    const size_t base = (size_t)row * per_row;
+    for (uint32_t p = threadIdx.x; p < per_row; p += blockDim.x) {
+        const uint4 q = w[base + p];
+        const float sc = srow[p / si16];
+        const uint32_t wq[4] = {q.x, q.y, q.z, q.w};
+        f32x2 f[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            f[2 * k] = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq[k], false) * sc;
+            f[2 * k + 1] = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq[k], true) * sc;
+        }
+        if constexpr (OUT_BF16) {
+            uint32_t pk[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const bf16x2 h = __builtin_convertvector(f[k], bf16x2);
+                pk[k] = __builtin_bit_cast(uint32_t, h);
+            }
+            uint4* dst = reinterpret_cast<uint4*>(out) + 2 * (base + p);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        } else {
+            float4* dst = reinterpret_cast<float4*>(out) + 4 * (base + p);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                dst[k] = make_float4(f[2 * k].x, f[2 * k].y, f[2 * k + 1].x, f[2 * k + 1].y);
+        }
+    }
+}
+
 // 1:4 codes + keep-masks -> the inference layout of bitpacking_sparsegptq14.cu:58-107: for
 // every row and every 32-column word one u64
 //   bf16(scale) << 48 | idx16 << 32 | qw32
@@ -295,6 +341,23 @@ extern "C" int forge_fp8_e4m3_block_dequant(const uint8_t* w, const float* scale
     forge::KernelTiming timing("fp8_block_dequant", (hipStream_t)stream,
                                (double)batch * O * I * (out_dtype == FORGE_BF16 ? 3.0 : 5.0),
                                forge::WORK_BYTES);
+    if (I % 16 == 0 && si % 16 == 0 && (reinterpret_cast<uintptr_t>(w) % 16) == 0 &&
+        (reinterpret_cast<uintptr_t>(out) % 16) == 0 && batch * O < (1LL << 31) && I < (1LL << 32) &&
+        so < (1LL << 32) && si < (1LL << 32) && nO < (1LL << 32)) {
+        const uint32_t per_row = (uint32_t)(I / 16);
+        const dim3 rows((unsigned)(batch * O));
+        const dim3 block((unsigned)std::min<int64_t>(1024, forge::ceil_div((int64_t)per_row, 64) * 64));
+        if (out_dtype == FORGE_BF16)
+            fp8_block_dequant_rows_kernel<true><<<rows, block, 0, (hipStream_t)stream>>>(
+                (const uint4*)w, scale_inv, out, (uint32_t)O, per_row, (uint32_t)so, (uint32_t)(si / 16),
+                (uint32_t)nO, (uint32_t)nI);
+        else
+            fp8_block_dequant_rows_kernel<false><<<rows, block, 0, (hipStream_t)stream>>>(
+                (const uint4*)w, scale_inv, out, (uint32_t)O, per_row, (uint32_t)so, (uint32_t)(si / 16),
+                (uint32_t)nO, (uint32_t)nI);
+        FORGE_LAUNCH_CHECK();
+        return FORGE_OK;
+    }
     dim3 grid((unsigned)forge::ceil_div(n, 256));
     if (out_dtype == FORGE_BF16)
         fp8_block_dequant_kernel<true><<<grid, dim3(256), 0, (hipStream_t)stream>>>(

@@ -325,6 +325,42 @@ __global__ __launch_bounds__(256) void pack_int4_fast_kernel(const uint8_t* __re
     packed[idx] = (int32_t)word;
 }
 
+// The four codes in the bytes of x, each plus its row's bias modulo 16, as four nibbles.
+__device__ __forceinline__ uint32_t four_nibbles(uint32_t x, uint32_t bias4) {
+    const uint32_t v = ((x & 0x0F0F0F0Fu) + bias4) & 0x0F0F0F0Fu;
+    const uint32_t t = (v | (v >> 4)) & 0x00FF00FFu;
+    return (t | (t >> 8)) & 0xFFFFu;
+}
+
+// C and the group size multiples of 16, codes 16-byte aligned, fewer than 2^32 pieces: the
+// code array is one run of 16-byte pieces, a thread packs one piece into two words.  32-bit
+// index arithmetic throughout (with 64-bit divisions per thread the kernel is bound by them,
+// not by memory).  EVEN: the groups tile the row exactly, so piece / (gs / 16) numbers the
+// zero points.
+template <bool EVEN>
+__global__ __launch_bounds__(256) void pack_int4_wide_kernel(const uint4* __restrict__ codes,
+                                                             const float* __restrict__ qzeros,
+                                                             uint2* __restrict__ packed, uint32_t pieces,
+                                                             uint32_t per_row, uint32_t gs16, uint32_t G) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= pieces) return;
+    const uint4 cc = codes[idx];
+    int z = 8;
+    if (qzeros) {
+        uint32_t zi;
+        if constexpr (EVEN) {
+            zi = idx / gs16;
+        } else {
+            const uint32_t r = idx / per_row;
+            zi = r * G + (idx - r * per_row) / gs16;
+        }
+        z = (int)qzeros[zi];
+    }
+    const uint32_t bias4 = ((uint32_t)(8 - z) & 0xFu) * 0x01010101u;
+    packed[idx] = make_uint2(four_nibbles(cc.x, bias4) | (four_nibbles(cc.y, bias4) << 16),
+                             four_nibbles(cc.z, bias4) | (four_nibbles(cc.w, bias4) << 16));
+}
+
 }  // namespace
 
 static int weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, int64_t ldw,
@@ -506,6 +542,22 @@ extern "C" int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_
     const int64_t n = R * ((C + 7) / 8);
     forge::KernelTiming timing("pack_int4", (hipStream_t)stream,
                                1.5 * R * C + 4.0 * R * forge::ceil_div(C, gs), forge::WORK_BYTES);
+    if (C % 16 == 0 && gs % 16 == 0 && (reinterpret_cast<uintptr_t>(codes) % 16) == 0 &&
+        (reinterpret_cast<uintptr_t>(packed) % 8) == 0 && n / 2 < (1LL << 32) - 256 && gs < (1LL << 32) &&
+        R * forge::ceil_div(C, gs) < (1LL << 32)) {
+        const uint32_t pieces = (uint32_t)(n / 2), per_row = (uint32_t)(C / 16);
+        const dim3 grid((unsigned)forge::ceil_div((int64_t)pieces, 256));
+        if (C % gs == 0)
+            pack_int4_wide_kernel<true><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
+                (const uint4*)codes, qzeros, (uint2*)packed, pieces, per_row, (uint32_t)(gs / 16),
+                (uint32_t)(C / gs));
+        else
+            pack_int4_wide_kernel<false><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
+                (const uint4*)codes, qzeros, (uint2*)packed, pieces, per_row, (uint32_t)(gs / 16),
+                (uint32_t)forge::ceil_div(C, gs));
+        FORGE_LAUNCH_CHECK();
+        return FORGE_OK;
+    }
     if (C % 8 == 0 && gs % 8 == 0 && (reinterpret_cast<uintptr_t>(codes) % 8) == 0 &&
         forge::ceil_div(n, 256) < (1LL << 31)) {
         pack_int4_fast_kernel<<<dim3((unsigned)forge::ceil_div(n, 256)), dim3(256), 0,

@@ -78,7 +78,8 @@ def test_gpu_sparse_pack_bit_exact(hip, R, C):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("O,I,dtype", [(256, 512, torch.bfloat16), (300, 384, torch.bfloat16),
-                                       (77, 128, torch.float32)])
+                                       (77, 128, torch.float32), (50, 200, torch.bfloat16),
+                                       (40, 136, torch.float32), (3, 20480, torch.bfloat16)])
 def test_gpu_fp8_block_dequant_bit_exact(hip, O, I, dtype):
     g = torch.Generator().manual_seed(O)
     raw = torch.randint(0, 256, (2, O, I), dtype=torch.uint8, generator=g)      # every byte pattern

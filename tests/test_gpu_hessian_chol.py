@@ -202,17 +202,18 @@ def test_pack_int4_layout(hip):
     assert torch.equal(pk8.to(torch.int64) & 0xFFFFFFFF, sum(sh[:, :, k] << (4 * k) for k in range(8)))
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("gs", [128, 32])
-def test_pack_int4_aligned_rows(hip, gs):
-    """C and the group size multiples of 8: the 8-byte-load form, same words as the general one."""
-    R, C = 96, 1024
+@pytest.mark.parametrize("C,gs", [(1024, 128), (1024, 32), (1040, 128), (1008, 48), (1000, 40), (1000, 64)])
+def test_pack_int4_aligned_rows(hip, C, gs):
+    """C and the group size multiples of 16 (16-byte loads, groups tiling the row or not) or of
+    8 (8-byte loads): same words as the general form."""
+    R = 96
     g = torch.Generator().manual_seed(2)
     codes = torch.randint(0, 16, (R, C), dtype=torch.uint8, generator=g)
-    G = C // gs
+    G = (C + gs - 1) // gs
     z = torch.randint(0, 16, (R * G,), generator=g).float()
     for zeros in (z, None):
         pk = hip.pack_int4(codes.to(DEV), None if zeros is None else zeros.to(DEV), gs).cpu()
-        zz = 8 if zeros is None else z.view(R, G).repeat_interleave(gs, 1).to(torch.int64)
+        zz = 8 if zeros is None else z.view(R, G).repeat_interleave(gs, 1)[:, :C].to(torch.int64)
         sh = ((codes.to(torch.int64) - zz + 8) & 0xF).view(R, -1, 8)
         ref = sum(sh[:, :, k] << (4 * k) for k in range(8))
         assert torch.equal(pk.to(torch.int64) & 0xFFFFFFFF, ref)
