@@ -276,6 +276,46 @@ __global__ __launch_bounds__(256) void dequantize_groups_kernel(
     }
 }
 
+// C and the group size multiples of 16, codes and output 16-byte aligned: one workgroup per
+// row, a 16-byte piece of codes per thread and turn, 32-bit indices, bf16 rounding (to nearest
+// even, as f32_to_bf16_rne) by the hardware's packed conversion.
+template <bool OUT_BF16>
+__global__ __launch_bounds__(1024) void dequantize_groups_rows_kernel(
+    const uint4* __restrict__ q, const float* __restrict__ scales, const float* __restrict__ qzeros,
+    void* __restrict__ out, uint32_t per_row, uint32_t gs16, uint32_t G) {
+    const size_t row = blockIdx.x;                    // batch * R + r
+    const float* __restrict__ s = scales + row * G;
+    const float* __restrict__ z = qzeros + row * G;
+    const size_t base = row * per_row;
+    for (uint32_t p = threadIdx.x; p < per_row; p += blockDim.x) {
+        const uint4 v = q[base + p];
+        const uint32_t g = p / gs16;
+        const float zz = z[g], ss = s[g];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        float val[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) val[k] = ((float)((w[k >> 2] >> (8 * (k & 3))) & 0xFFu) - zz) * ss;
+        if constexpr (OUT_BF16) {
+            uint32_t pk[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                f32x2 pair;
+                pair.x = val[2 * k];
+                pair.y = val[2 * k + 1];
+                pk[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+            }
+            uint4* dst = reinterpret_cast<uint4*>(out) + 2 * (base + p);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        } else {
+            float4* dst = reinterpret_cast<float4*>(out) + 4 * (base + p);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                dst[k] = make_float4(val[4 * k], val[4 * k + 1], val[4 * k + 2], val[4 * k + 3]);
+        }
+    }
+}
+
 // out[i][:] = X[row_idx[i]][:] * weight[i]; one workgroup per output row, 8 bytes per lane.
 template <typename T, bool SCALE>
 __global__ __launch_bounds__(256) void gather_scaled_rows_kernel(
@@ -400,6 +440,21 @@ extern "C" int forge_dequantize_groups(const uint8_t* q, const float* scales, co
     forge::KernelTiming timing("dequantize_groups", (hipStream_t)stream,
                                (double)batch * R * (C * (out_dtype == FORGE_BF16 ? 3.0 : 5.0) + 8.0 * G),
                                forge::WORK_BYTES);
+    if (C % 16 == 0 && gs % 16 == 0 && (reinterpret_cast<uintptr_t>(q) % 16) == 0 &&
+        (reinterpret_cast<uintptr_t>(out) % 16) == 0 && batch * R < (1LL << 31) && C < (1LL << 32) &&
+        gs < (1LL << 32)) {
+        const uint32_t per_row = (uint32_t)(C / 16);
+        const dim3 rows((unsigned)(batch * R));
+        const dim3 block((unsigned)std::min<int64_t>(1024, forge::ceil_div((int64_t)per_row, 64) * 64));
+        if (out_dtype == FORGE_BF16)
+            dequantize_groups_rows_kernel<true><<<rows, block, 0, (hipStream_t)stream>>>(
+                (const uint4*)q, scales, qzeros, out, per_row, (uint32_t)(gs / 16), (uint32_t)G);
+        else
+            dequantize_groups_rows_kernel<false><<<rows, block, 0, (hipStream_t)stream>>>(
+                (const uint4*)q, scales, qzeros, out, per_row, (uint32_t)(gs / 16), (uint32_t)G);
+        FORGE_LAUNCH_CHECK();
+        return FORGE_OK;
+    }
     const dim3 grid((unsigned)forge::ceil_div(n, 256));
     if (out_dtype == FORGE_BF16)
         dequantize_groups_kernel<true><<<grid, dim3(256), 0, (hipStream_t)stream>>>(q, scales, qzeros, out,

@@ -52,7 +52,8 @@ def test_oracle_routed_rows_brute_force():
 
 # ------------------------------------------------------------------ HIP parity (bit-exact)
 @pytest.mark.gpu
-@pytest.mark.parametrize("B,R,C,gs", [(1, 33, 300, 128), (3, 64, 1024, 128), (2, 7, 70, 32)])
+@pytest.mark.parametrize("B,R,C,gs", [(1, 33, 300, 128), (3, 64, 1024, 128), (2, 7, 70, 32),
+                                      (2, 5, 1040, 128), (1, 3, 20480, 48), (2, 9, 1024, 40)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_dequantize_groups_matches_oracle(hip, B, R, C, gs, dtype):
     g = torch.Generator().manual_seed(C)
