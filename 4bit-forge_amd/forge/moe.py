@@ -334,9 +334,11 @@ class ExpertGroupGPTQ:
                     lr_stream = lr_side if lr_side is not None and dn_ids else main
                     lr_stream.wait_stream(main)
                 with torch.cuda.stream(lr_stream):
-                    # by the number of rows the kernels are compiled for: 4, 16, 32, 64 or 128
+                    # by the number of rows the kernels are compiled for: 4, 16, 32, 64 or 128; the
+                    # largest first: the sweep's workgroups start in launch order and run in
+                    # proportion to their rows, the short ones fill in behind the long ones
                     buckets = []
-                    for lo, nr in ((0, 4), (4, 16), (16, 32), (32, 64), (64, 128)):
+                    for lo, nr in ((64, 128), (32, 64), (16, 32), (4, 16), (0, 4)):
                         ids = [i for i in lr_ids if lo < self.num_samples[e0 + i] <= nr]
                         if ids:
                             buckets.append((nr, ids))
