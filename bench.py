@@ -289,8 +289,9 @@ def mfma_ceiling():
 
 
 def hbm_kernels(wl):
-    """min/max grid, int4 pack and fp8 block dequant on the chunk's gate_proj stack (chunk x 2048
-    x 7168): achieved GB/s of the algorithmic bytes against 8 TB/s."""
+    """min/max grid, int4 pack, fp8 block dequant and write-back dequant on the chunk's gate_proj
+    stack (chunk x 2048 x 7168), the 1:4 packer on an eighth of it and the routed-row gather on the
+    layer's calibration rows: achieved GB/s of the algorithmic bytes against 8 TB/s."""
     import torch
     from forge.backend.hip import kernels
     Wg = wl["Wg"]
@@ -301,11 +302,27 @@ def hbm_kernels(wl):
     w8 = Wg.float().clamp(-0.05, 0.05).mul(448 / 0.05).to(torch.float8_e4m3fn).view(torch.uint8)
     sinv = torch.full((B, (O + 127) // 128, (I + 127) // 128), 0.05 / 448, device="cuda")
 
+    G = (I + 127) // 128
+    scales = torch.full((B, O * G), 0.01, device="cuda")
+    codes3 = codes.view(B, O, I)
+    # the 1:4 packer on one expert's tall matrix, every group of four keeping its first column
+    G32 = I // 32
+    keep = torch.full((G32, B * O // 8), 0x11111111, dtype=torch.int32, device="cuda").view(torch.uint32)
+    sc32 = torch.full((G32, B * O // 8), 0.01, device="cuda")
+    codes_tall = codes[:B * O // 8]
+    # routed-row gather: every calibration row once, in a random order, with its routing weight
+    xs = wl["xs"]
+    order = torch.randperm(xs.shape[0], generator=g, device="cuda")
+    gate = torch.rand(xs.shape[0], generator=g, device="cuda").to(xs.dtype)
+
     def work():
         for _ in range(3):
             kernels.quant_grid(Wg, 128, 4, False, False)
             kernels.pack_int4(codes, zeros, 128)
             kernels.fp8_block_dequant(w8, sinv)
+            kernels.dequantize_groups(codes3, scales, zeros.view(B, O * G), 128, torch.bfloat16)
+            kernels.pack_sparsegptq14_to_u64x2(codes_tall, keep, sc32)
+            kernels.gather_scaled_rows(xs, order, gate)
 
     work()
     stats = timing_pass(work)
