@@ -261,22 +261,49 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
     if (search) {
         const float xmin = symmetric ? 0.0f : -(sg * q0g);
         float best_loss = 3.402823466e+38f;
+        // The group's extreme values are two of the summands; shrinking the scale clips them
+        // first.  A single summand is a lower bound of the (monotone, non-negative) fp32 sum,
+        // so once it reaches the best loss for every group of the wavefront the candidate is
+        // out without touching the other gs-2 elements.
+        //
+        // Symmetric grids (the zero point does not move with the candidate) make that test
+        // before the candidate's reciprocal is even divided out, on |diff| instead of the loss:
+        // `reach` is the |diff| from which one element's loss is certain to reach best_loss
+        // (its 1/norm-th power plus a margin of 1e-4 against the few ulp of the log/exp pair;
+        // the power is monotone for norm >= 1).  An extreme whose quotient by the approximate
+        // reciprocal lies a whole level beyond the clamp is clamped under the exact reciprocal
+        // as well (the two quotients differ by a few 1e-6), and then fma(bound, s, -x) IS its
+        // diff.  Anything less clear counts as 0, which only means that the candidate is
+        // evaluated: the test is an optimisation, candidate_loss decides.
+        const bool early = symmetric && norm >= 1.0f;
+        const float inv_norm = 1.0f / norm;
+        const float top = maxq - q0g, bot = -q0g;
+        float reach = 3.402823466e+38f;
         for (int p = 0; p < P; ++p) {
             const float s = sg * cand[p];
+            if (early) {
+                const float approx = __builtin_amdgcn_rcpf(s + kEps);
+                const float over = (hi * approx >= top + 1.0f) ? -__builtin_fmaf(top, s, -hi) : 0.0f;
+                const float under = (lo * approx <= bot - 1.0f) ? __builtin_fmaf(bot, s, -lo) : 0.0f;
+                if (__builtin_amdgcn_ballot_w64(!(fmaxf(over, under) >= reach)) == 0) continue;
+            }
             const float rcp = 1.0f / (s + kEps);
             const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
-            // The group's extreme values are two of the summands; shrinking the scale clips
-            // them first.  A single summand is a lower bound of the (monotone, non-negative)
-            // fp32 sum, so once it reaches the best loss for every group of the wavefront
-            // the candidate is out without touching the other gs-2 elements.
-            const float clip = fmaxf(element_loss<FLOOR>(lo, s, rcp, q0, maxq, norm),
-                                     element_loss<FLOOR>(hi, s, rcp, q0, maxq, norm));
-            if (__builtin_amdgcn_ballot_w64(clip < best_loss) == 0) continue;
+            if (!early) {
+                const float clip = fmaxf(element_loss<FLOOR>(lo, s, rcp, q0, maxq, norm),
+                                         element_loss<FLOOR>(hi, s, rcp, q0, maxq, norm));
+                if (__builtin_amdgcn_ballot_w64(clip < best_loss) == 0) continue;
+            }
             const float loss = candidate_loss<GS, FLOOR>(v, s, rcp, q0, maxq, norm, best_loss);
             if (loss < best_loss) {
                 best_loss = loss;
                 best_s = s;
                 best_q = q0;
+                // (a loss of exactly 0 cannot be improved on: everything is out; losses down
+                // where the log would see a denormal: no early test)
+                reach = loss == 0.0f ? 0.0f
+                        : loss < 1e-30f ? 3.402823466e+38f
+                        : __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(loss) * inv_norm) * 1.0001f;
             }
         }
     }

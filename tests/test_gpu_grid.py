@@ -135,3 +135,29 @@ def test_full_size_scale_search_properties(hip):
     G = 7168 // 128
     pick = (rows[:, None] * G + torch.arange(G)[None, :]).flatten().to(DEV)
     _check_mse(s0, z0, L, s[pick], z[pick], p.cpu(), sm)
+
+
+def test_symmetric_search_at_config3_shape(hip):
+    """One expert's projection of config 3 (2048 x 7168 bf16 out of the fp8 block round trip,
+    symmetric grid: the zero point stays put, so the search tests the clipped extremes before it
+    divides): every chosen scale is a candidate, and a sample of rows against the oracle."""
+    from forge import synth
+    g = torch.Generator().manual_seed(11)
+    W = synth.fp8_block_roundtrip((0.02 * torch.randn(2048, 7168, generator=g)).bfloat16()).to(DEV)
+    p = torch.linspace(1.0, 0.2, 100, device=DEV)
+    s_mm, z_mm = hip.quant_grid(W, 128, 4, True, False)
+    s, z = hip.quant_grid(W, 128, 4, True, True, p, 2.4)
+    assert torch.equal(z, z_mm) and bool((z == 8).all())
+    idx = torch.bucketize(-(s / s_mm), -p).clamp(0, 99)
+    ok = torch.zeros_like(s, dtype=torch.bool)
+    for d in (-1, 0, 1):
+        ok |= s == s_mm * p[(idx + d).clamp(0, 99)]
+    assert bool(ok.all())
+    rows = torch.arange(0, 2048, 64)
+    Wg = W[rows].float().cpu().reshape(-1, 128)
+    s0, z0 = oracle.build_group_meta_packed(Wg, 4, True)
+    sm = s0.clone()
+    s0, z0, L = oracle.mse_scale_groups_packed(Wg, s0, z0, p.cpu(), 2.4, 4, True, return_losses=True)
+    G = 7168 // 128
+    pick = (rows[:, None] * G + torch.arange(G)[None, :]).flatten().to(DEV)
+    _check_mse(s0, z0, L, s[pick], z[pick], p.cpu(), sm)
