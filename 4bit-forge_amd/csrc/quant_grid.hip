@@ -279,13 +279,33 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
         const float inv_norm = 1.0f / norm;
         const float top = maxq - q0g, bot = -q0g;
         float reach = 3.402823466e+38f;
+        // Both |diff| grow as the scale shrinks and best_loss only changes when a candidate is
+        // evaluated: a candidate that is out for the whole wavefront, each lane by an extreme
+        // that is clamped with room to spare (1.01 levels: the next, smaller scale keeps it
+        // beyond 1), takes every later candidate with a factor no larger out with it.
+        bool rest_out = false;
+        float out_from = 0.0f;
         for (int p = 0; p < P; ++p) {
-            const float s = sg * cand[p];
+            const float factor = cand[p];
+            if (rest_out && factor <= out_from) continue;
+            const float s = sg * factor;
             if (early) {
                 const float approx = __builtin_amdgcn_rcpf(s + kEps);
-                const float over = (hi * approx >= top + 1.0f) ? -__builtin_fmaf(top, s, -hi) : 0.0f;
-                const float under = (lo * approx <= bot - 1.0f) ? __builtin_fmaf(bot, s, -lo) : 0.0f;
-                if (__builtin_amdgcn_ballot_w64(!(fmaxf(over, under) >= reach)) == 0) continue;
+                const float qh = hi * approx, ql = lo * approx;
+                const float over = (qh >= top + 1.0f) ? -__builtin_fmaf(top, s, -hi) : 0.0f;
+                const float under = (ql <= bot - 1.0f) ? __builtin_fmaf(bot, s, -lo) : 0.0f;
+                if (__builtin_amdgcn_ballot_w64(!(fmaxf(over, under) >= reach)) == 0) {
+                    // (a grid handed in with its zero point outside [0, maxq] or a scale below
+                    // zero would turn the growth around: never settled)
+                    const bool settled = sg > 0.0f && top >= 0.0f && bot <= 0.0f &&
+                                         ((qh >= top + 1.01f && over >= reach) ||
+                                          (ql <= bot - 1.01f && under >= reach));
+                    if (__builtin_amdgcn_ballot_w64(!settled) == 0) {
+                        rest_out = true;
+                        out_from = factor;
+                    }
+                    continue;
+                }
             }
             const float rcp = 1.0f / (s + kEps);
             const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
