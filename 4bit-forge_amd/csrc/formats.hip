@@ -136,12 +136,12 @@ __global__ __launch_bounds__(1024) void fp8_block_dequant_rows_kernel(
 // The three inputs want different lane orders: the codes are row-major [R, C] (a word's 32
 // bytes are contiguous, neighbouring words of one row follow each other), while masks,
 // scales and the output are word-major ([word][row]: neighbouring rows are contiguous).  So a
-// workgroup takes a tile of 32 rows x 32 words, brings the tile's codes into LDS with lanes
-// running along the columns (1 KiB contiguous per row, 16 bytes per lane), and then switches
-// to lanes running along the rows for everything else: 128-byte runs of masks and scales,
-// 512-byte runs of output, and byte reads from LDS whose row pitch (1040 bytes) spreads the
-// 32 rows over the banks.
-constexpr int SP_ROWS = 32, SP_WORDS = 32, SP_COLS = SP_WORDS * 32, SP_PITCH = SP_COLS + 16;
+// workgroup takes a tile of 128 rows x 8 words, brings the tile's codes into LDS with lanes
+// running along the columns (256 bytes contiguous per row, 16 bytes per lane), and then
+// switches to lanes running along the rows for everything else: 512-byte runs of masks and
+// scales, 2 KiB runs of output, and 16-byte reads from LDS (row pitch 272 bytes).
+constexpr int SP_ROWS = 128, SP_WORDS = 8, SP_COLS = SP_WORDS * 32, SP_PITCH = SP_COLS + 16;
+constexpr int SP_PAIRS_PER_TURN = 256 / SP_ROWS;     // word pairs that the 256 threads build at a time
 
 __global__ __launch_bounds__(256) void pack_sparse14_tile_kernel(
     const uint8_t* __restrict__ codes, const uint32_t* __restrict__ keep,
@@ -178,8 +178,8 @@ __global__ __launch_bounds__(256) void pack_sparse14_tile_kernel(
     if (r >= R) return;
     const uint8_t* trow = &tile[lr * SP_PITCH];
 #pragma unroll
-    for (int it = 0; it < SP_WORDS / 2 / 8; ++it) {
-        const int lpair = (tid >> 5) + 8 * it;                 // pair of words inside the tile
+    for (int it = 0; it < SP_WORDS / 2 / SP_PAIRS_PER_TURN; ++it) {
+        const int lpair = tid / SP_ROWS + SP_PAIRS_PER_TURN * it;   // pair of words inside the tile
         const int64_t pair = word0 / 2 + lpair;
         if (2 * pair >= n_words) break;
         uint64_t both[2];
@@ -189,17 +189,22 @@ __global__ __launch_bounds__(256) void pack_sparse14_tile_kernel(
             uint64_t packed = 0ull;
             if (word < n_words) {
                 const uint32_t mask = keep[word * R + r];
-                const uint8_t* tw = trow + (2 * lpair + h) * 32;
+                // the word's 32 codes as two 16-byte reads, a group of four = one register;
+                // no branch below: a data-dependent byte read inside a branch is a branch and
+                // an LDS round trip per group, one after the other
+                const uint4* tw = reinterpret_cast<const uint4*>(trow + (2 * lpair + h) * 32);
+                const uint4 lo4 = tw[0], hi4 = tw[1];
+                const uint32_t fours[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+                const int64_t col = word * 32;
                 uint32_t where = 0u, kept = 0u;
 #pragma unroll
                 for (int grp = 0; grp < 8; ++grp) {
                     const uint32_t four = (mask >> (4 * grp)) & 0xFu;
-                    uint32_t code = 8u, pos = 0u;
-                    if (four != 0u) {
-                        pos = (uint32_t)__builtin_ctz(four);   // first kept column of the group
-                        // columns past C hold no code: the slot keeps the code of zero
-                        if (word * 32 + 4 * grp + pos < C) code = tw[4 * grp + pos] & 0xFu;
-                    }
+                    // first kept column of the group (0 where it kept nothing)
+                    const uint32_t pos = (uint32_t)__builtin_ctz(four | 16u) & 3u;
+                    // columns past C hold no code: the slot keeps the code of zero
+                    const bool has = four != 0u && col + 4 * grp + pos < C;
+                    const uint32_t code = has ? (fours[grp] >> (8 * pos)) & 0xFu : 8u;
                     where |= pos << (2 * grp);
                     kept |= code << (4 * grp);
                 }
