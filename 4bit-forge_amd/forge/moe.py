@@ -34,6 +34,23 @@ class ExpertGroupGPTQ:
     MAX_IN_FLIGHT = 2
     _in_flight = collections.deque()
     _in_flight_lock = threading.Lock()
+    # The device runs the kernels of one hardware queue one after the other, and a process has
+    # four such queues for all of its streams: a fresh pair of side streams per call ends up
+    # sharing queues with the callers' streams in patterns that change from call to call (a
+    # chain of small kernels then waits behind a 20 ms scale search).  So every group of a
+    # device shares ONE stream for the scale searches (each fills the device: they run one
+    # after the other anyway, in the order of the quantize() calls) and ONE for the low-rank
+    # experts' chains: with two callers' streams that is four streams, one queue each.
+    _side_streams = {}
+    _side_streams_lock = threading.Lock()
+
+    @classmethod
+    def _streams_of(cls, dev):
+        key = dev.index if dev.index is not None else torch.cuda.current_device()
+        with cls._side_streams_lock:
+            if key not in cls._side_streams:
+                cls._side_streams[key] = (torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev))
+            return cls._side_streams[key]                   # default priority
 
     def __init__(self, weights: Sequence[torch.Tensor], bits: int = 4, group_size: int = 128,
                  symmetric: bool = False, quantization_scale: str = "mse",
@@ -91,6 +108,7 @@ class ExpertGroupGPTQ:
         self._kept: Optional[torch.Tensor] = None
         self._non_invertible = torch.zeros(self.E, dtype=torch.bool)
         self._pending_info = []                          # (expert ids, device flags) not yet fetched
+        self._prepared = None                            # what prepare() queued, until quantize() uses it
 
     @property
     def issue_non_invertible(self) -> torch.Tensor:
@@ -115,6 +133,7 @@ class ExpertGroupGPTQ:
         offsets[e]:offsets[e+1].  Running mean per expert as in forge/gptq.py:61-80."""
         if len(offsets) != self.E + 1:
             raise ValueError("offsets must have E+1 entries")
+        self._prepared = None
         X = X.to(self.device)
         if X.dtype not in (torch.bfloat16, torch.float32):
             X = X.float()
@@ -163,18 +182,15 @@ class ExpertGroupGPTQ:
 
     # ------------------------------------------------------------------ solve
     @torch.no_grad()
-    def quantize(self, chunk: int = 32, max_shrink: float = 0.2, n_grid: int = 100,
-                 norm: float = 2.4, overlap_scale_search: bool = True):
-        """Returns one (qweight [E,R,C] u8, scales [E,R*G] f32, qzeros [E,R*G] f32) per stack;
-        with algorithm="sparsegptq" a fourth element M [E, ceil(C/32), R] u32 (bit i of word w
-        <-> column 32 w + i of the SOLVER order, as the reference returns it).
-        overlap_scale_search=False keeps the scale search on the caller's stream instead of a
-        side stream (same results; for per-kernel timing, where no kernel's time should include
-        another stream's work)."""
-        E, C, gs, dev = self.E, self.C, self.group_size, self.device
-        G = (C + gs - 1) // gs
-        mse = self.quantization_scale == "mse"
-        cand = torch.linspace(1.0, max_shrink, n_grid, dtype=torch.float32, device=dev) if mse else None
+    def prepare(self):
+        """Queues what quantize() has to know on the host before it can queue the solve (which
+        experts have no usable Hessian, which have dead features, which may have all-zero
+        weight columns) and the transfer of those few flags, and returns without waiting.
+        quantize() calls it itself; a caller that calls it earlier, right after its last
+        update() and on the same stream, with other work queued behind it, finds the flags
+        there when it calls quantize(), which then neither waits for that other work nor makes
+        its scale search wait for it.  Another update() discards it."""
+        E, C, dev = self.E, self.C, self.device
         if self.H is None:
             self.H = torch.empty((E, C, C), dtype=torch.float32, device=dev)
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
@@ -182,6 +198,7 @@ class ExpertGroupGPTQ:
         diag_all = self.H.diagonal(dim1=1, dim2=2)                        # [E, C] view
         lr_host = list(self.low_rank)
         any_lr = any(lr_host)
+        lr_dev = alpha32 = None
         if any_lr:
             # low-rank experts: diag(H) = (2/n) sum of squares of their kept rows (float64, rounded
             # once, as the Hessian kernel does for the others); H[e] itself holds nothing
@@ -199,10 +216,38 @@ class ExpertGroupGPTQ:
         # can only be all zero if its first rows are: one look at 8 rows of every expert (fp8-
         # or int-derived weights do contain single zeros) and at the Hessian diagonals tells
         # which experts need the full pass over their weights at all.  These flags and `bad`
-        # reach the host in ONE transfer, the only synchronisation before the solve.
+        # reach the host in ONE transfer (pinned memory, asynchronous), the only thing that
+        # quantize() waits for before it queues the solve.
         dead_any = ((diag_all == 0) & ~bad[:, None]).any(dim=1)
         maybe_zero = [(W[:, :8, :] == 0).all(dim=1).any(dim=1) for W in self.W]
-        host_flags = torch.stack([bad, dead_any] + maybe_zero).cpu()       # [2 + stacks, E]
+        flags = torch.stack([bad, dead_any] + maybe_zero)                  # [2 + stacks, E]
+        host_flags = torch.empty(flags.shape, dtype=flags.dtype, pin_memory=True)
+        host_flags.copy_(flags, non_blocking=True)
+        ready = torch.cuda.Event()
+        ready.record()
+        self._prepared = dict(diag_all=diag_all, bad=bad, host_flags=host_flags, ready=ready,
+                              lr_host=lr_host, any_lr=any_lr, lr_dev=lr_dev, alpha32=alpha32,
+                              keep=flags)
+        return self._prepared
+
+    @torch.no_grad()
+    def quantize(self, chunk: int = 32, max_shrink: float = 0.2, n_grid: int = 100,
+                 norm: float = 2.4, overlap_scale_search: bool = True):
+        """Returns one (qweight [E,R,C] u8, scales [E,R*G] f32, qzeros [E,R*G] f32) per stack;
+        with algorithm="sparsegptq" a fourth element M [E, ceil(C/32), R] u32 (bit i of word w
+        <-> column 32 w + i of the SOLVER order, as the reference returns it).
+        overlap_scale_search=False keeps the scale search on the caller's stream instead of a
+        side stream (same results; for per-kernel timing, where no kernel's time should include
+        another stream's work)."""
+        E, C, gs, dev = self.E, self.C, self.group_size, self.device
+        G = (C + gs - 1) // gs
+        mse = self.quantization_scale == "mse"
+        prep = self._prepared if self._prepared is not None else self.prepare()
+        self._prepared = None
+        prep["ready"].synchronize()        # the only wait for the GPU before the solve is queued
+        diag_all, bad, host_flags = prep["diag_all"], prep["bad"], prep["host_flags"]
+        lr_host, any_lr = prep["lr_host"], prep["any_lr"]
+        lr_dev, alpha32 = prep["lr_dev"], prep["alpha32"]
         # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
         # fraction of the fill rate)
         for e in host_flags[0].nonzero().flatten().tolist():
@@ -213,10 +258,11 @@ class ExpertGroupGPTQ:
             diag_all = self.H.diagonal(dim1=1, dim2=2) if not any_lr else diag_all.index_fill(
                 0, self._dev([e]), 1.0)
         failed = []
-        side = torch.cuda.Stream(device=dev) if overlap_scale_search else None   # default priority
+        cand = None                                   # the shrink factors, made on the search stream
+        side, lr_shared = self._streams_of(dev) if overlap_scale_search else (None, None)
         # the low-rank experts' kernels are chains of dependent steps on a few wavefronts: on a
         # stream of their own they run beside the other experts' matrix products
-        lr_side = torch.cuda.Stream(device=dev) if overlap_scale_search and any_lr else None
+        lr_side = lr_shared if any_lr else None
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
@@ -283,8 +329,16 @@ class ExpertGroupGPTQ:
                 # its VALU/transcendental work shares the CUs with the MFMA-bound factorisation
                 main = torch.cuda.current_stream()
                 search = side if side is not None else main
-                search.wait_stream(main)
+                # the search reads the weights and, where features are dead, their mask: without
+                # dead features it only waits for what prepare() saw queued, not for whatever
+                # the caller has queued on this stream since
+                if has_dead:
+                    search.wait_stream(main)
+                else:
+                    search.wait_event(prep["ready"])
                 with torch.cuda.stream(search):
+                    if mse and cand is None:
+                        cand = torch.linspace(1.0, max_shrink, n_grid, dtype=torch.float32, device=dev)
                     parts = []
                     for i in job:
                         # pruned columns are zero in the reference's W before the grid is built

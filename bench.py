@@ -43,7 +43,6 @@ import re
 import statistics
 import sys
 import time
-from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
@@ -114,9 +113,10 @@ def make_workload(name, cfg, chunk, seed=0):
 STREAMS = []
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128):
-    """Hot path for experts [step*chunk, (step+1)*chunk) of the layer.  overlap=False runs the
-    jobs one after the other (per-kernel event times are then exclusive)."""
+def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_tokens=128):
+    """First half of the hot path for experts [step*chunk, (step+1)*chunk) of the layer: the
+    expert groups, their Hessian updates and the look at the result that the solve starts from
+    (ExpertGroupGPTQ.prepare), queued on the jobs' streams."""
     import torch
     from forge.moe import ExpertGroupGPTQ
     E = cfg["n_experts"]
@@ -137,39 +137,53 @@ def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct"
     kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"],
               quantization_scale="mse" if mse else "absmax", quantization_order=cfg["order"],
               rel_damp=0.01, device="cuda", factor_route=factor_route, low_rank_tokens=low_rank_tokens)
-    # gate/up (shared Hessian) and down are independent: one host thread and one HIP stream
-    # each, so that the MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale
-    # search and the latency-bound diagonal blocks of the other
+    # gate/up (shared Hessian) and down are independent: one HIP stream each, so that the
+    # MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale search and the
+    # latency-bound diagonal blocks of the other.  One host thread queues both (quantize() does
+    # not wait for the GPU), gate/up first: its scale searches are the first on the groups'
+    # shared search stream, and its sweep is the longest chain of the step.
     cur = torch.cuda.current_stream()
     for s in STREAMS:
         s.wait_stream(cur)
     nsub = max(1, len(STREAMS) // 2)              # sub-batches of experts, each on its own streams
     per = (chunk + nsub - 1) // nsub
-    jobs = []
-    with ThreadPoolExecutor(max_workers=len(STREAMS)) as pool:
-        for j in range(nsub):
-            a, b = j * per, min(chunk, (j + 1) * per)
-            if a >= b:
-                continue
-            sub_offs = [o - offs[a] for o in offs[a:b + 1]]
+    staged = []
+    for j in range(nsub):
+        a, b = j * per, min(chunk, (j + 1) * per)
+        if a >= b:
+            continue
+        sub_offs = [o - offs[a] for o in offs[a:b + 1]]
+        for weights, rows, stream in (([wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]),
+                                      ([wl["Wd"]], hs, STREAMS[2 * j + 1])):
+            with torch.cuda.stream(stream):
+                grp = ExpertGroupGPTQ([w[a:b] for w in weights], **kw)
+                grp.update(rows[offs[a]:offs[b]], sub_offs)
+                grp.prepare()
+            staged.append((grp, stream, b - a))
+    return staged
 
-            def solve_sub(weights, rows, stream, a=a, b=b, sub_offs=sub_offs):
-                with torch.cuda.stream(stream):
-                    grp = ExpertGroupGPTQ([w[a:b] for w in weights], **kw)
-                    grp.update(rows[offs[a]:offs[b]], sub_offs)
-                    return grp.quantize(chunk=b - a, overlap_scale_search=overlap)
 
-            for weights, rows, stream in (([wl["Wg"], wl["Wu"]], xs, STREAMS[2 * j]),
-                                          ([wl["Wd"]], hs, STREAMS[2 * j + 1])):
-                job = pool.submit(solve_sub, weights, rows, stream)
-                if not overlap:
-                    job.result()
-                    stream.synchronize()
-                jobs.append(job)
-        results = [j.result() for j in jobs]
+def solve_step(staged, overlap=True):
+    """Second half: scale search, factorisation, sweep and layout of the staged groups.
+    overlap=False runs the jobs one after the other (per-kernel event times are then
+    exclusive)."""
+    import torch
+    cur = torch.cuda.current_stream()
+    results = []
+    for grp, stream, n in staged:
+        with torch.cuda.stream(stream):
+            results.append(grp.quantize(chunk=n, overlap_scale_search=overlap))
+        if not overlap:
+            stream.synchronize()
     for s in STREAMS:
         cur.wait_stream(s)
     return results[0::2], results[1::2]
+
+
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128):
+    """One whole step (both halves) of the hot path."""
+    return solve_step(stage_step(wl, cfg, chunk, step, mse=mse, factor_route=factor_route,
+                                 low_rank_tokens=low_rank_tokens), overlap=overlap)
 
 
 def route_counts(wl, chunk, low_rank_tokens):
@@ -185,9 +199,17 @@ def timed_steps(wl, cfg, chunk, steps, warmup, first_step=0, **kw):
     for i in range(warmup):
         run_step(wl, cfg, chunk, first_step + i, **kw)
     torch.cuda.synchronize()
+    # The K steps as a caller with a layer (or a model) of chunks would queue them: the Hessian
+    # updates of chunk i+1 go onto the streams before the solve of chunk i, so that the solve of
+    # chunk i+1 finds what it has to see on the host already there and its scale search starts
+    # while the last sweeps of chunk i still run.  Every step's work is inside the timed region.
+    overlap = kw.pop("overlap", True)
     t0 = time.perf_counter()
+    staged = stage_step(wl, cfg, chunk, first_step + warmup, **kw) if steps else None
     for i in range(steps):
-        run_step(wl, cfg, chunk, first_step + warmup + i, **kw)
+        ahead = stage_step(wl, cfg, chunk, first_step + warmup + i + 1, **kw) if i + 1 < steps else None
+        solve_step(staged, overlap=overlap)
+        staged = ahead
     torch.cuda.synchronize()
     return time.perf_counter() - t0
 

@@ -258,3 +258,48 @@ def test_expert_group_low_rank_route_against_the_dense_route_and_the_oracle():
                 # rows are independent and part ways at a rounding tie: the low-rank route must
                 # not lose more rows to ties than the route through the Hessian does
                 assert rl <= rd + 0.05, (e, rl, rd)
+
+
+@pytest.mark.parametrize("dead", [False, True])
+def test_prepare_ahead_of_other_work_changes_nothing(dead):
+    """prepare() right after update(), then unrelated work on the same stream (another group's
+    update, a large product), then quantize(): the same codes, scales and zeros as quantize()
+    alone, with and without a dead input feature (with one the scale search waits for the
+    stream after all); an update() after prepare() discards what was prepared."""
+    from forge.moe import ExpertGroupGPTQ
+    g0 = torch.Generator().manual_seed(21)
+    C, R = 512, 128
+    ns = (0, 3, 16, 40, 200)
+    W = (0.02 * torch.randn(len(ns), R, C, generator=g0)).bfloat16().to(DEV)
+    xs = [torch.randn(n, C, generator=g0).bfloat16() for n in ns]
+    if dead:
+        for x in xs:
+            x[:, 33] = 0
+    X = torch.cat(xs).to(DEV)
+    offs = np.concatenate([[0], np.cumsum(ns)]).tolist()
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
+              quantization_order="activation", rel_damp=0.01, device=DEV)
+    plain = ExpertGroupGPTQ([W], **kw)
+    plain.update(X, offs)
+    want = [t.cpu() for t in plain.quantize(chunk=8)[0]]
+
+    early = ExpertGroupGPTQ([W], **kw)
+    early.update(X, offs)
+    early.prepare()
+    other = ExpertGroupGPTQ([W.flip(0).contiguous()], **kw)       # unrelated work behind it
+    other.update(X, offs)
+    big = torch.randn(4096, 4096, device=DEV)
+    for _ in range(8):
+        big = (big @ big).clamp(-1, 1)
+    got = [t.cpu() for t in early.quantize(chunk=8)[0]]
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
+
+    again = ExpertGroupGPTQ([W], **kw)
+    again.update(X[:offs[3]], offs[:4] + [offs[3]] * 2)           # the first three experts' rows
+    again.prepare()
+    again.update(X[offs[3]:], [0, 0, 0, 0, ns[3], ns[3] + ns[4]])  # the rest: prepare() is void
+    assert again._prepared is None
+    got = [t.cpu() for t in again.quantize(chunk=8)[0]]
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
