@@ -14,6 +14,9 @@ by chunk (128 experts a step; their routed-token lists differ).  Experts with at
 routed rows (most of them: 8192 tokens over 256 experts with Zipf popularity) take the
 library's low-rank route, which reaches the same result from the rows themselves without a
 C x C Hessian; `config.experts_by_route` counts them.
+The timed steps are queued as a caller with a layer of chunks would queue them: chunk i+1's
+Hessian updates go onto the streams before chunk i's solve (all K updates and all K solves lie
+inside the timed region).
 value = experts quantised per second = steps * chunk / elapsed.
 
 After the timed steps:
@@ -27,7 +30,8 @@ After the timed steps:
   sweep: every integer stage bit-exact against the CPU oracle);
 * `every_expert_through_its_hessian`: the same steps with the low-rank route switched off;
 * `hessian_buckets`: the rank-k kernel alone at 16 / 256 / 1024 / 4096 tokens per expert;
-* `hbm_kernels`: min/max grid, int4 pack, fp8 block dequant at benchmark shapes;
+* `hbm_kernels`: min/max grid, int4 pack, fp8 block dequant, write-back dequant, routed-row
+  gather and the 1:4 packer at benchmark shapes;
 * `other_configs`: configs 1, 2, 4, 5 of the benchmark definition, end to end;
 * `cpu_baseline`: the CPU oracle in the reference's structure (32-column C kernel + BLAS
   SGEMM trailing update, LAPACK potrf/potri/potrf, OpenMP grid search) on four experts of
