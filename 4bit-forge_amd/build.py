@@ -7,7 +7,10 @@ into one shared library with a plain C ABI (see include/forge_hip.h).
 from __future__ import annotations
 
 import argparse
+import json
 import os
+import re
+import shutil
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -26,11 +29,72 @@ FLAGS = [
     # the register-resident sweep relies on `#pragma unroll` of large bodies being honoured
     "-mllvm", "-pragma-unroll-threshold=200000",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    # one remark block per kernel with its registers, spills and scratch bytes (parsed below)
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# Kernels that must keep everything in registers.  A kernel with a private segment (spilled
+# registers, or a register array that ended up in scratch memory) needs a scratch allocation at
+# its first dispatch, which fails -- and takes the queue down with it -- when device memory is
+# nearly full, and pays memory latency inside chains that are bound by latency already.
+# Matched against the demangled-ish kernel name; the build fails when one of them spills.
+NO_SCRATCH = (
+    "lowrank_block_wide_kernel", "lowrank_block_kernel", "lowrank_gram_kernel",
+    "lowrank_gram_wide_kernel", "lowrank_sweep_kernel", "mse_grid_kernel",
+    "split_gemm_kernel", "chain_gemm_fast_kernel", "syrk_bf16_big_kernel", "syrk_bf16_kernel",
+    "diag_block_kernel",
+    # the LDS-staged variants of the in-block chain (sixth template argument, TAIL, false)
+    re.compile(r"sweep_block_kernel<\d+, \d+, \w+, \w+, \w+, false"),
+)
 
 
 def sources():
     return sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
+
+
+_FIELDS = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch",
+           "SGPRs Spill": "sgpr_spill", "VGPRs Spill": "vgpr_spill",
+           "Occupancy [waves/SIMD]": "occupancy", "LDS Size [bytes/block]": "lds"}
+_REMARK = re.compile(r"remark:\s+(.*?):\s*(\S+) \[-Rpass-analysis=kernel-resource-usage\]")
+
+
+def parse_resource_usage(text: str) -> dict:
+    """{kernel name: {vgprs, agprs, scratch, sgpr_spill, vgpr_spill, occupancy, lds}} from the
+    compiler's kernel-resource-usage remarks (names demangled with c++filt when it is there)."""
+    out, cur = {}, None
+    for line in text.splitlines():
+        m = _REMARK.search(line)
+        if not m:
+            continue
+        key, val = m.group(1).strip(), m.group(2)
+        if key == "Function Name" or key == "Name":
+            cur = out.setdefault(val, {v: 0 for v in _FIELDS.values()})
+        elif cur is not None and key in _FIELDS:
+            cur[_FIELDS[key]] = int(val)
+    if out and shutil.which("c++filt"):
+        names = list(out)
+        r = subprocess.run(["c++filt", *names], capture_output=True, text=True)
+        plain = r.stdout.splitlines()
+        if r.returncode == 0 and len(plain) == len(names):
+            out = {p: out[n] for p, n in zip(plain, names)}
+    return out
+
+
+def strip_remarks(text: str):
+    """compiler output without the resource-usage remark blocks (three lines each: the remark,
+    the source line, the caret) and without the host pass's note on the packed-fp32 feature"""
+    lines, skip = [], 0
+    for l in text.splitlines():
+        if skip:
+            skip -= 1
+            continue
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            continue
+        if "packed-fp32-ops" in l:
+            continue
+        lines.append(l)
+    return [l for l in lines if not re.match(r"^\s+\d* \|", l) and l.strip() != "^"
+            and not re.match(r"^\d+ warnings? generated", l)]
 
 
 def _stale(obj: Path, deps) -> bool:
@@ -58,18 +122,32 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
         if src.suffix == ".cpp":
             cmd = [HIPCC, "-O2", "-std=c++17", "-fPIC", "-c", str(src), "-o", str(obj)]
         r = subprocess.run(cmd, capture_output=True, text=True)
-        msgs = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
-                         if "packed-fp32-ops" not in l)
-        return src, r.returncode, msgs
+        text = r.stdout + r.stderr
+        usage = parse_resource_usage(text)
+        msgs = "\n".join(strip_remarks(text))
+        return src, r.returncode, msgs, usage
 
+    usage_file = bdir / "resource_usage.json"
+    table = json.loads(usage_file.read_text()) if usage_file.exists() and not force else {}
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        for src, rc, msgs in ex.map(compile_one, todo):
+        for src, rc, msgs, usage in ex.map(compile_one, todo):
             if verbose and msgs.strip():
                 print(msgs, file=sys.stderr)
             if rc != 0:
                 raise RuntimeError(f"hipcc failed on {src.name}")
+            if src.suffix == ".hip":
+                table[src.name] = usage
             if verbose:
                 print(f"[build] compiled {src.name}")
+    if todo:
+        usage_file.write_text(json.dumps(table, indent=1, sort_keys=True))
+    # (scalar registers spilled into lanes of a vector register touch no memory: not counted)
+    spilled = [f"{f}: {k} ({u['scratch']} B/lane, {u['vgpr_spill']} VGPRs spilled)"
+               for f, ks in sorted(table.items()) for k, u in sorted(ks.items())
+               if any((n.search(k) if hasattr(n, "search") else n in k) for n in NO_SCRATCH)
+               and (u["scratch"] or u["vgpr_spill"])]
+    if spilled:
+        raise RuntimeError("kernels that must stay in registers use scratch memory:\n  " + "\n  ".join(spilled))
     if todo or force or not OUT.exists():
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
         subprocess.run(cmd, check=True)

@@ -120,6 +120,7 @@ const OptionInfo kOptions[OPT_COUNT] = {
     {"fp32_blocked_sum", "FORGE_FP32_BLOCKED_SUM", 0, 1, 0},
     {"sweep_update_products", "FORGE_SWEEP_UPDATE_PRODUCTS", 0, 6, 0},
     {"factor_pieces", "FORGE_FACTOR_PIECES", 0, 1, 0},
+    {"mse_reference_quantiser", "FORGE_MSE_REFERENCE_QUANTISER", 0, 1, 0},
 };
 std::atomic<int64_t> g_options[OPT_COUNT];
 

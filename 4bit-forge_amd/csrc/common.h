@@ -37,6 +37,7 @@ enum Option {
     OPT_FP32_BLOCKED_SUM = 1,  // 1 = blocked sums stay on the fp32 matrix instruction
     OPT_SWEEP_PRODUCTS = 2,    // piece products per fp32 product in the direct sweep's updates
     OPT_FACTOR_PIECES = 3,     // 0 = fp16 halves where the operand bound is known, 1 = bf16 thirds
+    OPT_MSE_REFERENCE_QUANTISER = 4,   // 1 = the shrink search rounds fma(x, 1/s, zero) as the reference does
     OPT_COUNT
 };
 int64_t option(Option o);

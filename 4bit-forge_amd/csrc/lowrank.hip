@@ -305,14 +305,19 @@ __global__ __launch_bounds__(WN * WS) void lowrank_block_wide_kernel(const float
         const double* __restrict__ src = later + ((b * nblk + blk) * WN + row) * WN + qt * WQ;
 #pragma unroll
         for (int j = 0; j < WQ; ++j) S[j] += src[j];
+        // (the quarter of the pivot is a run-time loop, the position inside it unrolled: S is
+        // indexed with constants, and the code is a quarter of the fully unrolled form's)
+#pragma unroll 1
+        for (int mq = 0; mq < WS; ++mq)
 #pragma unroll
-        for (int m = 0; m < WN; ++m) {
+        for (int mi = 0; mi < WQ; ++mi) {
+            const int m = mq * WQ + mi;
             __syncthreads();                       // the previous pivot row and column have been read
             if (row == m) {
 #pragma unroll
                 for (int j = 0; j < WQ; ++j) rowsh[qt * WQ + j] = S[j];
             }
-            if (qt == m / WQ) colsh[row] = S[m % WQ];
+            if (qt == mq) colsh[row] = S[mi];
             __syncthreads();
             double piv[WQ];
 #pragma unroll
@@ -329,7 +334,7 @@ __global__ __launch_bounds__(WN * WS) void lowrank_block_wide_kernel(const float
             const double g = is_m ? rp : -(colsh[row] * rp);
 #pragma unroll
             for (int j = 0; j < WQ; ++j) S[j] = __builtin_fma(g, piv[j], keep * S[j]);
-            if (qt == m / WQ) S[m % WQ] = g;
+            if (qt == mq) S[mi] = g;
         }
     }
 

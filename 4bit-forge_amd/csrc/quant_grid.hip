@@ -147,14 +147,16 @@ __device__ __forceinline__ float pow_abs(float e, float norm) {
 // max(|diff|, 1e-20): for norm >= 2.3 the floor's own loss 1e-20^norm is below the smallest
 // fp32 denormal, i.e. 0, which is also what |diff| = 0 gives without it (log2 0 = -inf,
 // exp2 -inf = 0); the launcher chooses.
-template <bool FLOOR>
+template <bool FLOOR, bool REFQ = false>
 __device__ __forceinline__ float element_loss(float x, float s, float rcp, float q0, float maxq,
                                               float norm) {
     // q - q0 directly: round(x*rcp) clamped to [-q0, maxq - q0].  q0 is a small integer, so
     // this is the reference's clamp(round(fma(x, rcp, q0)), 0, maxq) - q0 except where the
     // fma's own rounding lands x*rcp + q0 on a half-integer that x*rcp is not; there the two
-    // neighbouring levels are equally far from x to within one ulp of the sum.
-    const float qc = __builtin_amdgcn_fmed3f(__builtin_rintf(x * rcp), -q0, maxq - q0);
+    // neighbouring levels are equally far from x to within one ulp of the sum.  REFQ is the
+    // reference's form itself (one more instruction per weight and candidate).
+    const float qc = REFQ ? __builtin_amdgcn_fmed3f(__builtin_rintf(__builtin_fmaf(x, rcp, q0)), 0.0f, maxq) - q0
+                          : __builtin_amdgcn_fmed3f(__builtin_rintf(x * rcp), -q0, maxq - q0);
     const float diff = __builtin_fmaf(qc, s, -x);
     return pow_abs(FLOOR ? fmaxf(fabsf(diff), 1e-20f) : fabsf(diff), norm);
 }
@@ -162,7 +164,7 @@ __device__ __forceinline__ float element_loss(float x, float s, float rcp, float
 // Sum over the 8 "reference lanes" l = Q, Q+4, ..., Q+28 (each the in-order sum of its
 // GS/32 elements), combined exactly as the reference's halving tree combines them:
 // ((p[Q] + p[Q+16]) + (p[Q+8] + p[Q+24])) + ((p[Q+4] + p[Q+20]) + (p[Q+12] + p[Q+28])).
-template <int GS, int Q, bool FLOOR>
+template <int GS, int Q, bool FLOOR, bool REFQ>
 __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, float rcp, float q0,
                                               float maxq, float norm) {
     constexpr int VPL = GS / 32;
@@ -171,9 +173,9 @@ __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, flo
     for (int j = 0; j < 8; ++j) {
         const int l = Q + 4 * j;
         // (the reference starts from 0 and adds: the same value, every term being >= +0)
-        float loss = element_loss<FLOOR>(v[l], s, rcp, q0, maxq, norm);
+        float loss = element_loss<FLOOR, REFQ>(v[l], s, rcp, q0, maxq, norm);
 #pragma unroll
-        for (int i = 1; i < VPL; ++i) loss += element_loss<FLOOR>(v[l + 32 * i], s, rcp, q0, maxq, norm);
+        for (int i = 1; i < VPL; ++i) loss += element_loss<FLOOR, REFQ>(v[l + 32 * i], s, rcp, q0, maxq, norm);
         p[j] = loss;
     }
     return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
@@ -185,23 +187,23 @@ __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, flo
 // once it reaches `bound` for every group of the wavefront the candidate cannot be a new
 // strict minimum and the rest of its evaluation is skipped (returns +inf for it).  The
 // selected candidate and its loss are exactly those of the full evaluation.
-template <int GS, bool FLOOR>
+template <int GS, bool FLOOR, bool REFQ>
 __device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, float rcp,
                                                 float q0, float maxq, float norm, float bound) {
     constexpr float kInf = __builtin_inff();
-    const float a0 = quarter_loss<GS, 0, FLOOR>(v, s, rcp, q0, maxq, norm);
+    const float a0 = quarter_loss<GS, 0, FLOOR, REFQ>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(a0 < bound) == 0) return kInf;
-    const float h0 = a0 + quarter_loss<GS, 2, FLOOR>(v, s, rcp, q0, maxq, norm);
+    const float h0 = a0 + quarter_loss<GS, 2, FLOOR, REFQ>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(h0 < bound) == 0) return kInf;
-    const float a1 = quarter_loss<GS, 1, FLOOR>(v, s, rcp, q0, maxq, norm);
+    const float a1 = quarter_loss<GS, 1, FLOOR, REFQ>(v, s, rcp, q0, maxq, norm);
     if (__builtin_amdgcn_ballot_w64(h0 + a1 < bound) == 0) return kInf;
-    const float h1 = a1 + quarter_loss<GS, 3, FLOOR>(v, s, rcp, q0, maxq, norm);
+    const float h1 = a1 + quarter_loss<GS, 3, FLOOR, REFQ>(v, s, rcp, q0, maxq, norm);
     return h0 + h1;
 }
 
 // One lane per group.  FUSED: derive (sg, q0g) from the group's own extrema first;
 // otherwise read them from scales/qzeros (the reference's two-call protocol).
-template <typename T, int GS, bool FUSED, bool FLOOR>
+template <typename T, int GS, bool FUSED, bool FLOOR, bool REFQ>
 __global__ __launch_bounds__(64) void mse_grid_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t G,
     int64_t n_groups, const float* __restrict__ cand, int P, float maxq, float norm,
@@ -310,11 +312,11 @@ __global__ __launch_bounds__(64) void mse_grid_kernel(
             const float rcp = 1.0f / (s + kEps);
             const float q0 = symmetric ? q0g : clampf(__builtin_rintf(-xmin * rcp), 0.0f, maxq);
             if (!early) {
-                const float clip = fmaxf(element_loss<FLOOR>(lo, s, rcp, q0, maxq, norm),
-                                         element_loss<FLOOR>(hi, s, rcp, q0, maxq, norm));
+                const float clip = fmaxf(element_loss<FLOOR, REFQ>(lo, s, rcp, q0, maxq, norm),
+                                         element_loss<FLOOR, REFQ>(hi, s, rcp, q0, maxq, norm));
                 if (__builtin_amdgcn_ballot_w64(clip < best_loss) == 0) continue;
             }
-            const float loss = candidate_loss<GS, FLOOR>(v, s, rcp, q0, maxq, norm, best_loss);
+            const float loss = candidate_loss<GS, FLOOR, REFQ>(v, s, rcp, q0, maxq, norm, best_loss);
             if (loss < best_loss) {
                 best_loss = loss;
                 best_s = s;
@@ -342,16 +344,17 @@ int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, 
                                (double)n_groups * (gs * sizeof(T) + 8.0 + (FUSED ? 0.0 : 8.0)),
                                forge::WORK_BYTES);
     const bool floor_needed = !(norm >= 2.3f);
+    const bool refq = forge::option(forge::OPT_MSE_REFERENCE_QUANTISER) != 0;
+#define FORGE_MSE_LAUNCH(GS, FL, RQ)                                                          \
+    mse_grid_kernel<T, GS, FUSED, FL, RQ><<<grid, block, 0, st>>>(                            \
+        W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric, search,     \
+        scales, qzeros)
 #define FORGE_MSE_CASE(GS)                                                                    \
     case GS:                                                                                  \
-        if (floor_needed)                                                                     \
-            mse_grid_kernel<T, GS, FUSED, true><<<grid, block, 0, st>>>(                      \
-                W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric,     \
-                search, scales, qzeros);                                                      \
-        else                                                                                  \
-            mse_grid_kernel<T, GS, FUSED, false><<<grid, block, 0, st>>>(                     \
-                W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric,     \
-                search, scales, qzeros);                                                      \
+        if (floor_needed && refq) FORGE_MSE_LAUNCH(GS, true, true);                           \
+        else if (floor_needed) FORGE_MSE_LAUNCH(GS, true, false);                             \
+        else if (refq) FORGE_MSE_LAUNCH(GS, false, true);                                     \
+        else FORGE_MSE_LAUNCH(GS, false, false);                                              \
         break;
     switch (gs) {
         FORGE_MSE_CASE(32)
@@ -362,6 +365,7 @@ int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, 
                                (long long)gs);
     }
 #undef FORGE_MSE_CASE
+#undef FORGE_MSE_LAUNCH
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

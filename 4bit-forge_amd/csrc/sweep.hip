@@ -86,9 +86,8 @@ __device__ __forceinline__ float dpp_source(float u) {
 // those 32 errors are pushed into the block's remaining columns, then x[] is shifted down
 // by 32 so that the next sub-block again sits in x[0..31] (this keeps the unrolled code at
 // one sub-block's size).  U[t,k] is the same for every lane: the workgroup stages the
-// 32-row panel of U that a sub-block needs in LDS (the next panel is fetched into
-// registers while the current one is used) and every fma takes its U operand from a
-// broadcast ds_read.  TAIL is the guarded, slower variant (U straight from global memory)
+// block's rows of U in LDS once, before the first column, and every fma takes its U operand
+// from there.  TAIL is the guarded, slower variant (U straight from global memory)
 // for blocks that are not a whole number of 32-column sub-blocks or whose U rows are not
 // 16-byte aligned.
 //
@@ -105,12 +104,37 @@ __device__ __forceinline__ float dpp_source(float u) {
 __device__ __forceinline__ float w0_as_f32(const float* p) { return *p; }
 __device__ __forceinline__ float w0_as_f32(const uint16_t* p) { return __uint_as_float((uint32_t)*p << 16); }
 
+// The LDS-staged variants reach memory through buffer instructions: the matrix's base address
+// sits in scalar registers (one descriptor per array), the lane's row is ONE 32-bit register
+// and the column a scalar offset, where pointers cost two registers per array and lane -- the
+// registers that x[], the scales and the errors leave no room for.  Offsets are bytes from the
+// descriptor's base and stay below 2^31 (the launcher checks the shape).
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ rsrc_t row_rsrc(const void* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00027000);
+}
+__device__ __forceinline__ float buf_ld_f32(rsrc_t rs, int voff, int soff) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0));
+}
+__device__ __forceinline__ float buf_ld_w0(rsrc_t rs, int row, int64_t col_elems, const float*) {
+    return buf_ld_f32(rs, row * 4, (int)(col_elems * 4));
+}
+__device__ __forceinline__ float buf_ld_w0(rsrc_t rs, int row, int64_t col_elems, const uint16_t*) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row * 2, (int)(col_elems * 2), 0) << 16);
+}
+__device__ __forceinline__ void buf_st_f32(float v, rsrc_t rs, int voff, int soff) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rs, voff, soff, 0);
+}
+
 template <int BW, int NT, bool SPARSE, bool PER_ELEM, bool ERR_IN_A, bool TAIL, bool DISP = false,
           typename W0T = float>
-__global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
+__global__ __launch_bounds__(NT, (TAIL || NT >= 256) ? 2 : 1) void sweep_block_kernel(SweepArgs a) {
     constexpr int SB = 32, NSB = BW / SB;
     constexpr int RING = FORGE_SWEEP_RING;   // LDS read-ahead: RING-1 steps of 16 columns
-    __shared__ __attribute__((aligned(16))) float Up[TAIL ? 1 : 2][TAIL ? 1 : SB][TAIL ? 4 : BW];
+    // (all of the block's rows of U at once, 64 KB for 128 columns: a panel per sub-block, fetched
+    // one sub-block ahead, held the next panel in registers across the serial chain, and those
+    // twelve registers were the ones that no longer fitted beside x[], the scales and the errors)
+    __shared__ __attribute__((aligned(16))) float Up[TAIL ? 1 : BW][TAIL ? 4 : BW];
     // Lanes past the last row leave at once; that only happens in the TAIL variant (the
     // LDS-staged variants are launched for whole wavefronts only: every lane loads its
     // share of the panel and meets the others at the barriers).
@@ -133,18 +157,34 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
     const float maxq = (float)a.maxq;
     float dmax = 0.0f;     // largest |d| this lane hands on in this block
 
-    float x[BW];
-#pragma unroll
-    for (int i = 0; i < BW; ++i) x[i] = (i < bw) ? A[(a.c0 + i) * R] : 0.0f;
+    // (fast variants only) descriptors at the matrix's first row of this block
+    const int row = (int)r;
+    const rsrc_t rsA = row_rsrc(a.A + b * C * R + a.c0 * R);
+    const rsrc_t rsB = row_rsrc(ERR_IN_A ? nullptr : a.B + b * C * R + a.c0 * R);
+    const rsrc_t rsQ = row_rsrc(a.q + b * C * R + a.c0 * R);
+    const rsrc_t rsS = row_rsrc(a.scales + b * (PER_ELEM ? C * R : a.G * R) + (PER_ELEM ? a.c0 * R : 0));
+    const rsrc_t rsZ = row_rsrc(a.qzeros + b * (PER_ELEM ? C * R : a.G * R) + (PER_ELEM ? a.c0 * R : 0));
+    const rsrc_t rsW = row_rsrc(DISP ? static_cast<const W0T*>(a.W0) + b * C * R + a.c0 * R : nullptr);
+    const rsrc_t rsM = row_rsrc(SPARSE ? a.M + b * ((C + 31) / 32) * R : nullptr);
 
-    int buf = 0;
+    float x[BW];
+    if constexpr (TAIL) {
+#pragma unroll
+        for (int i = 0; i < BW; ++i) x[i] = (i < bw) ? A[(a.c0 + i) * R] : 0.0f;
+    } else {
+#pragma unroll
+        for (int i = 0; i < BW; ++i) x[i] = (i < bw) ? buf_ld_f32(rsA, row * 4, (int)(i * R * 4)) : 0.0f;
+    }
+
     if constexpr (!TAIL) {
-        // first panel: rows c0..c0+31, columns c0..c0+bw-1
-        const int w4 = bw / 4;
-        for (int idx = threadIdx.x; idx < SB * w4; idx += NT) {
-            const int t = idx / w4, j = idx - t * w4;
-            *reinterpret_cast<float4*>(&Up[0][t][4 * j]) =
-                *reinterpret_cast<const float4*>(U + (a.c0 + t) * C + a.c0 + 4 * j);
+        // rows c0..c0+bw-1 of U; of the 32 rows of sub-block i the columns from that sub-block on
+        for (int i = 0; i < nsub; ++i) {
+            const int w4 = (bw - i * SB) / 4;
+            for (int idx = threadIdx.x; idx < SB * w4; idx += NT) {
+                const int t = i * SB + idx / w4, j = idx % w4;
+                *reinterpret_cast<float4*>(&Up[t][i * SB + 4 * j]) =
+                    *reinterpret_cast<const float4*>(U + (a.c0 + t) * C + a.c0 + i * SB + 4 * j);
+            }
         }
         __syncthreads();
     }
@@ -159,12 +199,12 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             for (int t = 0; t < SB; ++t) {
                 const int64_t c = c_first + t;
                 if constexpr (PER_ELEM) {
-                    sv[t] = sc[c * R];
-                    qv[t] = qz[c * R];
+                    sv[t] = buf_ld_f32(rsS, row * 4, (int)((c - a.c0) * R * 4));
+                    qv[t] = buf_ld_f32(rsZ, row * 4, (int)((c - a.c0) * R * 4));
                 } else {
                     const int64_t g = gi[c];
-                    sv[t] = sc[g * R];
-                    qv[t] = qz[g * R];
+                    sv[t] = buf_ld_f32(rsS, row * 4, (int)(g * R * 4));
+                    qv[t] = buf_ld_f32(rsZ, row * 4, (int)(g * R * 4));
                 }
             }
         }
@@ -176,6 +216,8 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
         const int rem = bw - sb * SB;                 // block columns from cs on
         float err[SB];
         uint32_t mask = 0u;
+        // this sub-block's rows of U, from its own first column on
+        const float* __restrict__ Ub = &Up[0][0] + (TAIL ? 0 : sb * (SB * BW + SB));
 
         auto select_and_quantize = [&](int t, int64_t c, float s, float q0) {
             bool keep = true;
@@ -194,7 +236,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                         // block of N = I - strict(V).
                         auto vv = [&](int j, int k) -> float {
                             if constexpr (TAIL) return (c + k < C) ? U[(c + j) * C + c + k] : 0.0f;
-                            else return Up[buf][t + j][t + k];
+                            else return Ub[(t + j) * BW + t + k];
                         };
                         const float v01 = vv(0, 1), v02 = vv(0, 2), v03 = vv(0, 3);
                         const float v12 = vv(1, 2), v13 = vv(1, 3), v23 = vv(2, 3);
@@ -231,34 +273,35 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             }
             err[t] = e;
             if constexpr (DISP) dmax = fmaxf(dmax, fabsf(e));
-            q[c * R] = (uint8_t)qf;
-            if constexpr (ERR_IN_A) {
-                A[c * R] = e;
+            if constexpr (TAIL) {
+                q[c * R] = (uint8_t)qf;
+                if constexpr (ERR_IN_A) {
+                    A[c * R] = e;
+                } else {
+                    A[c * R] = deq;
+                    Bo[c * R] = e;
+                }
             } else {
-                A[c * R] = deq;
-                Bo[c * R] = e;
+                const int col = (int)((c - a.c0) * R);
+                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)qf, rsQ, row, col, 0);
+                if constexpr (ERR_IN_A) {
+                    buf_st_f32(e, rsA, row * 4, col * 4);
+                } else {
+                    buf_st_f32(deq, rsA, row * 4, col * 4);
+                    buf_st_f32(e, rsB, row * 4, col * 4);
+                }
             }
         };
 
         if constexpr (!TAIL) {
+            // (the original weights of the sub-block's second half are requested when a quarter of
+            // the chain is done and as many scale/zero registers are free again: all 32 at the
+            // start were the registers that the kernel did not have)
             if constexpr (DISP) {
 #pragma unroll
-                for (int t = 0; t < SB; ++t) err[t] = w0_as_f32(W0 + (cs + t) * R);
+                for (int t = 0; t < SB / 2; ++t) err[t] = buf_ld_w0(rsW, row, (cs - a.c0 + t) * R, (const W0T*)nullptr);
             }
-            // fetch the next sub-block's panel (rows cs+32.., columns cs+32..) into registers
             const bool more = sb + 1 < nsub;
-            float4 nxt[(NSB - 1) * (256 / NT)];
-            if (more) {
-                const int w4 = (rem - SB) / 4;               // float4 per panel row
-#pragma unroll
-                for (int i = 0; i < (NSB - 1) * (256 / NT); ++i) {
-                    const int idx = threadIdx.x + i * NT;
-                    if (idx < SB * w4) {
-                        const int t = idx / w4, j = idx - t * w4;
-                        nxt[i] = *reinterpret_cast<const float4*>(U + (cs + SB + t) * C + cs + SB + 4 * j);
-                    }
-                }
-            }
             // U operands come from LDS 16 columns (4 broadcast ds_read_b128) at a time, read
             // two steps ahead of their use; scheduling barriers pin that distance (left
             // alone the scheduler hoists hundreds of reads and spills the x registers).
@@ -266,13 +309,19 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
             {
                 const int l16 = threadIdx.x & 15;
                 float ring[RING];
-                auto rd = [&](int step) { return Up[buf][step >> 1][(step & 1) * 16 + l16]; };
+                auto rd = [&](int step) { return Ub[(step >> 1) * BW + (step & 1) * 16 + l16]; };
                 ring[0] = rd(0);
                 if (RING > 2) ring[1] = rd(1);
 #pragma unroll
                 for (int step = 0; step < 2 * SB; ++step) {
                     const int t = step >> 1, h = step & 1;
                     if (step + RING - 1 < 2 * SB) ring[(step + RING - 1) % RING] = rd(step + RING - 1);
+                    if constexpr (DISP) {
+                        if (step == SB / 2) {
+#pragma unroll
+                            for (int i = SB / 2; i < SB; ++i) err[i] = buf_ld_w0(rsW, row, (cs - a.c0 + i) * R, (const W0T*)nullptr);
+                        }
+                    }
                     if (h == 0) select_and_quantize(t, cs + t, sv[t], qv[t]);
                     __builtin_amdgcn_sched_barrier(0);
                     const float u16 = dpp_source(ring[step % RING]);
@@ -283,7 +332,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            if constexpr (SPARSE) Mw[(cs >> 5) * R] = mask;
+            if constexpr (SPARSE) __builtin_amdgcn_raw_buffer_store_b32(mask, rsM, row * 4, (int)((cs >> 5) * R * 4), 0);
             if (more) load_meta(cs + SB);
             // push the 32 errors into the rest of the block
 #pragma unroll
@@ -291,7 +340,7 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                 if (sb + u < nsub) {
                     const int l16 = threadIdx.x & 15;
                     float ring[RING];
-                    auto rd = [&](int step) { return Up[buf][step >> 1][u * SB + (step & 1) * 16 + l16]; };
+                    auto rd = [&](int step) { return Ub[(step >> 1) * BW + u * SB + (step & 1) * 16 + l16]; };
                     ring[0] = rd(0);
                     if (RING > 2) ring[1] = rd(1);
 #pragma unroll
@@ -308,19 +357,6 @@ __global__ __launch_bounds__(NT, 2) void sweep_block_kernel(SweepArgs a) {
                     }
                 }
             }
-            if (more) {
-                const int w4 = (rem - SB) / 4;
-#pragma unroll
-                for (int i = 0; i < (NSB - 1) * (256 / NT); ++i) {
-                    const int idx = threadIdx.x + i * NT;
-                    if (idx < SB * w4) {
-                        const int t = idx / w4, j = idx - t * w4;
-                        *reinterpret_cast<float4*>(&Up[buf ^ 1][t][4 * j]) = nxt[i];
-                    }
-                }
-            }
-            __syncthreads();
-            buf ^= 1;
         } else {
             if constexpr (DISP) {
 #pragma unroll 1
@@ -432,8 +468,11 @@ int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
                                (double)a.bw * (a.bw - 1) * (double)a.R * (double)batch,
                                forge::WORK_FLOPS);
     // the LDS-staged variants need whole wavefronts (every lane helps to load the panel)
+    // (and their byte offsets from a block's or a matrix's first row fit 31 bits)
+    const int64_t far = 128 > a.G ? (128 > a.C / 32 + 1 ? 128 : a.C / 32 + 1)
+                                  : (a.G > a.C / 32 + 1 ? a.G : a.C / 32 + 1);
     const bool fast = a.bw % 32 == 0 && a.C % 4 == 0 && a.c0 % 4 == 0 && a.R % 64 == 0 &&
-                      (reinterpret_cast<uintptr_t>(a.U) % 16) == 0;
+                      (reinterpret_cast<uintptr_t>(a.U) % 16) == 0 && (far + 1) * a.R * 4 < (1LL << 31);
     if (fast && a.R % 256 == 0) {
         dim3 grid((unsigned)(a.R / 256), (unsigned)batch);
         sweep_block_kernel<forge_kBW, 256, SPARSE, PER_ELEM, ERR_IN_A, false, DISP, W0T>

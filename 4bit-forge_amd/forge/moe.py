@@ -71,7 +71,7 @@ class ExpertGroupGPTQ:
         see the module text; 0 = every expert through its Hessian.  At 65-128 rows the per-row
         vector sweep costs nearly what the route through the Hessian costs (measured: 1 % of a
         benchmark step in its favour).  ``self.H[e]`` of such an
-        expert is never written."""
+        expert is never written (uninitialised memory): read Hessians through ``hessian(e)``."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         if factor_route not in ("direct", "inverse"):
@@ -106,6 +106,7 @@ class ExpertGroupGPTQ:
         self._cap = next(n for n in (16, 32, 64, 128) if n >= max(self.low_rank_tokens, 1))
         self.low_rank = [self.low_rank_tokens > 0] * self.E
         self._kept: Optional[torch.Tensor] = None
+        self._kept_wide = [False] * self.E               # an f32 row among the kept ones
         self._non_invertible = torch.zeros(self.E, dtype=torch.bool)
         self._pending_info = []                          # (expert ids, device flags) not yet fetched
         self._prepared = None                            # what prepare() queued, until quantize() uses it
@@ -118,6 +119,20 @@ class ExpertGroupGPTQ:
             self._non_invertible[ids] |= (info > 0).cpu()
         self._pending_info = []
         return self._non_invertible
+
+    @torch.no_grad()
+    def hessian(self, e: int) -> torch.Tensor:
+        """H of expert e, [C, C] f32, as forge/gptq.py:61-80 would have accumulated it.  For an
+        expert on the low-rank route ``self.H[e]`` is never written (that is the point of the
+        route); its Hessian is formed here from the rows that were kept, (2/n) X^T X in float64
+        rounded once; an expert that saw nothing has none (the reference's ``H is None``)."""
+        n = self.num_samples[e]
+        if n == 0:
+            return None
+        if self.low_rank[e]:
+            X = self._kept[e, :n].double()
+            return ((2.0 / n) * X.t() @ X).float()
+        return self.H[e]
 
     def _dev(self, values, dtype=None):
         """A small host list as a device tensor without stopping the host: through pinned memory
@@ -152,6 +167,7 @@ class ExpertGroupGPTQ:
             self.num_samples[e] = total
             if self.low_rank[e] and total <= self.low_rank_tokens:
                 src.extend(range(o, o + new))                     # keep the rows, no Hessian
+                self._kept_wide[e] |= new > 0 and X.dtype == torch.float32
                 dst.extend(range(e * self._cap + n, e * self._cap + total))
                 new = 0
             elif self.low_rank[e]:
@@ -171,8 +187,11 @@ class ExpertGroupGPTQ:
             # new ones together, (2/total) X^T X, what the running mean equals
             parts, row0, counts, alpha = [], [0] * self.E, [0] * self.E, [0.0] * self.E
             at = 0
+            # kept rows that came in as f32 are not rounded to a later call's bf16: the route
+            # through the Hessian would have summed them in f32 too
+            dt = torch.float32 if any(self._kept_wide[e] for e, *_ in late) else X.dtype
             for e, n, o, new in late:
-                parts += [self._kept[e, :n].to(X.dtype), X[o:o + new]]
+                parts += [self._kept[e, :n].to(dt), X[o:o + new].to(dt)]
                 row0[e], counts[e], alpha[e] = at, n + new, 2.0 / (n + new)
                 at += n + new
                 self._kept[e].zero_()
@@ -206,7 +225,10 @@ class ExpertGroupGPTQ:
                 self._kept = torch.zeros((E, self._cap, C), dtype=torch.float32, device=dev)
             lr_dev = self._dev(lr_host)
             alpha32 = self._dev([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32)
-            d_lr = ((self._kept.double() ** 2).sum(dim=1) * alpha32.double()[:, None]).float()
+            # (32 experts at a time: the float64 squares of all kept rows at once are 2 x 0.9 GB
+            # for 128 experts of 7168 features)
+            d_lr = torch.cat([((self._kept[i:i + 32].double() ** 2).sum(dim=1)
+                               * alpha32[i:i + 32].double()[:, None]).float() for i in range(0, E, 32)])
             diag_all = torch.where(lr_dev[:, None], d_lr, diag_all)
         bad = (~seen) | torch.isnan(diag_all).any(dim=1)
         if any_lr:

@@ -84,6 +84,15 @@ int64_t forge_mfma_rate_probe_sink_floats(int workgroups);
  *                           scaled by a power of two from its diagonal entry, and three
  *                           products (fp32-grade: the halves hold 22+ bits); 1: three bf16 thirds
  *                           and six products everywhere, as forge_chol_inv_upper_batched always does
+ *   "mse_reference_quantiser" FORGE_MSE_REFERENCE_QUANTISER=1   how the shrink search (forge_quant_grid,
+ *                           forge_mse_scale_groups_packed) finds the level of a weight inside the
+ *                           candidate's loss.  0 (default): rint(x * rcp) clamped to [-zero, maxq - zero],
+ *                           one instruction less per weight and candidate; it picks the other of two
+ *                           levels only where the reference's single rounding of x * rcp + zero lands on
+ *                           a half-integer that x * rcp is not on, i.e. where both levels are equally
+ *                           far from x to one ulp (it moves the loss by ~1e-7 of one term).
+ *                           1: clamp(rint(fma(x, rcp, zero)), 0, maxq) - zero, quant_grid.cu:160-163
+ *                           literally (12 % slower)
  * forge_set_option returns FORGE_ERR_INVALID for an unknown name or a value out of range;
  * forge_get_option returns -1 for an unknown name. */
 int forge_set_option(const char* name, int64_t value);

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import linear, flip_rate
+from helpers import linear, flip_rate, codes_at_floor
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -255,9 +255,11 @@ def test_expert_group_low_rank_route_against_the_dense_route_and_the_oracle():
             elif e == 5:
                 assert torch.equal(ql, qd)                   # through the Hessian either way
             else:
-                # rows are independent and part ways at a rounding tie: the low-rank route must
-                # not lose more rows to ties than the route through the Hessian does
-                assert rl <= rd + 0.05, (e, rl, rd)
+                # the rule of the end-to-end tests: within max(1e-3, 1.5 x floor) of the oracle,
+                # the floor being what the reference's own codes move by between valid fp32
+                # realisations of its library calls; on matrices this small (one diverging row is
+                # 0.8 % of the codes) isolated rows that start from a one-level tie pass too
+                codes_at_floor(f"low-rank stack {i} expert {e}", qo, ql, Wi[e], [X], kw, order=o.perm)
 
 
 @pytest.mark.parametrize("dead", [False, True])
@@ -303,3 +305,64 @@ def test_prepare_ahead_of_other_work_changes_nothing(dead):
     got = [t.cpu() for t in again.quantize(chunk=8)[0]]
     for a, b in zip(want, got):
         assert torch.equal(a, b)
+
+
+def test_more_matrices_than_one_mixed_launch_holds(hip):
+    """forge_gptq_sweep_lowrank_mixed splits a batch of more than 96 matrices into several
+    launches, each with its own offsets into the weights, the vectors, the scales and the codes:
+    100 small matrices of all five sizes in one call must equal the same matrices swept one
+    by one."""
+    g = torch.Generator().manual_seed(13)
+    B, C, R, gs = 100, 128, 96, 128
+    sizes = (4, 16, 32, 64, 128)
+    ns = [sizes[int(i)] for i in torch.randint(0, 5, (B,), generator=g)]
+    ns[0], ns[95], ns[96], ns[99] = 128, 4, 64, 16           # both sides of the split, all lane widths
+    W0 = (0.02 * torch.randn(B, C, R, generator=g)).bfloat16().to(DEV)
+    sT = (0.002 + 0.004 * torch.rand(B, 1, R, generator=g)).to(DEV)
+    zT = torch.randint(5, 11, (B, 1, R), generator=g).float().to(DEV)
+    g_idx = torch.zeros(B, C, dtype=torch.int32, device=DEV)
+    Bps, Hms, infos = [], [], []
+    for b, n in enumerate(ns):
+        Bp, D = _problem(C, max(1, n - (b % 3)), 100 + b)    # some rows of the size left zero
+        assert Bp.shape[1] <= n
+        Bp = torch.nn.functional.pad(Bp, (0, n - Bp.shape[1]))
+        Hm, info = hip.lowrank_factor(Bp[None].to(DEV), D[None].to(DEV))
+        Bps.append(Bp.to(DEV))
+        Hms.append(Hm[0])
+        infos.append(info)
+    info = torch.cat(infos)
+    info[7] = 1                                              # one matrix swept uncoupled
+    q = hip.gptq_sweep_lowrank_mixed(W0, torch.cat([b.flatten() for b in Bps]),
+                                     torch.cat([h.flatten() for h in Hms]), ns, info, sT, zT, g_idx, 4)
+    for b in range(B):
+        one = hip.gptq_sweep_lowrank(W0[b:b + 1], Bps[b][None], Hms[b][None], info[b:b + 1],
+                                     sT[b:b + 1], zT[b:b + 1], g_idx[b:b + 1], 4)
+        assert torch.equal(q[b], one[0]), (b, ns[b])
+
+
+def test_rows_kept_in_f32_are_not_rounded_when_an_expert_leaves_the_route():
+    """An expert whose first rows came as f32 and whose later rows come as bf16 (and push it off
+    the low-rank route): its Hessian is the f32 sum over all of them, as the route through the
+    Hessian gives it, not the sum over kept rows rounded to bf16."""
+    from forge.moe import ExpertGroupGPTQ
+    g0 = torch.Generator().manual_seed(17)
+    C, R = 256, 64
+    W = (0.02 * torch.randn(2, R, C, generator=g0)).bfloat16().to(DEV)
+    first = torch.randn(10, C, generator=g0)                       # f32, not bf16-representable
+    later = torch.randn(30, C, generator=g0).bfloat16()
+    kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="absmax",
+              quantization_order="default", rel_damp=0.01, device=DEV)
+    Hs = {}
+    for lim in (16, 0):
+        grp = ExpertGroupGPTQ([W], low_rank_tokens=lim, **kw)
+        grp.update(first.to(DEV), [0, 10, 10])
+        grp.update(later.to(DEV), [0, 30, 30])
+        assert grp.low_rank == [False, lim > 0]
+        Hs[lim] = grp.hessian(0).cpu().double()
+        assert grp.hessian(1) is None
+    X = torch.cat([first.double(), later.double()])
+    want = (2.0 / 40) * X.t() @ X
+    for lim, H in Hs.items():
+        assert ((H - want).norm() / want.norm()).item() < 2e-6, lim
+    rounded = torch.cat([first.bfloat16().double(), later.double()])
+    assert (((2.0 / 40) * rounded.t() @ rounded - want).norm() / want.norm()).item() > 1e-4

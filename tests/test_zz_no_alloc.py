@@ -47,3 +47,27 @@ def test_static_entry_point_rejects_what_does_not_fit(hip):
     assert rc == 1 and b"exceeds the static workspace" in lib.forge_last_error()
     rc = lib.forge_hessian_update_static(X.data_ptr(), 0, 20000, 4, 20000, 1.0, 0.0, H.data_ptr(), None)
     assert rc == 1 and b"columns" in lib.forge_last_error()
+
+
+def test_static_entry_point_allocates_nothing_and_creates_no_events(hip):
+    """What the entry point is for: across its calls (after the first on the device, which looks
+    the array's address up) the device's free memory and torch's reserved memory do not move,
+    and with per-kernel timing switched on it files no record (a record is a pair of events)."""
+    g = torch.Generator().manual_seed(9)
+    X = torch.randn(300, 512, generator=g).bfloat16().to(DEV)
+    Xf = torch.randn(90, 512, generator=g).to(DEV)
+    H = torch.zeros(512, 512, device=DEV)
+    hip.hessian_update_static(X, H, 1.0, 0.0)              # first call on this device
+    torch.cuda.synchronize()
+    free0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    hip.timing_enable(True)
+    try:
+        for _ in range(3):
+            hip.hessian_update_static(X, H, 0.5, 0.5)
+            hip.hessian_update_static(Xf, H, 0.5, 0.5)
+        torch.cuda.synchronize()
+        records = hip.timing_collect()
+    finally:
+        hip.timing_enable(False)
+    assert records == {}
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_reserved() == reserved0
