@@ -45,6 +45,12 @@ struct GemmArgs {
     // Problems that do not take the piece path ignore it and start from X.
     const void* x_init;
     bool x_init_bf16;
+    // not null = the matrices of the batch differ in size inside their common, zero-padded
+    // allocation: lim[matrix] (a multiple of 128, device memory) replaces k1 (lim_k), m1 (lim_m)
+    // and/or n1 (lim_n) for that matrix where it is smaller.  Tiles that lie wholly beyond it
+    // are skipped; the host still sizes the grid for the largest matrix.
+    const int32_t* lim;
+    bool lim_k, lim_m, lim_n;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;

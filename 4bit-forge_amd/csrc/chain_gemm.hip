@@ -75,6 +75,11 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_kernel(GemmArgs g) {
     const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile % g.n_tiles : tile % g.n_tiles;
     const int nt = g.n0 + tn * TN;                  // first n of this tile
     int k0 = g.k0, k1 = g.k1;
+    if (g.lim != nullptr) {   // uniform over the workgroup; before any barrier
+        const int own = g.lim[bz];
+        if ((g.lim_m && mt >= own) || (g.lim_n && nt >= own)) return;
+        if (g.lim_k && k1 > own) k1 = own;
+    }
     if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
     if (g.b_lower_tri && k0 < nt) k0 = nt;
 
@@ -276,6 +281,11 @@ __global__ __launch_bounds__(256, 2) void chain_gemm_fast_kernel(GemmPair pair) 
     const int tn = g.b_upper_tri ? g.n_tiles - 1 - tile % g.n_tiles : tile % g.n_tiles;
     const int nt = g.n0 + tn * TN;
     int k0 = g.k0, k1 = g.k1;
+    if (g.lim != nullptr) {   // uniform over the workgroup; before any barrier
+        const int own = g.lim[bz];
+        if ((g.lim_m && mt >= own) || (g.lim_n && nt >= own)) return;
+        if (g.lim_k && k1 > own) k1 = own;
+    }
     if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
     if (g.b_lower_tri && k0 < nt) k0 = nt;
 
@@ -742,6 +752,11 @@ __global__ __launch_bounds__(512, 1) void split_gemm_kernel(SplitPair sp) {
     const int nt = g.n0 + tn * TN;
     const int k0 = g.k0;
     int k1 = g.k1;
+    if (g.lim != nullptr) {   // uniform over the workgroup; before any barrier
+        const int own = g.lim[bz];
+        if ((g.lim_m && m0 >= own) || (g.lim_n && nt >= own)) return;
+        if (g.lim_k && k1 > own) k1 = own;
+    }
     if (g.b_upper_tri && k1 > nt + TN) k1 = nt + TN;
     const int n_stage = (k1 - k0) / SPLIT_TK;     // a multiple of 4
 

@@ -604,3 +604,179 @@ extern "C" int forge_unit_upper_from_lower(const float* L, const int32_t* info, 
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }
+
+// ------------------------------------------------------------------ factor from the rows
+// A layer that saw n rows, n below its number of input features, has H = D + B^T B with B only n
+// rows tall (B = sqrt(2/N) X in solver order, D = damp, + 1 in pruned columns).  Eliminating the
+// columns from the last 128-column block upwards, the matrix that is left when block J is
+// reached is D + B^T S_J B with S_J = (I + B_> D_>^-1 B_>^T)^-1 (n x n; "_>" = the columns after
+// the block), so with Y = S_J B_J:
+//     T    = D_J + B_J^T Y              the block's own 128 x 128 matrix, = M_JJ^T M_JJ
+//     G    = Y M_JJ^-1                  n x 128
+//     M[k, t] = G[:, k] . b_t           every entry of the factor's rows k in J left of the block
+//     S_{J-1} = S_J - G G^T
+// Everything the displacement-form sweep reads of the factor follows: h_k = G[:, k] / M[k, k]
+// (M[k, t] / M[k, k] = h_k . b_t for t left of the block) and, inside the block,
+// -M[k, t] / M[k, k].  4 n^2 C multiply-adds instead of C^3 / 3, no C x C matrix, all of it
+// 128-wide products on the matrix pipe plus the 128 x 128 diagonal-block kernel above.  fp32
+// throughout: measured against the float64 factor the h_k . b_t come out 2-20 times CLOSER than
+// those of an fp32 Cholesky factorisation of the C x C matrix (56 rank-128 downdates of a
+// matrix that starts as the identity, against C^2 / 2 entries that each collect C / 2 products).
+namespace {
+
+// T[b] <- diag(D[b][c0 .. c0 + 127])
+__global__ __launch_bounds__(256) void rows_block_diag_kernel(float* __restrict__ T,
+                                                              const float* __restrict__ D, int64_t C,
+                                                              int64_t c0) {
+    const int64_t b = blockIdx.y;
+    const int e = blockIdx.x * 256 + threadIdx.x;           // 128 * 128 / 4 float4 per matrix
+    const int r = e >> 5, c4 = (e & 31) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (r >= c4 && r < c4 + 4) (&v.x)[r - c4] = D[b * C + c0 + r];
+    *reinterpret_cast<float4*>(T + b * NB * NB + r * NB + c4) = v;
+}
+
+// From the block's factor M (lower triangle of Mj) and its inverse Z:
+//   Zs[c][k] = Z[c][k] * (1 / M[k][k])                 (columns of the inverse, scaled: G -> h)
+//   V[c0 + t][k] = -(M[k][t] * (1 / M[k][k]))  (t < k), 0 otherwise     (the sweep's in-block rows)
+// and the next block's T = diag(D) (next_c0 >= 0).
+__global__ __launch_bounds__(256) void rows_block_scale_kernel(
+    const float* __restrict__ Mj, const float* __restrict__ Z, float* __restrict__ Zs,
+    float* __restrict__ V, float* __restrict__ T, const float* __restrict__ D, int64_t C, int64_t c0,
+    int64_t next_c0) {
+    __shared__ float rc[NB];
+    const int64_t b = blockIdx.y;
+    const float* __restrict__ Mb = Mj + b * NB * NB;
+    if (threadIdx.x < NB) rc[threadIdx.x] = 1.0f / Mb[threadIdx.x * NB + threadIdx.x];
+    __syncthreads();
+    for (int e = threadIdx.x; e < NB * NB; e += 256) {
+        const int r = e >> 7, c = e & (NB - 1);
+        Zs[b * NB * NB + e] = Z[b * NB * NB + e] * rc[c];
+        // V[t = r][k = c] from M[k][t] = Mb[c][r]
+        V[(b * C + c0 + r) * NB + c] = r < c ? -(Mb[c * NB + r] * rc[c]) : 0.0f;
+        if (next_c0 >= 0) T[b * NB * NB + e] = r == c ? D[b * C + next_c0 + r] : 0.0f;
+    }
+}
+
+__global__ __launch_bounds__(256) void rows_identity_kernel(float* __restrict__ S, int64_t n) {
+    const int64_t b = blockIdx.y;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * n; e += (int64_t)gridDim.x * 256)
+        S[b * n * n + e] = (e / n == e % n) ? 1.0f : 0.0f;
+}
+
+// A matrix whose factorisation met a pivot that is not positive is swept uncoupled
+// (gptq.py:172-175): its vectors and in-block rows become zero.
+__global__ __launch_bounds__(256) void rows_failed_kernel(float* __restrict__ HmT, float* __restrict__ V,
+                                                          const int32_t* __restrict__ info, int64_t n_hm,
+                                                          int64_t n_v) {
+    const int64_t b = blockIdx.y;
+    if (info[b] == 0) return;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n_hm; e += (int64_t)gridDim.x * 256)
+        HmT[b * n_hm + e] = 0.0f;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n_v; e += (int64_t)gridDim.x * 256)
+        V[b * n_v + e] = 0.0f;
+}
+
+}  // namespace
+
+extern "C" int64_t forge_rows_factor_workspace_bytes(int64_t batch, int64_t C, int64_t nmax) {
+    if (batch <= 0 || C <= 0 || nmax <= 0) return 0;
+    // S, Y, Y^T, G^T, and four 128 x 128 tiles per matrix: T, its factor, the inverse, the scaled inverse
+    return batch * (nmax * nmax + 3 * nmax * NB + 4 * NB * NB) * (int64_t)sizeof(float);
+}
+
+extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const int32_t* n_rows,
+                                         float* HmT, float* V, int32_t* info, int64_t batch, int64_t C,
+                                         int64_t nmax, void* ws, int64_t ws_bytes,
+                                         forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= NB && C < (1 << 22) && C % NB == 0,
+                  "bad shape batch=%lld C=%lld (C: a multiple of 128)", (long long)batch, (long long)C);
+    FORGE_REQUIRE(nmax >= NB && nmax <= 4096 && nmax % NB == 0, "nmax=%lld: a multiple of 128 up to 4096",
+                  (long long)nmax);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(BT && D && n_rows && HmT && V && info && ws, "null pointer");
+    FORGE_REQUIRE(ws_bytes >= forge_rows_factor_workspace_bytes(batch, C, nmax), "workspace too small");
+    FORGE_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 255u) == 0, "ws must be 256-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    float* S = (float*)ws;
+    float* Y = S + batch * nmax * nmax;
+    float* YT = Y + batch * nmax * NB;
+    float* GT = YT + batch * nmax * NB;
+    float* T = GT + batch * nmax * NB;
+    float* Mj = T + batch * NB * NB;
+    float* Z = Mj + batch * NB * NB;
+    float* Zs = Z + batch * NB * NB;
+    constexpr size_t kDiagLds = 2 * NB * LDP * sizeof(float);
+    FORGE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(diag_block_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDiagLds));
+    clear_info_kernel<<<dim3((unsigned)forge::ceil_div(batch, 256)), dim3(256), 0, st>>>(info, batch);
+    FORGE_LAUNCH_CHECK();
+    rows_identity_kernel<<<dim3((unsigned)(nmax * nmax / 256 < 1024 ? nmax * nmax / 256 : 1024), (unsigned)batch),
+                           dim3(256), 0, st>>>(S, nmax);
+    FORGE_LAUNCH_CHECK();
+    const dim3 tile_grid(NB * NB / 4 / 256, (unsigned)batch);
+    rows_block_diag_kernel<<<tile_grid, dim3(256), 0, st>>>(T, D, C, C - NB);
+    FORGE_LAUNCH_CHECK();
+
+    const int n = (int)nmax;
+    for (int64_t c0 = C - NB; c0 >= 0; c0 -= NB) {
+        // Y = S B_J and its transpose (each is an operand of a later product in that layout)
+        forge::GemmArgs ya{}, yb{};
+        ya.X = Y; ya.ldx = NB; ya.xs = nmax * NB;
+        ya.At = S; ya.lda = nmax; ya.as = nmax * nmax;
+        ya.Bm = BT + c0; ya.ldb = C; ya.bs = nmax * C;
+        ya.m1 = n; ya.n1 = NB; ya.k1 = n; ya.init_zero = true; ya.blocked_sum = true;
+        ya.lim = n_rows; ya.lim_m = ya.lim_k = true;
+        yb.X = YT; yb.ldx = nmax; yb.xs = nmax * NB;
+        yb.At = BT + c0; yb.lda = C; yb.as = nmax * C;
+        yb.Bm = S; yb.ldb = nmax; yb.bs = nmax * nmax;
+        yb.m1 = NB; yb.n1 = n; yb.k1 = n; yb.init_zero = true; yb.blocked_sum = true;
+        yb.lim = n_rows; yb.lim_n = yb.lim_k = true;
+        if (int e = forge::launch_chain_gemm_pair(ya, yb, batch, st)) return e;
+        // T = D_J + B_J^T Y
+        forge::GemmArgs t{};
+        t.X = T; t.ldx = NB; t.xs = NB * NB;
+        t.At = BT + c0; t.lda = C; t.as = nmax * C;
+        t.Bm = Y; t.ldb = NB; t.bs = nmax * NB;
+        t.m1 = NB; t.n1 = NB; t.k1 = n; t.blocked_sum = true;
+        t.lim = n_rows; t.lim_k = true;
+        if (int e = forge::launch_chain_gemm(t, batch, st)) return e;
+        // T = M^T M, Z = M^-1
+        {
+            forge::KernelTiming timing("chol_diag_block", st, 2.0 * NB * NB * NB * (double)batch,
+                                       forge::WORK_FLOPS);
+            diag_block_kernel<<<dim3((unsigned)batch), dim3(256), kDiagLds, st>>>(
+                T, nullptr, Z, nullptr, info, NB, 0, 1, Mj);
+            FORGE_LAUNCH_CHECK();
+        }
+        rows_block_scale_kernel<<<dim3(1, (unsigned)batch), dim3(256), 0, st>>>(Mj, Z, Zs, V, T, D, C, c0,
+                                                                                c0 - NB);
+        FORGE_LAUNCH_CHECK();
+        // G^T = Z^T Y^T (for the downdate) and the h_k = G[:, k] / M[k, k] into their columns of HmT
+        forge::GemmArgs ga{}, gb{};
+        ga.X = GT; ga.ldx = nmax; ga.xs = nmax * NB;
+        ga.At = Z; ga.lda = NB; ga.as = NB * NB;
+        ga.Bm = YT; ga.ldb = nmax; ga.bs = nmax * NB;
+        ga.m1 = NB; ga.n1 = n; ga.k1 = NB; ga.init_zero = true; ga.blocked_sum = true;
+        ga.lim = n_rows; ga.lim_n = true;
+        gb.X = HmT + c0; gb.ldx = C; gb.xs = nmax * C;
+        gb.At = YT; gb.lda = nmax; gb.as = nmax * NB;
+        gb.Bm = Zs; gb.ldb = NB; gb.bs = NB * NB;
+        gb.m1 = n; gb.n1 = NB; gb.k1 = NB; gb.init_zero = true; gb.blocked_sum = true;
+        gb.lim = n_rows; gb.lim_m = true;
+        if (int e = forge::launch_chain_gemm_pair(ga, gb, batch, st)) return e;
+        // S -= G G^T
+        if (c0 > 0) {
+            forge::GemmArgs s{};
+            s.X = S; s.ldx = nmax; s.xs = nmax * nmax;
+            s.At = GT; s.lda = nmax; s.as = nmax * NB;
+            s.Bm = GT; s.ldb = nmax; s.bs = nmax * NB;
+            s.m1 = n; s.n1 = n; s.k1 = NB; s.negate_a = true; s.blocked_sum = true;
+            s.lim = n_rows; s.lim_m = s.lim_n = true;
+            if (int e = forge::launch_chain_gemm(s, batch, st)) return e;
+        }
+    }
+    rows_failed_kernel<<<dim3(64, (unsigned)batch), dim3(256), 0, st>>>(HmT, V, info, nmax * C, C * NB);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}

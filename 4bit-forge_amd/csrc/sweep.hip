@@ -44,6 +44,10 @@ struct SweepArgs {
     const void* W0;        // [C,R] per matrix: the untouched weights (displacement form only),
     bool w0_bf16;          // as f32 or, when set, as bf16 (exact for weights that are bf16)
     float* dbound;         // [R] per matrix or null: running max |d| of each row (displacement form)
+    // U's pitch and batch stride; 0 = C and C*C.  u_band: row t holds the columns of its own
+    // 128-column block only, [C, 128] per matrix: entry (t, k) sits at U[t * ldu + k - c0].
+    int64_t ldu, u_stride;
+    bool u_band;
     int64_t C, R, G;
     int64_t c0;            // first column of this block
     int bw;                // columns in this block (<= BW)
@@ -144,7 +148,9 @@ __global__ __launch_bounds__(NT, (TAIL || NT >= 256) ? 2 : 1) void sweep_block_k
     const int64_t C = a.C, R = a.R;
     float* __restrict__ A = a.A + b * C * R + r;
     float* __restrict__ Bo = ERR_IN_A ? nullptr : a.B + b * C * R + r;
-    const float* __restrict__ U = a.U + b * C * C;
+    const int64_t ldu = a.ldu ? a.ldu : C;
+    // (band form: this block's columns start at 0 of every row)
+    const float* __restrict__ U = a.U + b * (a.ldu ? a.u_stride : C * C) - (a.u_band ? a.c0 : 0);
     const float* __restrict__ sc = a.scales + b * (PER_ELEM ? C * R : a.G * R) + r;
     const float* __restrict__ qz = a.qzeros + b * (PER_ELEM ? C * R : a.G * R) + r;
     const int32_t* __restrict__ gi = PER_ELEM ? nullptr : a.g_idx + b * C;
@@ -183,7 +189,7 @@ __global__ __launch_bounds__(NT, (TAIL || NT >= 256) ? 2 : 1) void sweep_block_k
             for (int idx = threadIdx.x; idx < SB * w4; idx += NT) {
                 const int t = i * SB + idx / w4, j = idx % w4;
                 *reinterpret_cast<float4*>(&Up[t][i * SB + 4 * j]) =
-                    *reinterpret_cast<const float4*>(U + (a.c0 + t) * C + a.c0 + i * SB + 4 * j);
+                    *reinterpret_cast<const float4*>(U + (a.c0 + t) * ldu + a.c0 + i * SB + 4 * j);
             }
         }
         __syncthreads();
@@ -235,7 +241,7 @@ __global__ __launch_bounds__(NT, (TAIL || NT >= 256) ? 2 : 1) void sweep_block_k
                         // w0_k + sum_{j<=k} d_j A[j,k], A the inverse of the 4x4 unit diagonal
                         // block of N = I - strict(V).
                         auto vv = [&](int j, int k) -> float {
-                            if constexpr (TAIL) return (c + k < C) ? U[(c + j) * C + c + k] : 0.0f;
+                            if constexpr (TAIL) return (c + k < C) ? U[(c + j) * ldu + c + k] : 0.0f;
                             else return Ub[(t + j) * BW + t + k];
                         };
                         const float v01 = vv(0, 1), v02 = vv(0, 2), v03 = vv(0, 3);
@@ -376,7 +382,7 @@ __global__ __launch_bounds__(NT, (TAIL || NT >= 256) ? 2 : 1) void sweep_block_k
                         q0_t = qz[g * R];
                     }
                     select_and_quantize(t, cs + t, s_t, q0_t);
-                    const float* __restrict__ Urow = U + (cs + t) * C + cs;
+                    const float* __restrict__ Urow = U + (cs + t) * ldu + cs;
                     for (int k = t + 1; k < rem; ++k)
                         x[k] = __builtin_fmaf(-Urow[k], err[t], x[k]);
                 }
@@ -471,7 +477,7 @@ int launch_block(const SweepArgs& a, int64_t batch, hipStream_t st) {
     // (and their byte offsets from a block's or a matrix's first row fit 31 bits)
     const int64_t far = 128 > a.G ? (128 > a.C / 32 + 1 ? 128 : a.C / 32 + 1)
                                   : (a.G > a.C / 32 + 1 ? a.G : a.C / 32 + 1);
-    const bool fast = a.bw % 32 == 0 && a.C % 4 == 0 && a.c0 % 4 == 0 && a.R % 64 == 0 &&
+    const bool fast = a.bw % 32 == 0 && (a.ldu ? a.ldu : a.C) % 4 == 0 && a.c0 % 4 == 0 && a.R % 64 == 0 &&
                       (reinterpret_cast<uintptr_t>(a.U) % 16) == 0 && (far + 1) * a.R * 4 < (1LL << 31);
     if (fast && a.R % 256 == 0) {
         dim3 grid((unsigned)(a.R / 256), (unsigned)batch);
@@ -764,6 +770,73 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
     return forge_gptq_sweep_direct_batched_w0(X, W0, FORGE_F32, 0, V, nullptr, nullptr, scalesT, qzerosT, g_idx,
                                               qweight, M, mdiag, batch, C, R, G, bits, sparse14, ws,
                                               ws_bytes, stream);
+}
+
+// ------------------------------------------------------------------ sweep from the rows, blocked
+// The displacement-form sweep for matrices whose factor is given by forge_rows_factor_blocked:
+// the entries of the factor's row k left of k's own 128-column block are h_k . b_t, so all that
+// the earlier blocks hand to block J is the n x R matrix  A = sum_{t before J} b_t d_t^T  (d_t the
+// displacements of column t, one per output row):
+//     X_J  = W0_J + Hm_J A          128 x R, inner dimension n     (before the block is swept)
+//     A   += B_J^T D_J              n x R, inner dimension 128     (after it)
+// 4 n C R multiply-adds per matrix instead of C^2 R / 2, and the in-block chains unchanged.
+extern "C" int64_t forge_gptq_sweep_rows_workspace_bytes(int64_t batch, int64_t R, int64_t nmax) {
+    if (batch <= 0 || R <= 0 || nmax <= 0) return 0;
+    return batch * nmax * R * (int64_t)sizeof(float);
+}
+
+extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dtype, const float* HmT,
+                                             const float* Bp, const float* V, const int32_t* n_rows,
+                                             const float* scalesT, const float* qzerosT,
+                                             const int32_t* g_idx, uint8_t* qweight, int64_t batch,
+                                             int64_t C, int64_t R, int64_t G, int bits, int64_t nmax,
+                                             void* ws, int64_t ws_bytes, forge_stream_t stream) {
+    if (int e = check_sweep_shape(C, R, bits)) return e;
+    FORGE_REQUIRE(batch >= 0 && batch < 65536 && G >= 1, "bad batch=%lld G=%lld", (long long)batch,
+                  (long long)G);
+    FORGE_REQUIRE(C % forge::kBW == 0 && R % 128 == 0, "C=%lld and R=%lld must be multiples of 128",
+                  (long long)C, (long long)R);
+    FORGE_REQUIRE(nmax >= 128 && nmax % 128 == 0, "nmax=%lld: a multiple of 128", (long long)nmax);
+    FORGE_REQUIRE(w0_dtype == FORGE_F32 || w0_dtype == FORGE_BF16, "w0_dtype=%d", w0_dtype);
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(X && W0 && HmT && Bp && V && n_rows && scalesT && qzerosT && g_idx && qweight && ws,
+                  "null pointer");
+    FORGE_REQUIRE(ws_bytes >= forge_gptq_sweep_rows_workspace_bytes(batch, R, nmax), "workspace too small");
+    hipStream_t st = (hipStream_t)stream;
+    float* A = (float*)ws;
+    const bool w0_bf16 = w0_dtype == FORGE_BF16;
+    for (int64_t start = 0; start < C; start += forge::kBW) {
+        if (start > 0) {
+            forge::GemmArgs g{};
+            g.X = X; g.ldx = R; g.xs = C * R;
+            g.At = HmT; g.lda = C; g.as = nmax * C;
+            g.Bm = A; g.ldb = R; g.bs = nmax * R;
+            g.m0 = (int)start; g.m1 = (int)(start + forge::kBW); g.n1 = (int)R; g.k1 = (int)nmax;
+            g.blocked_sum = true;
+            g.lim = n_rows; g.lim_k = true;
+            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        }
+        SweepArgs a{};
+        a.A = X; a.U = V; a.ldu = forge::kBW; a.u_stride = C * forge::kBW; a.u_band = true;
+        a.scales = scalesT; a.qzeros = qzerosT; a.g_idx = g_idx; a.q = qweight;
+        a.C = C; a.R = R; a.G = G; a.c0 = start; a.bw = forge::kBW;
+        a.W0 = W0; a.w0_bf16 = w0_bf16; a.maxq = (1 << bits) - 1;
+        if (int e = w0_bf16 ? launch_block<false, false, true, uint16_t>(a, batch, st)
+                            : launch_block<false, false, true>(a, batch, st))
+            return e;
+        if (start + forge::kBW < C) {
+            forge::GemmArgs g{};
+            g.X = A; g.ldx = R; g.xs = nmax * R;
+            g.At = Bp; g.lda = nmax; g.as = C * nmax;
+            g.Bm = X; g.ldb = R; g.bs = C * R;
+            g.m1 = (int)nmax; g.n1 = (int)R; g.k0 = (int)start; g.k1 = (int)(start + forge::kBW);
+            g.init_zero = start == 0;
+            g.blocked_sum = true;
+            g.lim = n_rows; g.lim_m = true;
+            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+        }
+    }
+    return FORGE_OK;
 }
 
 // ------------------------------------------------------------------ Babai (nearest plane)

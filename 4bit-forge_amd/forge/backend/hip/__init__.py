@@ -71,6 +71,11 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_codes_to_layer_order_scatter": ([vp, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_gptq_sweep_lowrank": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i64,
                                       vp], i32),
+        "forge_rows_factor_blocked": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, vp, i64, vp], i32),
+        "forge_rows_factor_workspace_bytes": ([i64, i64, i64], i64),
+        "forge_gptq_sweep_rows_blocked": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
+                                           i32, i64, vp, i64, vp], i32),
+        "forge_gptq_sweep_rows_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
         "forge_hessian_update_static_max_rows": ([i64, i32], i64),
         "forge_chol_inv_upper_batched": ([vp, vp, vp, vp, vp, i64, i64, i32, vp, i64, vp], i32),
@@ -124,6 +129,8 @@ EXPORTED_SYMBOLS = (
     "forge_gptq_sweep_lowrank", "forge_round_to_nearest", "forge_lowrank_workspace_bytes",
     "forge_gptq_sweep_lowrank_mixed", "forge_hessian_permute_gather",
     "forge_weight_to_solver_order_gather", "forge_codes_to_layer_order_scatter",
+    "forge_rows_factor_blocked", "forge_rows_factor_workspace_bytes",
+    "forge_gptq_sweep_rows_blocked", "forge_gptq_sweep_rows_workspace_bytes",
 )
 
 
@@ -498,6 +505,53 @@ class _HipKernels:
             self._check(self._lib.forge_gptq_sweep_lowrank(
                 _ptr(W0), _dtype_code(W0), _ptr(Bp), _ptr(Hm), _ptr(info), _ptr(scalesT), _ptr(qzerosT),
                 _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), n, _stream()))
+        return q
+
+    def rows_factor_blocked(self, BT, D, n_rows):
+        """BT [B,nmax,C] f32 (row j = sqrt(2/n) x_j in solver order, zero rows beyond a matrix's own),
+        D [B,C] f32, n_rows [B] int32 on the device (each a multiple of 128, <= nmax) ->
+        (HmT [B,nmax,C], V [B,C,128], info [B] i32): the factor of D + BT^T BT as the blocked
+        sweep reads it (see forge_rows_factor_blocked in forge_hip.h)."""
+        _need_cuda(BT, D, n_rows)
+        B, nmax, C = BT.shape
+        assert BT.is_contiguous() and BT.dtype == torch.float32 and nmax % 128 == 0 and C % 128 == 0
+        assert D.is_contiguous() and D.dtype == torch.float32 and tuple(D.shape) == (B, C)
+        assert n_rows.is_contiguous() and n_rows.dtype == torch.int32 and n_rows.numel() == B
+        HmT = torch.empty_like(BT)
+        V = torch.empty((B, C, 128), dtype=torch.float32, device=BT.device)
+        info = torch.empty(B, dtype=torch.int32, device=BT.device)
+        nbytes = int(self._lib.forge_rows_factor_workspace_bytes(B, C, nmax))
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=BT.device)
+        with torch.cuda.device(BT.device):
+            self._check(self._lib.forge_rows_factor_blocked(_ptr(BT), _ptr(D), _ptr(n_rows), _ptr(HmT),
+                                                            _ptr(V), _ptr(info), B, C, nmax, _ptr(ws),
+                                                            nbytes, _stream()))
+        return HmT, V, info
+
+    def gptq_sweep_rows_blocked(self, X, W0, HmT, Bp, V, n_rows, scalesT, qzerosT, g_idx, bits):
+        """X [B,C,R] f32 (weights in solver order; displacements on return), W0 the same untouched
+        (f32/bf16), HmT [B,nmax,C], Bp [B,C,nmax], V [B,C,128], n_rows [B] i32 (device),
+        scalesT/qzerosT [B,G,R], g_idx [B,C] i32 -> codes [B,C,R] u8."""
+        _need_cuda(X, W0, HmT, Bp, V, n_rows, scalesT, qzerosT, g_idx)
+        B, C, R = X.shape
+        nmax = HmT.shape[1]
+        G = scalesT.shape[1]
+        assert X.is_contiguous() and X.dtype == torch.float32 and W0.is_contiguous() and W0.shape == X.shape
+        assert HmT.is_contiguous() and tuple(HmT.shape) == (B, nmax, C) and HmT.dtype == torch.float32
+        assert Bp.is_contiguous() and tuple(Bp.shape) == (B, C, nmax) and Bp.dtype == torch.float32
+        assert V.is_contiguous() and tuple(V.shape) == (B, C, 128) and V.dtype == torch.float32
+        assert n_rows.is_contiguous() and n_rows.dtype == torch.int32 and n_rows.numel() == B
+        assert scalesT.is_contiguous() and qzerosT.is_contiguous() and tuple(scalesT.shape) == (B, G, R)
+        assert tuple(qzerosT.shape) == (B, G, R) and scalesT.dtype == torch.float32
+        assert g_idx.dtype == torch.int32 and g_idx.is_contiguous() and tuple(g_idx.shape) == (B, C)
+        q = torch.empty((B, C, R), dtype=torch.uint8, device=X.device)
+        nbytes = int(self._lib.forge_gptq_sweep_rows_workspace_bytes(B, R, nmax))
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=X.device)
+        with torch.cuda.device(X.device):
+            self._check(self._lib.forge_gptq_sweep_rows_blocked(
+                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(HmT), _ptr(Bp), _ptr(V), _ptr(n_rows),
+                _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), nmax,
+                _ptr(ws), nbytes, _stream()))
         return q
 
     def hessian_update_static(self, X, H, alpha, beta):

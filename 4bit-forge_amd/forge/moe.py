@@ -194,8 +194,10 @@ class ExpertGroupGPTQ:
                 parts += [self._kept[e, :n].to(dt), X[o:o + new].to(dt)]
                 row0[e], counts[e], alpha[e] = at, n + new, 2.0 / (n + new)
                 at += n + new
+            rows = torch.cat(parts)               # (a copy: the kept rows are cleared next)
+            for e, *_ in late:
                 self._kept[e].zero_()
-            kernels.hessian_update_ranges(torch.cat(parts), row0, counts, self.H, alpha, [0.0] * self.E)
+            kernels.hessian_update_ranges(rows, row0, counts, self.H, alpha, [0.0] * self.E)
 
     add_batch = update
 

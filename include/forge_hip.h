@@ -256,6 +256,39 @@ int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, cons
                              const int32_t* g_idx, uint8_t* qweight, int64_t batch, int64_t C,
                              int64_t R, int64_t G, int bits, int64_t n, forge_stream_t stream);
 
+/* GPTQ.quantize for a layer that saw 129 .. ~1000 calibration rows, fewer than a fraction of its
+ * input features (gptq.py:128-166 with solver.cu:9-154), again without the C x C Hessian: the
+ * closed forms of forge_lowrank_factor as 128-column blocked products on the matrix pipe.
+ *   forge_rows_factor_blocked: BT [batch][nmax][C] f32 = the rows of forge_lowrank_factor's Bp,
+ *     transposed (row j = sqrt(2/n) x_j in solver order, 0 in pruned columns; zero rows beyond a
+ *     layer's own count), D [batch][C], n_rows [batch] int32 on the DEVICE = each matrix's own row
+ *     count rounded up to a multiple of 128 (<= nmax; products skip what lies beyond it)
+ *     -> HmT [batch][nmax][C] (HmT[j][k] = entry j of h_k: h_k . b_t = M[k][t] / M[k][k] for t
+ *     left of k's 128-column block), V [batch][C][128] (V[t][k - c0] = -M[k][t] / M[k][k] for t < k
+ *     inside the block that starts at c0; 0 elsewhere) and info [batch] (1-based position of a pivot that is not
+ *     positive; that matrix's HmT and V are then zero: swept uncoupled, gptq.py:172-175).
+ *     fp32; C a multiple of 128, nmax a multiple of 128; ws of forge_rows_factor_workspace_bytes,
+ *     256-byte aligned.
+ *   forge_gptq_sweep_rows_blocked: X [batch][C][R] f32 holding the weights in solver order on
+ *     entry and the displacements on exit, W0 the same weights untouched (f32 or bf16), Bp
+ *     [batch][C][nmax] (the transpose of BT) -> qweight [batch][C][R] u8.  Before a block is swept
+ *     its columns receive Hm_J A, after it A += B_J^T (displacements), A [nmax][R] per matrix in
+ *     ws (forge_gptq_sweep_rows_workspace_bytes); the block itself runs the in-block chain of
+ *     forge_gptq_sweep_direct_batched on V.  R a multiple of 128.
+ * No counterpart in the reference, which forms and factors the C x C matrix whatever the number
+ * of rows. */
+int forge_rows_factor_blocked(const float* BT, const float* D, const int32_t* n_rows, float* HmT,
+                              float* V, int32_t* info, int64_t batch, int64_t C, int64_t nmax,
+                              void* ws, int64_t ws_bytes, forge_stream_t stream);
+int64_t forge_rows_factor_workspace_bytes(int64_t batch, int64_t C, int64_t nmax);
+int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dtype, const float* HmT,
+                                  const float* Bp, const float* V, const int32_t* n_rows,
+                                  const float* scalesT, const float* qzerosT, const int32_t* g_idx,
+                                  uint8_t* qweight, int64_t batch, int64_t C, int64_t R, int64_t G,
+                                  int bits, int64_t nmax, void* ws, int64_t ws_bytes,
+                                  forge_stream_t stream);
+int64_t forge_gptq_sweep_rows_workspace_bytes(int64_t batch, int64_t R, int64_t nmax);
+
 /* Replaces kernels.babai_solver (kernels.cpp:46-56,147-149; solver_babai.cu:123-322).
  * W [C, R] f32 solver-order weights (read only; the reference also overwrites its private
  * copy with the dequantised values), A [C, C] f32 upper Cholesky factor of H (H = A^T A),
