@@ -507,6 +507,16 @@ class _HipKernels:
                 _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), n, _stream()))
         return q
 
+    def workspace_bytes(self, what: str, *dims) -> int:
+        """The size queries of forge_hip.h: what = "chol" (batch, C), "sweep_direct" (batch, C, R),
+        "lowrank" (batch, C, n), "rows_factor" (batch, C, nmax), "sweep_rows" (batch, R, nmax)."""
+        fn = {"chol": self._lib.forge_chol_workspace_bytes,
+              "sweep_direct": self._lib.forge_gptq_sweep_direct_workspace_bytes,
+              "lowrank": self._lib.forge_lowrank_workspace_bytes,
+              "rows_factor": self._lib.forge_rows_factor_workspace_bytes,
+              "sweep_rows": self._lib.forge_gptq_sweep_rows_workspace_bytes}[what]
+        return int(fn(*[int(d) for d in dims]))
+
     def rows_factor_blocked(self, BT, D, n_rows):
         """BT [B,nmax,C] f32 (row j = sqrt(2/n) x_j in solver order, zero rows beyond a matrix's own),
         D [B,C] f32, n_rows [B] int32 on the device (each a multiple of 128, <= nmax) ->

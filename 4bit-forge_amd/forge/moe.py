@@ -13,7 +13,11 @@ Experts that saw at most ``low_rank_tokens`` rows (most experts of a large route
 handful of the calibration tokens, many none) never get a C x C Hessian: their rows are kept,
 and the solve runs on the closed form that H = D + B^T B has in those few rows
 (``kernels.lowrank_factor`` / ``kernels.gptq_sweep_lowrank``): the same result in exact
-arithmetic.
+arithmetic.  Experts with more rows than that, but still few against their number of input
+features (``rows_route_tokens``), take the same closed form in its blocked shape
+(``kernels.rows_factor_blocked`` / ``kernels.gptq_sweep_rows_blocked``): products of inner
+dimension n on the matrix pipe instead of a C x C factorisation and products of inner
+dimension C.
 """
 from __future__ import annotations
 
@@ -32,6 +36,11 @@ class ExpertGroupGPTQ:
     # ahead of the device, each call holding tens of GB of workspace that cannot be reused before
     # its kernels have run: every call waits for the call before the last MAX_IN_FLIGHT to finish.
     MAX_IN_FLIGHT = 2
+    # The blocked closed form costs 4 n C R multiply-adds on the fp32 matrix instruction against
+    # C^2 R / 2 + C^3 / 6 of the route through the Hessian on the (three times faster) 16-bit
+    # pipe, plus that route's Hessian, permutation and panel passes: measured on the
+    # DeepSeek-V3-shaped layer it wins while n (a multiple of 128) times this factor is at most C.
+    ROWS_ROUTE_COST = 7
     _in_flight = collections.deque()
     _in_flight_lock = threading.Lock()
     # The device runs the kernels of one hardware queue one after the other, and a process has
@@ -56,7 +65,7 @@ class ExpertGroupGPTQ:
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
                  algorithm: str = "gptq", device=None, factor_route: str = "direct",
-                 low_rank_tokens: int = 128):
+                 low_rank_tokens: int = 128, rows_route_tokens: Optional[int] = None):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
@@ -70,8 +79,13 @@ class ExpertGroupGPTQ:
         experts with at most this many calibration rows are solved from the rows themselves,
         see the module text; 0 = every expert through its Hessian.  At 65-128 rows the per-row
         vector sweep costs nearly what the route through the Hessian costs (measured: 1 % of a
-        benchmark step in its favour).  ``self.H[e]`` of such an
-        expert is never written (uninitialised memory): read Hessians through ``hessian(e)``."""
+        benchmark step in its favour).  Such an expert has no stored Hessian: read Hessians
+        through ``hessian(e)``.
+        rows_route_tokens (needs low_rank_tokens > 0, C and every R a multiple of 128): experts
+        with more rows than low_rank_tokens and at most this many, rounded up to a multiple of
+        128, are solved from their rows by the blocked closed form, as long as that count times
+        ``ROWS_ROUTE_COST`` does not exceed C (beyond that the route through the Hessian is the
+        cheaper one).  0 or None = off (the default: see ROWS_ROUTE_COST)."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         if factor_route not in ("direct", "inverse"):
@@ -94,13 +108,29 @@ class ExpertGroupGPTQ:
         self.quantization_scale = quantization_scale
         self.quantization_order = quantization_order
         self.rel_damp = rel_damp
-        self.H: Optional[torch.Tensor] = None           # [E, C, C] f32
+        # Hessians of the experts that go through one, [slots, C, C] f32: expert e owns
+        # _Hpool[_slot[e]] (-1: none yet).  Experts that are solved from their rows never get one
+        # (a DeepSeek-V3 layer: 38 of 256 experts x 205 MB instead of 256).
+        self._Hpool: Optional[torch.Tensor] = None
+        self._slot = [-1] * self.E
+        self._slot_expert: List[int] = []
         self.num_samples = [0] * self.E                 # host-side counts
         if not 0 <= int(low_rank_tokens) <= 128:
             raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..128")
         ok = algorithm == "gptq" and factor_route == "direct" and self.C % 16 == 0 \
             and len({w.dtype for w in self.W}) == 1
         self.low_rank_tokens = int(low_rank_tokens) if ok else 0
+        rows_ok = self.low_rank_tokens > 0 and self.C % 128 == 0 and all(w.shape[1] % 128 == 0 for w in self.W)
+        want = 0 if rows_route_tokens is None else int(rows_route_tokens)
+        if want < 0 or want % 128 != 0:
+            raise ValueError(f"rows_route_tokens={rows_route_tokens}: a multiple of 128")
+        self.rows_route_tokens = min(want, self.C // self.ROWS_ROUTE_COST // 128 * 128) if rows_ok else 0
+        if self.rows_route_tokens <= self.low_rank_tokens:
+            self.rows_route_tokens = 0
+        # experts on the blocked route: rows_route[e], their rows as they came (a list of [k, C]
+        # tensors per expert, copies)
+        self.rows_route = [False] * self.E
+        self._rows = [[] for _ in range(self.E)]
         # rows of the experts that are still on the low-rank route, [E, _cap, C] f32 (zero rows
         # beyond num_samples[e]); low_rank[e] turns False for good once an expert has seen more
         self._cap = next(n for n in (16, 32, 64, 128) if n >= max(self.low_rank_tokens, 1))
@@ -122,9 +152,9 @@ class ExpertGroupGPTQ:
 
     @torch.no_grad()
     def hessian(self, e: int) -> torch.Tensor:
-        """H of expert e, [C, C] f32, as forge/gptq.py:61-80 would have accumulated it.  For an
-        expert on the low-rank route ``self.H[e]`` is never written (that is the point of the
-        route); its Hessian is formed here from the rows that were kept, (2/n) X^T X in float64
+        """H of expert e, [C, C] f32, as forge/gptq.py:61-80 would have accumulated it.  An
+        expert that is solved from its rows has no stored Hessian (that is the point of those
+        routes); it is formed here from the rows that were kept, (2/n) X^T X in float64
         rounded once; an expert that saw nothing has none (the reference's ``H is None``)."""
         n = self.num_samples[e]
         if n == 0:
@@ -132,7 +162,61 @@ class ExpertGroupGPTQ:
         if self.low_rank[e]:
             X = self._kept[e, :n].double()
             return ((2.0 / n) * X.t() @ X).float()
-        return self.H[e]
+        if self.rows_route[e]:
+            X = torch.cat(self._rows[e]).double()
+            return ((2.0 / n) * X.t() @ X).float()
+        return self._Hpool[self._slot[e]]
+
+    def _give_slots(self, experts):
+        """Hessian storage for these experts (those that have none yet); the pool grows by what
+        is asked for, existing Hessians are copied over."""
+        fresh = [e for e in experts if self._slot[e] < 0]
+        if not fresh:
+            return
+        have = len(self._slot_expert)
+        if self._Hpool is None or self._Hpool.shape[0] < have + len(fresh):
+            pool = torch.empty((have + len(fresh), self.C, self.C), dtype=torch.float32, device=self.device)
+            if have:
+                pool[:have] = self._Hpool[:have]
+            self._Hpool = pool
+        for e in fresh:
+            self._slot[e] = len(self._slot_expert)
+            self._slot_expert.append(e)
+
+    def workspace_bytes(self, n_dense: int, n_low: int, n_rows: int, rows_nmax: int, R: int) -> int:
+        """Device memory that quantize() allocates while one of its jobs is in flight (a job = the
+        stacks that share a factor, R rows in all) for n_dense experts through their Hessians,
+        n_low solved from at most 128 rows and n_rows by the blocked closed form with up to
+        rows_nmax rows: permuted Hessian, factor band, solver-order weights (fp32 and their own
+        type), codes and the kernels' workspaces.  The three routes run on two streams, so their
+        needs add up."""
+        C, esz = self.C, self.W[0].element_size()
+        per_matrix = C * R * (4 + esz + 1)                    # X, W0, codes
+        need = 0
+        if n_dense:
+            need += n_dense * (2 * C * C * 4 + per_matrix) + kernels.workspace_bytes("chol", n_dense, C) \
+                + kernels.workspace_bytes("sweep_direct", n_dense, C, R)
+        if n_low:
+            need += n_low * (C * R * (esz + 1) + 2 * C * 128 * 4) + kernels.workspace_bytes("lowrank", n_low, C, 128)
+        if n_rows:
+            need += n_rows * (per_matrix + 3 * rows_nmax * C * 4 + C * 128 * 4) \
+                + kernels.workspace_bytes("rows_factor", n_rows, C, rows_nmax) \
+                + kernels.workspace_bytes("sweep_rows", n_rows, R, rows_nmax)
+        return need
+
+    def _require_memory(self, need: int):
+        """Raises before anything is queued when the device cannot hold a solve's workspace: a
+        kernel that meets a full device in the middle of the queue takes the queue down with it."""
+        free, _ = torch.cuda.mem_get_info(self.device)
+        cached = torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+        if need > free + cached:
+            raise RuntimeError(
+                f"ExpertGroupGPTQ.quantize needs about {need / 2**30:.1f} GiB of workspace for a chunk, "
+                f"{(free + cached) / 2**30:.1f} GiB are free on {self.device}: pass a smaller `chunk`")
+
+    def _per_slot(self, per_expert):
+        """a per-expert host list rearranged by Hessian slot"""
+        return [per_expert[e] for e in self._slot_expert]
 
     def _dev(self, values, dtype=None):
         """A small host list as a device tensor without stopping the host: through pinned memory
@@ -154,10 +238,10 @@ class ExpertGroupGPTQ:
             X = X.float()
         if X.stride(-1) != 1:
             X = X.contiguous()
-        if self.H is None:
-            self.H = torch.empty((self.E, self.C, self.C), dtype=torch.float32, device=self.device)
         if self._kept is None and self.low_rank_tokens:
             self._kept = torch.zeros((self.E, self._cap, self.C), dtype=torch.float32, device=self.device)
+        if not self.low_rank_tokens:
+            self._give_slots(range(self.E))          # every expert through its Hessian, in order
         row0, counts, alpha, beta = [], [], [], []
         src, dst, late = [], [], []
         for e in range(self.E):
@@ -170,18 +254,32 @@ class ExpertGroupGPTQ:
                 self._kept_wide[e] |= new > 0 and X.dtype == torch.float32
                 dst.extend(range(e * self._cap + n, e * self._cap + total))
                 new = 0
-            elif self.low_rank[e]:
-                self.low_rank[e] = False
+            elif (self.low_rank[e] or self.rows_route[e]) and total <= self.rows_route_tokens:
+                if self.low_rank[e]:                              # outgrew the per-row-vector sizes
+                    self.low_rank[e], self.rows_route[e] = False, True
+                    if n > 0:
+                        self._rows[e].append(self._kept[e, :n].clone())
+                        self._kept[e].zero_()
+                if new > 0:
+                    self._rows[e].append(X[o:o + new].clone())
+                new = 0
+            elif self.low_rank[e] or self.rows_route[e]:
                 if n > 0:
                     late.append((e, n, o, new))                   # H[e] was never written
                     new = 0
+                else:
+                    self.low_rank[e] = self.rows_route[e] = False
             row0.append(o)
             counts.append(new)
             alpha.append(2.0 / max(total, 1))
             beta.append(n / max(total, 1))
         if src:
             self._kept.view(self.E * self._cap, self.C)[self._dev(dst)] = X[self._dev(src)].float()
-        kernels.hessian_update_ranges(X, row0, counts, self.H, alpha, beta)
+        self._give_slots([e for e in range(self.E) if counts[e] > 0] + [e for e, *_ in late])
+        if any(counts):
+            kernels.hessian_update_ranges(X, self._per_slot(row0), self._per_slot(counts),
+                                          self._Hpool[:len(self._slot_expert)], self._per_slot(alpha),
+                                          self._per_slot(beta))
         if late:
             # experts that leave the low-rank route: their Hessian from the kept rows and the
             # new ones together, (2/total) X^T X, what the running mean equals
@@ -190,14 +288,23 @@ class ExpertGroupGPTQ:
             # kept rows that came in as f32 are not rounded to a later call's bf16: the route
             # through the Hessian would have summed them in f32 too
             dt = torch.float32 if any(self._kept_wide[e] for e, *_ in late) else X.dtype
+            dt = torch.float32 if any(r.dtype == torch.float32 for e, *_ in late for r in self._rows[e]) else dt
             for e, n, o, new in late:
-                parts += [self._kept[e, :n].to(dt), X[o:o + new].to(dt)]
+                if self.rows_route[e]:
+                    parts += [r.to(dt) for r in self._rows[e]] + [X[o:o + new].to(dt)]
+                else:
+                    parts += [self._kept[e, :n].to(dt), X[o:o + new].to(dt)]
                 row0[e], counts[e], alpha[e] = at, n + new, 2.0 / (n + new)
                 at += n + new
             rows = torch.cat(parts)               # (a copy: the kept rows are cleared next)
             for e, *_ in late:
-                self._kept[e].zero_()
-            kernels.hessian_update_ranges(rows, row0, counts, self.H, alpha, [0.0] * self.E)
+                if self.low_rank[e]:
+                    self._kept[e].zero_()
+                self._rows[e] = []
+                self.low_rank[e] = self.rows_route[e] = False
+            kernels.hessian_update_ranges(rows, self._per_slot(row0), self._per_slot(counts),
+                                          self._Hpool[:len(self._slot_expert)], self._per_slot(alpha),
+                                          [0.0] * len(self._slot_expert))
 
     add_batch = update
 
@@ -212,12 +319,19 @@ class ExpertGroupGPTQ:
         there when it calls quantize(), which then neither waits for that other work nor makes
         its scale search wait for it.  Another update() discards it."""
         E, C, dev = self.E, self.C, self.device
-        if self.H is None:
-            self.H = torch.empty((E, C, C), dtype=torch.float32, device=dev)
+        lr_host = list(self.low_rank)
+        rr_host = list(self.rows_route)
+        # every expert that is not solved from its rows has a Hessian (one that saw nothing gets
+        # the identity written into its slot by quantize())
+        self._give_slots([e for e in range(E) if not (lr_host[e] or rr_host[e])])
         # experts that never saw a token (or whose Hessian went NaN) fall back to H = I
         seen = self._dev([n > 0 for n in self.num_samples])
-        diag_all = self.H.diagonal(dim1=1, dim2=2)                        # [E, C] view
-        lr_host = list(self.low_rank)
+        if self._slot_expert == list(range(E)):
+            diag_all = self._Hpool.diagonal(dim1=1, dim2=2)                # [E, C] view
+        else:
+            diag_all = torch.zeros((E, C), dtype=torch.float32, device=dev)
+            if self._slot_expert:
+                diag_all[self._dev(self._slot_expert)] = self._Hpool[:len(self._slot_expert)].diagonal(dim1=1, dim2=2)
         any_lr = any(lr_host)
         lr_dev = alpha32 = None
         if any_lr:
@@ -232,9 +346,20 @@ class ExpertGroupGPTQ:
             d_lr = torch.cat([((self._kept[i:i + 32].double() ** 2).sum(dim=1)
                                * alpha32[i:i + 32].double()[:, None]).float() for i in range(0, E, 32)])
             diag_all = torch.where(lr_dev[:, None], d_lr, diag_all)
+        rows_cat = {}
+        if any(rr_host):
+            # experts on the blocked route: the same diagonal from their own rows
+            d_rr = torch.zeros((E, C), dtype=torch.float32, device=dev)
+            for e in range(E):
+                if rr_host[e]:
+                    rows_cat[e] = self._rows[e][0] if len(self._rows[e]) == 1 else torch.cat(self._rows[e])
+                    self._rows[e] = [rows_cat[e]]
+                    d_rr[e] = ((rows_cat[e].double() ** 2).sum(dim=0) * (2.0 / self.num_samples[e])).float()
+            diag_all = torch.where(self._dev(rr_host)[:, None], d_rr, diag_all)
         bad = (~seen) | torch.isnan(diag_all).any(dim=1)
-        if any_lr:
-            diag_all = torch.where((bad & lr_dev)[:, None], torch.ones((), device=dev), diag_all)
+        if any_lr or any(rr_host):
+            off_h = self._dev([a or b for a, b in zip(lr_host, rr_host)])
+            diag_all = torch.where((bad & off_h)[:, None], torch.ones((), device=dev), diag_all)
         # Weights with pruned columns zeroed decide the (unpermuted-index) zero-column mask
         # that the reference applies to the permuted Hessian (forge/gptq.py:145-149).  A column
         # can only be all zero if its first rows are: one look at 8 rows of every expert (fp8-
@@ -251,7 +376,7 @@ class ExpertGroupGPTQ:
         ready.record()
         self._prepared = dict(diag_all=diag_all, bad=bad, host_flags=host_flags, ready=ready,
                               lr_host=lr_host, any_lr=any_lr, lr_dev=lr_dev, alpha32=alpha32,
-                              keep=flags)
+                              rr_host=rr_host, rows_cat=rows_cat, keep=flags)
         return self._prepared
 
     @torch.no_grad()
@@ -272,21 +397,34 @@ class ExpertGroupGPTQ:
         diag_all, bad, host_flags = prep["diag_all"], prep["bad"], prep["host_flags"]
         lr_host, any_lr = prep["lr_host"], prep["any_lr"]
         lr_dev, alpha32 = prep["lr_dev"], prep["alpha32"]
+        rr_host, rows_cat = prep["rr_host"], prep["rows_cat"]
+        any_rr = any(rr_host)
         # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
         # fraction of the fill rate)
         for e in host_flags[0].nonzero().flatten().tolist():
-            if lr_host[e]:
+            if lr_host[e] or rr_host[e]:
                 continue                       # no matrix: its rows count as none (below)
-            self.H[e].zero_()
-            self.H[e].diagonal().fill_(1.0)
-            diag_all = self.H.diagonal(dim1=1, dim2=2) if not any_lr else diag_all.index_fill(
-                0, self._dev([e]), 1.0)
+            He = self._Hpool[self._slot[e]]
+            He.zero_()
+            He.diagonal().fill_(1.0)
+            diag_all = diag_all.index_fill(0, self._dev([e]), 1.0)
+        # the largest chunk's workspace must fit before anything is queued
+        sizes_all = sum(int(W.shape[1]) for W in self.W)
+        need = 0
+        for c0 in range(0, E, chunk):
+            ids = range(c0, min(E, c0 + chunk))
+            rr = [self.num_samples[e] for e in ids if rr_host[e] and not bool(host_flags[0, e])]
+            need = max(need, self.workspace_bytes(
+                sum(1 for e in ids if not (lr_host[e] or rr_host[e])),
+                sum(1 for e in ids if lr_host[e] and not bool(host_flags[0, e])),
+                len(rr), max([(n + 127) // 128 * 128 for n in rr], default=0), sizes_all))
+        self._require_memory(need)
         failed = []
         cand = None                                   # the shrink factors, made on the search stream
         side, lr_shared = self._streams_of(dev) if overlap_scale_search else (None, None)
         # the low-rank experts' kernels are chains of dependent steps on a few wavefronts: on a
         # stream of their own they run beside the other experts' matrix products
-        lr_side = lr_shared if any_lr else None
+        lr_side = lr_shared if (any_lr or any_rr) else None
 
         sizes = [int(W.shape[1]) for W in self.W]
         sparse = self.algorithm == "sparsegptq"
@@ -339,9 +477,10 @@ class ExpertGroupGPTQ:
                 if babai:   # positions of the reference's order -> positions of the reversed one
                     masks = [m.flip(1).contiguous() for m in masks]
             # the experts of the chunk by route (positions in the chunk, ascending)
-            none_ids = [e - e0 for e in range(e0, e1) if lr_host[e] and bool(host_flags[0, e])]
+            none_ids = [e - e0 for e in range(e0, e1) if (lr_host[e] or rr_host[e]) and bool(host_flags[0, e])]
             lr_ids = [e - e0 for e in range(e0, e1) if lr_host[e] and not bool(host_flags[0, e])]
-            dn_ids = [e - e0 for e in range(e0, e1) if not lr_host[e]]
+            rr_ids = [e - e0 for e in range(e0, e1) if rr_host[e] and not bool(host_flags[0, e])]
+            dn_ids = [e - e0 for e in range(e0, e1) if not (lr_host[e] or rr_host[e])]
             # stacks that share the factor are swept as ONE tall matrix (rows are independent)
             jobs = [list(range(len(self.W)))] if shared else [[i] for i in range(len(self.W))]
             for job in jobs:
@@ -408,7 +547,7 @@ class ExpertGroupGPTQ:
 
                 # ---------------------------------------------------------- low-rank experts
                 lr_stream = main
-                if lr_ids or none_ids:
+                if lr_ids or none_ids or rr_ids:
                     lr_stream = lr_side if lr_side is not None and dn_ids else main
                     lr_stream.wait_stream(main)
                 with torch.cuda.stream(lr_stream):
@@ -446,10 +585,36 @@ class ExpertGroupGPTQ:
                         layout_in(ids, W0[pos:pos + len(ids)], skip_out=True)
                         pos += len(ids)
                         at += len(ids) * C * nr
-                    if lr_ids or none_ids:
+                    # ---------------------------------------------------- blocked closed form
+                    if rr_ids:
+                        ri = self._dev(rr_ids)
+                        msk = mask[ri].bool()                               # [Br, C], solver order
+                        n_own = [self.num_samples[e0 + i] for i in rr_ids]
+                        nmax = max((n + 127) // 128 * 128 for n in n_own)
+                        n_rows = self._dev([(n + 127) // 128 * 128 for n in n_own], dtype=torch.int32)
+                        BT = torch.zeros((len(rr_ids), nmax, C), dtype=torch.float32, device=dev)
+                        perm_r = perm[ri]
+                        for b, (i, n) in enumerate(zip(rr_ids, n_own)):
+                            rows = (rows_cat[e0 + i].double() * (2.0 / n) ** 0.5).float()
+                            BT[b, :n] = rows.index_select(1, perm_r[b]).masked_fill(msk[b][None, :], 0)
+                        dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[ri], 1, perm_r))
+                        D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
+                        HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows)
+                        Bp_r = BT.transpose(1, 2).contiguous()
+                        del BT
+                        failed.append((torch.tensor([e0 + i for i in rr_ids]), info_r))
+                        Xr = torch.empty((len(rr_ids), C, R), dtype=torch.float32, device=dev)
+                        W0r = torch.empty((len(rr_ids), C, R), dtype=self.W[job[0]].dtype, device=dev)
+                        layout_in(rr_ids, W0r, Xr)
+                    if lr_ids or none_ids or rr_ids:
                         lr_stream.wait_stream(search)
                         for t in (scales, qzeros, sT, zT) + tuple(x for p in parts for x in p):
                             t.record_stream(lr_stream)
+                    if rr_ids:
+                        q = kernels.gptq_sweep_rows_blocked(Xr, W0r, HmT, Bp_r, V, n_rows, sT[ri], zT[ri],
+                                                            g_idx[ri].contiguous(), self.bits)
+                        layout_out(rr_ids, q)
+                        del Xr, W0r, HmT, Bp_r, V, q
                     if ids_all:
                         failed.append((torch.tensor([e0 + i for i in ids_all]), info))
                         la = self._dev(ids_all)
@@ -474,8 +639,21 @@ class ExpertGroupGPTQ:
                     pick = (lambda t: t) if whole else (lambda t: t[di].contiguous())
                     Bd = len(dn_ids)
                     # the factorisations read their input's lower triangle in 128 x 128 blocks only
-                    Hp, damp = kernels.hessian_permute(self.H[e0:e1], perm, mask, float(self.rel_damp),
-                                                       lower_blocks=True, index=di)
+                    slots = [self._slot[e0 + i] for i in dn_ids]
+                    if slots == list(range(e0, e1)) and self._Hpool.shape[0] >= e1:
+                        Hp, damp = kernels.hessian_permute(self._Hpool[e0:e1], perm, mask, float(self.rel_damp),
+                                                           lower_blocks=True)
+                    else:
+                        # the kernel takes ONE index for the Hessian, the order and the mask: the
+                        # latter two are laid out by slot as well
+                        si = self._dev(slots)
+                        n_slots = len(self._slot_expert)
+                        perm_s = torch.empty((n_slots, C), dtype=perm.dtype, device=dev)
+                        mask_s = torch.empty((n_slots, C), dtype=mask.dtype, device=dev)
+                        perm_s[si] = pick(perm)
+                        mask_s[si] = pick(mask)
+                        Hp, damp = kernels.hessian_permute(self._Hpool[:n_slots], perm_s, mask_s,
+                                                           float(self.rel_damp), lower_blocks=True, index=si)
                     if babai:
                         L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                         U = kernels.unit_upper_from_lower(L, info, upper_only=True)

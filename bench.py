@@ -117,7 +117,8 @@ def make_workload(name, cfg, chunk, seed=0):
 STREAMS = []
 
 
-def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_tokens=128):
+def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_tokens=128,
+               rows_route_tokens=None):
     """First half of the hot path for experts [step*chunk, (step+1)*chunk) of the layer: the
     expert groups, their Hessian updates and the look at the result that the solve starts from
     (ExpertGroupGPTQ.prepare), queued on the jobs' streams."""
@@ -140,7 +141,8 @@ def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_t
         offs.append(offs[-1] + wl["counts"][e])
     kw = dict(bits=4, group_size=128, symmetric=cfg["symmetric"],
               quantization_scale="mse" if mse else "absmax", quantization_order=cfg["order"],
-              rel_damp=0.01, device="cuda", factor_route=factor_route, low_rank_tokens=low_rank_tokens)
+              rel_damp=0.01, device="cuda", factor_route=factor_route, low_rank_tokens=low_rank_tokens,
+              rows_route_tokens=rows_route_tokens)
     # gate/up (shared Hessian) and down are independent: one HIP stream each, so that the
     # MFMA-bound factorisation/sweep of one overlaps the VALU-bound scale search and the
     # latency-bound diagonal blocks of the other.  One host thread queues both (quantize() does
@@ -184,18 +186,30 @@ def solve_step(staged, overlap=True):
     return results[0::2], results[1::2]
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128):
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128,
+             rows_route_tokens=None):
     """One whole step (both halves) of the hot path."""
     return solve_step(stage_step(wl, cfg, chunk, step, mse=mse, factor_route=factor_route,
-                                 low_rank_tokens=low_rank_tokens), overlap=overlap)
+                                 low_rank_tokens=low_rank_tokens, rows_route_tokens=rows_route_tokens),
+                      overlap=overlap)
 
 
-def route_counts(wl, chunk, low_rank_tokens):
-    """How many of the layer's experts take which route (whole layer, by routed rows)."""
+def route_counts(wl, cfg, low_rank_tokens, rows_route_tokens):
+    """How many of the layer's experts take which route (whole layer, by routed rows): the
+    limits that ExpertGroupGPTQ derives for the gate/up group (C = hidden) and for the down
+    group (C = inter)."""
+    from forge.moe import ExpertGroupGPTQ
     c = wl["counts"]
     none = sum(1 for n in c if n == 0) if low_rank_tokens else 0
     low = sum(1 for n in c if 0 < n <= low_rank_tokens)
-    return dict(no_rows=none, low_rank=low, through_hessian=len(c) - none - low)
+    out = dict(no_rows=none, low_rank=low)
+    want = 0 if rows_route_tokens is None else rows_route_tokens
+    for name, C in (("gate_up", cfg["hidden"]), ("down", cfg["inter"])):
+        lim = min(want, C // ExpertGroupGPTQ.ROWS_ROUTE_COST // 128 * 128) if low_rank_tokens else 0
+        rows = sum(1 for n in c if low_rank_tokens < n <= lim)
+        out[f"rows_blocked_{name}"] = rows
+        out[f"through_hessian_{name}"] = len(c) - none - low - rows
+    return out
 
 
 def timed_steps(wl, cfg, chunk, steps, warmup, first_step=0, **kw):
@@ -493,6 +507,10 @@ def main():
     ap.add_argument("--low-rank-tokens", type=int, default=128,
                     help="experts with at most this many routed rows are solved from the rows themselves "
                          "(0: every expert through its Hessian)")
+    ap.add_argument("--rows-route-tokens", type=int, default=None,
+                    help="experts with more rows than --low-rank-tokens and at most this many (a multiple "
+                         "of 128) take the blocked closed form while it is cheaper than the route through "
+                         "the Hessian (default 0: off)")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run of "
@@ -518,7 +536,8 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    route = dict(factor_route=a.factor_route, low_rank_tokens=a.low_rank_tokens)
+    route = dict(factor_route=a.factor_route, low_rank_tokens=a.low_rank_tokens,
+                 rows_route_tokens=a.rows_route_tokens)
     elapsed = timed_steps(wl, cfg, chunk, a.steps, a.warmup, mse=mse, **route)
     peak_gb = torch.cuda.max_memory_reserved() / 1e9      # workload and the steps in flight
 
@@ -565,7 +584,9 @@ def main():
                                f" {'mse' if mse else 'absmax'} grid",
                    "experts_per_step": chunk, "factor_route": a.factor_route,
                    "low_rank_tokens": a.low_rank_tokens if a.factor_route == "direct" else 0,
-                   "experts_by_route": route_counts(wl, chunk, a.low_rank_tokens if a.factor_route == "direct" else 0)},
+                   "rows_route_tokens": a.rows_route_tokens,
+                   "experts_by_route": route_counts(wl, cfg, a.low_rank_tokens if a.factor_route == "direct" else 0,
+                                                    a.rows_route_tokens)},
         "roofline": roofline,
         "kernels": breakdown,
         "peak_device_memory_gb": round(peak_gb, 1),

@@ -3,7 +3,7 @@
 One ``ExpertGroupGPTQ.quantize()`` call per projection carries experts of every kind that a
 step of the benchmark layer holds: experts without a single routed row (plain rounding),
 with 3 .. 128 rows (solved from the rows, all sizes of the per-row-vector sweep in ONE mixed
-launch), and with more rows than that (through the Hessian or the blocked closed form).  gate_proj
+launch), with 200 rows (the blocked closed form) and with 1536 (through the Hessian).  gate_proj
 and up_proj are two stacks that share one factor (C = 7168; 256 of their 2048 rows each, rows
 being independent); down_proj has its full shape, R = 7168, C = 2048.  Every expert is then
 compared with ``oracle.GPTQ`` (forge/gptq.py:128-139 on the handles that quant.py:386-396
@@ -50,11 +50,11 @@ def gate_up():
                       for _ in range(E)]) for _ in range(2)]
     xs = _rows(32, C)
     offs = np.concatenate([[0], np.cumsum(NS)]).tolist()
-    grp = ExpertGroupGPTQ([w.to(DEV) for w in W], device=DEV, **KW)
+    grp = ExpertGroupGPTQ([w.to(DEV) for w in W], device=DEV, rows_route_tokens=1024, **KW)
     grp.update(torch.cat(xs).to(DEV), offs)
     outs = [tuple(t.cpu() for t in o) for o in grp.quantize(chunk=E)]
     assert not grp.issue_non_invertible.any()
-    routes = list(grp.low_rank)
+    routes = (list(grp.low_rank), list(grp.rows_route))
     del grp
     torch.cuda.empty_cache()
     return W, xs, outs, routes
@@ -69,11 +69,11 @@ def down():
                      for _ in range(E)])
     xs = _rows(34, C)
     offs = np.concatenate([[0], np.cumsum(NS)]).tolist()
-    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, **KW)
+    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, rows_route_tokens=1024, **KW)
     grp.update(torch.cat(xs).to(DEV), offs)
     outs = [tuple(t.cpu() for t in o) for o in grp.quantize(chunk=E)]
     assert not grp.issue_non_invertible.any()
-    routes = list(grp.low_rank)
+    routes = (list(grp.low_rank), list(grp.rows_route))
     del grp
     torch.cuda.empty_cache()
     return W, xs, outs, routes
@@ -109,11 +109,12 @@ def _against_the_oracle(tag, W, X, q, s, z):
 
 
 def test_routes_taken(gate_up, down):
-    """What the step is meant to mix: no-row and few-row experts off the Hessian route, the
-    others on it, in one call."""
-    for _, _, _, routes in (gate_up, down):
-        assert [r for r, n in zip(routes, NS) if n <= 128] == [True] * sum(n <= 128 for n in NS)
-        assert not any(r for r, n in zip(routes, NS) if n > 128)
+    """What the step is meant to mix in one call: experts without rows and with few rows solved
+    from the rows themselves, the expert with 200 rows by the blocked closed form (256 x 7 does
+    not exceed 2048 nor 7168), the one with 1536 rows through its Hessian."""
+    for _, _, _, (low, blocked) in (gate_up, down):
+        assert low == [n <= 128 for n in NS]
+        assert blocked == [n == 200 for n in NS]
 
 
 @pytest.mark.parametrize("e", GATE_UP_CASES)

@@ -581,3 +581,25 @@ def test_config2_qwen3_experts_at_full_shape(hip):
     print(f"config2 experts: worst flips {worst:.2e}, worst per-expert error deviation "
           f"{worst_ratio:.2e}, layer error ratio {sum_g / sum_o:.5f}")
     assert worst_ratio < 0.01 and abs(sum_g / sum_o - 1) < 0.01
+
+
+def test_quantize_refuses_a_chunk_whose_workspace_does_not_fit(monkeypatch):
+    """quantize() adds up what its largest chunk allocates and raises before it queues anything
+    when the device cannot hold it (a kernel that meets a full device mid-queue takes the queue
+    down with it); a smaller chunk then goes through."""
+    from forge.moe import ExpertGroupGPTQ
+    g0 = torch.Generator().manual_seed(2)
+    W = (0.02 * torch.randn(4, 128, 256, generator=g0)).bfloat16().to(DEV)
+    X = torch.randn(600, 256, generator=g0).bfloat16().to(DEV)
+    grp = ExpertGroupGPTQ([W], device=DEV, bits=4, group_size=128, symmetric=True,
+                          quantization_scale="absmax", quantization_order="activation")
+    grp.update(X, [0, 200, 400, 403, 600])
+    need = grp.workspace_bytes(3, 1, 0, 0, 128)
+    assert need > 3 * (2 * 256 * 256 * 4 + 256 * 128 * 7)
+    real = ExpertGroupGPTQ.workspace_bytes
+    monkeypatch.setattr(ExpertGroupGPTQ, "workspace_bytes",
+                        lambda self, nd, *a: (1 << 50) if nd > 2 else real(self, nd, *a))
+    with pytest.raises(RuntimeError, match="smaller `chunk`"):
+        grp.quantize(chunk=4)
+    (q, s, z), = grp.quantize(chunk=2)
+    assert tuple(q.shape) == (4, 128, 256) and not grp.issue_non_invertible.any()

@@ -236,7 +236,7 @@ def test_expert_group_low_rank_route_against_the_dense_route_and_the_oracle():
         if lim:
             X4 = torch.cat([xs[4], extra]).double()
             H4 = (2.0 / 21) * X4.t() @ X4
-            assert ((grp.H[4].cpu().double() - H4).norm() / H4.norm()).item() < 2e-6
+            assert ((grp.hessian(4).cpu().double() - H4).norm() / H4.norm()).item() < 2e-6
     for i, Wi in enumerate((W, W2)):
         assert torch.equal(out[16][i][1], out[0][i][1]) and torch.equal(out[16][i][2], out[0][i][2])
         for e, n in enumerate(ns):
