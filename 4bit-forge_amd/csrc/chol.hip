@@ -644,12 +644,13 @@ __global__ __launch_bounds__(256) void rows_block_scale_kernel(
     const float* __restrict__ Mj, const float* __restrict__ Z, float* __restrict__ Zs,
     float* __restrict__ V, float* __restrict__ T, const float* __restrict__ D, int64_t C, int64_t c0,
     int64_t next_c0) {
+    // sixteen workgroups per matrix, eight rows of the tile each
     __shared__ float rc[NB];
     const int64_t b = blockIdx.y;
     const float* __restrict__ Mb = Mj + b * NB * NB;
     if (threadIdx.x < NB) rc[threadIdx.x] = 1.0f / Mb[threadIdx.x * NB + threadIdx.x];
     __syncthreads();
-    for (int e = threadIdx.x; e < NB * NB; e += 256) {
+    for (int e = blockIdx.x * (NB * NB / 16) + threadIdx.x; e < (blockIdx.x + 1) * (NB * NB / 16); e += 256) {
         const int r = e >> 7, c = e & (NB - 1);
         Zs[b * NB * NB + e] = Z[b * NB * NB + e] * rc[c];
         // V[t = r][k = c] from M[k][t] = Mb[c][r]
@@ -749,8 +750,8 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
                 T, nullptr, Z, nullptr, info, NB, 0, 1, Mj);
             FORGE_LAUNCH_CHECK();
         }
-        rows_block_scale_kernel<<<dim3(1, (unsigned)batch), dim3(256), 0, st>>>(Mj, Z, Zs, V, T, D, C, c0,
-                                                                                c0 - NB);
+        rows_block_scale_kernel<<<dim3(16, (unsigned)batch), dim3(256), 0, st>>>(Mj, Z, Zs, V, T, D, C, c0,
+                                                                                 c0 - NB);
         FORGE_LAUNCH_CHECK();
         // G^T = Z^T Y^T (for the downdate) and the h_k = G[:, k] / M[k, k] into their columns of HmT
         forge::GemmArgs ga{}, gb{};

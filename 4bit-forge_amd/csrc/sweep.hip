@@ -782,7 +782,9 @@ extern "C" int forge_gptq_sweep_direct_batched(float* X, const float* W0, const 
 // 4 n C R multiply-adds per matrix instead of C^2 R / 2, and the in-block chains unchanged.
 extern "C" int64_t forge_gptq_sweep_rows_workspace_bytes(int64_t batch, int64_t R, int64_t nmax) {
     if (batch <= 0 || R <= 0 || nmax <= 0) return 0;
-    return batch * nmax * R * (int64_t)sizeof(float);
+    // A, and the 16-bit pieces of a block's h vectors (the shared operand of its product)
+    return (batch * nmax * R * (int64_t)sizeof(float) + 255) / 256 * 256 +
+           forge::split_gemm_workspace_bytes(batch, nmax);
 }
 
 extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dtype, const float* HmT,
@@ -804,17 +806,26 @@ extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dt
     FORGE_REQUIRE(ws_bytes >= forge_gptq_sweep_rows_workspace_bytes(batch, R, nmax), "workspace too small");
     hipStream_t st = (hipStream_t)stream;
     float* A = (float*)ws;
+    void* split_ws = (char*)ws + (batch * nmax * R * (int64_t)sizeof(float) + 255) / 256 * 256;
+    const int64_t split_bytes = forge::split_gemm_workspace_bytes(batch, nmax);
     const bool w0_bf16 = w0_dtype == FORGE_BF16;
     for (int64_t start = 0; start < C; start += forge::kBW) {
         if (start > 0) {
+            // on the 16-bit matrix pipe from two rounded bf16 pieces per operand (three products,
+            // within ~2^-17 of the fp32 product: what the route through the Hessian takes for
+            // its block updates from 4096 columns on), starting from the untouched weights;
+            // fp32 matrix instruction from X where the option fp32_blocked_sum asks for it
             forge::GemmArgs g{};
             g.X = X; g.ldx = R; g.xs = C * R;
             g.At = HmT; g.lda = C; g.as = nmax * C;
             g.Bm = A; g.ldb = R; g.bs = nmax * R;
             g.m0 = (int)start; g.m1 = (int)(start + forge::kBW); g.n1 = (int)R; g.k1 = (int)nmax;
             g.blocked_sum = true;
+            g.products = 3;
+            g.x_init = W0; g.x_init_bf16 = w0_bf16;
             g.lim = n_rows; g.lim_k = true;
-            if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
+            if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, split_ws, split_bytes))
+                return e;
         }
         SweepArgs a{};
         a.A = X; a.U = V; a.ldu = forge::kBW; a.u_stride = C * forge::kBW; a.u_band = true;

@@ -36,10 +36,12 @@ class ExpertGroupGPTQ:
     # ahead of the device, each call holding tens of GB of workspace that cannot be reused before
     # its kernels have run: every call waits for the call before the last MAX_IN_FLIGHT to finish.
     MAX_IN_FLIGHT = 2
-    # The blocked closed form costs 4 n C R multiply-adds on the fp32 matrix instruction against
-    # C^2 R / 2 + C^3 / 6 of the route through the Hessian on the (three times faster) 16-bit
-    # pipe, plus that route's Hessian, permutation and panel passes: measured on the
-    # DeepSeek-V3-shaped layer it wins while n (a multiple of 128) times this factor is at most C.
+    # The blocked closed form costs 4 n C R multiply-adds, half of them as products of inner
+    # dimension 128 that are bound by the traffic of the n x R accumulator, plus a chain of small
+    # launches per 128-column block, against C^2 R / 2 + C^3 / 6 of the route through the
+    # Hessian: measured on the DeepSeek-V3-shaped layer (256 experts a step) it wins up to 512
+    # rows at C = 7168 (232.4 / 231.2 / 237.1 ms with a limit of 256 / 512 / 1024 against 235.6
+    # without), i.e. while n (a multiple of 128) times this factor is at most C.
     ROWS_ROUTE_COST = 7
     _in_flight = collections.deque()
     _in_flight_lock = threading.Lock()
@@ -85,7 +87,7 @@ class ExpertGroupGPTQ:
         with more rows than low_rank_tokens and at most this many, rounded up to a multiple of
         128, are solved from their rows by the blocked closed form, as long as that count times
         ``ROWS_ROUTE_COST`` does not exceed C (beyond that the route through the Hessian is the
-        cheaper one).  0 or None = off (the default: see ROWS_ROUTE_COST)."""
+        cheaper one).  None = 512; 0 = off."""
         if algorithm not in ("gptq", "sparsegptq", "babai"):
             raise NotImplementedError(f"algorithm={algorithm!r}: 'gptq', 'sparsegptq' or 'babai'")
         if factor_route not in ("direct", "inverse"):
@@ -121,7 +123,7 @@ class ExpertGroupGPTQ:
             and len({w.dtype for w in self.W}) == 1
         self.low_rank_tokens = int(low_rank_tokens) if ok else 0
         rows_ok = self.low_rank_tokens > 0 and self.C % 128 == 0 and all(w.shape[1] % 128 == 0 for w in self.W)
-        want = 0 if rows_route_tokens is None else int(rows_route_tokens)
+        want = 512 if rows_route_tokens is None else int(rows_route_tokens)
         if want < 0 or want % 128 != 0:
             raise ValueError(f"rows_route_tokens={rows_route_tokens}: a multiple of 128")
         self.rows_route_tokens = min(want, self.C // self.ROWS_ROUTE_COST // 128 * 128) if rows_ok else 0

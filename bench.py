@@ -84,7 +84,7 @@ KERNEL_BOUND = {
 
 CONFIGS = {
     "deepseek_v3": dict(n_experts=256, hidden=7168, inter=2048, tokens=8192, fp8=True,
-                        symmetric=True, order="activation", chunk=128),
+                        symmetric=True, order="activation", chunk=256),
     "qwen3": dict(n_experts=128, hidden=2048, inter=768, tokens=4096, fp8=False,
                   symmetric=False, order="default", chunk=128),
 }
@@ -203,7 +203,7 @@ def route_counts(wl, cfg, low_rank_tokens, rows_route_tokens):
     none = sum(1 for n in c if n == 0) if low_rank_tokens else 0
     low = sum(1 for n in c if 0 < n <= low_rank_tokens)
     out = dict(no_rows=none, low_rank=low)
-    want = 0 if rows_route_tokens is None else rows_route_tokens
+    want = 512 if rows_route_tokens is None else rows_route_tokens
     for name, C in (("gate_up", cfg["hidden"]), ("down", cfg["inter"])):
         lim = min(want, C // ExpertGroupGPTQ.ROWS_ROUTE_COST // 128 * 128) if low_rank_tokens else 0
         rows = sum(1 for n in c if low_rank_tokens < n <= lim)
@@ -510,7 +510,7 @@ def main():
     ap.add_argument("--rows-route-tokens", type=int, default=None,
                     help="experts with more rows than --low-rank-tokens and at most this many (a multiple "
                          "of 128) take the blocked closed form while it is cheaper than the route through "
-                         "the Hessian (default 0: off)")
+                         "the Hessian (default 512; 0: off)")
     ap.add_argument("--no-mse", action="store_true", help="min/max grid only (not the default config)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run of "

@@ -4,7 +4,7 @@ One ``ExpertGroupGPTQ.quantize()`` call per projection carries experts of every 
 step of the benchmark layer holds: experts without a single routed row (plain rounding),
 with 3 .. 128 rows (solved from the rows, all sizes of the per-row-vector sweep in ONE mixed
 launch), with 200 rows (the blocked closed form) and with 1536 (through the Hessian).  gate_proj
-and up_proj are two stacks that share one factor (C = 7168; 256 of their 2048 rows each, rows
+and up_proj are two stacks that share one factor (C = 7168; 128 of their 2048 rows each, rows
 being independent); down_proj has its full shape, R = 7168, C = 2048.  Every expert is then
 compared with ``oracle.GPTQ`` (forge/gptq.py:128-139 on the handles that quant.py:386-396
 creates) under the rules of test_gpu_gptq: scales equal up to candidate near-ties, codes
@@ -31,9 +31,10 @@ KW = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
           quantization_order="activation", rel_damp=0.01)
 #        rows each expert saw: none, the per-row-vector sizes 4/16/32/64/128, then beyond
 NS = (0, 3, 16, 40, 100, 128, 200, 1536, 0, 64, 128, 5)
-# experts compared with the oracle (the others add to the batch: both n = 128, both n = 0)
-GATE_UP_CASES = (0, 1, 3, 4, 5, 6, 7)
-DOWN_CASES = (8, 2, 10, 6, 7)
+# experts compared with the oracle (a CPU solve and the floor's realisations at C = 7168 take
+# about a minute each; the others add to the batch and to the mixed launch's sizes)
+GATE_UP_CASES = (0, 1, 5, 6, 7)
+DOWN_CASES = (8, 6, 7)
 
 
 def _rows(seed, C):
@@ -45,7 +46,7 @@ def _rows(seed, C):
 def gate_up():
     from forge.moe import ExpertGroupGPTQ
     g = torch.Generator().manual_seed(31)
-    E, R, C = len(NS), 256, 7168
+    E, R, C = len(NS), 128, 7168
     W = [torch.stack([synth.fp8_block_roundtrip((0.02 * torch.randn(R, C, generator=g)).bfloat16())
                       for _ in range(E)]) for _ in range(2)]
     xs = _rows(32, C)
