@@ -9,11 +9,11 @@ g128, act-order, MSE scale search (the GPTQ class default), damp 0.01; built by
 forge.synth.deepseek_v3_moe (seed 0) on the GPU.  One STEP = one pass of the hot path over
 one chunk of experts, everything already resident in HBM: ragged Hessian accumulation for
 gate/up and for down, then per expert two factorisations (gate and up share theirs), three
-scale searches and three sweeps.  Successive steps walk through the layer's experts chunk
-by chunk (128 experts a step; their routed-token lists differ).  Experts with at most 128
+scale searches and three sweeps.  A step is the layer's 256 experts (--chunk 128: half of
+them, successive steps then walk through the layer chunk by chunk).  Experts with at most 128
 routed rows (most of them: 8192 tokens over 256 experts with Zipf popularity) take the
 library's low-rank route, which reaches the same result from the rows themselves without a
-C x C Hessian; `config.experts_by_route` counts them.
+C x C Hessian, those with up to 512 its blocked form; `config.experts_by_route` counts them.
 The timed steps are queued as a caller with a layer of chunks would queue them: chunk i+1's
 Hessian updates go onto the streams before chunk i's solve (all K updates and all K solves lie
 inside the timed region).
@@ -21,9 +21,11 @@ value = experts quantised per second = steps * chunk / elapsed.
 
 After the timed steps:
 * one more step runs with the library's per-kernel HIP-event timing switched on (events on
-  the stream each kernel is launched on); the longest-running kernel that an HBM or a
-  matrix-pipe roofline bounds gives `roofline`, every kernel a line in `kernels` with its
-  algorithmic rate and the fraction of the peak that bounds it;
+  the stream each kernel is launched on); the kernel with the largest total time gives
+  `roofline` (the scale search: bound by the vector ALU, so the line carries its nominal HBM
+  rate and the vector-ALU counters of the committed profile), the longest one on the matrix
+  pipe `roofline_matrix_pipe`, every kernel a line in `kernels` with its algorithmic rate and
+  the fraction of the peak that bounds it;
 * `mfma_ceiling`: what the matrix pipe itself sustains on this device, with operands of ones
   and with random operands;
 * `reference_route`: the same steps on the reference's route (factor of inv(H), fp32-chain
@@ -54,9 +56,11 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "4bit-forge_amd"))
 
 PEAK = {"mfma_f32": 157.3, "mfma_bf16": 2500.0, "valu_f32": 157.3, "hbm": 8000.0}   # TFLOP/s ... GB/s
-# Transcendental issue rate: v_log_f32 / v_exp_f32 run at a quarter of the fp32 rate, 16 lanes
-# per clock and SIMD: 256 CUs x 4 SIMDs x 4 per clock x 2.4 GHz.
-PEAK_TRANSCENDENTALS = 256 * 4 * 4 * 2.4e9
+# Transcendental issue rate: v_log_f32 / v_exp_f32 take eight cycles per 64-lane instruction
+# (SQ_ACTIVE_INST_VALU against SQ_INSTS_VALU in the scale search: 1.24 four-cycle units per
+# instruction with two transcendentals in eight), half the fp32 rate: 256 CUs x 4 SIMDs x 8 lanes
+# per clock x 2.4 GHz.
+PEAK_TRANSCENDENTALS = 256 * 4 * 8 * 2.4e9
 
 # kernel name (as the library's timing records call it) -> (bound, peak key, executed / counted)
 # The library counts ALGORITHMIC work per launch: 2*M*N*K for the GEMMs whatever the number
@@ -169,16 +173,18 @@ def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_t
     return staged
 
 
-def solve_step(staged, overlap=True):
+def solve_step(staged, overlap=True, inner=0):
     """Second half: scale search, factorisation, sweep and layout of the staged groups.
     overlap=False runs the jobs one after the other (per-kernel event times are then
-    exclusive)."""
+    exclusive).  inner > 0: quantize() works through a group in chunks of that many experts
+    (the runs with every expert through its Hessian: 256 permuted Hessians and factors of
+    205 MB each do not fit beside the layer)."""
     import torch
     cur = torch.cuda.current_stream()
     results = []
     for grp, stream, n in staged:
         with torch.cuda.stream(stream):
-            results.append(grp.quantize(chunk=n, overlap_scale_search=overlap))
+            results.append(grp.quantize(chunk=min(n, inner) if inner else n, overlap_scale_search=overlap))
         if not overlap:
             stream.synchronize()
     for s in STREAMS:
@@ -187,11 +193,11 @@ def solve_step(staged, overlap=True):
 
 
 def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128,
-             rows_route_tokens=None):
+             rows_route_tokens=None, inner=0):
     """One whole step (both halves) of the hot path."""
     return solve_step(stage_step(wl, cfg, chunk, step, mse=mse, factor_route=factor_route,
                                  low_rank_tokens=low_rank_tokens, rows_route_tokens=rows_route_tokens),
-                      overlap=overlap)
+                      overlap=overlap, inner=inner)
 
 
 def route_counts(wl, cfg, low_rank_tokens, rows_route_tokens):
@@ -216,17 +222,19 @@ def timed_steps(wl, cfg, chunk, steps, warmup, first_step=0, **kw):
     import torch
     for i in range(warmup):
         run_step(wl, cfg, chunk, first_step + i, **kw)
+    kw = dict(kw)
     torch.cuda.synchronize()
     # The K steps as a caller with a layer (or a model) of chunks would queue them: the Hessian
     # updates of chunk i+1 go onto the streams before the solve of chunk i, so that the solve of
     # chunk i+1 finds what it has to see on the host already there and its scale search starts
     # while the last sweeps of chunk i still run.  Every step's work is inside the timed region.
     overlap = kw.pop("overlap", True)
+    inner = kw.pop("inner", 0)
     t0 = time.perf_counter()
     staged = stage_step(wl, cfg, chunk, first_step + warmup, **kw) if steps else None
     for i in range(steps):
         ahead = stage_step(wl, cfg, chunk, first_step + warmup + i + 1, **kw) if i + 1 < steps else None
-        solve_step(staged, overlap=overlap)
+        solve_step(staged, overlap=overlap, inner=inner)
         staged = ahead
     torch.cuda.synchronize()
     return time.perf_counter() - t0
@@ -262,6 +270,24 @@ def measured_traffic(config, chunk, kernel):
         m = re.match(r"traffic\s+(\S+)\s+(\d+)\s+(\S+)\s+([0-9.eE+]+)", line.strip())
         if m and m.group(1) == config and int(m.group(2)) == chunk and m.group(3) == kernel:
             return float(m.group(4))
+    return None
+
+
+def measured_valu(config, chunk, kernel):
+    """What the vector ALU did in `kernel`, from the committed rocprofv3 --pmc summary of this
+    file's default command (a line `valu <config> <chunk> <kernel> <wave instructions per launch>
+    <issue fraction> <busy fraction>`), or None.  Issue fraction = SQ_INSTS_VALU / (active cycles
+    x 1024 SIMDs) / 0.25 (a SIMD takes four cycles per 64-lane instruction); busy fraction =
+    4 x SQ_ACTIVE_INST_VALU / (active cycles x 1024): above the issue fraction where
+    instructions take more than four cycles (the transcendentals take eight)."""
+    path = ROOT / "profiles" / f"bench_{config}_valu_pmc.txt"
+    if not path.exists():
+        return None
+    for line in path.read_text().splitlines():
+        m = re.match(r"valu\s+(\S+)\s+(\d+)\s+(\S+)\s+([0-9.eE+]+)\s+([0-9.]+)\s+([0-9.]+)", line.strip())
+        if m and m.group(1) == config and int(m.group(2)) == chunk and m.group(3) == kernel:
+            return dict(wave_instructions_per_launch=float(m.group(4)), issue_frac=float(m.group(5)),
+                        busy_frac=float(m.group(6)))
     return None
 
 
@@ -545,29 +571,40 @@ def main():
     # jobs run one after the other so that no kernel's time includes another stream's work
     stats = timing_pass(lambda: run_step(wl, cfg, chunk, a.warmup + a.steps, mse, overlap=False, **route))
     breakdown = kernel_table(stats)
-    # `roofline` describes the longest-running kernel among those that an HBM or a matrix-pipe
-    # roofline bounds; a kernel bound by the vector ALU (the shrink search, the in-block chains)
-    # has no such line and is reported under `kernels` / `mse_grid_search`
-    by_time = next(iter(breakdown))
-    dom = next(k for k, v in breakdown.items() if v["bound"] in ("mfma", "hbm"))
-    d = breakdown[dom]
-    bound, peak_key, executed = KERNEL_BOUND.get(dom, ("hbm", "hbm", 1.0))
-    roofline = dict(kernel=dom, bound="mfma" if bound == "mfma" else "hbm", achieved=d["rate"],
+    # `roofline` describes the kernel with the largest total time.  That is the shrink search,
+    # which neither an HBM nor a matrix-pipe roofline bounds: it reads every weight once and then
+    # evaluates 100 candidates on it in registers, so its line carries the nominal HBM rate (its
+    # algorithmic bytes / time) AND what the vector ALU did (counters of the committed profile).
+    # `roofline_matrix_pipe` is the same line for the longest kernel on the matrix pipe.
+    default_run = a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 128 \
+        and a.rows_route_tokens is None
+
+    def roofline_of(name):
+        d = breakdown[name]
+        bound, peak_key, executed = KERNEL_BOUND.get(name, ("hbm", "hbm", 1.0))
+        line = dict(kernel=name, bound=bound if bound in ("mfma", "valu") else "hbm", achieved=d["rate"],
                     peak=PEAK[peak_key], unit=d["rate_unit"], frac=d["frac"],
-                    traffic=measured_traffic(a.config, chunk, dom)
-                    if a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 128 else None,
-                    avg_launch_us=d["avg_us"], launches=d["launches"],
-                    note="achieved = algorithmic work (2*M*N*K counted once per fp32 product) / event time")
-    if by_time != dom:
-        roofline["longest_kernel"] = by_time
-        roofline["longest_kernel_note"] = (
-            f"{by_time} ({breakdown[by_time]['ms']} ms against {d['ms']} ms) is bound by the vector ALU: "
-            "neither roofline applies to it; see mse_grid_search")
-    if executed != 1.0:
-        roofline["executed_frac"] = d["executed_frac"]
-        roofline["executed_note"] = (f"every fp32 product is formed from {int(executed)} 16-bit piece products: "
+                    traffic=measured_traffic(a.config, chunk, name) if default_run else None,
+                    avg_launch_us=d["avg_us"], launches=d["launches"], share_of_kernel_time=d["share"])
+        if bound == "mfma":
+            line["note"] = "achieved = algorithmic work (2*M*N*K counted once per fp32 product) / event time"
+        if executed != 1.0:
+            line["executed_frac"] = d["executed_frac"]
+            line["executed_note"] = (f"every fp32 product is formed from {int(executed)} 16-bit piece products: "
                                      f"{executed:.0f} x achieved is what the matrix pipe executes; with random "
                                      "operands the pipe itself sustains what mfma_ceiling reports")
+        if bound == "valu":
+            line["note"] = ("bound by the vector ALU: `achieved` / `frac` are the kernel's algorithmic bytes over "
+                            "its time against the HBM peak (nominal); `valu` holds the counters")
+            valu = measured_valu(a.config, chunk, name) if default_run else None
+            if valu:
+                line["valu"] = valu
+        return line
+
+    by_time = next(iter(breakdown))
+    roofline = roofline_of(by_time)
+    dom = next((k for k, v in breakdown.items() if v["bound"] == "mfma"), None)
+    roofline_mfma = roofline_of(dom) if dom and dom != by_time else None
 
     out = {
         "metric": "experts quantized/sec (GPTQ 4-bit g128)",
@@ -588,6 +625,7 @@ def main():
                    "experts_by_route": route_counts(wl, cfg, a.low_rank_tokens if a.factor_route == "direct" else 0,
                                                     a.rows_route_tokens)},
         "roofline": roofline,
+        "roofline_matrix_pipe": roofline_mfma,
         "kernels": breakdown,
         "peak_device_memory_gb": round(peak_gb, 1),
     }
@@ -595,27 +633,38 @@ def main():
         # nominal candidate evaluations: P = 100 shrink factors for every weight of the step
         n_w = chunk * 3 * cfg["inter"] * cfg["hidden"]
         evals = 100.0 * n_w / (breakdown["mse_grid"]["ms"] * 1e-3)
-        out["mse_grid_search"] = dict(
-            candidate_evals_per_s=round(evals, 0),
-            frac_of_transcendental_rate=round(2.0 * evals / PEAK_TRANSCENDENTALS, 4),
-            note="nominal evaluations (100 candidates x weights) per second; each costs two "
-                 "transcendentals (v_log_f32, v_exp_f32); candidates dropped by the exact "
-                 "partial-sum pruning count as evaluated, so the fraction can exceed 1")
+        search = dict(
+            nominal_candidate_evals_per_s=round(evals, 0),
+            note="nominal = 100 candidates x weights; the exact pruning (partial sums and clipped "
+                 "extremes are lower bounds of a candidate's loss) leaves `executed_fraction` of them")
+        valu = measured_valu(a.config, chunk, "mse_grid") if default_run else None
+        if valu:
+            # an executed evaluation is 1060 vector instructions per 128-weight group (7 per
+            # weight, 129 additions, the candidate's own 35): lane instructions / 8.28
+            lane_instr = valu["wave_instructions_per_launch"] * 64 * breakdown["mse_grid"]["launches"]
+            executed = lane_instr / (1060.0 / 128.0)
+            search["executed_fraction"] = round(executed / (100.0 * n_w), 3)
+            search["executed_candidate_evals_per_s"] = round(executed / (breakdown["mse_grid"]["ms"] * 1e-3), 0)
+            # two transcendentals per executed evaluation
+            search["frac_of_transcendental_rate"] = round(
+                2.0 * search["executed_candidate_evals_per_s"] / PEAK_TRANSCENDENTALS, 4)
+        out["mse_grid_search"] = search
     if not a.no_extras:
         other = "inverse" if a.factor_route == "direct" else "direct"
-        dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route=other)
+        dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route=other, inner=64)
         out["reference_route" if other == "inverse" else "direct_route"] = dict(
             factor_route=other, ms_per_step=round(1e3 * dt / a.steps, 2),
             value=round(a.steps * chunk / dt, 3), unit="experts/s")
         if a.factor_route == "direct" and a.low_rank_tokens:
-            dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route="direct", low_rank_tokens=0)
+            dt = timed_steps(wl, cfg, chunk, a.steps, 1, mse=mse, factor_route="direct", low_rank_tokens=0,
+                             inner=64)
             dense = kernel_table(timing_pass(lambda: run_step(
-                wl, cfg, chunk, 0, mse, overlap=False, factor_route="direct", low_rank_tokens=0)))
+                wl, cfg, chunk, 0, mse, overlap=False, factor_route="direct", low_rank_tokens=0, inner=64)))
             out["every_expert_through_its_hessian"] = dict(
                 low_rank_tokens=0, ms_per_step=round(1e3 * dt / a.steps, 2),
                 value=round(a.steps * chunk / dt, 3), unit="experts/s",
-                note="the two three-product GEMMs with all of the step's experts in their batch "
-                     "(the default run leaves them the experts with more rows than low_rank_tokens)",
+                note="every expert through its Hessian, 64 experts per factorisation and sweep batch "
+                     "(the default run leaves that route the experts with more than 512 rows, 20 per layer)",
                 kernels={k: v for k, v in dense.items() if k.startswith("split_gemm")})
         out["hessian_buckets"] = hessian_buckets(cfg["hidden"], min(chunk, 64))
         out["hbm_kernels"] = hbm_kernels(wl)
