@@ -1,4 +1,6 @@
-// Matrix-pipe rate probe (benchmark helper, no counterpart in the reference).
+// Matrix-pipe rate probe: a benchmark helper of its own, built into libforge_probe.so beside
+// this file and loaded by bench.py only; not part of libforge_hip.so and of no use to a caller
+// of the library.
 //
 // The split GEMMs of this library run at about half of the published bf16 / fp16 matrix rate
 // although their matrix instructions are issued back to back.  This kernel measures what the
@@ -8,7 +10,8 @@
 // mantissa and several exponent bits toggle between consecutive instructions, as with real
 // weights); without, every operand is 1.0.  The difference between the two is the device's power
 // management, and the random-operand rate is the ceiling that a GEMM on real data can reach.
-#include "common.h"
+#include <hip/hip_runtime.h>
+#include <cstdint>
 
 namespace {
 
@@ -72,21 +75,19 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int random_bi
 
 }  // namespace
 
-extern "C" int64_t forge_mfma_rate_probe_sink_floats(int workgroups) {
+// sink: probe_sink_floats(workgroups) floats of device memory.  *flops receives the work of the
+// launch; the caller times it with events on `stream`.  Returns 0, or 1 for a bad argument or a
+// failed launch.
+extern "C" int64_t probe_sink_floats(int workgroups) {
     return workgroups > 0 ? (int64_t)workgroups * 256 : 0;
 }
 
-extern "C" int forge_mfma_rate_probe(int f16, int random_bits, int iters, int workgroups, float* sink,
-                                     double* flops, forge_stream_t stream) {
-    FORGE_REQUIRE(iters >= 1 && iters <= (1 << 24) && workgroups >= 1 && workgroups <= 65535, "bad size");
-    FORGE_REQUIRE(sink && flops, "null pointer");
+extern "C" int probe_mfma_rate(int f16, int random_bits, int iters, int workgroups, float* sink,
+                               double* flops, void* stream) {
+    if (iters < 1 || iters > (1 << 24) || workgroups < 1 || workgroups > 65535 || !sink || !flops) return 1;
     hipStream_t st = (hipStream_t)stream;
     *flops = 2.0 * 32 * 32 * 16 * kProbeAcc * (double)iters * 4.0 * (double)workgroups;
-    forge::KernelTiming timing(f16 ? (random_bits ? "mfma_rate_f16_random" : "mfma_rate_f16_ones")
-                                   : (random_bits ? "mfma_rate_bf16_random" : "mfma_rate_bf16_ones"),
-                               st, *flops, forge::WORK_FLOPS);
     if (f16) mfma_rate_kernel<true><<<dim3((unsigned)workgroups), dim3(256), 0, st>>>(iters, random_bits, sink);
     else mfma_rate_kernel<false><<<dim3((unsigned)workgroups), dim3(256), 0, st>>>(iters, random_bits, sink);
-    FORGE_LAUNCH_CHECK();
-    return FORGE_OK;
+    return hipGetLastError() == hipSuccess ? 0 : 1;
 }

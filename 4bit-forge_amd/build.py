@@ -19,6 +19,9 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 CSRC = ROOT / "csrc"
 OUT = CSRC / "libforge_hip.so"
+# bench.py's matrix-pipe rate probe: a library of its own, not part of the product
+PROBE_SRC = ROOT / "bench_probe" / "mfma_rate_probe.hip"
+PROBE_OUT = ROOT / "bench_probe" / "libforge_probe.so"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # -ffp-contract=off: every fused multiply-add in the kernels is written explicitly, so
@@ -148,6 +151,15 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
                and (u["scratch"] or u["vgpr_spill"])]
     if spilled:
         raise RuntimeError("kernels that must stay in registers use scratch memory:\n  " + "\n  ".join(spilled))
+    if PROBE_SRC.exists() and (force or _stale(PROBE_OUT, [PROBE_SRC])):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", str(PROBE_SRC), "-o", str(PROBE_OUT)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            print(r.stdout + r.stderr, file=sys.stderr)
+            raise RuntimeError("hipcc failed on the bench probe")
+        if verbose:
+            print(f"[build] built {PROBE_OUT}")
     if todo or force or not OUT.exists():
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
         subprocess.run(cmd, check=True)

@@ -36,8 +36,6 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_last_error": ([], ctypes.c_char_p),
         "forge_kernel_timing_enable": ([i32], i32),
         "forge_kernel_timing_collect": ([], i32),
-        "forge_mfma_rate_probe": ([i32, i32, i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp], i32),
-        "forge_mfma_rate_probe_sink_floats": ([i32], i64),
         "forge_kernel_timing_get": ([i32, ctypes.c_char_p, i32, ctypes.POINTER(i64),
                                      ctypes.POINTER(ctypes.c_double),
                                      ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i32)], i32),
@@ -107,8 +105,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
 
 EXPORTED_SYMBOLS = (
     "forge_hip_abi_version", "forge_last_error", "forge_kernel_timing_enable",
-    "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_mfma_rate_probe",
-    "forge_mfma_rate_probe_sink_floats", "forge_set_option",
+    "forge_kernel_timing_collect", "forge_kernel_timing_get", "forge_set_option",
     "forge_get_option", "forge_build_group_meta_packed",
     "forge_mse_scale_groups_packed", "forge_quant_grid", "forge_gptq_solver",
     "forge_sparsegptq14_solver", "forge_gptq_sweep_batched", "forge_gptq_sweep_direct_batched",
@@ -208,20 +205,6 @@ class _HipKernels:
                                             unit="flop" if kind.value == 0 else "byte")
         return out
 
-    def mfma_rate_probe(self, f16: bool, random_bits: bool, iters: int = 20000, workgroups: int = 512,
-                        device="cuda"):
-        """Launches the matrix-pipe rate probe once (forge_mfma_rate_probe) and returns the
-        flops of the launch; time it with timing_enable / timing_collect."""
-        n = int(self._lib.forge_mfma_rate_probe_sink_floats(int(workgroups)))
-        sink = torch.empty(n, dtype=torch.float32, device=device)
-        flops = ctypes.c_double()
-        with torch.cuda.device(sink.device):
-            self._check(self._lib.forge_mfma_rate_probe(int(bool(f16)), int(bool(random_bits)), int(iters),
-                                                        int(workgroups), _ptr(sink), ctypes.byref(flops),
-                                                        _stream()))
-        return flops.value
-
-    # -- reference-signature operators -------------------------------------------------
     def build_group_meta_packed(self, X, bit_width, symmetric):
         _need_cuda(X)
         if X.dtype != torch.float32 or not X.is_contiguous() or X.dim() != 2:

@@ -336,19 +336,42 @@ def hessian_buckets(C=7168, E=64):
 
 
 def mfma_ceiling():
-    """What the matrix pipe itself sustains on this device (forge_mfma_rate_probe: back-to-back
-    32x32x16 matrix instructions from registers, nothing else): with operands of ones, and with
-    pseudo-random operands, whose toggling bits make the device's power management slow the
-    pipe.  The random-operand rate is the ceiling of any GEMM on real data."""
-    from forge.backend.hip import kernels
+    """What the matrix pipe itself sustains on this device (4bit-forge_amd/bench_probe: back-to-back
+    32x32x16 matrix instructions from registers, nothing else; a helper library of this
+    benchmark, not part of the product): with operands of ones, and with pseudo-random operands,
+    whose toggling bits make the device's power management slow the pipe.  The random-operand
+    rate is the ceiling of any GEMM on real data.  Timed with events on the launch stream."""
+    import ctypes
+    import torch
+    path = ROOT / "4bit-forge_amd" / "bench_probe" / "libforge_probe.so"
+    if not path.exists():
+        return dict(note=f"{path.name} is not built (python 4bit-forge_amd/build.py)")
+    lib = ctypes.CDLL(str(path))
+    lib.probe_sink_floats.restype = ctypes.c_int64
+    lib.probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                    ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    wgs, iters = 512, 20000
+    sink = torch.empty(int(lib.probe_sink_floats(wgs)), dtype=torch.float32, device="cuda")
+    flops = ctypes.c_double()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def launch(f16, rnd):
+        rc = lib.probe_mfma_rate(int(f16), int(rnd), iters, wgs, ctypes.c_void_p(sink.data_ptr()),
+                                 ctypes.byref(flops), stream)
+        assert rc == 0, "probe launch failed"
+
     out = {}
     for name, f16, rnd in (("bf16_ones", False, False), ("bf16_random", False, True),
                            ("f16_ones", True, False), ("f16_random", True, True)):
-        kernels.mfma_rate_probe(f16, rnd)                                          # warm-up
-        stats = timing_pass(lambda: [kernels.mfma_rate_probe(f16, rnd) for _ in range(3)])
-        s = stats["mfma_rate_" + name]
-        out[name] = dict(tflops=round(s["work"] / s["ms"] / 1e9, 1),
-                         frac_of_published_peak=round(s["work"] / s["ms"] / 1e9 / PEAK["mfma_bf16"], 4))
+        launch(f16, rnd)                                                          # warm-up
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(3):
+            launch(f16, rnd)
+        t1.record()
+        t1.synchronize()
+        tflops = 3 * flops.value / (t0.elapsed_time(t1) * 1e-3) / 1e12
+        out[name] = dict(tflops=round(tflops, 1), frac_of_published_peak=round(tflops / PEAK["mfma_bf16"], 4))
     out["note"] = ("executed TFLOP/s of v_mfma_f32_32x32x16 issued back to back from registers on "
                    "every CU, ~7 ms per launch; published peak 2500")
     return out

@@ -48,18 +48,6 @@ int forge_kernel_timing_collect(void);
 int forge_kernel_timing_get(int index, char* name, int name_cap, int64_t* launches,
                             double* total_ms, double* work, int* work_kind);
 
-/* Matrix-pipe rate probe, for benchmarks (no counterpart in the reference): `workgroups`
- * workgroups of four wavefronts issue `iters` x 8 v_mfma_f32_32x32x16 (bf16, or fp16 when f16 != 0)
- * each, on independent accumulators, from operands held in registers; random_bits != 0 fills the
- * operands with pseudo-random numbers in (-1, 1), 0 with ones.  *flops receives the work of the
- * launch; time it with events on `stream` (or through forge_kernel_timing_*: names
- * mfma_rate_{bf16,f16}_{random,ones}).  sink: forge_mfma_rate_probe_sink_floats(workgroups)
- * floats of device memory.  What the pipe sustains with random operands is the ceiling for any
- * GEMM on real data on that device. */
-int forge_mfma_rate_probe(int f16, int random_bits, int iters, int workgroups, float* sink,
-                          double* flops, forge_stream_t stream);
-int64_t forge_mfma_rate_probe_sink_floats(int workgroups);
-
 /* Library-wide settings; no counterpart in the reference.  Each starts from an environment
  * variable that is read once, when the library is loaded, and is changed afterwards only
  * through forge_set_option (an atomic store; a launch reads the value it finds).

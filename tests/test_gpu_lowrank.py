@@ -366,3 +366,4 @@ def test_rows_kept_in_f32_are_not_rounded_when_an_expert_leaves_the_route():
         assert ((H - want).norm() / want.norm()).item() < 2e-6, lim
     rounded = torch.cat([first.bfloat16().double(), later.double()])
     assert (((2.0 / 40) * rounded.t() @ rounded - want).norm() / want.norm()).item() > 1e-4
+
