@@ -67,7 +67,7 @@ class ExpertGroupGPTQ:
                  symmetric: bool = False, quantization_scale: str = "mse",
                  quantization_order: str = "activation", rel_damp: float = 1e-2,
                  algorithm: str = "gptq", device=None, factor_route: str = "direct",
-                 low_rank_tokens: int = 128, rows_route_tokens: Optional[int] = None):
+                 low_rank_tokens: Optional[int] = None, rows_route_tokens: Optional[int] = None):
         """weights: stacks [E, R_i, C] (bf16 or f32) that share the input features C.
         algorithm: "gptq", "sparsegptq" (1:4 joint solve; quantize() then also returns the
         keep-masks M [E, ceil(C/32), R_i] u32 per stack) or "babai".
@@ -79,10 +79,12 @@ class ExpertGroupGPTQ:
         near-tie.
         low_rank_tokens (0..128; algorithm "gptq" on the direct route, C a multiple of 16):
         experts with at most this many calibration rows are solved from the rows themselves,
-        see the module text; 0 = every expert through its Hessian.  At 65-128 rows the per-row
-        vector sweep costs nearly what the route through the Hessian costs (measured: 1 % of a
-        benchmark step in its favour).  Such an expert has no stored Hessian: read Hessians
-        through ``hessian(e)``.
+        see the module text; 0 = every expert through its Hessian.  None = 64 where the blocked
+        closed form can take over from there (rows_route_tokens), else 128: at 65-128 rows the
+        per-row-vector sweep, which runs on the vector ALU, costs more than the blocked form's
+        matrix products and in-block chains (benchmark layer: 230.7 ms a step with 128, 223.7
+        with 64, 228.1 with 32).  Such an expert has no stored Hessian: read Hessians through
+        ``hessian(e)``.
         rows_route_tokens (needs low_rank_tokens > 0, C and every R a multiple of 128): experts
         with more rows than low_rank_tokens and at most this many, rounded up to a multiple of
         128, are solved from their rows by the blocked closed form, as long as that count times
@@ -117,16 +119,18 @@ class ExpertGroupGPTQ:
         self._slot = [-1] * self.E
         self._slot_expert: List[int] = []
         self.num_samples = [0] * self.E                 # host-side counts
-        if not 0 <= int(low_rank_tokens) <= 128:
+        if low_rank_tokens is not None and not 0 <= int(low_rank_tokens) <= 128:
             raise ValueError(f"low_rank_tokens={low_rank_tokens}: 0..128")
         ok = algorithm == "gptq" and factor_route == "direct" and self.C % 16 == 0 \
             and len({w.dtype for w in self.W}) == 1
-        self.low_rank_tokens = int(low_rank_tokens) if ok else 0
-        rows_ok = self.low_rank_tokens > 0 and self.C % 128 == 0 and all(w.shape[1] % 128 == 0 for w in self.W)
+        rows_ok = ok and low_rank_tokens != 0 and self.C % 128 == 0 and all(w.shape[1] % 128 == 0 for w in self.W)
         want = 512 if rows_route_tokens is None else int(rows_route_tokens)
         if want < 0 or want % 128 != 0:
             raise ValueError(f"rows_route_tokens={rows_route_tokens}: a multiple of 128")
         self.rows_route_tokens = min(want, self.C // self.ROWS_ROUTE_COST // 128 * 128) if rows_ok else 0
+        if low_rank_tokens is None:
+            low_rank_tokens = 64 if self.rows_route_tokens >= 128 else 128
+        self.low_rank_tokens = int(low_rank_tokens) if ok else 0
         if self.rows_route_tokens <= self.low_rank_tokens:
             self.rows_route_tokens = 0
         # experts on the blocked route: rows_route[e], their rows as they came (a list of [k, C]

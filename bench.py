@@ -10,10 +10,11 @@ forge.synth.deepseek_v3_moe (seed 0) on the GPU.  One STEP = one pass of the hot
 one chunk of experts, everything already resident in HBM: ragged Hessian accumulation for
 gate/up and for down, then per expert two factorisations (gate and up share theirs), three
 scale searches and three sweeps.  A step is the layer's 256 experts (--chunk 128: half of
-them, successive steps then walk through the layer chunk by chunk).  Experts with at most 128
+them, successive steps then walk through the layer chunk by chunk).  Experts with at most 64
 routed rows (most of them: 8192 tokens over 256 experts with Zipf popularity) take the
 library's low-rank route, which reaches the same result from the rows themselves without a
-C x C Hessian, those with up to 512 its blocked form; `config.experts_by_route` counts them.
+C x C Hessian, those with up to 512 (256 for down_proj) its blocked form;
+`config.experts_by_route` counts them.
 The timed steps are queued as a caller with a layer of chunks would queue them: chunk i+1's
 Hessian updates go onto the streams before chunk i's solve (all K updates and all K solves lie
 inside the timed region).
@@ -121,7 +122,7 @@ def make_workload(name, cfg, chunk, seed=0):
 STREAMS = []
 
 
-def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_tokens=128,
+def stage_step(wl, cfg, chunk, step, mse=True, factor_route="direct", low_rank_tokens=64,
                rows_route_tokens=None):
     """First half of the hot path for experts [step*chunk, (step+1)*chunk) of the layer: the
     expert groups, their Hessian updates and the look at the result that the solve starts from
@@ -192,7 +193,7 @@ def solve_step(staged, overlap=True, inner=0):
     return results[0::2], results[1::2]
 
 
-def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=128,
+def run_step(wl, cfg, chunk, step, mse=True, overlap=True, factor_route="direct", low_rank_tokens=64,
              rows_route_tokens=None, inner=0):
     """One whole step (both halves) of the hot path."""
     return solve_step(stage_step(wl, cfg, chunk, step, mse=mse, factor_route=factor_route,
@@ -553,9 +554,9 @@ def main():
     ap.add_argument("--factor-route", default="direct", choices=["direct", "inverse"],
                     help="direct (default): sweep fed by the factor of H itself; inverse: the "
                          "reference's factor of inv(H) and fp32-chain sweep")
-    ap.add_argument("--low-rank-tokens", type=int, default=128,
-                    help="experts with at most this many routed rows are solved from the rows themselves "
-                         "(0: every expert through its Hessian)")
+    ap.add_argument("--low-rank-tokens", type=int, default=64,
+                    help="experts with at most this many routed rows are solved from the rows themselves, "
+                         "column by column (0: every expert through its Hessian)")
     ap.add_argument("--rows-route-tokens", type=int, default=None,
                     help="experts with more rows than --low-rank-tokens and at most this many (a multiple "
                          "of 128) take the blocked closed form while it is cheaper than the route through "
@@ -599,7 +600,7 @@ def main():
     # evaluates 100 candidates on it in registers, so its line carries the nominal HBM rate (its
     # algorithmic bytes / time) AND what the vector ALU did (counters of the committed profile).
     # `roofline_matrix_pipe` is the same line for the longest kernel on the matrix pipe.
-    default_run = a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 128 \
+    default_run = a.split == 1 and a.factor_route == "direct" and mse and a.low_rank_tokens == 64 \
         and a.rows_route_tokens is None
 
     def roofline_of(name):

@@ -2,8 +2,9 @@
 
 One ``ExpertGroupGPTQ.quantize()`` call per projection carries experts of every kind that a
 step of the benchmark layer holds: experts without a single routed row (plain rounding),
-with 3 .. 128 rows (solved from the rows, all sizes of the per-row-vector sweep in ONE mixed
-launch), with 200 rows (the blocked closed form) and with 1536 (through the Hessian).  gate_proj
+with 3 .. 64 rows (solved from the rows, the sizes of the per-row-vector sweep in ONE mixed
+launch), with 100, 128 and 200 rows (the blocked closed form, sizes 128 and 256 in one batch)
+and with 1536 (through the Hessian).  gate_proj
 and up_proj are two stacks that share one factor (C = 7168; 128 of their 2048 rows each, rows
 being independent); down_proj has its full shape, R = 7168, C = 2048.  Every expert is then
 compared with ``oracle.GPTQ`` (forge/gptq.py:128-139 on the handles that quant.py:386-396
@@ -29,7 +30,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 KW = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
           quantization_order="activation", rel_damp=0.01)
-#        rows each expert saw: none, the per-row-vector sizes 4/16/32/64/128, then beyond
+#        rows each expert saw: none, the per-row-vector sizes 4/16/32/64, then beyond
 NS = (0, 3, 16, 40, 100, 128, 200, 1536, 0, 64, 128, 5)
 # experts compared with the oracle (a CPU solve and the floor's realisations at C = 7168 take
 # about a minute each; the others add to the batch and to the mixed launch's sizes)
@@ -51,7 +52,7 @@ def gate_up():
                       for _ in range(E)]) for _ in range(2)]
     xs = _rows(32, C)
     offs = np.concatenate([[0], np.cumsum(NS)]).tolist()
-    grp = ExpertGroupGPTQ([w.to(DEV) for w in W], device=DEV, rows_route_tokens=1024, **KW)
+    grp = ExpertGroupGPTQ([w.to(DEV) for w in W], device=DEV, **KW)
     grp.update(torch.cat(xs).to(DEV), offs)
     outs = [tuple(t.cpu() for t in o) for o in grp.quantize(chunk=E)]
     assert not grp.issue_non_invertible.any()
@@ -70,7 +71,7 @@ def down():
                      for _ in range(E)])
     xs = _rows(34, C)
     offs = np.concatenate([[0], np.cumsum(NS)]).tolist()
-    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, rows_route_tokens=1024, **KW)
+    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, **KW)
     grp.update(torch.cat(xs).to(DEV), offs)
     outs = [tuple(t.cpu() for t in o) for o in grp.quantize(chunk=E)]
     assert not grp.issue_non_invertible.any()
@@ -110,12 +111,13 @@ def _against_the_oracle(tag, W, X, q, s, z):
 
 
 def test_routes_taken(gate_up, down):
-    """What the step is meant to mix in one call: experts without rows and with few rows solved
-    from the rows themselves, the expert with 200 rows by the blocked closed form (256 x 7 does
-    not exceed 2048 nor 7168), the one with 1536 rows through its Hessian."""
+    """What the step is meant to mix in one call: experts without rows and with up to 64 rows
+    solved from the rows themselves column by column, those with 100, 128 and 200 rows by the
+    blocked closed form (256 x 7 does not exceed 2048 nor 7168), the one with 1536 rows through
+    its Hessian."""
     for _, _, _, (low, blocked) in (gate_up, down):
-        assert low == [n <= 128 for n in NS]
-        assert blocked == [n == 200 for n in NS]
+        assert low == [n <= 64 for n in NS]
+        assert blocked == [64 < n <= 256 for n in NS]
 
 
 @pytest.mark.parametrize("e", GATE_UP_CASES)

@@ -457,12 +457,18 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     # it, so that this is the arithmetic the benchmark times
     kernels.set_option("sweep_schedule", 1)
     try:
-        for route in ("inverse", "direct"):
-            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **kw)
+        # (128 rows: the default takes the blocked closed form from 65 rows on; with
+        # low_rank_tokens=128 the column-by-column form with eight lanes per row of the sweep)
+        variants = [("inverse", {}), ("direct", {})] + ([("direct", dict(low_rank_tokens=128))] if n_tokens == 128 else [])
+        for route, extra in variants:
+            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **extra, **kw)
             grp.update(X.to(DEV), [0, n_tokens])
             (q, s, z), = grp.quantize(chunk=1)
             assert not grp.issue_non_invertible.any()
-            check(f"batched {route}", q[0], s[0], z[0])
+            if route == "direct":
+                assert grp.low_rank == [n_tokens <= (extra.get("low_rank_tokens", 64))]
+                assert grp.rows_route == [extra.get("low_rank_tokens", 64) < n_tokens <= 512]
+            check(f"batched {route} {extra}", q[0], s[0], z[0])
             del grp
     finally:
         kernels.set_option("sweep_schedule", 0)
