@@ -51,6 +51,9 @@ struct GemmArgs {
     // are skipped; the host still sizes the grid for the largest matrix.
     const int32_t* lim;
     bool lim_k, lim_m, lim_n;
+    // with lim: the share of the nominal 2*M*N*K (largest matrix's sizes times the batch) that
+    // the batch's own sizes amount to, for the timing records' work figure; 0 = all of it
+    double work_frac;
     // filled in by launch_chain_gemm
     int n_tiles, m_tiles;
     bool xcd_map;

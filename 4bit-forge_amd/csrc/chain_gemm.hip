@@ -1101,7 +1101,7 @@ Prepared prepare(const GemmArgs& g_in, int64_t batch) {
         const int ncols = (g.n1 - nt) < TN ? (g.n1 - nt) : TN;
         if (k1 > k0) kn += (double)(k1 - k0) * ncols;
     }
-    p.flops = 2.0 * (g.m1 - g.m0) * kn * (double)batch;
+    p.flops = 2.0 * (g.m1 - g.m0) * kn * (double)batch * (g.work_frac > 0.0 ? g.work_frac : 1.0);
     return p;
 }
 

@@ -687,9 +687,9 @@ extern "C" int64_t forge_rows_factor_workspace_bytes(int64_t batch, int64_t C, i
 }
 
 extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const int32_t* n_rows,
-                                         float* HmT, float* V, int32_t* info, int64_t batch, int64_t C,
-                                         int64_t nmax, void* ws, int64_t ws_bytes,
-                                         forge_stream_t stream) {
+                                         const int32_t* n_rows_host, float* HmT, float* V, int32_t* info,
+                                         int64_t batch, int64_t C, int64_t nmax, void* ws,
+                                         int64_t ws_bytes, forge_stream_t stream) {
     FORGE_REQUIRE(batch >= 0 && batch < 65536 && C >= NB && C < (1 << 22) && C % NB == 0,
                   "bad shape batch=%lld C=%lld (C: a multiple of 128)", (long long)batch, (long long)C);
     FORGE_REQUIRE(nmax >= NB && nmax <= 4096 && nmax % NB == 0, "nmax=%lld: a multiple of 128 up to 4096",
@@ -720,6 +720,18 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
     FORGE_LAUNCH_CHECK();
 
     const int n = (int)nmax;
+    // (for the timing records only: what the batch's own sizes leave of the nominal work)
+    double f1 = 1.0, f2 = 1.0;
+    if (n_rows_host) {
+        f1 = f2 = 0.0;
+        for (int64_t b = 0; b < batch; ++b) {
+            FORGE_REQUIRE(n_rows_host[b] >= NB && n_rows_host[b] <= nmax && n_rows_host[b] % NB == 0,
+                          "n_rows[%lld]=%d: a multiple of 128 up to nmax", (long long)b, n_rows_host[b]);
+            const double r = (double)n_rows_host[b] / (double)nmax;
+            f1 += r / (double)batch;
+            f2 += r * r / (double)batch;
+        }
+    }
     for (int64_t c0 = C - NB; c0 >= 0; c0 -= NB) {
         // Y = S B_J and its transpose (each is an operand of a later product in that layout)
         forge::GemmArgs ya{}, yb{};
@@ -727,12 +739,12 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
         ya.At = S; ya.lda = nmax; ya.as = nmax * nmax;
         ya.Bm = BT + c0; ya.ldb = C; ya.bs = nmax * C;
         ya.m1 = n; ya.n1 = NB; ya.k1 = n; ya.init_zero = true; ya.blocked_sum = true;
-        ya.lim = n_rows; ya.lim_m = ya.lim_k = true;
+        ya.lim = n_rows; ya.lim_m = ya.lim_k = true; ya.work_frac = f2;
         yb.X = YT; yb.ldx = nmax; yb.xs = nmax * NB;
         yb.At = BT + c0; yb.lda = C; yb.as = nmax * C;
         yb.Bm = S; yb.ldb = nmax; yb.bs = nmax * nmax;
         yb.m1 = NB; yb.n1 = n; yb.k1 = n; yb.init_zero = true; yb.blocked_sum = true;
-        yb.lim = n_rows; yb.lim_n = yb.lim_k = true;
+        yb.lim = n_rows; yb.lim_n = yb.lim_k = true; yb.work_frac = f2;
         if (int e = forge::launch_chain_gemm_pair(ya, yb, batch, st)) return e;
         // T = D_J + B_J^T Y
         forge::GemmArgs t{};
@@ -740,7 +752,7 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
         t.At = BT + c0; t.lda = C; t.as = nmax * C;
         t.Bm = Y; t.ldb = NB; t.bs = nmax * NB;
         t.m1 = NB; t.n1 = NB; t.k1 = n; t.blocked_sum = true;
-        t.lim = n_rows; t.lim_k = true;
+        t.lim = n_rows; t.lim_k = true; t.work_frac = f1;
         if (int e = forge::launch_chain_gemm(t, batch, st)) return e;
         // T = M^T M, Z = M^-1
         {
@@ -759,12 +771,12 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
         ga.At = Z; ga.lda = NB; ga.as = NB * NB;
         ga.Bm = YT; ga.ldb = nmax; ga.bs = nmax * NB;
         ga.m1 = NB; ga.n1 = n; ga.k1 = NB; ga.init_zero = true; ga.blocked_sum = true;
-        ga.lim = n_rows; ga.lim_n = true;
+        ga.lim = n_rows; ga.lim_n = true; ga.work_frac = f1;
         gb.X = HmT + c0; gb.ldx = C; gb.xs = nmax * C;
         gb.At = YT; gb.lda = nmax; gb.as = nmax * NB;
         gb.Bm = Zs; gb.ldb = NB; gb.bs = NB * NB;
         gb.m1 = n; gb.n1 = NB; gb.k1 = NB; gb.init_zero = true; gb.blocked_sum = true;
-        gb.lim = n_rows; gb.lim_m = true;
+        gb.lim = n_rows; gb.lim_m = true; gb.work_frac = f1;
         if (int e = forge::launch_chain_gemm_pair(ga, gb, batch, st)) return e;
         // S -= G G^T
         if (c0 > 0) {
@@ -773,7 +785,7 @@ extern "C" int forge_rows_factor_blocked(const float* BT, const float* D, const 
             s.At = GT; s.lda = nmax; s.as = nmax * NB;
             s.Bm = GT; s.ldb = nmax; s.bs = nmax * NB;
             s.m1 = n; s.n1 = n; s.k1 = NB; s.negate_a = true; s.blocked_sum = true;
-            s.lim = n_rows; s.lim_m = s.lim_n = true;
+            s.lim = n_rows; s.lim_m = s.lim_n = true; s.work_frac = f2;
             if (int e = forge::launch_chain_gemm(s, batch, st)) return e;
         }
     }

@@ -789,7 +789,8 @@ extern "C" int64_t forge_gptq_sweep_rows_workspace_bytes(int64_t batch, int64_t 
 
 extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dtype, const float* HmT,
                                              const float* Bp, const float* V, const int32_t* n_rows,
-                                             const float* scalesT, const float* qzerosT,
+                                             const int32_t* n_rows_host, const float* scalesT,
+                                             const float* qzerosT,
                                              const int32_t* g_idx, uint8_t* qweight, int64_t batch,
                                              int64_t C, int64_t R, int64_t G, int bits, int64_t nmax,
                                              void* ws, int64_t ws_bytes, forge_stream_t stream) {
@@ -806,6 +807,15 @@ extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dt
     FORGE_REQUIRE(ws_bytes >= forge_gptq_sweep_rows_workspace_bytes(batch, R, nmax), "workspace too small");
     hipStream_t st = (hipStream_t)stream;
     float* A = (float*)ws;
+    double f1 = 1.0;         // for the timing records only: the batch's own share of the nominal work
+    if (n_rows_host) {
+        f1 = 0.0;
+        for (int64_t b = 0; b < batch; ++b) {
+            FORGE_REQUIRE(n_rows_host[b] >= 128 && n_rows_host[b] <= nmax && n_rows_host[b] % 128 == 0,
+                          "n_rows[%lld]=%d: a multiple of 128 up to nmax", (long long)b, n_rows_host[b]);
+            f1 += (double)n_rows_host[b] / (double)nmax / (double)batch;
+        }
+    }
     void* split_ws = (char*)ws + (batch * nmax * R * (int64_t)sizeof(float) + 255) / 256 * 256;
     const int64_t split_bytes = forge::split_gemm_workspace_bytes(batch, nmax);
     const bool w0_bf16 = w0_dtype == FORGE_BF16;
@@ -823,7 +833,7 @@ extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dt
             g.blocked_sum = true;
             g.products = 3;
             g.x_init = W0; g.x_init_bf16 = w0_bf16;
-            g.lim = n_rows; g.lim_k = true;
+            g.lim = n_rows; g.lim_k = true; g.work_frac = f1;
             if (int e = forge::launch_chain_gemm_pair(g, forge::GemmArgs{}, batch, st, split_ws, split_bytes))
                 return e;
         }
@@ -843,7 +853,7 @@ extern "C" int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dt
             g.m1 = (int)nmax; g.n1 = (int)R; g.k0 = (int)start; g.k1 = (int)(start + forge::kBW);
             g.init_zero = start == 0;
             g.blocked_sum = true;
-            g.lim = n_rows; g.lim_m = true;
+            g.lim = n_rows; g.lim_m = true; g.work_frac = f1;
             if (int e = forge::launch_chain_gemm(g, batch, st)) return e;
         }
     }

@@ -69,9 +69,9 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_codes_to_layer_order_scatter": ([vp, i64, i64, vp, vp, vp, i64, i64, i64, vp], i32),
         "forge_gptq_sweep_lowrank": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i64,
                                       vp], i32),
-        "forge_rows_factor_blocked": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, vp, i64, vp], i32),
+        "forge_rows_factor_blocked": ([vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, vp, i64, vp], i32),
         "forge_rows_factor_workspace_bytes": ([i64, i64, i64], i64),
-        "forge_gptq_sweep_rows_blocked": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
+        "forge_gptq_sweep_rows_blocked": ([vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                            i32, i64, vp, i64, vp], i32),
         "forge_gptq_sweep_rows_workspace_bytes": ([i64, i64, i64], i64),
         "forge_hessian_update_static": ([vp, i32, i64, i64, i64, f32, f32, vp, vp], i32),
@@ -500,11 +500,12 @@ class _HipKernels:
               "sweep_rows": self._lib.forge_gptq_sweep_rows_workspace_bytes}[what]
         return int(fn(*[int(d) for d in dims]))
 
-    def rows_factor_blocked(self, BT, D, n_rows):
+    def rows_factor_blocked(self, BT, D, n_rows, n_rows_host=None):
         """BT [B,nmax,C] f32 (row j = sqrt(2/n) x_j in solver order, zero rows beyond a matrix's own),
         D [B,C] f32, n_rows [B] int32 on the device (each a multiple of 128, <= nmax) ->
         (HmT [B,nmax,C], V [B,C,128], info [B] i32): the factor of D + BT^T BT as the blocked
-        sweep reads it (see forge_rows_factor_blocked in forge_hip.h)."""
+        sweep reads it (see forge_rows_factor_blocked in forge_hip.h).  n_rows_host: the same
+        numbers as a host list (only the timing records' work figures use them)."""
         _need_cuda(BT, D, n_rows)
         B, nmax, C = BT.shape
         assert BT.is_contiguous() and BT.dtype == torch.float32 and nmax % 128 == 0 and C % 128 == 0
@@ -516,12 +517,14 @@ class _HipKernels:
         nbytes = int(self._lib.forge_rows_factor_workspace_bytes(B, C, nmax))
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=BT.device)
         with torch.cuda.device(BT.device):
-            self._check(self._lib.forge_rows_factor_blocked(_ptr(BT), _ptr(D), _ptr(n_rows), _ptr(HmT),
+            nh = (ctypes.c_int32 * B)(*[int(n) for n in n_rows_host]) if n_rows_host is not None else None
+            self._check(self._lib.forge_rows_factor_blocked(_ptr(BT), _ptr(D), _ptr(n_rows), nh, _ptr(HmT),
                                                             _ptr(V), _ptr(info), B, C, nmax, _ptr(ws),
                                                             nbytes, _stream()))
         return HmT, V, info
 
-    def gptq_sweep_rows_blocked(self, X, W0, HmT, Bp, V, n_rows, scalesT, qzerosT, g_idx, bits):
+    def gptq_sweep_rows_blocked(self, X, W0, HmT, Bp, V, n_rows, scalesT, qzerosT, g_idx, bits,
+                                n_rows_host=None):
         """X [B,C,R] f32 (weights in solver order; displacements on return), W0 the same untouched
         (f32/bf16), HmT [B,nmax,C], Bp [B,C,nmax], V [B,C,128], n_rows [B] i32 (device),
         scalesT/qzerosT [B,G,R], g_idx [B,C] i32 -> codes [B,C,R] u8."""
@@ -541,8 +544,9 @@ class _HipKernels:
         nbytes = int(self._lib.forge_gptq_sweep_rows_workspace_bytes(B, R, nmax))
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=X.device)
         with torch.cuda.device(X.device):
+            nh = (ctypes.c_int32 * B)(*[int(n) for n in n_rows_host]) if n_rows_host is not None else None
             self._check(self._lib.forge_gptq_sweep_rows_blocked(
-                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(HmT), _ptr(Bp), _ptr(V), _ptr(n_rows),
+                _ptr(X), _ptr(W0), _dtype_code(W0), _ptr(HmT), _ptr(Bp), _ptr(V), _ptr(n_rows), nh,
                 _ptr(scalesT), _ptr(qzerosT), _ptr(g_idx), _ptr(q), B, C, R, G, int(bits), nmax,
                 _ptr(ws), nbytes, _stream()))
         return q

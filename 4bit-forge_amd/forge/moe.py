@@ -597,7 +597,8 @@ class ExpertGroupGPTQ:
                         msk = mask[ri].bool()                               # [Br, C], solver order
                         n_own = [self.num_samples[e0 + i] for i in rr_ids]
                         nmax = max((n + 127) // 128 * 128 for n in n_own)
-                        n_rows = self._dev([(n + 127) // 128 * 128 for n in n_own], dtype=torch.int32)
+                        n_pad = [(n + 127) // 128 * 128 for n in n_own]
+                        n_rows = self._dev(n_pad, dtype=torch.int32)
                         BT = torch.zeros((len(rr_ids), nmax, C), dtype=torch.float32, device=dev)
                         perm_r = perm[ri]
                         for b, (i, n) in enumerate(zip(rr_ids, n_own)):
@@ -605,7 +606,7 @@ class ExpertGroupGPTQ:
                             BT[b, :n] = rows.index_select(1, perm_r[b]).masked_fill(msk[b][None, :], 0)
                         dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[ri], 1, perm_r))
                         D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
-                        HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows)
+                        HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows, n_pad)
                         Bp_r = BT.transpose(1, 2).contiguous()
                         del BT
                         failed.append((torch.tensor([e0 + i for i in rr_ids]), info_r))
@@ -618,7 +619,7 @@ class ExpertGroupGPTQ:
                             t.record_stream(lr_stream)
                     if rr_ids:
                         q = kernels.gptq_sweep_rows_blocked(Xr, W0r, HmT, Bp_r, V, n_rows, sT[ri], zT[ri],
-                                                            g_idx[ri].contiguous(), self.bits)
+                                                            g_idx[ri].contiguous(), self.bits, n_pad)
                         layout_out(rr_ids, q)
                         del Xr, W0r, HmT, Bp_r, V, q
                     if ids_all:

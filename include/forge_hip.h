@@ -250,7 +250,9 @@ int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, cons
  *   forge_rows_factor_blocked: BT [batch][nmax][C] f32 = the rows of forge_lowrank_factor's Bp,
  *     transposed (row j = sqrt(2/n) x_j in solver order, 0 in pruned columns; zero rows beyond a
  *     layer's own count), D [batch][C], n_rows [batch] int32 on the DEVICE = each matrix's own row
- *     count rounded up to a multiple of 128 (<= nmax; products skip what lies beyond it)
+ *     count rounded up to a multiple of 128 (<= nmax; products skip what lies beyond it),
+ *     n_rows_host the same numbers on the host (may be NULL: only the work figures of the
+ *     forge_kernel_timing_* records use it, which otherwise count every matrix as nmax rows)
  *     -> HmT [batch][nmax][C] (HmT[j][k] = entry j of h_k: h_k . b_t = M[k][t] / M[k][k] for t
  *     left of k's 128-column block), V [batch][C][128] (V[t][k - c0] = -M[k][t] / M[k][k] for t < k
  *     inside the block that starts at c0; 0 elsewhere) and info [batch] (1-based position of a pivot that is not
@@ -265,13 +267,15 @@ int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, cons
  *     forge_gptq_sweep_direct_batched on V.  R a multiple of 128.
  * No counterpart in the reference, which forms and factors the C x C matrix whatever the number
  * of rows. */
-int forge_rows_factor_blocked(const float* BT, const float* D, const int32_t* n_rows, float* HmT,
-                              float* V, int32_t* info, int64_t batch, int64_t C, int64_t nmax,
-                              void* ws, int64_t ws_bytes, forge_stream_t stream);
+int forge_rows_factor_blocked(const float* BT, const float* D, const int32_t* n_rows,
+                              const int32_t* n_rows_host, float* HmT, float* V, int32_t* info,
+                              int64_t batch, int64_t C, int64_t nmax, void* ws, int64_t ws_bytes,
+                              forge_stream_t stream);
 int64_t forge_rows_factor_workspace_bytes(int64_t batch, int64_t C, int64_t nmax);
 int forge_gptq_sweep_rows_blocked(float* X, const void* W0, int w0_dtype, const float* HmT,
                                   const float* Bp, const float* V, const int32_t* n_rows,
-                                  const float* scalesT, const float* qzerosT, const int32_t* g_idx,
+                                  const int32_t* n_rows_host, const float* scalesT,
+                                  const float* qzerosT, const int32_t* g_idx,
                                   uint8_t* qweight, int64_t batch, int64_t C, int64_t R, int64_t G,
                                   int bits, int64_t nmax, void* ws, int64_t ws_bytes,
                                   forge_stream_t stream);
