@@ -688,7 +688,8 @@ def main():
                 low_rank_tokens=0, ms_per_step=round(1e3 * dt / a.steps, 2),
                 value=round(a.steps * chunk / dt, 3), unit="experts/s",
                 note="every expert through its Hessian, 64 experts per factorisation and sweep batch "
-                     "(the default run leaves that route the experts with more than 512 rows, 20 per layer)",
+                     "(the default run leaves that route only the experts beyond the closed forms' row "
+                     "limits: see config.experts_by_route)",
                 kernels={k: v for k, v in dense.items() if k.startswith("split_gemm")})
         out["hessian_buckets"] = hessian_buckets(cfg["hidden"], min(chunk, 64))
         out["hbm_kernels"] = hbm_kernels(wl)
