@@ -85,21 +85,39 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
     const uint16_t* __restrict__ Wb = W + sb * w_stride;
-    {   // 16 lanes x 8 bytes cover one 128-byte row piece; 16 rows per pass
-        const int rr = tid >> 4, c4 = (tid & 15) * 4;
+    {   // 16 lanes x 8 bytes cover one 128-byte row piece.  A lane takes a block of 4 rows x 4
+        // columns, transposes it in registers and stores four rows of r into LDS, 8 bytes each
+        const int rb = tid >> 4, c4 = (tid & 15) * 4;
         uint32_t keep = 0xF;
         if (dead) {
             const uint8_t* d = dead + sb * C + c0 + c4;
             keep = (d[0] ? 0u : 1u) | (d[1] ? 0u : 2u) | (d[2] ? 0u : 4u) | (d[3] ? 0u : 8u);
         }
-#pragma unroll 4
-        for (int p = 0; p < TR / 16; ++p) {
-            const int r = 16 * p + rr;
-            const uint2 v = *reinterpret_cast<const uint2*>(Wb + (r0 + r) * ldw + c0 + c4);
-            tile[c4 + 0][r] = (keep & 1u) ? (uint16_t)(v.x & 0xFFFFu) : (uint16_t)0;
-            tile[c4 + 1][r] = (keep & 2u) ? (uint16_t)(v.x >> 16) : (uint16_t)0;
-            tile[c4 + 2][r] = (keep & 4u) ? (uint16_t)(v.y & 0xFFFFu) : (uint16_t)0;
-            tile[c4 + 3][r] = (keep & 8u) ? (uint16_t)(v.y >> 16) : (uint16_t)0;
+#pragma unroll
+        for (int p = 0; p < TR / 64; ++p) {
+            const int r = 4 * (16 * p + rb);
+            const uint16_t* src = Wb + (r0 + r) * ldw + c0 + c4;
+            const uint2 v0 = *reinterpret_cast<const uint2*>(src);
+            const uint2 v1 = *reinterpret_cast<const uint2*>(src + ldw);
+            const uint2 v2 = *reinterpret_cast<const uint2*>(src + 2 * ldw);
+            const uint2 v3 = *reinterpret_cast<const uint2*>(src + 3 * ldw);
+            // perm(hi, lo, sel): result byte i = byte sel[i] of {hi, lo} (0..3 = lo, 4..7 = hi)
+            uint2 o0 = make_uint2(__builtin_amdgcn_perm(v1.x, v0.x, 0x05040100u),    // column c4
+                                  __builtin_amdgcn_perm(v3.x, v2.x, 0x05040100u));
+            uint2 o1 = make_uint2(__builtin_amdgcn_perm(v1.x, v0.x, 0x07060302u),    // c4 + 1
+                                  __builtin_amdgcn_perm(v3.x, v2.x, 0x07060302u));
+            uint2 o2 = make_uint2(__builtin_amdgcn_perm(v1.y, v0.y, 0x05040100u),    // c4 + 2
+                                  __builtin_amdgcn_perm(v3.y, v2.y, 0x05040100u));
+            uint2 o3 = make_uint2(__builtin_amdgcn_perm(v1.y, v0.y, 0x07060302u),    // c4 + 3
+                                  __builtin_amdgcn_perm(v3.y, v2.y, 0x07060302u));
+            if (!(keep & 1u)) o0 = make_uint2(0u, 0u);
+            if (!(keep & 2u)) o1 = make_uint2(0u, 0u);
+            if (!(keep & 4u)) o2 = make_uint2(0u, 0u);
+            if (!(keep & 8u)) o3 = make_uint2(0u, 0u);
+            *reinterpret_cast<uint2*>(&tile[c4 + 0][r]) = o0;
+            *reinterpret_cast<uint2*>(&tile[c4 + 1][r]) = o1;
+            *reinterpret_cast<uint2*>(&tile[c4 + 2][r]) = o2;
+            *reinterpret_cast<uint2*>(&tile[c4 + 3][r]) = o3;
         }
     }
     __syncthreads();
@@ -118,36 +136,52 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     }
 }
 
-// 128 (c) x 256 (r) byte tile.  LDS holds it as [c][r]; a row of the result is gathered
-// back four bytes (four values of c) per lane.
+// 128 (c) x 256 (r) byte tile.  LDS holds it as [c][r]; each lane takes a 4 x 4 byte block out
+// of it (four words, one per source row), transposes it in registers with byte permutes and
+// stores one word into each of four rows of the result.
 __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
     const uint8_t* __restrict__ qin, const int64_t* __restrict__ perm_inv,
     uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride,
     const int64_t* __restrict__ index) {
     constexpr int TC = 128, TR = 256, PITCH = TR + 4;    // 65 words per row: odd
-    __shared__ __attribute__((aligned(4))) uint8_t tile[TC][PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[TC][PITCH];
     const int64_t b = blockIdx.z, sb = index ? index[b] : b;
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
-    {   // a wavefront reads the 256 bytes of one source row per instruction
-        const int cw = tid >> 6, r4 = (tid & 63) * 4;
-#pragma unroll 4
-        for (int cc = 0; cc < TC; cc += 4) {
-            const int c = cc + cw;
-            const uint32_t v = *reinterpret_cast<const uint32_t*>(
-                qin + b * i_stride + perm_inv[sb * C + c0 + c] * ldi + r0 + r4);
-            *reinterpret_cast<uint32_t*>(&tile[c][r4]) = v;
+    {   // 16 lanes x 16 bytes read the 256 bytes of one source row; all eight loads of a lane
+        // are in flight before the first is stored
+        const int cw = tid >> 4, r16 = (tid & 15) * 16;
+        uint4 v[TC / 16];
+#pragma unroll
+        for (int p = 0; p < TC / 16; ++p)
+            v[p] = *reinterpret_cast<const uint4*>(
+                qin + b * i_stride + perm_inv[sb * C + c0 + 16 * p + cw] * ldi + r0 + r16);
+#pragma unroll
+        for (int p = 0; p < TC / 16; ++p) {
+            uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[16 * p + cw][r16]);   // rows are 4-aligned
+            dst[0] = v[p].x; dst[1] = v[p].y; dst[2] = v[p].z; dst[3] = v[p].w;
         }
     }
     __syncthreads();
-    {   // 32 lanes x 4 bytes cover one 128-byte row piece; 8 rows per pass
-        const int rr = tid >> 5, c4 = (tid & 31) * 4;
-#pragma unroll 4
-        for (int p = 0; p < TR / 8; ++p) {
-            const int r = 8 * p + rr;
-            const uint32_t v = (uint32_t)tile[c4][r] | ((uint32_t)tile[c4 + 1][r] << 8) |
-                               ((uint32_t)tile[c4 + 2][r] << 16) | ((uint32_t)tile[c4 + 3][r] << 24);
-            *reinterpret_cast<uint32_t*>(qout + sb * R * C + (r0 + r) * C + c0 + c4) = v;
+    {   // 32 lanes x 4 bytes cover one 128-byte row piece; a lane's block is rows r4 .. r4 + 3
+        const int rg = tid >> 5, c4 = (tid & 31) * 4;
+#pragma unroll 2
+        for (int p = 0; p < TR / 32; ++p) {
+            const int r4 = 4 * (8 * p + rg);
+            const uint32_t w0 = *reinterpret_cast<const uint32_t*>(&tile[c4 + 0][r4]);
+            const uint32_t w1 = *reinterpret_cast<const uint32_t*>(&tile[c4 + 1][r4]);
+            const uint32_t w2 = *reinterpret_cast<const uint32_t*>(&tile[c4 + 2][r4]);
+            const uint32_t w3 = *reinterpret_cast<const uint32_t*>(&tile[c4 + 3][r4]);
+            // perm(hi, lo, sel): result byte i = byte sel[i] of {hi, lo} (0..3 = lo, 4..7 = hi)
+            const uint32_t a = __builtin_amdgcn_perm(w1, w0, 0x05010400u);   // w0.0 w1.0 w0.1 w1.1
+            const uint32_t bq = __builtin_amdgcn_perm(w3, w2, 0x05010400u);  // w2.0 w3.0 w2.1 w3.1
+            const uint32_t cq = __builtin_amdgcn_perm(w1, w0, 0x07030602u);  // w0.2 w1.2 w0.3 w1.3
+            const uint32_t d = __builtin_amdgcn_perm(w3, w2, 0x07030602u);   // w2.2 w3.2 w2.3 w3.3
+            uint8_t* out = qout + sb * R * C + (r0 + r4) * C + c0 + c4;
+            *reinterpret_cast<uint32_t*>(out) = __builtin_amdgcn_perm(bq, a, 0x05040100u);
+            *reinterpret_cast<uint32_t*>(out + C) = __builtin_amdgcn_perm(bq, a, 0x07060302u);
+            *reinterpret_cast<uint32_t*>(out + 2 * C) = __builtin_amdgcn_perm(d, cq, 0x05040100u);
+            *reinterpret_cast<uint32_t*>(out + 3 * C) = __builtin_amdgcn_perm(d, cq, 0x07060302u);
         }
     }
 }
@@ -447,8 +481,8 @@ static int codes_to_layer_order(const uint8_t* qin, int64_t ldi, int64_t i_strid
     FORGE_REQUIRE(grid.y < 65536, "R too large");
     forge::KernelTiming timing("codes_to_layer_order", (hipStream_t)stream, 2.0 * batch * R * C,
                                forge::WORK_BYTES);
-    const bool fast = (R % 256) == 0 && (C % 128) == 0 && (reinterpret_cast<uintptr_t>(qin) % 4) == 0 &&
-                      (reinterpret_cast<uintptr_t>(qout) % 4) == 0 && (ldi % 4) == 0 && (i_stride % 4) == 0;
+    const bool fast = (R % 256) == 0 && (C % 128) == 0 && (reinterpret_cast<uintptr_t>(qin) % 16) == 0 &&
+                      (reinterpret_cast<uintptr_t>(qout) % 4) == 0 && (ldi % 16) == 0 && (i_stride % 16) == 0;
     if (fast) {
         const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
         to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C,
@@ -568,6 +602,111 @@ extern "C" int forge_pack_int4(const uint8_t* codes, const float* qzeros, int32_
     }
     pack_int4_kernel<<<dim3((unsigned)forge::ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream>>>(
         codes, qzeros, packed, R, C, gs, forge::ceil_div(C, gs));
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Front end of the blocked closed form: its operands straight from the calibration rows.
+namespace {
+
+// BT[b][r][j] = Bp[b][j][r] = (float)((double)rows[row0[b] + r][perm[b][j]] * root[b]) for r below
+// the matrix's own row count and a column that is not pruned, else 0: the rows of
+// sqrt(2/n) X (forge/gptq.py:70-79 sums their products into H) in solver order, once row-major
+// (the factor's K-major operand) and once column-major (the sweep's).  32 x 32 tiles: the gather
+// along the permuted columns and the row-major store by lanes along j, the transposed store by
+// lanes along r.  Every element of both outputs is written (zeros beyond n[b]); BT may be null.
+template <typename T>
+__global__ __launch_bounds__(256) void rows_operands_kernel(
+    const T* __restrict__ rows, const int64_t* __restrict__ row0, const int32_t* __restrict__ n,
+    const double* __restrict__ root, const int64_t* __restrict__ perm,
+    const uint8_t* __restrict__ dead, float* __restrict__ BT, float* __restrict__ Bp, int64_t C,
+    int64_t nmax) {
+    __shared__ float tile[32][33];
+    const int64_t b = blockIdx.z;
+    const int64_t j0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int64_t j = j0 + tx;
+    const int nb = n[b];
+    const double sc = root[b];
+    const bool live = j < C && !dead[b * C + j];
+    const int64_t src = live ? perm[b * C + j] : 0;
+    const T* __restrict__ Xb = rows + row0[b] * C;
+#pragma unroll
+    for (int i = ty; i < 32; i += 8) {
+        const int64_t r = r0 + i;
+        float v = 0.0f;
+        if (live && r < nb) v = (float)((double)ld_as_f32(Xb + r * C + src) * sc);
+        tile[i][tx] = v;
+        if (BT && j < C && r < nmax) BT[(b * nmax + r) * C + j] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = ty; i < 32; i += 8) {
+        const int64_t jj = j0 + i, r = r0 + tx;
+        if (jj < C && r < nmax) Bp[(b * C + jj) * nmax + r] = tile[tx][i];
+    }
+}
+
+// out[b][c] = (float)(alpha[b] * sum_r (double)x[r][c]^2): the diagonal of (2/n) X^T X summed
+// in float64 and rounded once.  One lane per feature, rows in sequence: the loads of a
+// wavefront are one contiguous piece of a row.
+template <typename T>
+__global__ __launch_bounds__(256) void rows_diagonal_kernel(
+    const T* __restrict__ rows, const int64_t* __restrict__ row0, const int32_t* __restrict__ n,
+    const double* __restrict__ alpha, float* __restrict__ out, int64_t C) {
+    const int64_t b = blockIdx.y;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const T* __restrict__ Xb = rows + row0[b] * C + c;
+    const int nb = n[b];
+    double acc = 0.0;
+    for (int r = 0; r < nb; ++r) {
+        const double x = (double)ld_as_f32(Xb + (int64_t)r * C);
+        acc = __builtin_fma(x, x, acc);
+    }
+    out[b * C + c] = (float)(acc * alpha[b]);
+}
+
+}  // namespace
+
+extern "C" int forge_rows_operands(const void* rows, int x_dtype, const int64_t* row0,
+                                   const int32_t* n, const double* root, const int64_t* perm,
+                                   const uint8_t* dead, float* BT, float* Bp, int64_t batch,
+                                   int64_t C, int64_t nmax, forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && C >= 1 && nmax >= 1, "bad shape");
+    FORGE_REQUIRE(x_dtype == FORGE_BF16 || x_dtype == FORGE_F32, "rows must be bf16 or f32");
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(rows && row0 && n && root && perm && dead && Bp, "null pointer");
+    FORGE_REQUIRE(batch <= 65535 && forge::ceil_div(nmax, 32) <= 65535, "batch or nmax too large for one grid");
+    hipStream_t st = (hipStream_t)stream;
+    forge::KernelTiming timing("rows_operands", st, (BT ? 8.0 : 4.0) * batch * nmax * C, forge::WORK_BYTES);
+    const dim3 grid((unsigned)forge::ceil_div(C, 32), (unsigned)forge::ceil_div(nmax, 32), (unsigned)batch);
+    if (x_dtype == FORGE_BF16)
+        rows_operands_kernel<__hip_bfloat16><<<grid, dim3(256), 0, st>>>(
+            (const __hip_bfloat16*)rows, row0, n, root, perm, dead, BT, Bp, C, nmax);
+    else
+        rows_operands_kernel<float><<<grid, dim3(256), 0, st>>>((const float*)rows, row0, n, root, perm,
+                                                                dead, BT, Bp, C, nmax);
+    FORGE_LAUNCH_CHECK();
+    return FORGE_OK;
+}
+
+extern "C" int forge_rows_diagonal(const void* rows, int x_dtype, const int64_t* row0,
+                                   const int32_t* n, const double* alpha, float* out, int64_t batch,
+                                   int64_t C, forge_stream_t stream) {
+    FORGE_REQUIRE(batch >= 0 && C >= 1, "bad shape");
+    FORGE_REQUIRE(x_dtype == FORGE_BF16 || x_dtype == FORGE_F32, "rows must be bf16 or f32");
+    if (batch == 0) return FORGE_OK;
+    FORGE_REQUIRE(rows && row0 && n && alpha && out, "null pointer");
+    FORGE_REQUIRE(batch <= 65535, "batch too large for one grid");
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)forge::ceil_div(C, 256), (unsigned)batch);
+    if (x_dtype == FORGE_BF16)
+        rows_diagonal_kernel<__hip_bfloat16><<<grid, dim3(256), 0, st>>>(
+            (const __hip_bfloat16*)rows, row0, n, alpha, out, C);
+    else
+        rows_diagonal_kernel<float><<<grid, dim3(256), 0, st>>>((const float*)rows, row0, n, alpha, out, C);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;
 }

@@ -96,6 +96,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
         "forge_pack_sparsegptq14_to_u64x2": ([vp, vp, vp, vp, i64, i64, vp], i32),
         "forge_dequantize_groups": ([vp, vp, vp, vp, i32, i64, i64, i64, i64, vp], i32),
         "forge_gather_scaled_rows": ([vp, i32, i64, i64, i64, vp, vp, vp, i64, vp], i32),
+        "forge_rows_operands": ([vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, vp], i32),
+        "forge_rows_diagonal": ([vp, i32, vp, vp, vp, vp, i64, i64, vp], i32),
     }
     for name, (args, res) in sigs.items():
         fn = getattr(lib, name)          # AttributeError here = library/header mismatch
@@ -128,6 +130,7 @@ EXPORTED_SYMBOLS = (
     "forge_weight_to_solver_order_gather", "forge_codes_to_layer_order_scatter",
     "forge_rows_factor_blocked", "forge_rows_factor_workspace_bytes",
     "forge_gptq_sweep_rows_blocked", "forge_gptq_sweep_rows_workspace_bytes",
+    "forge_rows_operands", "forge_rows_diagonal",
 )
 
 
@@ -522,6 +525,44 @@ class _HipKernels:
                                                             _ptr(V), _ptr(info), B, C, nmax, _ptr(ws),
                                                             nbytes, _stream()))
         return HmT, V, info
+
+    def rows_operands(self, rows, row0, n, root, perm, dead, nmax, want_bt=True, out=None):
+        """rows [*, C] bf16/f32 (matrix b owns rows row0[b] .. row0[b]+n[b]-1; row0 [B] i64, n [B]
+        i32, root [B] f64 = sqrt(2/n), all on the device), perm [B,C] i64, dead [B,C] u8 or bool
+        in solver order -> (BT [B,nmax,C] or None, Bp [B,C,nmax]) f32: sqrt(2/n) X in solver
+        order with pruned columns zero, row-major and column-major.  out: Bp's storage."""
+        _need_cuda(rows, row0, n, root, perm, dead)
+        B, C = perm.shape
+        assert rows.dim() == 2 and rows.shape[1] == C and rows.is_contiguous()
+        assert row0.dtype == torch.int64 and n.dtype == torch.int32 and root.dtype == torch.float64
+        assert row0.numel() == B and n.numel() == B and root.numel() == B
+        assert perm.dtype == torch.int64 and perm.is_contiguous()
+        if dead.dtype == torch.bool:
+            dead = dead.view(torch.uint8)
+        assert dead.dtype == torch.uint8 and dead.is_contiguous() and tuple(dead.shape) == (B, C)
+        BT = torch.empty((B, nmax, C), dtype=torch.float32, device=rows.device) if want_bt else None
+        Bp = out if out is not None else torch.empty((B, C, nmax), dtype=torch.float32, device=rows.device)
+        assert Bp.is_contiguous() and Bp.dtype == torch.float32 and tuple(Bp.shape) == (B, C, nmax)
+        with torch.cuda.device(rows.device):
+            self._check(self._lib.forge_rows_operands(
+                _ptr(rows), _dtype_code(rows), _ptr(row0), _ptr(n), _ptr(root), _ptr(perm), _ptr(dead),
+                _ptr(BT), _ptr(Bp), B, C, int(nmax), _stream()))
+        return BT, Bp
+
+    def rows_diagonal(self, rows, row0, n, alpha):
+        """diag((2/n) X^T X) per matrix, summed in float64 and rounded once: rows [*, C] bf16/f32,
+        row0 [B] i64, n [B] i32, alpha [B] f64 (device) -> [B, C] f32."""
+        _need_cuda(rows, row0, n, alpha)
+        C = rows.shape[1]
+        B = row0.numel()
+        assert rows.dim() == 2 and rows.is_contiguous()
+        assert row0.dtype == torch.int64 and n.dtype == torch.int32 and alpha.dtype == torch.float64
+        assert n.numel() == B and alpha.numel() == B
+        out = torch.empty((B, C), dtype=torch.float32, device=rows.device)
+        with torch.cuda.device(rows.device):
+            self._check(self._lib.forge_rows_diagonal(_ptr(rows), _dtype_code(rows), _ptr(row0), _ptr(n),
+                                                      _ptr(alpha), _ptr(out), B, C, _stream()))
+        return out
 
     def gptq_sweep_rows_blocked(self, X, W0, HmT, Bp, V, n_rows, scalesT, qzerosT, g_idx, bits,
                                 n_rows_host=None):

@@ -249,7 +249,7 @@ class ExpertGroupGPTQ:
         if not self.low_rank_tokens:
             self._give_slots(range(self.E))          # every expert through its Hessian, in order
         row0, counts, alpha, beta = [], [], [], []
-        src, dst, late = [], [], []
+        src, dst, late, keep = [], [], [], []
         for e in range(self.E):
             o, new = int(offsets[e]), int(offsets[e + 1]) - int(offsets[e])
             n = self.num_samples[e]
@@ -267,7 +267,7 @@ class ExpertGroupGPTQ:
                         self._rows[e].append(self._kept[e, :n].clone())
                         self._kept[e].zero_()
                 if new > 0:
-                    self._rows[e].append(X[o:o + new].clone())
+                    keep.append((e, o, new))
                 new = 0
             elif self.low_rank[e] or self.rows_route[e]:
                 if n > 0:
@@ -281,6 +281,13 @@ class ExpertGroupGPTQ:
             beta.append(n / max(total, 1))
         if src:
             self._kept.view(self.E * self._cap, self.C)[self._dev(dst)] = X[self._dev(src)].float()
+        if keep:
+            # one copy for all of them; each expert holds a view of its rows
+            block = torch.cat([X[o:o + new] for _, o, new in keep])
+            at = 0
+            for e, _, new in keep:
+                self._rows[e].append(block[at:at + new])
+                at += new
         self._give_slots([e for e in range(self.E) if counts[e] > 0] + [e for e, *_ in late])
         if any(counts):
             kernels.hessian_update_ranges(X, self._per_slot(row0), self._per_slot(counts),
@@ -347,21 +354,31 @@ class ExpertGroupGPTQ:
                 self._kept = torch.zeros((E, self._cap, C), dtype=torch.float32, device=dev)
             lr_dev = self._dev(lr_host)
             alpha32 = self._dev([2.0 / max(n, 1) for n in self.num_samples], dtype=torch.float32)
-            # (32 experts at a time: the float64 squares of all kept rows at once are 2 x 0.9 GB
-            # for 128 experts of 7168 features)
-            d_lr = torch.cat([((self._kept[i:i + 32].double() ** 2).sum(dim=1)
-                               * alpha32[i:i + 32].double()[:, None]).float() for i in range(0, E, 32)])
+            cap = self._cap
+            d_lr = kernels.rows_diagonal(
+                self._kept.view(E * cap, C), self._dev([e * cap for e in range(E)]),
+                self._dev([n if lr else 0 for n, lr in zip(self.num_samples, lr_host)], dtype=torch.int32),
+                alpha32.double())
             diag_all = torch.where(lr_dev[:, None], d_lr, diag_all)
-        rows_cat = {}
-        if any(rr_host):
-            # experts on the blocked route: the same diagonal from their own rows
-            d_rr = torch.zeros((E, C), dtype=torch.float32, device=dev)
-            for e in range(E):
-                if rr_host[e]:
-                    rows_cat[e] = self._rows[e][0] if len(self._rows[e]) == 1 else torch.cat(self._rows[e])
-                    self._rows[e] = [rows_cat[e]]
-                    d_rr[e] = ((rows_cat[e].double() ** 2).sum(dim=0) * (2.0 / self.num_samples[e])).float()
-            diag_all = torch.where(self._dev(rr_host)[:, None], d_rr, diag_all)
+        rows_all, rows_at = None, {}
+        rr_list = [e for e in range(E) if rr_host[e]]
+        if rr_list:
+            # experts on the blocked route: the same diagonal from their own rows, which from
+            # here on lie end to end in ONE tensor (each expert keeps a view of its part)
+            pieces = [p for e in rr_list for p in self._rows[e]]
+            if any(p.dtype == torch.float32 for p in pieces):
+                pieces = [p.float() for p in pieces]
+            rows_all = pieces[0] if len(pieces) == 1 else torch.cat(pieces)
+            at = 0
+            for e in rr_list:
+                rows_at[e] = at
+                self._rows[e] = [rows_all[at:at + self.num_samples[e]]]
+                at += self.num_samples[e]
+            d_rr = kernels.rows_diagonal(
+                rows_all, self._dev([rows_at[e] for e in rr_list]),
+                self._dev([self.num_samples[e] for e in rr_list], dtype=torch.int32),
+                self._dev([2.0 / self.num_samples[e] for e in rr_list], dtype=torch.float64))
+            diag_all = diag_all.index_copy(0, self._dev(rr_list), d_rr)
         bad = (~seen) | torch.isnan(diag_all).any(dim=1)
         if any_lr or any(rr_host):
             off_h = self._dev([a or b for a, b in zip(lr_host, rr_host)])
@@ -382,7 +399,7 @@ class ExpertGroupGPTQ:
         ready.record()
         self._prepared = dict(diag_all=diag_all, bad=bad, host_flags=host_flags, ready=ready,
                               lr_host=lr_host, any_lr=any_lr, lr_dev=lr_dev, alpha32=alpha32,
-                              rr_host=rr_host, rows_cat=rows_cat, keep=flags)
+                              rr_host=rr_host, rows_all=rows_all, rows_at=rows_at, keep=flags)
         return self._prepared
 
     @torch.no_grad()
@@ -403,7 +420,7 @@ class ExpertGroupGPTQ:
         diag_all, bad, host_flags = prep["diag_all"], prep["bad"], prep["host_flags"]
         lr_host, any_lr = prep["lr_host"], prep["any_lr"]
         lr_dev, alpha32 = prep["lr_dev"], prep["alpha32"]
-        rr_host, rows_cat = prep["rr_host"], prep["rows_cat"]
+        rr_host, rows_all, rows_at = prep["rr_host"], prep["rows_all"], prep["rows_at"]
         any_rr = any(rr_host)
         # (per expert: an indexed assignment of a broadcast identity moves the same bytes at a
         # fraction of the fill rate)
@@ -577,13 +594,14 @@ class ExpertGroupGPTQ:
                     for nr, ids in buckets:
                         li = self._dev(ids)
                         msk = mask[li].bool()                               # [Bl, C], solver order
-                        root = alpha32[e0:e1][li].double().sqrt()[:, None, None]
-                        Bp = torch.gather((self._kept[e0:e1][li][:, :nr].double() * root).float(), 2,
-                                          perm[li][:, None, :].expand(-1, nr, -1))
-                        Bp = Bp.masked_fill(msk[:, None, :], 0).transpose(1, 2)            # [Bl, C, nr]
                         span = slice(at, at + len(ids) * C * nr)
                         Bpv = Bp_all[span].view(len(ids), C, nr)
-                        Bpv.copy_(Bp)
+                        own = [self.num_samples[e0 + i] for i in ids]
+                        # sqrt(2/n) X in solver order with pruned columns zero, [Bl, C, nr]
+                        kernels.rows_operands(
+                            self._kept.view(E * self._cap, C), self._dev([(e0 + i) * self._cap for i in ids]),
+                            self._dev(own, dtype=torch.int32), alpha32[e0:e1][li].double().sqrt(),
+                            perm[li], mask[li], nr, want_bt=False, out=Bpv)
                         dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[li], 1, perm[li]))
                         D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
                         kernels.lowrank_factor(Bpv, D.contiguous(),
@@ -599,15 +617,15 @@ class ExpertGroupGPTQ:
                         nmax = max((n + 127) // 128 * 128 for n in n_own)
                         n_pad = [(n + 127) // 128 * 128 for n in n_own]
                         n_rows = self._dev(n_pad, dtype=torch.int32)
-                        BT = torch.zeros((len(rr_ids), nmax, C), dtype=torch.float32, device=dev)
                         perm_r = perm[ri]
-                        for b, (i, n) in enumerate(zip(rr_ids, n_own)):
-                            rows = (rows_cat[e0 + i].double() * (2.0 / n) ** 0.5).float()
-                            BT[b, :n] = rows.index_select(1, perm_r[b]).masked_fill(msk[b][None, :], 0)
+                        BT, Bp_r = kernels.rows_operands(
+                            rows_all, self._dev([rows_at[e0 + i] for i in rr_ids]),
+                            self._dev(n_own, dtype=torch.int32),
+                            self._dev([(2.0 / n) ** 0.5 for n in n_own], dtype=torch.float64),
+                            perm_r, mask[ri], nmax)
                         dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[ri], 1, perm_r))
                         D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
                         HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows, n_pad)
-                        Bp_r = BT.transpose(1, 2).contiguous()
                         del BT
                         failed.append((torch.tensor([e0 + i for i in rr_ids]), info_r))
                         Xr = torch.empty((len(rr_ids), C, R), dtype=torch.float32, device=dev)

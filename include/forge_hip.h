@@ -244,6 +244,29 @@ int forge_gptq_sweep_lowrank(const void* W0, int w0_dtype, const float* Bp, cons
                              const int32_t* g_idx, uint8_t* qweight, int64_t batch, int64_t C,
                              int64_t R, int64_t G, int bits, int64_t n, forge_stream_t stream);
 
+/* Front end of the two closed forms (layers that saw fewer calibration rows than they have
+ * features): their operands straight from the rows the layer saw, without the Hessian that the
+ * reference sums from them (forge/gptq.py:61-80: H = (2/n) X^T X as the running mean of
+ * X^T (alpha X)).  rows [*, C] (x_dtype FORGE_BF16 or FORGE_F32, row pitch C): matrix b owns the
+ * rows row0[b] .. row0[b] + n[b] - 1.  row0 [batch] int64, n [batch] int32, device memory.
+ *
+ * forge_rows_operands: root [batch] f64 (sqrt(2 / n[b]) as the caller rounds it), perm
+ * [batch, C] int64 (solver column j is feature perm[b][j]), dead [batch, C] u8 in solver order
+ * (pruned columns, gptq.py:145-149, read as zero).
+ *   BT[b][r][j] = Bp[b][j][r] = (float)((double)rows[row0[b] + r][perm[b][j]] * root[b])
+ * for r < n[b] and dead[b][j] == 0, else 0; BT [batch, nmax, C] f32 (may be NULL), Bp
+ * [batch, C, nmax] f32, every element written.
+ *
+ * forge_rows_diagonal: out[b][c] = (float)(alpha[b] * sum_r (double)rows[row0[b] + r][c]^2),
+ * the diagonal of H summed in float64 and rounded once (what the activation order and the
+ * damping are taken from, gptq.py:100-108,151-153).  alpha [batch] f64, out [batch, C] f32. */
+int forge_rows_operands(const void* rows, int x_dtype, const int64_t* row0, const int32_t* n,
+                        const double* root, const int64_t* perm, const uint8_t* dead, float* BT,
+                        float* Bp, int64_t batch, int64_t C, int64_t nmax, forge_stream_t stream);
+int forge_rows_diagonal(const void* rows, int x_dtype, const int64_t* row0, const int32_t* n,
+                        const double* alpha, float* out, int64_t batch, int64_t C,
+                        forge_stream_t stream);
+
 /* GPTQ.quantize for a layer that saw 129 .. ~1000 calibration rows, fewer than a fraction of its
  * input features (gptq.py:128-166 with solver.cu:9-154), again without the C x C Hessian: the
  * closed forms of forge_lowrank_factor as 128-column blocked products on the matrix pipe.

@@ -407,7 +407,7 @@ def test_config5_sparse14_full_size():
 
 @pytest.mark.parametrize("n_tokens", [1536, 200, 128, 40])
 def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
-    """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 512 of
+    """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 256 of
     its 2048 rows, rows being independent, to keep the CPU oracle's sweeps short) with a heavy
     expert's tokens, with 200 (Hessian of rank 200 before damping; the batched front end's default
     route then takes the blocked closed form) and with 128 and 40 (that route then solves from the
@@ -424,7 +424,7 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     from forge.gptq import GPTQ
     from forge.moe import ExpertGroupGPTQ
     g0 = torch.Generator().manual_seed(11)
-    W = synth.fp8_block_roundtrip((0.02 * torch.randn(512, 7168, generator=g0)).bfloat16())
+    W = synth.fp8_block_roundtrip((0.02 * torch.randn(256, 7168, generator=g0)).bfloat16())
     X = torch.randn(1536, 7168, generator=g0).bfloat16()[:n_tokens].contiguous()
     kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
               quantization_order="activation", rel_damp=0.01)
@@ -461,7 +461,7 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
         # low_rank_tokens=128 the column-by-column form with eight lanes per row of the sweep)
         variants = [("inverse", {}), ("direct", {})] + ([("direct", dict(low_rank_tokens=128))] if n_tokens == 128 else [])
         for route, extra in variants:
-            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **extra, **kw)
+            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 256, 7168)], device=DEV, factor_route=route, **extra, **kw)
             grp.update(X.to(DEV), [0, n_tokens])
             (q, s, z), = grp.quantize(chunk=1)
             assert not grp.issue_non_invertible.any()
@@ -539,55 +539,79 @@ def test_expert_group_few_tokens_routes_agree():
             assert err(q, s, z) < 0.5 * rtn
 
 
-def test_config2_qwen3_experts_at_full_shape(hip):
+@pytest.fixture(scope="module")
+def config2_step(hip):
     """Eight Qwen3-30B-A3B-shaped experts (768x2048 / 2048x768 bf16, asymmetric, MSE) with the
-    layer's ragged routing, batched, against per-expert oracle handles.  With the left-looking
-    schedule that the layer's 128 experts take (eight alone would be swept right-looking): long
-    products from fp16 halves, their V operand from the factor's rows, X never laid out."""
+    layer's ragged routing, batched.  With the left-looking schedule that the layer's 128
+    experts take (eight alone would be swept right-looking): long products from fp16 halves,
+    their V operand from the factor's rows, X never laid out."""
     from forge.moe import ExpertGroupGPTQ
     moe = synth.qwen3_moe(experts=8, seed=6)
     E = 8
     xs, hs = zip(*(moe.expert_inputs(e) for e in range(E)))
     offs = np.concatenate([[0], np.cumsum([x.shape[0] for x in xs])])
-    kw = dict(bits=4, group_size=128, symmetric=False, quantization_scale="mse",
-              quantization_order="default")
-    gu = ExpertGroupGPTQ([moe.Wg.to(DEV), moe.Wu.to(DEV)], device=DEV, **kw)
-    dn = ExpertGroupGPTQ([moe.Wd.to(DEV)], device=DEV, **kw)
+    gu = ExpertGroupGPTQ([moe.Wg.to(DEV), moe.Wu.to(DEV)], device=DEV, **CONFIG2_KW)
+    dn = ExpertGroupGPTQ([moe.Wd.to(DEV)], device=DEV, **CONFIG2_KW)
     gu.update(torch.cat(xs).to(DEV), offs)
     dn.update(torch.cat(hs).to(DEV), offs)
     hip.set_option("sweep_schedule", 1)
     try:
         assert hip.sweep_direct_reads_band_only(8, 2048, 1536) and hip.sweep_direct_reads_band_only(8, 768, 2048)
-        (qg, sg, zg), (qu, su, zu) = gu.quantize(chunk=8)
-        (qd, sd, zd), = dn.quantize(chunk=8)
+        outs = [tuple(t.cpu() for t in o) for o in gu.quantize(chunk=8)]
+        outs += [tuple(t.cpu() for t in o) for o in dn.quantize(chunk=8)]
     finally:
         hip.set_option("sweep_schedule", 0)
-    # ||WX - QX||^2 summed over the tokens each expert saw: the layer's output error.  Per
-    # expert the ratio is only meaningful with enough tokens (an expert that saw 3 tokens has
-    # a rank-3 Hessian and its error moves by several % between equally good solutions).
-    worst, worst_ratio, sum_o, sum_g = 0.0, 0.0, 0.0, 0.0
-    for e in range(E):
-        for W, X, (q, s, z) in ((moe.Wg[e], xs[e], (qg, sg, zg)), (moe.Wu[e], xs[e], (qu, su, zu)),
-                                (moe.Wd[e], hs[e], (qd, sd, zd))):
-            o = oracle.GPTQ(linear(W), **kw)
-            o.update(X)
-            n = X.shape[0]
-            H = o.H.double().numpy().copy() if o.H is not None else np.eye(W.shape[1])
-            qo, so, zo = o.quantize()
-            assert float((so != s[e].cpu()).float().mean()) <= 2e-3
-            worst = max(worst, flip_rate(qo, q[e]))
-            if n:
-                _codes_at_floor(f"config2 expert {e} {tuple(W.shape)} n={n}", qo, q[e], W, [X], kw)
-            Wf = W.float().numpy()
-            eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H) * n / 2
-            eg = mathref.layer_error(Wf, oracle.dequantize(q[e].cpu(), s[e].cpu(), z[e].cpu(), 128).numpy(), H) * n / 2
-            sum_o += eo
-            sum_g += eg
-            if n >= 128:
-                worst_ratio = max(worst_ratio, abs(eg / eo - 1))
-    print(f"config2 experts: worst flips {worst:.2e}, worst per-expert error deviation "
-          f"{worst_ratio:.2e}, layer error ratio {sum_g / sum_o:.5f}")
-    assert worst_ratio < 0.01 and abs(sum_g / sum_o - 1) < 0.01
+    del gu, dn
+    torch.cuda.empty_cache()
+    return moe, xs, hs, outs, {}
+
+
+CONFIG2_KW = dict(bits=4, group_size=128, symmetric=False, quantization_scale="mse",
+                  quantization_order="default")
+
+
+def _config2_expert(step, e, floors):
+    """One expert's three matrices against per-expert oracle handles: (error of the oracle's
+    codes, error of the GPU's) as ||WX - QX||^2 summed over the tokens the expert saw."""
+    moe, xs, hs, (og, ou, od), errors = step
+    if e in errors and not floors:
+        return errors[e]
+    sum_o = sum_g = 0.0
+    for W, X, (q, s, z) in ((moe.Wg[e], xs[e], og), (moe.Wu[e], xs[e], ou), (moe.Wd[e], hs[e], od)):
+        o = oracle.GPTQ(linear(W), **CONFIG2_KW)
+        o.update(X)
+        n = X.shape[0]
+        H = o.H.double().numpy().copy() if o.H is not None else np.eye(W.shape[1])
+        qo, so, zo = o.quantize()
+        assert float((so != s[e]).float().mean()) <= 2e-3
+        if n and floors:
+            _codes_at_floor(f"config2 expert {e} {tuple(W.shape)} n={n}", qo, q[e], W, [X], CONFIG2_KW)
+        Wf = W.float().numpy()
+        eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H) * n / 2
+        eg = mathref.layer_error(Wf, oracle.dequantize(q[e], s[e], z[e], 128).numpy(), H) * n / 2
+        # Per expert the ratio is only meaningful with enough tokens (an expert that saw 3 tokens
+        # has a rank-3 Hessian and its error moves by several % between equally good solutions).
+        if floors and n >= 128:
+            assert abs(eg / eo - 1) < 0.01, (e, tuple(W.shape), eg / eo)
+        sum_o += eo
+        sum_g += eg
+    errors[e] = (sum_o, sum_g)
+    return errors[e]
+
+
+@pytest.mark.parametrize("e", range(8))
+def test_config2_qwen3_expert_at_full_shape(config2_step, e):
+    """Scales equal up to candidate near-ties, codes under the floor rule, the expert's output
+    error within 1 % of the oracle's where it saw at least 128 tokens."""
+    _config2_expert(config2_step, e, floors=True)
+
+
+def test_config2_qwen3_layer_error(config2_step):
+    """The layer's output error over all eight experts: within 1 % of the oracle's."""
+    sums = [_config2_expert(config2_step, e, floors=False) for e in range(8)]
+    so, sg = sum(a for a, _ in sums), sum(b for _, b in sums)
+    print(f"config2 layer error ratio {sg / so:.5f}")
+    assert abs(sg / so - 1) < 0.01
 
 
 def test_quantize_refuses_a_chunk_whose_workspace_does_not_fit(monkeypatch):

@@ -115,3 +115,75 @@ def test_blocked_sweep_matches_float64_gptq_on_the_dense_factor(hip, n, dtype):
         # what is left in X: the displacements w0 - deq of the codes that were chosen
         deq = (q[b].float() - zT[b][g_idx.long()]) * sT[b][g_idx.long()]
         assert torch.allclose(X[b].cpu(), W0[b].float() - deq, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rows_operands_and_diagonal_match_their_definitions(hip, dtype):
+    """The front end of the closed forms: sqrt(2/n) X in solver order, pruned columns zero, in
+    both layouts, and the float64-summed diagonal of (2/n) X^T X, straight from rows that lie
+    end to end in one tensor (ragged counts, a feature count that is no multiple of the tile).
+    Element by element against the definition in float64, rounded once: bit-exact for the
+    operands; the diagonal's sum may be ordered differently, one ulp of f32 is allowed."""
+    g = torch.Generator().manual_seed(3)
+    C, nmax = 200, 96
+    ns = [5, 96, 40, 1]
+    row0 = [7, 20, 130, 0]                                   # not in batch order, with gaps
+    rows = torch.randn(180, C, generator=g).to(dtype)
+    perm = torch.stack([torch.randperm(C, generator=g) for _ in ns])
+    dead = torch.rand(len(ns), C, generator=g) < 0.1
+    root = torch.tensor([(2.0 / n) ** 0.5 for n in ns], dtype=torch.float64)
+    BT, Bp = hip.rows_operands(rows.to(DEV), torch.tensor(row0).to(DEV), torch.tensor(ns, dtype=torch.int32).to(DEV),
+                               root.to(DEV), perm.to(DEV), dead.to(DEV), nmax)
+    _, Bp_only = hip.rows_operands(rows.to(DEV), torch.tensor(row0).to(DEV),
+                                   torch.tensor(ns, dtype=torch.int32).to(DEV), root.to(DEV), perm.to(DEV),
+                                   dead.to(torch.uint8).to(DEV), nmax, want_bt=False)
+    want = torch.zeros(len(ns), nmax, C)
+    for b, n in enumerate(ns):
+        x = rows[row0[b]:row0[b] + n].double()[:, perm[b]] * root[b]
+        want[b, :n] = x.float().masked_fill(dead[b][None, :], 0)
+    assert torch.equal(BT.cpu(), want)
+    assert torch.equal(Bp.cpu(), want.transpose(1, 2)) and torch.equal(Bp_only.cpu(), want.transpose(1, 2))
+    alpha = torch.tensor([2.0 / n for n in ns], dtype=torch.float64)
+    d = hip.rows_diagonal(rows.to(DEV), torch.tensor(row0).to(DEV), torch.tensor(ns, dtype=torch.int32).to(DEV),
+                          alpha.to(DEV)).cpu()
+    ref = torch.stack([(rows[row0[b]:row0[b] + n].double() ** 2).sum(0) * alpha[b] for b, n in enumerate(ns)])
+    assert ((d.double() - ref).abs() <= 6e-8 * ref).all()
+    assert (d == ref.float()).float().mean() > 0.99
+
+
+def test_rows_that_arrive_in_several_updates_and_change_route():
+    """Rows of one expert spread over several update() calls, in f32 and bf16, with experts that
+    move from the per-row-vector form to the blocked form and from there to their Hessian:
+    every expert ends up where the oracle, fed the same rows in the same pieces
+    (forge/gptq.py:61-80), ends up, under the rule of the end-to-end tests."""
+    from forge.moe import ExpertGroupGPTQ
+    from helpers import linear, codes_at_floor
+    g0 = torch.Generator().manual_seed(23)
+    C, R = 1024, 128
+    W = (0.02 * torch.randn(3, R, C, generator=g0)).bfloat16()
+    first = [torch.randn(10, C, generator=g0), torch.randn(50, C, generator=g0), torch.randn(30, C, generator=g0)]
+    later = [torch.randn(30, C, generator=g0).bfloat16(), torch.randn(20, C, generator=g0).bfloat16(),
+             torch.randn(100, C, generator=g0).bfloat16()]
+    first[1] = first[1].bfloat16().float()
+    first[2] = first[2].bfloat16().float()                  # only expert 0's first rows need f32
+    kw = dict(bits=4, group_size=128, symmetric=False, quantization_scale="absmax",
+              quantization_order="activation", rel_damp=0.01)
+    grp = ExpertGroupGPTQ([W.to(DEV)], device=DEV, low_rank_tokens=16, **kw)
+    grp.update(torch.cat(first).to(DEV), [0, 10, 60, 90])
+    assert grp.low_rank == [True, False, False] and grp.rows_route == [False, True, True]
+    grp.prepare()                                           # lays the kept rows end to end; discarded below
+    grp.update(torch.cat(later).to(DEV), [0, 30, 50, 150])
+    # 40 and 70 rows: blocked form (up to 128 rows at 1024 features); 130 rows: through the Hessian
+    assert grp.low_rank == [False] * 3 and grp.rows_route == [True, True, False]
+    X2 = torch.cat([first[2].double(), later[2].double()])
+    H2 = (2.0 / 130) * X2.t() @ X2
+    assert ((grp.hessian(2).cpu().double() - H2).norm() / H2.norm()).item() < 2e-6
+    q = grp.quantize(chunk=3)[0][0].cpu()
+    assert not grp.issue_non_invertible.any()
+    for e in range(3):
+        o = oracle.GPTQ(linear(W[e]), **kw)
+        o.update(first[e])
+        o.update(later[e].float())
+        qo = o.quantize()[0]
+        codes_at_floor(f"expert {e}", qo, q[e], W[e], [torch.cat([first[e], later[e].float()])], kw,
+                       order=o.perm)
