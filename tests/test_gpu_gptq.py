@@ -407,7 +407,7 @@ def test_config5_sparse14_full_size():
 
 @pytest.mark.parametrize("n_tokens", [1536, 200, 128, 40])
 def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
-    """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 256 of
+    """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 512 of
     its 2048 rows, rows being independent, to keep the CPU oracle's sweeps short) with a heavy
     expert's tokens, with 200 (Hessian of rank 200 before damping; the batched front end's default
     route then takes the blocked closed form) and with 128 and 40 (that route then solves from the
@@ -424,7 +424,7 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     from forge.gptq import GPTQ
     from forge.moe import ExpertGroupGPTQ
     g0 = torch.Generator().manual_seed(11)
-    W = synth.fp8_block_roundtrip((0.02 * torch.randn(256, 7168, generator=g0)).bfloat16())
+    W = synth.fp8_block_roundtrip((0.02 * torch.randn(512, 7168, generator=g0)).bfloat16())
     X = torch.randn(1536, 7168, generator=g0).bfloat16()[:n_tokens].contiguous()
     kw = dict(bits=4, group_size=128, symmetric=True, quantization_scale="mse",
               quantization_order="activation", rel_damp=0.01)
@@ -436,6 +436,11 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     bound = max(1e-3, FLOORS * floor)
     Wf = W.float().numpy()
     eo = mathref.layer_error(Wf, oracle.dequantize(qo, so, zo, 128).numpy(), H)
+    # with fewer rows than the group size the error only sees the few directions the rows span
+    # and is driven almost to zero: it then moves by a per cent between equally valid solutions,
+    # the oracle's own float64-stage realisation included
+    e64 = mathref.layer_error(Wf, oracle.dequantize(*out64[:3], 128).numpy(), H)
+    allowed = 0.01 if n_tokens >= 128 else max(0.01, 2 * abs(e64 / eo - 1))
 
     def check(tag, q, s, z):
         q, s, z = q.cpu(), s.cpu(), z.cpu()
@@ -443,8 +448,8 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
         flips, to64 = flip_rate(qo, q), flip_rate(out64[0], q)
         eg = mathref.layer_error(Wf, oracle.dequantize(q, s, z, 128).numpy(), H)
         print(f"config3 n={n_tokens} {tag}: flips vs oracle {flips:.2e}, vs float64 stages {to64:.2e}, "
-              f"floor {floor:.2e}, error ratio {eg / eo:.5f}")
-        assert abs(eg / eo - 1) < 0.01
+              f"floor {floor:.2e}, error ratio {eg / eo:.5f} (the float64-stage oracle's: {e64 / eo:.5f})")
+        assert abs(eg / eo - 1) <= allowed, (tag, eg / eo, e64 / eo)
         assert flips <= bound and to64 <= bound
 
     g = GPTQ(linear(W).to(DEV), device=DEV, **kw)
@@ -461,7 +466,7 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
         # low_rank_tokens=128 the column-by-column form with eight lanes per row of the sweep)
         variants = [("inverse", {}), ("direct", {})] + ([("direct", dict(low_rank_tokens=128))] if n_tokens == 128 else [])
         for route, extra in variants:
-            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 256, 7168)], device=DEV, factor_route=route, **extra, **kw)
+            grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **extra, **kw)
             grp.update(X.to(DEV), [0, n_tokens])
             (q, s, z), = grp.quantize(chunk=1)
             assert not grp.issue_non_invertible.any()
