@@ -17,8 +17,8 @@ output error within 1 % (experts with a handful of rows: within twice what the o
 float64-stage realisation moves by, as in test_expert_group_few_tokens_routes_agree).
 
 The GPU side runs once per module; each parametrised case is one expert's CPU comparison
-(an oracle solve and the realisations of the floor: the factorisations of a 7168 x 7168
-Hessian take most of a minute).
+(an oracle solve and the realisations of the floor, each with its factorisations of a
+7168 x 7168 Hessian: about ten seconds).
 """
 import numpy as np
 import pytest
