@@ -5,9 +5,9 @@ step of the benchmark layer holds: experts without a single routed row (plain ro
 with 3 .. 64 rows (solved from the rows, the sizes of the per-row-vector sweep in ONE mixed
 launch), with 100, 128 and 200 rows (the blocked closed form, sizes 128 and 256 in one batch)
 and with 1536 (through the Hessian).  gate_proj
-and up_proj are two stacks that share one factor (C = 7168; 512 of their 2048 rows each, rows
-being independent); down_proj has its full shape, R = 7168, C = 2048.  The oracle checks a
-regular subset of each expert's rows (every second of gate/up's, every seventh of down's: the
+and up_proj are two stacks of their full shape that share one factor (R = 2048 each, C = 7168);
+down_proj has its full shape too, R = 7168, C = 2048.  The oracle checks a
+regular subset of each expert's rows (every eighth of gate/up's, every seventh of down's: the
 grid is per row and group, the sweep per row, gptq.py:128-139 / solver.cu:9-154), which
 touches every row tile of the kernels and keeps an expert's CPU side to a few seconds.  Every expert is then
 compared with ``oracle.GPTQ`` (forge/gptq.py:128-139 on the handles that quant.py:386-396
@@ -48,7 +48,7 @@ def _rows(seed, C):
 def gate_up():
     from forge.moe import ExpertGroupGPTQ
     g = torch.Generator().manual_seed(31)
-    E, R, C = len(NS), 512, 7168
+    E, R, C = len(NS), 2048, 7168
     W = [torch.stack([synth.fp8_block_roundtrip((0.02 * torch.randn(R, C, generator=g)).bfloat16())
                       for _ in range(E)]) for _ in range(2)]
     xs = _rows(32, C)
@@ -128,7 +128,7 @@ def test_gate_up_expert_against_the_oracle(gate_up, e):
     stacked, with the owner's single damping, as the batched front end defines the unit of work."""
     W, xs, outs, _ = gate_up
     R, G = W[0].shape[1], W[0].shape[2] // 128
-    rows = torch.arange(0, R, 2)
+    rows = torch.arange(0, R, 8)
     pick = lambda t: t[e].view(R, G)[rows].reshape(-1)
     Wst = torch.cat([W[0][e][rows], W[1][e][rows]])
     q = torch.cat([outs[0][0][e][rows], outs[1][0][e][rows]])
