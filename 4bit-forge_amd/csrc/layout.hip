@@ -8,6 +8,15 @@ namespace {
 
 constexpr int64_t kPermuteLdsFloats = 16384;   // 64 KB of LDS per workgroup at most
 
+// First statement of the movers that are meant to run BESIDE the scale search (another stream's
+// kernel that saturates the vector ALU with three wavefronts of 160 registers per SIMD).  Measured
+// on gfx950: a kernel gets onto such a SIMD when its wavefronts need no more than the 32 registers
+// left (16 for two of them), and it makes progress there only when it asks the instruction
+// arbiter for precedence: the older wavefronts of the scale search are ready in nearly every cycle
+// (layout pass beside the search: 14.6 ms one after the other, 14.0 ms together without the
+// priority, 9.5 ms with it, 7.6 ms being the search alone).
+__device__ __forceinline__ void run_beside_the_search() { __builtin_amdgcn_s_setprio(3); }
+
 __device__ __forceinline__ float ld_as_f32(const float* p) { return *p; }
 __device__ __forceinline__ float ld_as_f32(const __hip_bfloat16* p) {
     return __uint_as_float(static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(p)) << 16);
@@ -74,26 +83,36 @@ __global__ __launch_bounds__(256) void to_layer_order_kernel(
 // wavefront moves whole 128..1024-byte runs on both sides, with 4..16 bytes per lane.
 
 // 64 (c) x 256 (r) tile, bf16 in, f32 out.  LDS holds the tile as [c][r] 16-bit words.
+template <bool DEAD, bool XOUT>
 __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw,
     const int64_t* __restrict__ perm_inv, const uint8_t* __restrict__ dead,
     float* __restrict__ Xout, uint16_t* __restrict__ W0out, int64_t R, int64_t C, int64_t ldo,
     int64_t o_stride, const int64_t* __restrict__ index) {
     constexpr int TC = 64, TR = 256, PITCH = TR + 4;     // rows stay 8-byte aligned
-    __shared__ __attribute__((aligned(8))) uint16_t tile[TC][PITCH];
+    // (LDS asked for at launch, not declared: for a kernel whose declared LDS limits its
+    // occupancy the compiler raises the register count in the kernel descriptor to what that
+    // occupancy allows -- 97 for 33 KB -- and the wavefronts no longer fit beside the search's)
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint16_t (*tile)[PITCH] = reinterpret_cast<uint16_t (*)[PITCH]>(lds_raw);
+    run_beside_the_search();
     const int64_t b = blockIdx.z, sb = index ? index[b] : b;
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
     const uint16_t* __restrict__ Wb = W + sb * w_stride;
     {   // 16 lanes x 8 bytes cover one 128-byte row piece.  A lane takes a block of 4 rows x 4
-        // columns, transposes it in registers and stores four rows of r into LDS, 8 bytes each
+        // columns, transposes it in registers and stores four rows of r into LDS, 8 bytes each.
+        // (One pass at a time, and one output row at a time below: 18 registers, which fit into
+        // the 32 that three wavefronts of the scale search leave free on a SIMD.  Two rows at a
+        // time -- 16 registers, two wavefronts beside the search -- moved 22 % less alone and
+        // gained nothing beside it.)
         const int rb = tid >> 4, c4 = (tid & 15) * 4;
         uint32_t keep = 0xF;
-        if (dead) {
+        if constexpr (DEAD) {
             const uint8_t* d = dead + sb * C + c0 + c4;
             keep = (d[0] ? 0u : 1u) | (d[1] ? 0u : 2u) | (d[2] ? 0u : 4u) | (d[3] ? 0u : 8u);
         }
-#pragma unroll
+#pragma unroll 1
         for (int p = 0; p < TR / 64; ++p) {
             const int r = 4 * (16 * p + rb);
             const uint16_t* src = Wb + (r0 + r) * ldw + c0 + c4;
@@ -110,10 +129,12 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
                                   __builtin_amdgcn_perm(v3.y, v2.y, 0x05040100u));
             uint2 o3 = make_uint2(__builtin_amdgcn_perm(v1.y, v0.y, 0x07060302u),    // c4 + 3
                                   __builtin_amdgcn_perm(v3.y, v2.y, 0x07060302u));
-            if (!(keep & 1u)) o0 = make_uint2(0u, 0u);
-            if (!(keep & 2u)) o1 = make_uint2(0u, 0u);
-            if (!(keep & 4u)) o2 = make_uint2(0u, 0u);
-            if (!(keep & 8u)) o3 = make_uint2(0u, 0u);
+            if constexpr (DEAD) {
+                if (!(keep & 1u)) o0 = make_uint2(0u, 0u);
+                if (!(keep & 2u)) o1 = make_uint2(0u, 0u);
+                if (!(keep & 4u)) o2 = make_uint2(0u, 0u);
+                if (!(keep & 8u)) o3 = make_uint2(0u, 0u);
+            }
             *reinterpret_cast<uint2*>(&tile[c4 + 0][r]) = o0;
             *reinterpret_cast<uint2*>(&tile[c4 + 1][r]) = o1;
             *reinterpret_cast<uint2*>(&tile[c4 + 2][r]) = o2;
@@ -123,15 +144,16 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     __syncthreads();
     {   // a wavefront writes the 256 floats (1 KiB) of one output row per instruction
         const int cw = tid >> 6, r4 = (tid & 63) * 4;
-#pragma unroll 4
+#pragma unroll 1
         for (int cc = 0; cc < TC; cc += 4) {
             const int c = cc + cw;
             const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
-            const float4 o = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
-                                         __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
             const int64_t at = b * o_stride + perm_inv[sb * C + c0 + c] * ldo + r0 + r4;
-            if (Xout) *reinterpret_cast<float4*>(Xout + at) = o;
             if (W0out) *reinterpret_cast<uint2*>(W0out + at) = v;
+            if constexpr (XOUT)
+                *reinterpret_cast<float4*>(Xout + at) =
+                    make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
+                                __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
         }
     }
 }
@@ -144,28 +166,33 @@ __global__ __launch_bounds__(256) void to_layer_order_fast_kernel(
     uint8_t* __restrict__ qout, int64_t R, int64_t C, int64_t ldi, int64_t i_stride,
     const int64_t* __restrict__ index) {
     constexpr int TC = 128, TR = 256, PITCH = TR + 4;    // 65 words per row: odd
-    __shared__ __attribute__((aligned(16))) uint8_t tile[TC][PITCH];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];   // (at launch: see above)
+    uint8_t (*tile)[PITCH] = reinterpret_cast<uint8_t (*)[PITCH]>(lds_raw);
+    run_beside_the_search();
     const int64_t b = blockIdx.z, sb = index ? index[b] : b;
     const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
     const int tid = threadIdx.x;
-    {   // 16 lanes x 16 bytes read the 256 bytes of one source row; all eight loads of a lane
-        // are in flight before the first is stored
+    {   // 16 lanes x 16 bytes read the 256 bytes of one source row; four loads of a lane are in
+        // flight before the first is stored (eight would put the kernel beyond 32 registers)
         const int cw = tid >> 4, r16 = (tid & 15) * 16;
-        uint4 v[TC / 16];
+#pragma unroll 1
+        for (int h = 0; h < TC / 64; ++h) {
+            uint4 v[4];
 #pragma unroll
-        for (int p = 0; p < TC / 16; ++p)
-            v[p] = *reinterpret_cast<const uint4*>(
-                qin + b * i_stride + perm_inv[sb * C + c0 + 16 * p + cw] * ldi + r0 + r16);
+            for (int p = 0; p < 4; ++p)
+                v[p] = *reinterpret_cast<const uint4*>(
+                    qin + b * i_stride + perm_inv[sb * C + c0 + 64 * h + 16 * p + cw] * ldi + r0 + r16);
 #pragma unroll
-        for (int p = 0; p < TC / 16; ++p) {
-            uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[16 * p + cw][r16]);   // rows are 4-aligned
-            dst[0] = v[p].x; dst[1] = v[p].y; dst[2] = v[p].z; dst[3] = v[p].w;
+            for (int p = 0; p < 4; ++p) {
+                uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[64 * h + 16 * p + cw][r16]);   // rows are 4-aligned
+                dst[0] = v[p].x; dst[1] = v[p].y; dst[2] = v[p].z; dst[3] = v[p].w;
+            }
         }
     }
     __syncthreads();
     {   // 32 lanes x 4 bytes cover one 128-byte row piece; a lane's block is rows r4 .. r4 + 3
         const int rg = tid >> 5, c4 = (tid & 31) * 4;
-#pragma unroll 2
+#pragma unroll 1
         for (int p = 0; p < TR / 32; ++p) {
             const int r4 = 4 * (8 * p + rg);
             const uint32_t w0 = *reinterpret_cast<const uint32_t*>(&tile[c4 + 0][r4]);
@@ -418,9 +445,15 @@ static int weight_to_solver_order(const void* W, int w_dtype, int64_t w_stride, 
                       (reinterpret_cast<uintptr_t>(W0out) % 8) == 0;
     if (fast) {
         const dim3 tiles((unsigned)(C / 64), (unsigned)(R / 256), (unsigned)batch);
-        to_solver_order_bf16_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(
-            (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, (uint16_t*)W0out, R, C, ldo, o_stride,
-            index);
+        constexpr size_t kLds = 64 * 260 * sizeof(uint16_t);
+#define FORGE_W2S(DEAD, XOUT)                                                                        \
+    to_solver_order_bf16_kernel<DEAD, XOUT><<<tiles, dim3(256), kLds, (hipStream_t)stream>>>(       \
+        (const uint16_t*)W, w_stride, ldw, perm_inv, dead, Xout, (uint16_t*)W0out, R, C, ldo, o_stride, index)
+        if (dead && Xout) FORGE_W2S(true, true);
+        else if (dead) FORGE_W2S(true, false);
+        else if (Xout) FORGE_W2S(false, true);
+        else FORGE_W2S(false, false);
+#undef FORGE_W2S
     } else if (w_dtype == FORGE_F32) {
         to_solver_order_kernel<float><<<grid, dim3(256), 0, (hipStream_t)stream>>>(
             (const float*)W, w_stride, ldw, perm_inv, dead, Xout, (float*)W0out, R, C, ldo, o_stride, index);
@@ -485,7 +518,7 @@ static int codes_to_layer_order(const uint8_t* qin, int64_t ldi, int64_t i_strid
                       (reinterpret_cast<uintptr_t>(qout) % 4) == 0 && (ldi % 16) == 0 && (i_stride % 16) == 0;
     if (fast) {
         const dim3 tiles((unsigned)(C / 128), (unsigned)(R / 256), (unsigned)batch);
-        to_layer_order_fast_kernel<<<tiles, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C,
+        to_layer_order_fast_kernel<<<tiles, dim3(256), 128 * 260, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C,
                                                                                  ldi, i_stride, index);
     } else {
         to_layer_order_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(qin, perm_inv, qout, R, C, ldi,
@@ -622,7 +655,9 @@ __global__ __launch_bounds__(256) void rows_operands_kernel(
     const double* __restrict__ root, const int64_t* __restrict__ perm,
     const uint8_t* __restrict__ dead, float* __restrict__ BT, float* __restrict__ Bp, int64_t C,
     int64_t nmax) {
-    __shared__ float tile[32][33];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];   // (at launch, as above)
+    float (*tile)[33] = reinterpret_cast<float (*)[33]>(lds_raw);
+    run_beside_the_search();
     const int64_t b = blockIdx.z;
     const int64_t j0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
@@ -655,6 +690,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void rows_diagonal_kernel(
     const T* __restrict__ rows, const int64_t* __restrict__ row0, const int32_t* __restrict__ n,
     const double* __restrict__ alpha, float* __restrict__ out, int64_t C) {
+    run_beside_the_search();
     const int64_t b = blockIdx.y;
     const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
@@ -683,10 +719,10 @@ extern "C" int forge_rows_operands(const void* rows, int x_dtype, const int64_t*
     forge::KernelTiming timing("rows_operands", st, (BT ? 8.0 : 4.0) * batch * nmax * C, forge::WORK_BYTES);
     const dim3 grid((unsigned)forge::ceil_div(C, 32), (unsigned)forge::ceil_div(nmax, 32), (unsigned)batch);
     if (x_dtype == FORGE_BF16)
-        rows_operands_kernel<__hip_bfloat16><<<grid, dim3(256), 0, st>>>(
+        rows_operands_kernel<__hip_bfloat16><<<grid, dim3(256), 32 * 33 * sizeof(float), st>>>(
             (const __hip_bfloat16*)rows, row0, n, root, perm, dead, BT, Bp, C, nmax);
     else
-        rows_operands_kernel<float><<<grid, dim3(256), 0, st>>>((const float*)rows, row0, n, root, perm,
+        rows_operands_kernel<float><<<grid, dim3(256), 32 * 33 * sizeof(float), st>>>((const float*)rows, row0, n, root, perm,
                                                                 dead, BT, Bp, C, nmax);
     FORGE_LAUNCH_CHECK();
     return FORGE_OK;

@@ -168,17 +168,21 @@ template <int GS, int Q, bool FLOOR, bool REFQ>
 __device__ __forceinline__ float quarter_loss(const float (&v)[GS], float s, float rcp, float q0,
                                               float maxq, float norm) {
     constexpr int VPL = GS / 32;
-    float p[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    auto lane_sum = [&](int j) {
         const int l = Q + 4 * j;
         // (the reference starts from 0 and adds: the same value, every term being >= +0)
         float loss = element_loss<FLOOR, REFQ>(v[l], s, rcp, q0, maxq, norm);
 #pragma unroll
         for (int i = 1; i < VPL; ++i) loss += element_loss<FLOOR, REFQ>(v[l + 32 * i], s, rcp, q0, maxq, norm);
-        p[j] = loss;
-    }
-    return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+        return loss;
+    };
+    // the two halves of the tree one after the other: four lane sums in flight instead of eight
+    // (the registers that saves are what lets small kernels of other streams share a SIMD with
+    // three wavefronts of this one)
+    const float even = (lane_sum(0) + lane_sum(4)) + (lane_sum(2) + lane_sum(6));
+    __builtin_amdgcn_sched_barrier(0);
+    const float odd = (lane_sum(1) + lane_sum(5)) + (lane_sum(3) + lane_sum(7));
+    return even + odd;
 }
 
 // Loss of one candidate in the reference's summation order (32 lane sums, then the
@@ -203,11 +207,14 @@ __device__ __forceinline__ float candidate_loss(const float (&v)[GS], float s, f
 
 // One lane per group.  FUSED: derive (sg, q0g) from the group's own extrema first;
 // otherwise read them from scales/qzeros (the reference's two-call protocol).
-template <typename T, int GS, bool FUSED, bool FLOOR, bool REFQ>
+// SYM: symmetric grids as a compile-time fact: the zero point (maxq + 1) / 2 and what derives
+// from it are then the same for every lane and live in scalar registers.
+template <typename T, int GS, bool FUSED, bool FLOOR, bool REFQ, bool SYM>
 __global__ __launch_bounds__(64) void mse_grid_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, int64_t G,
     int64_t n_groups, const float* __restrict__ cand, int P, float maxq, float norm,
-    bool symmetric, bool search, float* __restrict__ scales, float* __restrict__ qzeros) {
+    bool search, float* __restrict__ scales, float* __restrict__ qzeros) {
+    constexpr bool symmetric = SYM;
     // lanes past the end replay the last group (the wavefront votes together below)
     const int64_t g_raw = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t g = g_raw < n_groups ? g_raw : n_groups - 1;
@@ -346,15 +353,18 @@ int launch_mse(const T* W, int64_t w_stride, int64_t R, int64_t C, int64_t ldw, 
     const bool floor_needed = !(norm >= 2.3f);
     const bool refq = forge::option(forge::OPT_MSE_REFERENCE_QUANTISER) != 0;
 #define FORGE_MSE_LAUNCH(GS, FL, RQ)                                                          \
-    mse_grid_kernel<T, GS, FUSED, FL, RQ><<<grid, block, 0, st>>>(                            \
-        W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, symmetric, search,     \
-        scales, qzeros)
+    if (symmetric)                                                                            \
+        mse_grid_kernel<T, GS, FUSED, FL, RQ, true><<<grid, block, 0, st>>>(                  \
+            W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, search, scales, qzeros); \
+    else                                                                                      \
+        mse_grid_kernel<T, GS, FUSED, FL, RQ, false><<<grid, block, 0, st>>>(                 \
+            W, w_stride, R, C, ldw, G, n_groups, cand, (int)P, maxq, norm, search, scales, qzeros)
 #define FORGE_MSE_CASE(GS)                                                                    \
     case GS:                                                                                  \
-        if (floor_needed && refq) FORGE_MSE_LAUNCH(GS, true, true);                           \
-        else if (floor_needed) FORGE_MSE_LAUNCH(GS, true, false);                             \
-        else if (refq) FORGE_MSE_LAUNCH(GS, false, true);                                     \
-        else FORGE_MSE_LAUNCH(GS, false, false);                                              \
+        if (floor_needed && refq) { FORGE_MSE_LAUNCH(GS, true, true); }                       \
+        else if (floor_needed) { FORGE_MSE_LAUNCH(GS, true, false); }                         \
+        else if (refq) { FORGE_MSE_LAUNCH(GS, false, true); }                                 \
+        else { FORGE_MSE_LAUNCH(GS, false, false); }                                          \
         break;
     switch (gs) {
         FORGE_MSE_CASE(32)

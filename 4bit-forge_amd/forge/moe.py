@@ -604,9 +604,11 @@ class ExpertGroupGPTQ:
                             perm[li], mask[li], nr, want_bt=False, out=Bpv)
                         dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[li], 1, perm[li]))
                         D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
+                        # (the layout pass ahead of the factor: it runs beside the scale search,
+                        # which the factor's kernels, with their many registers, wait out)
+                        layout_in(ids, W0[pos:pos + len(ids)], skip_out=True)
                         kernels.lowrank_factor(Bpv, D.contiguous(),
                                                out=(Hm_all[span].view(len(ids), C, nr), info[pos:pos + len(ids)]))
-                        layout_in(ids, W0[pos:pos + len(ids)], skip_out=True)
                         pos += len(ids)
                         at += len(ids) * C * nr
                     # ---------------------------------------------------- blocked closed form
@@ -625,12 +627,12 @@ class ExpertGroupGPTQ:
                             perm_r, mask[ri], nmax)
                         dp = torch.where(msk, torch.ones((), device=dev), torch.gather(diag[ri], 1, perm_r))
                         D = (float(self.rel_damp) * dp.mean(dim=1))[:, None] + msk.float()
-                        HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows, n_pad)
-                        del BT
-                        failed.append((torch.tensor([e0 + i for i in rr_ids]), info_r))
                         Xr = torch.empty((len(rr_ids), C, R), dtype=torch.float32, device=dev)
                         W0r = torch.empty((len(rr_ids), C, R), dtype=self.W[job[0]].dtype, device=dev)
                         layout_in(rr_ids, W0r, Xr)
+                        HmT, V, info_r = kernels.rows_factor_blocked(BT, D.contiguous(), n_rows, n_pad)
+                        del BT
+                        failed.append((torch.tensor([e0 + i for i in rr_ids]), info_r))
                     if lr_ids or none_ids or rr_ids:
                         lr_stream.wait_stream(search)
                         for t in (scales, qzeros, sT, zT) + tuple(x for p in parts for x in p):
@@ -663,6 +665,18 @@ class ExpertGroupGPTQ:
                     di = None if whole else self._dev(dn_ids)
                     pick = (lambda t: t) if whole else (lambda t: t[di].contiguous())
                     Bd = len(dn_ids)
+                    X = torch.empty((Bd, C, R), dtype=torch.float32, device=dev)
+                    # the displacement form also reads the untouched weights: the layout pass writes
+                    # them a second time in their own type instead of X being copied afterwards
+                    W0 = None
+                    if direct and len({self.W[i].dtype for i in job}) == 1:
+                        W0 = torch.empty((Bd, C, R), dtype=self.W[job[0]].dtype, device=dev)
+                    # where every column block is first written by its long product, that product
+                    # starts from W0 and X is not laid out at all
+                    band = direct and not babai and kernels.sweep_direct_reads_band_only(Bd, C, R)
+                    lazy_x = W0 is not None and band
+                    # (ahead of the factorisation: see the closed forms above)
+                    layout_in(dn_ids, W0, X, skip_out=lazy_x)
                     # the factorisations read their input's lower triangle in 128 x 128 blocks only
                     slots = [self._slot[e0 + i] for i in dn_ids]
                     if slots == list(range(e0, e1)) and self._Hpool.shape[0] >= e1:
@@ -687,7 +701,6 @@ class ExpertGroupGPTQ:
                         L, info = kernels.chol_reverse_lower_batched(Hp, damp)
                         # the sweep's long products read V straight from L's rows; where that covers
                         # everything beyond one block of the diagonal, only that band of V is written
-                        band = kernels.sweep_direct_reads_band_only(Bd, C, R)
                         U = kernels.unit_upper_from_lower(L, info, negate=True, upper_only=True, band=band)
                         if sparse:
                             # 1/diag(U) of the mask score (solver_sparsegptq14.cu:153) is the
@@ -707,16 +720,6 @@ class ExpertGroupGPTQ:
                         U, _, info = kernels.chol_inv_upper_batched(Hp, damp, normalise=True, upper_only=True)
                     del Hp
                     failed.append((torch.tensor([e0 + i for i in dn_ids]), info))
-                    X = torch.empty((Bd, C, R), dtype=torch.float32, device=dev)
-                    # the displacement form also reads the untouched weights: the layout pass writes
-                    # them a second time in their own type instead of X being copied afterwards
-                    W0 = None
-                    if direct and len({self.W[i].dtype for i in job}) == 1:
-                        W0 = torch.empty((Bd, C, R), dtype=self.W[job[0]].dtype, device=dev)
-                    # where every column block is first written by its long product, that product
-                    # starts from W0 and X is not laid out at all
-                    lazy_x = W0 is not None and band
-                    layout_in(dn_ids, W0, X, skip_out=lazy_x)
                     main.wait_stream(search)
                     for t in (scales, qzeros, sT, zT):
                         t.record_stream(main)

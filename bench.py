@@ -577,7 +577,12 @@ def main():
     chunk = a.chunk or cfg["chunk"]
     wl = make_workload(a.config, cfg, chunk)
     mse = not a.no_mse
-    STREAMS.extend(torch.cuda.Stream() for _ in range(2 * a.split))   # default priority
+    # A process has four hardware queues for all of its streams, the default stream included, and
+    # kernels of streams that share a queue run one after the other.  The library brings two
+    # streams of its own (scale searches; closed-form experts): the gate/up job takes the default
+    # stream, the down job one new stream, so that each of the four has a queue to itself.
+    STREAMS.append(torch.cuda.current_stream())
+    STREAMS.extend(torch.cuda.Stream() for _ in range(2 * a.split - 1))   # default priority
 
     if a.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
