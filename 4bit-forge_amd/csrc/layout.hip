@@ -102,17 +102,18 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     const uint16_t* __restrict__ Wb = W + sb * w_stride;
     {   // 16 lanes x 8 bytes cover one 128-byte row piece.  A lane takes a block of 4 rows x 4
         // columns, transposes it in registers and stores four rows of r into LDS, 8 bytes each.
-        // (One pass at a time, and one output row at a time below: 18 registers, which fit into
-        // the 32 that three wavefronts of the scale search leave free on a SIMD.  Two rows at a
-        // time -- 16 registers, two wavefronts beside the search -- moved 22 % less alone and
-        // gained nothing beside it.)
+        // (Two passes in flight, and two output rows at a time below: 26 registers, which fit
+        // into the 32 that three wavefronts of the scale search leave free on a SIMD; all four
+        // passes in flight need 48 and gain 4 % alone.  Two rows x four columns per lane -- 16
+        // registers, two wavefronts beside the search -- moved 22 % less alone and gained nothing
+        // beside it.)
         const int rb = tid >> 4, c4 = (tid & 15) * 4;
         uint32_t keep = 0xF;
         if constexpr (DEAD) {
             const uint8_t* d = dead + sb * C + c0 + c4;
             keep = (d[0] ? 0u : 1u) | (d[1] ? 0u : 2u) | (d[2] ? 0u : 4u) | (d[3] ? 0u : 8u);
         }
-#pragma unroll 1
+#pragma unroll 2
         for (int p = 0; p < TR / 64; ++p) {
             const int r = 4 * (16 * p + rb);
             const uint16_t* src = Wb + (r0 + r) * ldw + c0 + c4;
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(256) void to_solver_order_bf16_kernel(
     __syncthreads();
     {   // a wavefront writes the 256 floats (1 KiB) of one output row per instruction
         const int cw = tid >> 6, r4 = (tid & 63) * 4;
-#pragma unroll 1
+#pragma unroll 2
         for (int cc = 0; cc < TC; cc += 4) {
             const int c = cc + cw;
             const uint2 v = *reinterpret_cast<const uint2*>(&tile[c][r4]);
