@@ -51,6 +51,16 @@ NO_SCRATCH = (
 )
 
 
+# Register ceilings that the step's schedule relies on (see csrc/layout.hip, csrc/quant_grid.hip):
+# three wavefronts of the scale search must leave 32 registers free on a SIMD, and the kernels that
+# are meant to run beside it must fit into those.
+MAX_VGPRS = (
+    (re.compile(r"mse_grid_kernel<\w+, \d+, "), 160),
+    ("to_solver_order_bf16_kernel", 32), ("to_layer_order_fast_kernel", 32),
+    ("rows_operands_kernel", 32), ("rows_diagonal_kernel", 32),
+)
+
+
 def sources():
     return sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
 
@@ -151,6 +161,12 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
                and (u["scratch"] or u["vgpr_spill"])]
     if spilled:
         raise RuntimeError("kernels that must stay in registers use scratch memory:\n  " + "\n  ".join(spilled))
+    wide = [f"{f}: {k} ({u['vgprs']} > {lim})"
+            for f, ks in sorted(table.items()) for k, u in sorted(ks.items())
+            for n, lim in MAX_VGPRS
+            if (n.search(k) if hasattr(n, "search") else n in k) and u["vgprs"] > lim]
+    if wide:
+        raise RuntimeError("kernels beyond their register ceiling:\n  " + "\n  ".join(wide))
     if PROBE_SRC.exists() and (force or _stale(PROBE_OUT, [PROBE_SRC])):
         cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", str(PROBE_SRC), "-o", str(PROBE_OUT)]
