@@ -176,7 +176,7 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
             raise RuntimeError("hipcc failed on the bench probe")
         if verbose:
             print(f"[build] built {PROBE_OUT}")
-    if todo or force or not OUT.exists():
+    if todo or force or _stale(OUT, objs):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(OUT), *map(str, objs)]
         subprocess.run(cmd, check=True)
         if verbose:
