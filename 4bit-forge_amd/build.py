@@ -57,7 +57,7 @@ NO_SCRATCH = (
 MAX_VGPRS = (
     (re.compile(r"mse_grid_kernel<\w+, \d+, "), 160),
     ("to_solver_order_bf16_kernel", 32), ("to_layer_order_fast_kernel", 32),
-    ("rows_operands_kernel", 32), ("rows_diagonal_kernel", 32),
+    ("rows_operands_kernel", 32), ("rows_diagonal_kernel", 32), ("round_to_nearest_bf16x8_kernel", 32),
 )
 
 

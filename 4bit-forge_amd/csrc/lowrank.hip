@@ -572,6 +572,35 @@ __global__ __launch_bounds__(256) void lowrank_sweep_kernel(
 // A layer that saw no rows at all has H = I (gptq.py:97-99): nothing couples its columns and the
 // sweep is the quantiser applied to every weight, in whatever order.  Layer layout in, layer
 // layout out; a thread takes eight consecutive columns of a row.
+// The same for bf16 weights whose rows, groups and addresses are multiples of eight columns: a
+// thread's eight columns lie in one group, one 16-byte load and one 8-byte store.  Few enough
+// registers (and the wave priority) to run beside another stream's scale search.
+__global__ __launch_bounds__(256) void round_to_nearest_bf16x8_kernel(
+    const uint16_t* __restrict__ W, int64_t w_stride, int64_t ldw, const float* __restrict__ scales,
+    const float* __restrict__ qzeros, uint8_t* __restrict__ q, int64_t R, int64_t C, uint32_t gs,
+    int64_t G, float maxq, const int64_t* __restrict__ index) {
+    __builtin_amdgcn_s_setprio(3);
+    const uint32_t c0 = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    if ((int64_t)c0 >= C) return;
+    const int64_t b = index ? index[blockIdx.z] : blockIdx.z;
+    const uint32_t g = c0 / gs;
+#pragma unroll 1
+    for (int64_t r = blockIdx.y; r < R; r += gridDim.y) {
+        const uint4 w = *reinterpret_cast<const uint4*>(W + b * w_stride + r * ldw + c0);
+        const float s = scales[(b * R + r) * G + g], z = qzeros[(b * R + r) * G + g];
+        const float rcp = 1.0f / (s + kEps);
+        auto code = [&](uint32_t bits) {
+            return (uint32_t)__builtin_amdgcn_fmed3f(
+                __builtin_rintf(__builtin_fmaf(__uint_as_float(bits), rcp, z)), 0.0f, maxq);
+        };
+        const uint32_t lo = code(w.x << 16) | (code(w.x & 0xffff0000u) << 8) | (code(w.y << 16) << 16) |
+                            (code(w.y & 0xffff0000u) << 24);
+        const uint32_t hi = code(w.z << 16) | (code(w.z & 0xffff0000u) << 8) | (code(w.w << 16) << 16) |
+                            (code(w.w & 0xffff0000u) << 24);
+        *reinterpret_cast<uint2*>(q + (b * R + r) * C + c0) = make_uint2(lo, hi);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void round_to_nearest_kernel(
     const T* __restrict__ W, int64_t w_stride, int64_t ldw, const float* __restrict__ scales,
@@ -650,7 +679,13 @@ extern "C" int forge_round_to_nearest(const void* W, int w_dtype, int64_t w_stri
     forge::KernelTiming timing("round_to_nearest", st,
                                (double)batch * R * C * ((w_dtype == FORGE_BF16 ? 2.0 : 4.0) + 1.0),
                                forge::WORK_BYTES);
-    if (w_dtype == FORGE_BF16)
+    const bool x8 = w_dtype == FORGE_BF16 && C % 8 == 0 && gs % 8 == 0 && ldw % 8 == 0 && w_stride % 8 == 0 &&
+                    (reinterpret_cast<uintptr_t>(W) & 15u) == 0 && (reinterpret_cast<uintptr_t>(qweight) & 7u) == 0 &&
+                    gs < (1LL << 31);
+    if (x8)
+        round_to_nearest_bf16x8_kernel<<<grid, block, 0, st>>>((const uint16_t*)W, w_stride, ldw, scales, qzeros,
+                                                               qweight, R, C, (uint32_t)gs, G, maxq, index);
+    else if (w_dtype == FORGE_BF16)
         round_to_nearest_kernel<uint16_t><<<grid, block, 0, st>>>((const uint16_t*)W, w_stride, ldw, scales,
                                                                   qzeros, qweight, R, C, gs, G, maxq, index);
     else
