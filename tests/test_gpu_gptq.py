@@ -405,15 +405,14 @@ def test_config5_sparse14_full_size():
     assert torch.equal(words, want)
 
 
-@pytest.mark.parametrize("n_tokens", [1536, 200, 128, 40])
+@pytest.mark.parametrize("n_tokens", [1536, 200, 128, 100, 40])
 def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     """DeepSeek-V3-shaped gate_proj (C = 7168, fp8 block round trip, act-order, MSE; 512 of
     its 2048 rows, rows being independent, to keep the CPU oracle's sweeps short) with a heavy
     expert's tokens, with 200 (Hessian of rank 200 before damping; the batched front end's default
     route then takes the blocked closed form) and with 128 and 40 (that route then solves from the
-    rows themselves, column by column: at 65-128 rows with four threads per row of the factor's
-    recurrence and eight lanes per row of the sweep, at 40 with one; 100 rows:
-    test_gpu_bench_step).  At
+    rows themselves, column by column: at 65-128 rows, i.e. 100 and 128 here, with four threads per
+    row of the factor's recurrence and eight lanes per row of the sweep, at 40 with one).  At
     this size the
     problem is ill conditioned: the oracle's own codes move by 1-2 % between two valid fp32
     realisations of its library stages (the floor).  Three GPU routes are held to that floor
@@ -462,9 +461,9 @@ def test_config3_all_routes_against_the_oracle_at_full_shape(n_tokens):
     # it, so that this is the arithmetic the benchmark times
     kernels.set_option("sweep_schedule", 1)
     try:
-        # (128 rows: the default takes the blocked closed form from 65 rows on; with
+        # (100 and 128 rows: the default takes the blocked closed form from 65 rows on; with
         # low_rank_tokens=128 the column-by-column form with eight lanes per row of the sweep)
-        variants = [("inverse", {}), ("direct", {})] + ([("direct", dict(low_rank_tokens=128))] if n_tokens == 128 else [])
+        variants = [("inverse", {}), ("direct", {})] + ([("direct", dict(low_rank_tokens=128))] if n_tokens in (100, 128) else [])
         for route, extra in variants:
             grp = ExpertGroupGPTQ([W.to(DEV).view(1, 512, 7168)], device=DEV, factor_route=route, **extra, **kw)
             grp.update(X.to(DEV), [0, n_tokens])
